@@ -1,0 +1,96 @@
+/*
+ * C ABI of the MI355X (gfx950) fused LM-head log-probability path.
+ *
+ * One shared library, plain pointers and sizes, no C++ or torch types in any signature.  Every device
+ * pointer is memory the caller owns (in practice a torch tensor's data_ptr()); the library never frees or
+ * keeps it after the call returns.  All work is enqueued asynchronously on the HIP stream passed in
+ * (hipStream_t as void*, NULL = the default stream).  The library allocates nothing: scratch comes in as
+ * `workspace`, sized by the two *_workspace_bytes queries, so a caller can observe that no T x V buffer exists.
+ *
+ * Math (T tokens, H hidden, V vocab; z = (hidden . weight^T) * rcp_temperature):
+ *     lse_t      = log sum_v exp z_tv
+ *     logprob_t  = z_{t,label_t} - lse_t            (0 when label_t is outside [0, V))
+ *     pz_t       = sum_v softmax(z_t)_v * z_tv
+ *     entropy_t  = lse_t - pz_t
+ *     dz_tv      = ( g_t * (1[v == label_t] - p_tv) - q_t * p_tv * (z_tv - pz_t) ) * rcp_temperature
+ *     d_hidden   = dz . weight     (bf16)            d_weight = dz^T . hidden   (fp32)
+ * with g = dlogprobs, q = dentropy.  dz is rounded to bf16 once before the two gradient GEMMs, as the
+ * reference does (model_utils.py:413); all accumulation is fp32.
+ *
+ * Reference interfaces these entry points stand in for (paths under the SkyRL tree,
+ * skyrl/backends/skyrl_train/distributed/megatron/):
+ *   skyrl_lmhead_fwd  <- efficient_entropy_forward            fused_linear_logprob_triton.py:614-803
+ *                        FusedLinearChunkedDistributedLogprob.forward            model_utils.py:302-359
+ *                        _fused_vocab_parallel_entropy_from_hidden               model_utils.py:1090-1121
+ *   skyrl_lmhead_bwd  <- efficient_entropy_backward           fused_linear_logprob_triton.py:1541-1753
+ *                        FusedLinearChunkedDistributedLogprob.backward           model_utils.py:361-428
+ *
+ * Status codes: 0 = ok; negative = argument error detected before anything was enqueued (table below);
+ * positive = a hipError_t returned by the HIP runtime.
+ */
+#ifndef SKYRL_LMHEAD_H
+#define SKYRL_LMHEAD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SKYRL_LMHEAD_OK 0
+#define SKYRL_LMHEAD_ERR_NULL (-1)      /* a required pointer is NULL */
+#define SKYRL_LMHEAD_ERR_SHAPE (-2)     /* T, V < 1, H not a positive multiple of 64, or a leading dimension < H */
+#define SKYRL_LMHEAD_ERR_ALIGN (-3)     /* a pointer is not 16-byte aligned or a leading dimension is not a multiple of 8 */
+#define SKYRL_LMHEAD_ERR_WORKSPACE (-4) /* workspace is NULL or smaller than the matching *_workspace_bytes() */
+#define SKYRL_LMHEAD_ERR_ARG (-5)       /* rcp_temperature not finite and positive, or vocab_chunk not a multiple of 256 */
+
+/* ABI version of this header (bumped on any signature change). */
+int skyrl_lmhead_version(void);
+
+/* Human-readable text for a status code returned by this library (never NULL). */
+const char* skyrl_lmhead_strerror(int status);
+
+/* Scratch needed by skyrl_lmhead_fwd: per-vocab-tile (max, sum-exp, sum z*exp) partials, 24 * T * ceil(V/256) bytes
+ * plus alignment slack.  (The reference allocates the same kind of buffers: `_max/_accu/_entropy_b [T, num_splits]`,
+ * fused_linear_logprob_triton.py:670-672.) */
+size_t skyrl_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V);
+
+/* Scratch needed by skyrl_lmhead_bwd for a given vocab chunk width (0 = library default):
+ * weight^T bf16 [H, V'], hidden^T bf16 [H, T'], an fp32 dHidden accumulator [T, H] and two bf16 dz panels
+ * [T', chunk] / [chunk, T'] (T', V' = T, V rounded up to 256).  Nothing in it scales with T * V.
+ * (Stands in for the `d_logits [T, 9504]` scratch of the reference's default backward,
+ * fused_linear_logprob_triton.py:1689-1748.) */
+size_t skyrl_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t vocab_chunk);
+
+/*
+ * Forward.  hidden: bf16 [T, ld_hidden]; weight: bf16 [V, ld_weight]; labels: int64 [T] (a value outside [0, V),
+ * e.g. INT64_MAX, means "no target": logprob 0, no one-hot term in backward).
+ * Outputs, all fp32 [T]: logprobs (required); entropy, row_lse, row_pz (each may be NULL).
+ * row_lse (and row_pz when an entropy gradient will be applied) are what skyrl_lmhead_bwd needs back.
+ * If entropy and row_pz are both NULL the sum p*z accumulation is skipped entirely.
+ */
+int skyrl_lmhead_fwd(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight,
+                     const int64_t* labels, int64_t T, int64_t H, int64_t V, float rcp_temperature,
+                     float* logprobs, float* entropy, float* row_lse, float* row_pz,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Backward.  Same hidden / weight / labels as the forward call; row_lse, row_pz from it (row_pz may be NULL
+ * iff dentropy is NULL); dlogprobs fp32 [T] (required), dentropy fp32 [T] or NULL.
+ * d_hidden: bf16 [T, H] contiguous, overwritten.  d_weight: fp32 [V, H] contiguous, overwritten, or added to
+ * when accumulate_dw != 0 (gradient accumulation across micro-batches).  Both gradients are with respect to
+ * the unscaled weight / hidden: the 1/temperature factor is already applied.
+ * vocab_chunk: width of the dz panel in vocab columns (multiple of 256; 0 = library default).
+ */
+int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight,
+                     const int64_t* labels, const float* row_lse, const float* row_pz,
+                     const float* dlogprobs, const float* dentropy,
+                     int64_t T, int64_t H, int64_t V, float rcp_temperature,
+                     void* d_hidden, float* d_weight, int accumulate_dw, int64_t vocab_chunk,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SKYRL_LMHEAD_H */

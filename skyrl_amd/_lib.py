@@ -1,0 +1,88 @@
+"""ctypes binding of the C-ABI library (``include/skyrl_lmhead.h``).
+
+The library is loaded from the source tree (``skyrl_amd/csrc/libskyrl_lmhead.so``).  There is no fallback: if it has not
+been built, or the symbol table does not match the header, loading raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libskyrl_lmhead.so")
+ABI_VERSION = 1
+
+_c_i64 = ctypes.c_int64
+_c_p = ctypes.c_void_p
+
+# name -> (restype, argtypes); mirrors include/skyrl_lmhead.h one to one.
+SIGNATURES = {
+    "skyrl_lmhead_version": (ctypes.c_int, []),
+    "skyrl_lmhead_strerror": (ctypes.c_char_p, [ctypes.c_int]),
+    "skyrl_lmhead_fwd_workspace_bytes": (ctypes.c_size_t, [_c_i64, _c_i64, _c_i64]),
+    "skyrl_lmhead_bwd_workspace_bytes": (ctypes.c_size_t, [_c_i64, _c_i64, _c_i64, _c_i64]),
+    "skyrl_lmhead_fwd": (
+        ctypes.c_int,
+        [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_i64, _c_i64, ctypes.c_float, _c_p, _c_p, _c_p, _c_p, _c_p,
+         ctypes.c_size_t, _c_p],
+    ),
+    "skyrl_lmhead_bwd": (
+        ctypes.c_int,
+        [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, ctypes.c_float, _c_p, _c_p,
+         ctypes.c_int, _c_i64, _c_p, ctypes.c_size_t, _c_p],
+    ),
+}
+
+_lock = threading.Lock()
+_lib = None
+
+
+class LmHeadLibraryError(RuntimeError):
+    """The HIP library is missing, stale, or returned a non-zero status."""
+
+
+def lib_path() -> str:
+    return _LIB_PATH
+
+
+def load() -> ctypes.CDLL:
+    """Load (once) and return the library.  Raises LmHeadLibraryError when it is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(_LIB_PATH):
+            raise LmHeadLibraryError(
+                f"{_LIB_PATH} is not built. Run `python -m skyrl_amd.csrc.build` (needs hipcc, targets gfx950). "
+                "There is no non-HIP fallback for the fused LM-head path."
+            )
+        lib = ctypes.CDLL(_LIB_PATH)
+        for name, (restype, argtypes) in SIGNATURES.items():
+            try:
+                fn = getattr(lib, name)
+            except AttributeError as exc:
+                raise LmHeadLibraryError(f"{_LIB_PATH} does not export {name}; rebuild it") from exc
+            fn.restype = restype
+            fn.argtypes = argtypes
+        got = lib.skyrl_lmhead_version()
+        if got != ABI_VERSION:
+            raise LmHeadLibraryError(f"{_LIB_PATH} has ABI version {got}, this package expects {ABI_VERSION}; rebuild it")
+        _lib = lib
+        return lib
+
+
+def strerror(status: int) -> str:
+    return load().skyrl_lmhead_strerror(int(status)).decode("utf-8", "replace")
+
+
+def check(status: int, what: str) -> None:
+    """Turn a non-zero status into an exception (argument errors -> ValueError, HIP errors -> LmHeadLibraryError)."""
+    if status == 0:
+        return
+    msg = f"{what} failed with status {status}: {strerror(status)}"
+    if status < 0:
+        raise ValueError(msg)
+    raise LmHeadLibraryError(msg)

@@ -1,0 +1,586 @@
+// HIP kernels (gfx950) and C-ABI entry points of the fused LM-head log-probability path.
+//
+// Forward  (2*T*V*H flop):
+//   lmhead_fwd_tiles   one 256(vocab) x 256(token) logits tile per workgroup: bf16 MFMA GEMM, then in registers
+//                      scale by 1/temperature, per-token max / sum-exp / sum z*exp over the tile's vocab rows;
+//                      writes one (max, sum, pz) partial per token per 128-row half tile.  Logits never leave VGPRs.
+//   lmhead_fwd_merge   per token: merges the partials (online log-sum-exp), gathers the label logit with an
+//                      fp32 dot product hidden[t] . weight[label], writes logprob / entropy / lse / pz.
+// Backward (6*T*V*H flop), looped over vocab chunks of `vocab_chunk` columns:
+//   transpose_bf16     weight^T and hidden^T once per call, so that every contraction is K-contiguous.
+//   lmhead_bwd_dz_tiles recomputes a logits tile and forms dz in registers; writes it (bf16) row-major and
+//                      transposed into two chunk-sized panels.
+//   gemm_nt_store      dHidden (+)= dz . weight   and   dW[chunk] = dz^T . hidden, fp32 accumulation.
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdint.h>
+
+#include "../../include/skyrl_lmhead.h"
+#include "gemm_core.hpp"
+
+using namespace lmhead;
+
+namespace {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr int kGroupM = 8;
+
+__host__ __device__ inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+
+// ------------------------------------------------------------------------------------------------------------
+// Forward tile kernel.  M axis = vocab (A = weight), N axis = tokens (B = hidden).
+// Online softmax statistics follow efficient_entropy_kernel_general_mainloop
+// (fused_linear_logprob_triton.py:296-385): scale, running max, sum exp, sum z*exp; vocab rows past V take no part.
+// The label-logit gather of that kernel (:364-385) is done in lmhead_fwd_merge instead.
+// ------------------------------------------------------------------------------------------------------------
+template <bool ENTROPY, bool MASKED>
+__device__ __forceinline__ void fwd_tile_stats(acc_t& acc, int j, int vbase, int V, float scale2, int khalf, float& m_out,
+                                               float& s_out, float& e_out) {
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      float z2 = acc[i][j][r] * scale2;
+      if (MASKED) {
+        const int v = vbase + i * 32 + (r >> 2) * 8 + khalf * 4 + (r & 3);
+        if (v >= V) z2 = -INFINITY;
+      }
+      acc[i][j][r] = z2;
+      mx = fmaxf(mx, z2);
+    }
+  mx = fmaxf(mx, shfl_xor32(mx));  // finite: the wave has at least one row below V
+  float s = 0.f, e = 0.f;
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float z2 = acc[i][j][r];
+      const float p = __builtin_amdgcn_exp2f(z2 - mx);
+      s += p;
+      if (ENTROPY) {
+        float zz = z2;
+        if (MASKED) zz = (z2 == -INFINITY) ? 0.f : z2;
+        e = fmaf(zz, p, e);
+      }
+    }
+  s += shfl_xor32(s);
+  if (ENTROPY) e += shfl_xor32(e);
+  m_out = mx * kLn2;
+  s_out = s;
+  e_out = e * kLn2;
+}
+
+template <bool ENTROPY>
+__global__ __launch_bounds__(NTHREADS) void lmhead_fwd_tiles(const uint16_t* __restrict__ W, int ldw,
+                                                             const uint16_t* __restrict__ Hd, int ldh, int T, int H, int V,
+                                                             float rcp_temp, float* __restrict__ part_max,
+                                                             float* __restrict__ part_sum, float* __restrict__ part_pz) {
+  __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
+  const int tiles_m = (V + BM - 1) / BM;
+  const int tiles_n = (T + BN - 1) / BN;
+  int tm, tn;
+  tile_coords(blockIdx.x, tiles_m, tiles_n, kGroupM, tm, tn);
+
+  Operand a{W, ldw, tm * BM, V};
+  Operand b{Hd, ldh, tn * BN, T};
+  acc_t acc;
+  zero_acc(acc);
+  mainloop(a, b, 0, H / BK, lds, acc);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int lrow = lane & 31, khalf = lane >> 5;
+  const int vbase = tm * BM + wm * WM;
+  const size_t part = (size_t)(tm * WAVES_M + wm) * (size_t)T;
+  const float scale2 = rcp_temp * kLog2e;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int t = tn * BN + wn * WN + j * 32 + lrow;
+    float m = -INFINITY, s = 0.f, e = 0.f;
+    if (vbase + WM <= V) {
+      fwd_tile_stats<ENTROPY, false>(acc, j, vbase, V, scale2, khalf, m, s, e);
+    } else if (vbase < V) {
+      fwd_tile_stats<ENTROPY, true>(acc, j, vbase, V, scale2, khalf, m, s, e);
+    }
+    if (khalf == 0 && t < T) {
+      part_max[part + t] = m;
+      part_sum[part + t] = s;
+      if (ENTROPY) part_pz[part + t] = e;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// Forward merge.  32 tokens per workgroup of 256 threads.
+// Merge algebra as in efficient_entropy_triton_kernel_epilogue (fused_linear_logprob_triton.py:417-467) except that
+// the running max starts at -inf (that kernel starts it at 0, which loses rows whose logits are all << 0).
+// Out-of-range labels give logprob 0 (model_utils.py:337; fused_linear_logprob_triton.py:1898-1905).
+// ------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void lmhead_fwd_merge(const float* __restrict__ part_max, const float* __restrict__ part_sum,
+                                                        const float* __restrict__ part_pz, int nparts, int T,
+                                                        const uint16_t* __restrict__ Hd, int ldh,
+                                                        const uint16_t* __restrict__ W, int ldw,
+                                                        const int64_t* __restrict__ labels, int H, int V, float rcp_temp,
+                                                        float* __restrict__ logprobs, float* __restrict__ entropy,
+                                                        float* __restrict__ row_lse, float* __restrict__ row_pz) {
+  __shared__ float sm_m[8][32], sm_s[8][32], sm_e[8][32];
+  __shared__ float sm_lse[32], sm_pz[32];
+  const int tid = threadIdx.x;
+  {
+    const int tl = tid & 31, grp = tid >> 5;
+    const int t = blockIdx.x * 32 + tl;
+    float M = -INFINITY, S = 0.f, E = 0.f;
+    if (t < T) {
+      for (int p = grp; p < nparts; p += 8) {
+        const size_t idx = (size_t)p * (size_t)T + t;
+        const float m = part_max[idx];
+        if (m > -INFINITY) {
+          const float s = part_sum[idx];
+          const float e = part_pz ? part_pz[idx] : 0.f;
+          const float Mn = fmaxf(M, m);
+          const float ca = expf(M - Mn), cb = expf(m - Mn);
+          S = S * ca + s * cb;
+          E = E * ca + e * cb;
+          M = Mn;
+        }
+      }
+    }
+    sm_m[grp][tl] = M;
+    sm_s[grp][tl] = S;
+    sm_e[grp][tl] = E;
+    __syncthreads();
+    if (grp == 0) {
+      float Mg = -INFINITY;
+#pragma unroll
+      for (int g = 0; g < 8; ++g) Mg = fmaxf(Mg, sm_m[g][tl]);
+      float Sg = 0.f, Eg = 0.f;
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {
+        const float m = sm_m[g][tl];
+        if (m > -INFINITY) {
+          const float c = expf(m - Mg);
+          Sg += sm_s[g][tl] * c;
+          Eg += sm_e[g][tl] * c;
+        }
+      }
+      sm_lse[tl] = Mg + logf(Sg);
+      sm_pz[tl] = Eg / Sg;
+    }
+    __syncthreads();
+  }
+  // Label logit: 8 lanes per token, 16-byte loads, fp32 accumulation.
+  const int tl = tid >> 3, sub = tid & 7;
+  const int t = blockIdx.x * 32 + tl;
+  float dot = 0.f;
+  bool has_label = false;
+  if (t < T) {
+    const int64_t y = labels[t];
+    has_label = (y >= 0 && y < (int64_t)V);
+    if (has_label) {
+      const uint16_t* hp = Hd + (size_t)t * (size_t)ldh;
+      const uint16_t* wp = W + (size_t)y * (size_t)ldw;
+      for (int c = sub * 8; c < H; c += 64) {
+        const uint4 hv = *(const uint4*)(hp + c);
+        const uint4 wv = *(const uint4*)(wp + c);
+        const uint32_t hh[4] = {hv.x, hv.y, hv.z, hv.w};
+        const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          dot = fmaf(__uint_as_float(hh[k] << 16), __uint_as_float(ww[k] << 16), dot);
+          dot = fmaf(__uint_as_float(hh[k] & 0xffff0000u), __uint_as_float(ww[k] & 0xffff0000u), dot);
+        }
+      }
+    }
+  }
+  dot += __shfl_xor(dot, 1, 64);
+  dot += __shfl_xor(dot, 2, 64);
+  dot += __shfl_xor(dot, 4, 64);
+  if (sub == 0 && t < T) {
+    const float lse = sm_lse[tl], pz = sm_pz[tl];
+    logprobs[t] = has_label ? dot * rcp_temp - lse : 0.f;
+    if (entropy) entropy[t] = lse - pz;
+    if (row_lse) row_lse[t] = lse;
+    if (row_pz) row_pz[t] = pz;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// Backward dz producer.  Same tile as the forward; the epilogue is purely element-wise because the row
+// statistics come from the forward pass.  Formula of efficient_entropy_backward_kernel_general_d_logits_split_N
+// (fused_linear_logprob_triton.py:1402-1538, the arithmetic is at :947-957 of the fused variant):
+//     p  = exp(z - lse);   dz = ( g*(onehot - p) - q*p*(z - pz) ) / temperature
+// written as  p * (c0 + c1*x) + onehot*g/temperature  with x the raw dot product.
+// Out-of-range labels get no one-hot term but keep -p*g (model_utils.py:405-411).
+// ------------------------------------------------------------------------------------------------------------
+template <bool ENTGRAD>
+__global__ __launch_bounds__(NTHREADS) void lmhead_bwd_dz_tiles(
+    const uint16_t* __restrict__ W, int ldw, const uint16_t* __restrict__ Hd, int ldh, int T, int H, int V, float rcp_temp,
+    const int64_t* __restrict__ labels, const float* __restrict__ row_lse, const float* __restrict__ row_pz,
+    const float* __restrict__ dlogprobs, const float* __restrict__ dentropy, int vc0, int tiles_m, int tiles_n,
+    uint16_t* __restrict__ D, int ldd, uint16_t* __restrict__ DT, int lddt) {
+  __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
+  int tm, tn;
+  tile_coords(blockIdx.x, tiles_m, tiles_n, kGroupM, tm, tn);
+
+  Operand a{W, ldw, vc0 + tm * BM, V};
+  Operand b{Hd, ldh, tn * BN, T};
+  acc_t acc;
+  zero_acc(acc);
+  mainloop(a, b, 0, H / BK, lds, acc);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int lrow = lane & 31, khalf = lane >> 5;
+  const int vloc_base = tm * BM + wm * WM;    // first vocab row of this wave inside the chunk panel
+  const int vbase = vc0 + vloc_base;          // ... and in the full vocab
+  const bool full = vbase + WM <= V;
+  const float scale2 = rcp_temp * kLog2e;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int t = tn * BN + wn * WN + j * 32 + lrow;  // < tiles_n * 256 = padded T: always inside the panels
+    const bool valid = t < T;
+    const float g = valid ? dlogprobs[t] : 0.f;
+    const float q = (ENTGRAD && valid) ? dentropy[t] : 0.f;
+    const float lse2 = valid ? row_lse[t] * kLog2e : INFINITY;
+    const float pz = (ENTGRAD && valid) ? row_pz[t] : 0.f;
+    const int64_t y = valid ? labels[t] : (int64_t)-1;
+    const int64_t yrel64 = y - (int64_t)vbase;
+    const int yrel = (y >= 0 && y < (int64_t)V && yrel64 >= 0 && yrel64 < WM) ? (int)yrel64 : -1;
+    const float gs = g * rcp_temp;
+    const float c0 = -(g - q * pz) * rcp_temp;
+    const float c1 = -q * rcp_temp * rcp_temp;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      float d[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float x = acc[i][j][r];
+        const float p = __builtin_amdgcn_exp2f(fmaf(x, scale2, -lse2));
+        d[r] = ENTGRAD ? p * fmaf(c1, x, c0) : p * c0;
+      }
+      const int rel = yrel - i * 32;
+      const bool hit = (yrel >= 0) && ((unsigned)rel < 32u);
+      if (__any(hit)) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row_r = (r >> 2) * 8 + khalf * 4 + (r & 3);
+          if (hit && rel == row_r) d[r] += gs;
+        }
+      }
+      if (!full) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int v = vbase + i * 32 + (r >> 2) * 8 + khalf * 4 + (r & 3);
+          if (v >= V) d[r] = 0.f;
+        }
+      }
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        const int vl = vloc_base + i * 32 + rg * 8 + khalf * 4;
+        f32x4 v4 = {d[rg * 4 + 0], d[rg * 4 + 1], d[rg * 4 + 2], d[rg * 4 + 3]};
+        const bf16x4 b4 = __builtin_convertvector(v4, bf16x4);
+        *(bf16x4*)(D + (size_t)t * (size_t)ldd + vl) = b4;
+        const uint16_t* bits = (const uint16_t*)&b4;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) DT[(size_t)(vl + k) * (size_t)lddt + t] = bits[k];
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// Plain NT GEMM with an fp32 / bf16 store epilogue:  C[M,N] (+)= A[M,K] . B[N,K]^T.
+//   load_c     add the existing fp32 C before storing (accumulation across vocab chunks / micro-batches)
+//   Cf != 0    store fp32;   Cb != 0  store bf16 (round-to-nearest-even)
+// ------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(NTHREADS) void gemm_nt_store(const uint16_t* __restrict__ A, int lda, int a_rows,
+                                                          const uint16_t* __restrict__ B, int ldb, int b_rows, int nk,
+                                                          int M, int N, const float* __restrict__ Cin, float* __restrict__ Cf,
+                                                          uint16_t* __restrict__ Cb, int ldc) {
+  __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
+  const int tiles_m = (M + BM - 1) / BM;
+  const int tiles_n = (N + BN - 1) / BN;
+  int tm, tn;
+  tile_coords(blockIdx.x, tiles_m, tiles_n, kGroupM, tm, tn);
+  Operand a{A, lda, tm * BM, a_rows};
+  Operand b{B, ldb, tn * BN, b_rows};
+  acc_t acc;
+  zero_acc(acc);
+  mainloop(a, b, 0, nk, lds, acc);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int lrow = lane & 31, khalf = lane >> 5;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int n = tn * BN + wn * WN + j * 32 + lrow;
+    if (n >= N) continue;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = tm * BM + wm * WM + i * 32 + (r >> 2) * 8 + khalf * 4 + (r & 3);
+        if (m < M) {
+          const size_t idx = (size_t)m * (size_t)ldc + n;
+          float v = acc[i][j][r];
+          if (Cin) v += Cin[idx];
+          if (Cf) Cf[idx] = v;
+          if (Cb) {
+            const __bf16 bv = (__bf16)v;
+            Cb[idx] = *(const uint16_t*)&bv;
+          }
+        }
+      }
+  }
+}
+
+// dst[c, r] = src[r, c] for r < R, c < C;  dst[c, r] = 0 for R <= r < Rpad.  bf16 bits, 64 x 64 tiles.
+__global__ __launch_bounds__(256) void transpose_bf16(const uint16_t* __restrict__ src, int lds_src, int R, int C,
+                                                      uint16_t* __restrict__ dst, int ld_dst, int Rpad) {
+  __shared__ uint16_t tile[64][66];
+  const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
+  const int tid = threadIdx.x;
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    const int idx = it * 256 + tid;  // 512 chunks of 8 elements
+    const int rr = idx >> 3, cc = (idx & 7) * 8;
+    const int r = r0 + rr, c = c0 + cc;
+    uint16_t v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (r < R) {
+      if (c + 8 <= C) {
+        const uint4 q = *(const uint4*)(src + (size_t)r * (size_t)lds_src + c);
+        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          v[2 * k] = (uint16_t)(w[k] & 0xffffu);
+          v[2 * k + 1] = (uint16_t)(w[k] >> 16);
+        }
+      } else {
+        for (int k = 0; k < 8; ++k)
+          if (c + k < C) v[k] = src[(size_t)r * (size_t)lds_src + c + k];
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) tile[rr][cc + k] = v[k];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    const int idx = it * 256 + tid;
+    const int cc = idx >> 3, rr = (idx & 7) * 8;  // output row = source column
+    const int c = c0 + cc, r = r0 + rr;
+    if (c < C && r < Rpad) {
+      uint32_t w[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) w[k] = (uint32_t)tile[rr + 2 * k][cc] | ((uint32_t)tile[rr + 2 * k + 1][cc] << 16);
+      *(uint4*)(dst + (size_t)c * (size_t)ld_dst + r) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// Host side
+// ------------------------------------------------------------------------------------------------------------
+struct Carver {
+  char* base;
+  size_t off = 0;
+  explicit Carver(void* p) : base((char*)p) {}
+  template <typename T>
+  T* take(size_t count) {
+    off = (size_t)round_up((int64_t)off, 256);
+    T* p = base ? (T*)(base + off) : nullptr;
+    off += count * sizeof(T);
+    return p;
+  }
+};
+
+inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+int check_common(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
+                 int64_t H, int64_t V, float rcp_temperature) {
+  if (!hidden || !weight || !labels) return SKYRL_LMHEAD_ERR_NULL;
+  if (T < 1 || V < 1 || H < BK || H % BK != 0 || ldh < H || ldw < H) return SKYRL_LMHEAD_ERR_SHAPE;
+  if (T > (int64_t)1 << 30 || V > (int64_t)1 << 30 || ldh > (int64_t)1 << 30 || ldw > (int64_t)1 << 30)
+    return SKYRL_LMHEAD_ERR_SHAPE;
+  if (!aligned16(hidden) || !aligned16(weight) || ((uintptr_t)labels & 7u) || ldh % 8 != 0 || ldw % 8 != 0)
+    return SKYRL_LMHEAD_ERR_ALIGN;
+  if (!(rcp_temperature > 0.f) || !isfinite(rcp_temperature)) return SKYRL_LMHEAD_ERR_ARG;
+  return SKYRL_LMHEAD_OK;
+}
+
+int64_t default_vocab_chunk(int64_t T, int64_t V) {
+  const int64_t Tpad = round_up(T, 256), Vpad = round_up(V, 256);
+  int64_t vc = ((int64_t)1 << 28) / Tpad / 256 * 256;  // ~512 MiB of bf16 per dz panel
+  if (vc < 2048) vc = 2048;
+  if (vc > Vpad) vc = Vpad;
+  return vc;
+}
+
+struct BwdWorkspace {
+  uint16_t *Wt, *Ht, *D, *DT;
+  float* dHacc;
+  size_t bytes;
+};
+
+BwdWorkspace carve_bwd(void* ws, int64_t T, int64_t H, int64_t V, int64_t vc) {
+  const int64_t Tpad = round_up(T, 256), Vpad = round_up(V, 256);
+  Carver c(ws);
+  BwdWorkspace w;
+  w.Wt = c.take<uint16_t>((size_t)H * Vpad);
+  w.Ht = c.take<uint16_t>((size_t)H * Tpad);
+  w.dHacc = c.take<float>((size_t)T * H);
+  w.D = c.take<uint16_t>((size_t)Tpad * vc);
+  w.DT = c.take<uint16_t>((size_t)vc * Tpad);
+  w.bytes = (size_t)round_up((int64_t)c.off, 256);
+  return w;
+}
+
+hipError_t launch_gemm(hipStream_t s, const uint16_t* A, int64_t lda, int64_t a_rows, const uint16_t* B, int64_t ldb,
+                       int64_t b_rows, int64_t nk, int64_t M, int64_t N, const float* Cin, float* Cf, uint16_t* Cb,
+                       int64_t ldc) {
+  const unsigned tiles = (unsigned)(((M + BM - 1) / BM) * ((N + BN - 1) / BN));
+  hipLaunchKernelGGL(gemm_nt_store, dim3(tiles), dim3(NTHREADS), 0, s, A, (int)lda, (int)a_rows, B, (int)ldb, (int)b_rows,
+                     (int)nk, (int)M, (int)N, Cin, Cf, Cb, (int)ldc);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+extern "C" {
+
+int skyrl_lmhead_version(void) { return 1; }
+
+const char* skyrl_lmhead_strerror(int status) {
+  switch (status) {
+    case SKYRL_LMHEAD_OK: return "ok";
+    case SKYRL_LMHEAD_ERR_NULL: return "a required pointer is NULL";
+    case SKYRL_LMHEAD_ERR_SHAPE: return "bad shape: need T >= 1, V >= 1, H a positive multiple of 64, leading dimensions >= H";
+    case SKYRL_LMHEAD_ERR_ALIGN: return "bad alignment: pointers must be 16-byte aligned, leading dimensions multiples of 8";
+    case SKYRL_LMHEAD_ERR_WORKSPACE: return "workspace is NULL or too small";
+    case SKYRL_LMHEAD_ERR_ARG: return "bad argument: rcp_temperature must be finite and > 0, vocab_chunk a multiple of 256";
+    default: break;
+  }
+  if (status > 0) return hipGetErrorString((hipError_t)status);
+  return "unknown skyrl_lmhead status";
+}
+
+size_t skyrl_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
+  (void)H;
+  if (T < 1 || V < 1) return 0;
+  const size_t nparts = (size_t)((V + BM - 1) / BM) * WAVES_M;
+  Carver c(nullptr);
+  c.take<float>(nparts * (size_t)T);
+  c.take<float>(nparts * (size_t)T);
+  c.take<float>(nparts * (size_t)T);
+  return (size_t)round_up((int64_t)c.off, 256);
+}
+
+size_t skyrl_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t vocab_chunk) {
+  if (T < 1 || V < 1 || H < 1 || vocab_chunk < 0 || vocab_chunk % 256 != 0) return 0;
+  int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(T, V);
+  if (vc > round_up(V, 256)) vc = round_up(V, 256);
+  return carve_bwd(nullptr, T, H, V, vc).bytes;
+}
+
+int skyrl_lmhead_fwd(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight, const int64_t* labels,
+                     int64_t T, int64_t H, int64_t V, float rcp_temperature, float* logprobs, float* entropy,
+                     float* row_lse, float* row_pz, void* workspace, size_t workspace_bytes, void* stream) {
+  int st = check_common(hidden, ld_hidden, weight, ld_weight, labels, T, H, V, rcp_temperature);
+  if (st) return st;
+  if (!logprobs) return SKYRL_LMHEAD_ERR_NULL;
+  if (!workspace || workspace_bytes < skyrl_lmhead_fwd_workspace_bytes(T, H, V)) return SKYRL_LMHEAD_ERR_WORKSPACE;
+  if ((uintptr_t)workspace & 255u) return SKYRL_LMHEAD_ERR_ALIGN;
+
+  hipStream_t s = (hipStream_t)stream;
+  const int tiles_m = (int)((V + BM - 1) / BM), tiles_n = (int)((T + BN - 1) / BN);
+  const size_t nparts = (size_t)tiles_m * WAVES_M;
+  Carver c(workspace);
+  float* pmax = c.take<float>(nparts * (size_t)T);
+  float* psum = c.take<float>(nparts * (size_t)T);
+  float* ppz = c.take<float>(nparts * (size_t)T);
+  const bool want_pz = entropy || row_pz;
+  const uint16_t* Wp = (const uint16_t*)weight;
+  const uint16_t* Hp = (const uint16_t*)hidden;
+  const dim3 grid((unsigned)(tiles_m * tiles_n)), block(NTHREADS);
+  if (want_pz)
+    hipLaunchKernelGGL(lmhead_fwd_tiles<true>, grid, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)T, (int)H,
+                       (int)V, rcp_temperature, pmax, psum, ppz);
+  else
+    hipLaunchKernelGGL(lmhead_fwd_tiles<false>, grid, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)T, (int)H,
+                       (int)V, rcp_temperature, pmax, psum, ppz);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return (int)e;
+  hipLaunchKernelGGL(lmhead_fwd_merge, dim3((unsigned)((T + 31) / 32)), dim3(256), 0, s, pmax, psum,
+                     want_pz ? ppz : (float*)nullptr, (int)nparts, (int)T, Hp, (int)ld_hidden, Wp, (int)ld_weight, labels,
+                     (int)H, (int)V, rcp_temperature, logprobs, entropy, row_lse, row_pz);
+  e = hipGetLastError();
+  return e == hipSuccess ? SKYRL_LMHEAD_OK : (int)e;
+}
+
+int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight, const int64_t* labels,
+                     const float* row_lse, const float* row_pz, const float* dlogprobs, const float* dentropy, int64_t T,
+                     int64_t H, int64_t V, float rcp_temperature, void* d_hidden, float* d_weight, int accumulate_dw,
+                     int64_t vocab_chunk, void* workspace, size_t workspace_bytes, void* stream) {
+  int st = check_common(hidden, ld_hidden, weight, ld_weight, labels, T, H, V, rcp_temperature);
+  if (st) return st;
+  if (!row_lse || !dlogprobs || !d_hidden || !d_weight) return SKYRL_LMHEAD_ERR_NULL;
+  if (dentropy && !row_pz) return SKYRL_LMHEAD_ERR_NULL;
+  if (!aligned16(d_hidden) || !aligned16(d_weight)) return SKYRL_LMHEAD_ERR_ALIGN;
+  if (vocab_chunk < 0 || vocab_chunk % 256 != 0) return SKYRL_LMHEAD_ERR_ARG;
+  const int64_t Tpad = round_up(T, 256), Vpad = round_up(V, 256);
+  int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(T, V);
+  if (vc > Vpad) vc = Vpad;
+  if (!workspace || workspace_bytes < skyrl_lmhead_bwd_workspace_bytes(T, H, V, vc)) return SKYRL_LMHEAD_ERR_WORKSPACE;
+  if ((uintptr_t)workspace & 255u) return SKYRL_LMHEAD_ERR_ALIGN;
+
+  hipStream_t s = (hipStream_t)stream;
+  const BwdWorkspace w = carve_bwd(workspace, T, H, V, vc);
+  const uint16_t* Wp = (const uint16_t*)weight;
+  const uint16_t* Hp = (const uint16_t*)hidden;
+  hipError_t e;
+
+  // weight^T [H, Vpad] and hidden^T [H, Tpad], zero in the padding columns.
+  hipLaunchKernelGGL(transpose_bf16, dim3((unsigned)(Vpad / 64), (unsigned)(H / 64)), dim3(256), 0, s, Wp, (int)ld_weight,
+                     (int)V, (int)H, w.Wt, (int)Vpad, (int)Vpad);
+  hipLaunchKernelGGL(transpose_bf16, dim3((unsigned)(Tpad / 64), (unsigned)(H / 64)), dim3(256), 0, s, Hp, (int)ld_hidden,
+                     (int)T, (int)H, w.Ht, (int)Tpad, (int)Tpad);
+  if ((e = hipGetLastError()) != hipSuccess) return (int)e;
+
+  const int tiles_t = (int)(Tpad / 256);
+  const int tiles_h = (int)((H + 255) / 256);
+  const int64_t nchunks = (Vpad + vc - 1) / vc;
+  for (int64_t ci = 0; ci < nchunks; ++ci) {
+    const int64_t vc0 = ci * vc;
+    const int64_t vcw = (Vpad - vc0) < vc ? (Vpad - vc0) : vc;  // multiple of 256
+    const int tiles_v = (int)(vcw / 256);
+    const dim3 grid_dz((unsigned)(tiles_v * tiles_t)), block(NTHREADS);
+    if (dentropy)
+      hipLaunchKernelGGL(lmhead_bwd_dz_tiles<true>, grid_dz, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)T,
+                         (int)H, (int)V, rcp_temperature, labels, row_lse, row_pz, dlogprobs, dentropy, (int)vc0, tiles_v,
+                         tiles_t, w.D, (int)vcw, w.DT, (int)Tpad);
+    else
+      hipLaunchKernelGGL(lmhead_bwd_dz_tiles<false>, grid_dz, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)T,
+                         (int)H, (int)V, rcp_temperature, labels, row_lse, row_pz, dlogprobs, dentropy, (int)vc0, tiles_v,
+                         tiles_t, w.D, (int)vcw, w.DT, (int)Tpad);
+    if ((e = hipGetLastError()) != hipSuccess) return (int)e;
+
+    // dHidden[T, H] (+)= D[T, vcw] . weight[vc0 : vc0 + vcw, :]    (B operand = weight^T rows, k offset vc0)
+    const bool first = ci == 0, last = ci == nchunks - 1;
+    e = launch_gemm(s, w.D, vcw, Tpad, w.Wt + vc0, Vpad, H, vcw / BK, T, H,
+                    first ? (const float*)nullptr : (const float*)w.dHacc, last ? (float*)nullptr : w.dHacc,
+                    last ? (uint16_t*)d_hidden : (uint16_t*)nullptr, H);
+    if (e != hipSuccess) return (int)e;
+
+    // dW[vc0 : vc0 + rows, :] (+)= D^T[vcw, Tpad] . hidden   (B operand = hidden^T rows)
+    const int64_t rows = (V - vc0) < vcw ? (V - vc0) : vcw;
+    float* dWc = d_weight + (size_t)vc0 * (size_t)H;
+    e = launch_gemm(s, w.DT, Tpad, vcw, w.Ht, Tpad, H, Tpad / BK, rows, H,
+                    accumulate_dw ? (const float*)dWc : (const float*)nullptr, dWc, (uint16_t*)nullptr, H);
+    if (e != hipSuccess) return (int)e;
+  }
+  return SKYRL_LMHEAD_OK;
+}
+
+}  // extern "C"

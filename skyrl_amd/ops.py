@@ -1,0 +1,202 @@
+"""torch.library custom ops over the C ABI: ``skyrl_amd::lmhead_fwd`` and ``skyrl_amd::lmhead_bwd``.
+
+These are the only two places Python touches the HIP kernels.  Tensors stay torch-owned; the ops pass raw device
+pointers, sizes and the current HIP stream through ctypes.  Scratch is a torch ``uint8`` tensor sized by the library's
+own ``*_workspace_bytes`` query, so ``torch.cuda.max_memory_allocated`` sees every byte the path uses.
+
+Shapes: hidden ``[T, H]`` bf16 (row stride a multiple of 8), weight ``[V, H]`` bf16, labels ``[T]`` int64 (a value
+outside ``[0, V)`` means "no target": logprob 0 and no one-hot term in the gradient, which is how the reference treats
+targets outside the vocab shard, model_utils.py:314-337, 405-411).
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+__all__ = ["lmhead_fwd", "lmhead_bwd", "fwd_workspace_bytes", "bwd_workspace_bytes"]
+
+
+def _require_device(*tensors: torch.Tensor) -> torch.device:
+    dev = tensors[0].device
+    if dev.type != "cuda":
+        raise RuntimeError(
+            "skyrl_amd fused LM-head ops run only on a ROCm GPU (device type 'cuda'); got a tensor on "
+            f"'{dev}'. There is no CPU implementation of this path."
+        )
+    for t in tensors:
+        if t.device != dev:
+            raise RuntimeError(f"all tensors must be on {dev}, got one on {t.device}")
+    return dev
+
+
+def _check_operands(hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor) -> Tuple[int, int, int]:
+    if hidden.dim() != 2 or weight.dim() != 2 or labels.dim() != 1:
+        raise ValueError(f"expected hidden [T,H], weight [V,H], labels [T]; got {tuple(hidden.shape)}, "
+                         f"{tuple(weight.shape)}, {tuple(labels.shape)}")
+    if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise TypeError(f"the HIP path computes in bf16: hidden and weight must be torch.bfloat16, got {hidden.dtype} and "
+                        f"{weight.dtype} (cast explicitly if a down-cast is intended)")
+    if labels.dtype != torch.int64:
+        raise TypeError(f"labels must be int64, got {labels.dtype}")
+    T, H = hidden.shape
+    V, H2 = weight.shape
+    if H != H2 or labels.shape[0] != T:
+        raise ValueError(f"shape mismatch: hidden {tuple(hidden.shape)}, weight {tuple(weight.shape)}, labels {tuple(labels.shape)}")
+    if hidden.stride(1) != 1 or weight.stride(1) != 1 or not labels.is_contiguous():
+        raise ValueError("hidden and weight must have unit stride in the last dimension and labels must be contiguous")
+    return int(T), int(H), int(V)
+
+
+def fwd_workspace_bytes(T: int, H: int, V: int) -> int:
+    return int(_lib.load().skyrl_lmhead_fwd_workspace_bytes(T, H, V))
+
+
+def bwd_workspace_bytes(T: int, H: int, V: int, vocab_chunk: int = 0) -> int:
+    return int(_lib.load().skyrl_lmhead_bwd_workspace_bytes(T, H, V, vocab_chunk))
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+@torch.library.custom_op("skyrl_amd::lmhead_fwd", mutates_args=())
+def lmhead_fwd(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    rcp_temperature: float,
+    want_entropy: bool,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Returns ``(logprobs, entropy, row_lse, row_pz)``, each fp32 ``[T]``.
+
+    With ``want_entropy=False`` the sum p*z accumulation is skipped and ``entropy`` / ``row_pz`` come back empty (0 elements).
+    """
+    T, H, V = _check_operands(hidden, weight, labels)
+    dev = _require_device(hidden, weight, labels)
+    lib = _lib.load()
+    f32 = dict(dtype=torch.float32, device=dev)
+    logprobs = torch.empty(T, **f32)
+    row_lse = torch.empty(T, **f32)
+    entropy = torch.empty(T if want_entropy else 0, **f32)
+    row_pz = torch.empty(T if want_entropy else 0, **f32)
+    ws_bytes = int(lib.skyrl_lmhead_fwd_workspace_bytes(T, H, V))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        st = lib.skyrl_lmhead_fwd(
+            hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), labels.data_ptr(), T, H, V,
+            float(rcp_temperature), logprobs.data_ptr(), _ptr(entropy if want_entropy else None), row_lse.data_ptr(),
+            _ptr(row_pz if want_entropy else None), ws.data_ptr(), ws_bytes, stream,
+        )
+    _lib.check(st, "skyrl_lmhead_fwd")
+    return logprobs, entropy, row_lse, row_pz
+
+
+@lmhead_fwd.register_fake
+def _(hidden, weight, labels, rcp_temperature, want_entropy):
+    T = hidden.shape[0]
+    f32 = dict(dtype=torch.float32, device=hidden.device)
+    n = T if want_entropy else 0
+    return torch.empty(T, **f32), torch.empty(n, **f32), torch.empty(T, **f32), torch.empty(n, **f32)
+
+
+@torch.library.custom_op("skyrl_amd::lmhead_bwd", mutates_args=())
+def lmhead_bwd(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    row_lse: torch.Tensor,
+    row_pz: Optional[torch.Tensor],
+    dlogprobs: torch.Tensor,
+    dentropy: Optional[torch.Tensor],
+    rcp_temperature: float,
+    vocab_chunk: int,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Returns ``(d_hidden bf16 [T,H], d_weight fp32 [V,H])``."""
+    T, H, V = _check_operands(hidden, weight, labels)
+    dev = _require_device(hidden, weight, labels, row_lse, dlogprobs)
+    lib = _lib.load()
+    d_hidden = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    d_weight = torch.empty((V, H), dtype=torch.float32, device=dev)
+    _bwd_into(lib, hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk, d_hidden,
+              d_weight, False)
+    return d_hidden, d_weight
+
+
+def _bwd_into(lib, hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk, d_hidden,
+              d_weight, accumulate_dw: bool) -> None:
+    T, H = hidden.shape
+    V = weight.shape[0]
+    dev = hidden.device
+    if dentropy is not None and (row_pz is None or row_pz.numel() != T):
+        raise ValueError("an entropy gradient needs row_pz from a forward call made with want_entropy=True")
+    for name, t in (("row_lse", row_lse), ("dlogprobs", dlogprobs), ("row_pz", row_pz), ("dentropy", dentropy)):
+        if t is None:
+            continue
+        if name == "row_pz" and dentropy is None:
+            continue
+        if t.dtype != torch.float32 or t.shape != (T,) or not t.is_contiguous():
+            raise ValueError(f"{name} must be a contiguous fp32 tensor of shape [{T}], got {t.dtype} {tuple(t.shape)}")
+    ws_bytes = int(lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, int(vocab_chunk)))
+    if ws_bytes == 0:
+        raise ValueError(f"bad vocab_chunk {vocab_chunk}: must be 0 (library default) or a multiple of 256")
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        st = lib.skyrl_lmhead_bwd(
+            hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), labels.data_ptr(),
+            row_lse.data_ptr(), _ptr(row_pz if dentropy is not None else None), dlogprobs.data_ptr(), _ptr(dentropy),
+            T, H, V, float(rcp_temperature), d_hidden.data_ptr(), d_weight.data_ptr(), int(bool(accumulate_dw)),
+            int(vocab_chunk), ws.data_ptr(), ws_bytes, stream,
+        )
+    _lib.check(st, "skyrl_lmhead_bwd")
+
+
+def lmhead_bwd_accumulate(hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature: float,
+                          d_weight_accum: torch.Tensor, vocab_chunk: int = 0) -> torch.Tensor:
+    """Backward that *adds* dW into an existing fp32 ``[V, H]`` buffer (Megatron's ``main_grad`` style accumulation
+    across micro-batches, the role of ``grad_weight.add_`` at model_utils.py:425) and returns ``d_hidden``."""
+    T, H, V = _check_operands(hidden, weight, labels)
+    dev = _require_device(hidden, weight, labels, row_lse, dlogprobs, d_weight_accum)
+    if d_weight_accum.dtype != torch.float32 or d_weight_accum.shape != (V, H) or not d_weight_accum.is_contiguous():
+        raise ValueError(f"d_weight_accum must be contiguous fp32 [{V},{H}]")
+    d_hidden = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    _bwd_into(_lib.load(), hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk,
+              d_hidden, d_weight_accum, True)
+    return d_hidden
+
+
+@lmhead_bwd.register_fake
+def _(hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk):
+    return (torch.empty_like(hidden, memory_format=torch.contiguous_format),
+            torch.empty(weight.shape, dtype=torch.float32, device=weight.device))
+
+
+def _setup_context(ctx, inputs, output):
+    hidden, weight, labels, rcp_temperature, want_entropy = inputs
+    _, _, row_lse, row_pz = output
+    ctx.save_for_backward(hidden, weight, labels, row_lse, row_pz)
+    ctx.rcp_temperature = rcp_temperature
+    ctx.want_entropy = want_entropy
+
+
+def _backward(ctx, d_logprobs, d_entropy, d_row_lse, d_row_pz):
+    hidden, weight, labels, row_lse, row_pz = ctx.saved_tensors
+    T = hidden.shape[0]
+    if d_logprobs is None:
+        d_logprobs = torch.zeros(T, dtype=torch.float32, device=hidden.device)
+    d_logprobs = d_logprobs.to(torch.float32).contiguous()
+    dent = None
+    if ctx.want_entropy and d_entropy is not None:
+        dent = d_entropy.to(torch.float32).contiguous()
+    d_hidden, d_weight = lmhead_bwd(hidden, weight, labels, row_lse, row_pz if dent is not None else None, d_logprobs,
+                                    dent, ctx.rcp_temperature, 0)
+    # grad_weight is handed back in the weight's dtype, as the reference does (model_utils.py:428).
+    return d_hidden, d_weight.to(weight.dtype), None, None, None
+
+
+lmhead_fwd.register_autograd(_backward, setup_context=_setup_context)
