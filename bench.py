@@ -1,0 +1,214 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused LM-head log-probability path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config NAME] [--no-cpu-baseline]
+
+A step is one forward + backward pass of the path over one synthetic micro-batch that is already resident in HBM: the
+Qwen2.5-7B-shaped LM head (T=16384 packed tokens, H=3584, V=152064, temperature 0.6, upstream gradients on both the
+log-probabilities and the entropy).  The step goes through the C ABI (``skyrl_lmhead_fwd`` then ``skyrl_lmhead_bwd``), exactly
+as the torch custom ops call it.  One JSON line is printed:
+
+  value / unit   tokens per second of forward + backward (whole job; one GPU)
+  roofline       the dominant kernel (the gradient GEMM ``gemm_nt_store``, 4*T*V*H of the 8*T*V*H flop) against the dense bf16
+                 MFMA peak of 2.5 PFLOP/s; its time is measured live with HIP events on the launch stream
+  step_roofline  the whole step (8*T*V*H algorithmic flop / step time) against the same peak
+  kernels        live HIP-event time per kernel and step
+  cpu_baseline   the CPU restatement of the reference's torch implementation, timed on this host on a bounded sample
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_DENSE_FLOPS = 2.5e15  # MI355X dense bf16 MFMA
+METRIC = "fused LM-head fwd+bwd tokens/sec on 1 MI355X; % bf16 MFMA peak"
+
+# HBM bytes per gemm_nt_store launch from `rocprofv3 --pmc` (FETCH_SIZE, then WRITE_SIZE) scaled by a copy kernel of known size;
+# None until measured for the workload.  Keyed by config name.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {}
+
+
+def cpu_baseline(cfg, sample_tokens: int):
+    """Time the oracle's reference-faithful torch path (bf16 matmul, fp32 softmax, 1 chunk) on ``sample_tokens`` tokens."""
+    import torch
+
+    from oracle import lmhead_oracle as O
+    from skyrl_amd.bench_inputs import make_inputs
+    import dataclasses
+
+    small = dataclasses.replace(cfg, T=sample_tokens, layout="dense", n_seqs=1, mask="none")
+    d = make_inputs(small)
+    g = d.get("dlogprobs") if cfg.backward else None
+    warm = {k: (v[:8] if k in ("hidden", "labels", "dlogprobs") else v) for k, v in d.items()}
+    O.reference_faithful_fwd_bwd(warm["hidden"], warm["weight"][:4096], warm["labels"] % 4096, cfg.temperature,
+                                 warm.get("dlogprobs") if cfg.backward else None, chunk_size=8, want_entropy=cfg.entropy)
+    t0 = time.perf_counter()
+    chunk = min(sample_tokens, 1024)  # the reference's default logprobs_chunk_size (skyrl/train/config/config.py:1482)
+    O.reference_faithful_fwd_bwd(d["hidden"], d["weight"], d["labels"], cfg.temperature, g, chunk_size=chunk,
+                                 want_entropy=cfg.entropy)
+    dt = time.perf_counter() - t0
+    return {
+        "value": sample_tokens / dt,
+        "unit": "tokens/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"{sample_tokens} of {cfg.T} tokens at full H={cfg.H}, V={cfg.V}: logprob forward + entropy metric"
+                  f"{' + backward' if cfg.backward else ''} in chunks of {chunk}, bf16 torch.matmul on CPU, {dt:.1f} s; the algorithm is a"
+                  " loop over independent token chunks, so tokens/s carries over to the full batch",
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--config", default="qwen2.5-7b-fwdbwd")
+    ap.add_argument("--vocab-chunk", type=int, default=0)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs the fused LM-head path on ONE GPU; --gpus N with N > 1 is not supported "
+              "(every GPU box of this project has one GPU, and the path has no collectives at tensor-parallel size 1).",
+              file=sys.stderr)
+        return 2
+
+    import torch
+
+    from skyrl_amd import _lib, ops
+    from skyrl_amd.bench_inputs import CONFIGS, make_inputs
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback.", file=sys.stderr)
+        return 3
+    cfg = CONFIGS[args.config]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    lib = _lib.load()
+
+    d = make_inputs(cfg)
+    T, H, V = cfg.T, cfg.H, cfg.V
+    rcp_t = 1.0 / cfg.temperature
+    want_ent = cfg.entropy or cfg.entropy_grad
+    hidden, weight, labels = d["hidden"].to(dev), d["weight"].to(dev), d["labels"].to(dev)
+    g = d["dlogprobs"].to(dev) if cfg.backward else None
+    q = d["dentropy"].to(dev) if cfg.entropy_grad else None
+
+    # Outputs and scratch are allocated once, outside the timed region, and passed by pointer: the timed region is the C ABI.
+    f32 = dict(dtype=torch.float32, device=dev)
+    logprobs, row_lse = torch.empty(T, **f32), torch.empty(T, **f32)
+    entropy = torch.empty(T, **f32) if want_ent else None
+    row_pz = torch.empty(T, **f32) if want_ent else None
+    ws_f = torch.empty(ops.fwd_workspace_bytes(T, H, V), dtype=torch.uint8, device=dev)
+    if cfg.backward:
+        d_hidden = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+        d_weight = torch.empty(V, H, **f32)
+        ws_b = torch.empty(ops.bwd_workspace_bytes(T, H, V, args.vocab_chunk), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    ptr = lambda t: None if t is None else t.data_ptr()  # noqa: E731
+
+    def step():
+        st = lib.skyrl_lmhead_fwd(hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), labels.data_ptr(),
+                                  T, H, V, rcp_t, logprobs.data_ptr(), ptr(entropy), row_lse.data_ptr(), ptr(row_pz),
+                                  ws_f.data_ptr(), ws_f.numel(), stream)
+        _lib.check(st, "skyrl_lmhead_fwd")
+        if cfg.backward:
+            st = lib.skyrl_lmhead_bwd(hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0),
+                                      labels.data_ptr(), row_lse.data_ptr(), ptr(row_pz) if q is not None else None,
+                                      g.data_ptr(), ptr(q), T, H, V, rcp_t, d_hidden.data_ptr(), d_weight.data_ptr(), 0,
+                                      args.vocab_chunk, ws_b.data_ptr(), ws_b.numel(), stream)
+            _lib.check(st, "skyrl_lmhead_bwd")
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    # Timed region: exactly K steps, bracketed by synchronize on both sides; per-kernel HIP events ride along.
+    with _lib.KernelProfile() as prof:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    tokens_per_s = T * args.steps / elapsed
+
+    kernels = {k: {"ms_per_step": ms / args.steps, "launches_per_step": n / args.steps, "avg_launch_ms": ms / n}
+               for k, (ms, n) in prof.results.items() if n}
+    step_flop = cfg.total_flop
+    step_roofline = {"bound": "mfma", "achieved": step_flop / (ms_per_step * 1e-3) / 1e12, "peak": PEAK_BF16_DENSE_FLOPS / 1e12,
+                     "unit": "TFLOP/s"}
+    step_roofline["frac"] = step_roofline["achieved"] / step_roofline["peak"]
+
+    # Dominant kernel.  With a backward pass it is gemm_nt_store (dHidden and dWeight launches, 2*T*V*H flop each in total);
+    # forward-only workloads are all lmhead_fwd_tiles.
+    if cfg.backward:
+        ks = [kernels[n] for n in ("gemm_nt_store(dHidden)", "gemm_nt_store(dWeight)")]
+        dom_name = "gemm_nt_store"
+        dom_ms = sum(k["ms_per_step"] for k in ks)
+        dom_launches = sum(k["launches_per_step"] for k in ks)
+        dom_flop = 4.0 * T * V * H
+    else:
+        k = kernels["lmhead_fwd_tiles"]
+        dom_name, dom_ms, dom_launches, dom_flop = "lmhead_fwd_tiles", k["ms_per_step"], k["launches_per_step"], 2.0 * T * V * H
+    achieved = dom_flop / (dom_ms * 1e-3) / 1e12
+    roofline = {
+        "kernel": dom_name,
+        "bound": "mfma",
+        "achieved": achieved,
+        "peak": PEAK_BF16_DENSE_FLOPS / 1e12,
+        "unit": "TFLOP/s",
+        "frac": achieved / (PEAK_BF16_DENSE_FLOPS / 1e12),
+        "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(cfg.name),
+        "flop_per_launch": dom_flop / dom_launches,
+        "avg_launch_ms": dom_ms / dom_launches,
+        "launches_per_step": dom_launches,
+    }
+
+    out = {
+        "metric": METRIC,
+        "value": tokens_per_s,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{cfg.name}: LM head T={T} H={H} V={V}, temperature {cfg.temperature}, "
+                        f"{'forward+backward' if cfg.backward else 'forward'}"
+                        f"{', entropy with upstream grad' if cfg.entropy_grad else (', entropy' if cfg.entropy else '')}",
+            "T": T, "H": H, "V": V, "temperature": cfg.temperature,
+            "vocab_chunk": args.vocab_chunk or "library default",
+            "device": torch.cuda.get_device_name(0),
+            "compute_units": torch.cuda.get_device_properties(0).multi_processor_count,
+        },
+        "tflops": step_roofline["achieved"],
+        "pct_of_bf16_mfma_peak": 100.0 * step_roofline["frac"],
+        "roofline": roofline,
+        "step_roofline": step_roofline,
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_sample_tokens)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -90,6 +90,19 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
                      void* d_hidden, float* d_weight, int accumulate_dw, int64_t vocab_chunk,
                      void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * Per-kernel timing for benchmarks (no counterpart in the reference, which times whole calls from Python with
+ * torch.cuda.synchronize, skyrl/benchmarks/bench_fused_linear_logprob.py:96-101).
+ * skyrl_lmhead_profile_begin() opens a profile on the calling thread and returns its handle (NULL if one is already open):
+ * until it is closed, every kernel launched by skyrl_lmhead_fwd / skyrl_lmhead_bwd from this thread is bracketed by HIP
+ * events on the launch stream.  skyrl_lmhead_profile_end() waits for those events, fills total_ms[k] and launches[k] for
+ * k < skyrl_lmhead_num_kernel_kinds() and frees the profile.  skyrl_lmhead_kernel_name(k) names kind k.
+ */
+int skyrl_lmhead_num_kernel_kinds(void);
+const char* skyrl_lmhead_kernel_name(int kind);
+void* skyrl_lmhead_profile_begin(void);
+int skyrl_lmhead_profile_end(void* handle, double* total_ms, int64_t* launches);
+
 #ifdef __cplusplus
 }
 #endif

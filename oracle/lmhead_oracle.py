@@ -1,0 +1,349 @@
+"""CPU restatement of SkyRL's fused LM-head log-probability path.  TEST INFRASTRUCTURE ONLY.
+
+This module is the checker for the HIP kernels, not a product path: only ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py`` may import it.  Nothing under ``skyrl_amd/`` does, and the product raises when the
+HIP library is missing instead of routing here.
+
+Every function restates one piece of the reference and cites it (paths relative to the SkyRL tree; ``MU`` =
+``skyrl/backends/skyrl_train/distributed/megatron/model_utils.py``, ``TR`` = ``.../megatron/fused_linear_logprob_triton.py``).
+Tensor-parallel all-reduces are identities here (one vocab shard holds the full vocabulary).
+
+What pins each function (all in ``tests/test_oracle.py``; none of them re-types the formula under test):
+  * log-softmax / logprob / entropy forward: ``torch.log_softmax`` + ``gather`` in fp64, the closed forms
+    ``W = 0 -> logprob = -ln V, entropy = ln V`` (the reference's own known answer is ``ln 4``,
+    tests/backends/skyrl_train/utils/test_torch_utils.py:31-35), ``sum_y exp(logprob(y)) = 1`` by brute force over every
+    target, shift invariance, chunk-size invariance over the reference's cases {1, 7, 64, 512}
+    (tests/backends/skyrl_train/gpu/gpu_ci/megatron/test_fused_linear_logprob.py:98).
+  * split merge: any partition of the vocabulary merges to the one-shot result (hypothesis).
+  * d_logits, dHidden, dW: torch autograd of the fp64 closed form, fp64 central finite differences, row sums of d_logits,
+    linearity in (g, q), the reference's tolerances (test_fused_linear_logprob.py:89-95).
+  * out-of-vocabulary targets: forward 0 / backward keeps -p*g, by construction of an autograd twin whose target logit is
+    multiplied by the in-vocabulary mask.
+  * packed-sequence roll and scatter-back: a per-sequence Python loop.
+No function is left "parity unpinned".
+"""
+
+from __future__ import annotations
+
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+
+OOV_LABEL_SENTINEL = torch.iinfo(torch.int64).max  # TR:1832
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# Torch backend of the reference: FusedLinearChunkedDistributedLogprob and helpers
+# ----------------------------------------------------------------------------------------------------------------------
+def distributed_log_softmax(logits: torch.Tensor) -> torch.Tensor:
+    """MU:28-63 with the MAX / SUM all-reduces as identities: amax, subtract, exp, sum (as float), subtract log."""
+    logits_max = torch.amax(logits, dim=-1, keepdim=True)
+    shifted = logits - logits_max
+    sum_exp = shifted.exp().sum(-1, keepdim=True).float()
+    return shifted - sum_exp.log_().to(shifted.dtype)
+
+
+def _mask_targets(target: torch.Tensor, vocab_start: int, vocab_end: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """MU:314-316: mask of targets outside the shard; masked targets re-based to the shard and zeroed."""
+    target_mask = (target < vocab_start) | (target >= vocab_end)
+    masked_target = target - vocab_start
+    masked_target[target_mask] = 0
+    return target_mask, masked_target
+
+
+def fused_chunked_logprob_forward(
+    hidden: torch.Tensor, weight: torch.Tensor, target: torch.Tensor, vocab_start: int, vocab_end: int, chunk_size: int
+) -> torch.Tensor:
+    """MU:302-359.  hidden [B,S,H], weight [V,H], target [B,S] (already shifted) -> logprobs [B,S] fp32.
+
+    Per sequence chunk: matmul in the weight dtype, cast to fp32, log-softmax, gather the target, force 0 where the target is
+    outside [vocab_start, vocab_end).
+    """
+    target_mask, masked_target = _mask_targets(target.clone(), vocab_start, vocab_end)
+    seq = int(hidden.shape[1])
+    out: List[torch.Tensor] = []
+    for c0 in range(0, seq, chunk_size):
+        c1 = min(seq, c0 + chunk_size)
+        logits = torch.matmul(hidden[:, c0:c1, :].to(weight.dtype), weight.t()).to(torch.float32)
+        lp = distributed_log_softmax(logits)
+        lp = torch.gather(lp, -1, masked_target[:, c0:c1].unsqueeze(-1)).squeeze(-1)
+        lp[target_mask[:, c0:c1]] = 0.0
+        out.append(lp)
+    return torch.cat(out, dim=1)
+
+
+def fused_chunked_logprob_backward(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    target: torch.Tensor,
+    vocab_start: int,
+    vocab_end: int,
+    chunk_size: int,
+    grad_output: torch.Tensor,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """MU:361-428.  Returns (grad_hidden in hidden dtype, grad_weight as the fp32 accumulator *before* the final cast to the
+    weight dtype at MU:428 -- callers cast if they want the reference's returned dtype).
+
+    Per chunk: recompute softmax, grad_logits = -softmax * g, scatter-add g at in-shard targets, cast to the weight dtype,
+    grad_hidden[chunk] = grad_logits @ W, grad_weight += (grad_logits^T @ h).float().
+    """
+    target_mask, masked_target = _mask_targets(target.clone(), vocab_start, vocab_end)
+    V, H = int(weight.shape[0]), int(weight.shape[1])
+    B, seq = int(hidden.shape[0]), int(hidden.shape[1])
+    grad_hidden = torch.empty_like(hidden)
+    grad_weight = torch.zeros((V, H), dtype=torch.float32)
+    for c0 in range(0, seq, chunk_size):
+        c1 = min(seq, c0 + chunk_size)
+        h_chunk = hidden[:, c0:c1, :]
+        logits = torch.matmul(h_chunk.to(weight.dtype), weight.t()).to(torch.float32)
+        grad_logits = distributed_log_softmax(logits).exp_().neg_()
+        g = grad_output[:, c0:c1]
+        grad_logits.mul_(g.unsqueeze(-1))
+        valid = ~target_mask[:, c0:c1]
+        # scatter-add of g at the chosen column (MU:396-411), written with 2-D indexing instead of flat offsets
+        b_idx, s_idx = valid.nonzero(as_tuple=True)
+        grad_logits[b_idx, s_idx, masked_target[:, c0:c1][b_idx, s_idx]] += g[b_idx, s_idx]
+        grad_logits = grad_logits.to(weight.dtype)
+        grad_hidden[:, c0:c1, :] = torch.matmul(grad_logits, weight)
+        gl2 = grad_logits.reshape(-1, V)
+        grad_weight.add_(torch.matmul(gl2.t(), h_chunk.reshape(-1, H).to(gl2.dtype)).to(torch.float32))
+    return grad_hidden, grad_weight
+
+
+def fused_entropy_from_hidden(
+    hidden: torch.Tensor, weight: torch.Tensor, chunk_size: Optional[int] = None, temperature: float = 1.0
+) -> torch.Tensor:
+    """MU:1090-1121 (no-grad entropy metric): H = max + log(sum exp) - sum softmax*logits per token, weight divided by the
+    temperature first (in the weight dtype)."""
+    if temperature != 1.0:
+        weight = weight / temperature
+    B, S = int(hidden.shape[0]), int(hidden.shape[1])
+    out = torch.empty((B, S), dtype=torch.float32)
+    eff = chunk_size if (chunk_size is not None and chunk_size < S) else S
+    for c0 in range(0, S, eff):
+        c1 = min(S, c0 + eff)
+        logits = torch.matmul(hidden[:, c0:c1, :].to(weight.dtype), weight.t()).to(torch.float32)
+        logits_max = logits.max(dim=-1, keepdim=True).values
+        e = (logits - logits_max).exp_()
+        sum_exp = e.sum(dim=-1, keepdim=True)
+        softmax = e / sum_exp
+        spz = (softmax * logits).sum(dim=-1, keepdim=True)
+        out[:, c0:c1] = (logits_max + sum_exp.log() - spz).squeeze(-1)
+    return out
+
+
+def vocab_parallel_entropy_backward(logits: torch.Tensor, grad_entropy: torch.Tensor) -> torch.Tensor:
+    """MU:1339-1345: d entropy / d logits = softmax * (sum softmax*logits - logits) * grad."""
+    p = torch.softmax(logits, dim=-1)
+    spz = (p * logits).sum(dim=-1, keepdim=True)
+    return p * (spz - logits) * grad_entropy.unsqueeze(-1)
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# Triton backend of the reference (vendored verl kernels): split statistics, merge, d_logits
+# ----------------------------------------------------------------------------------------------------------------------
+def split_statistics(logits: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """TR:296-385 for one vocab split, logits already scaled by 1/temperature: (max, sum exp(z - max), sum z*exp(z - max))."""
+    m = logits.max(dim=-1).values
+    e = (logits - m.unsqueeze(-1)).exp()
+    return m, e.sum(-1), (e * logits).sum(-1)
+
+
+def merge_split_statistics(
+    maxes: torch.Tensor, accus: torch.Tensor, entropy_bs: torch.Tensor
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """TR:417-446: merge per-split (max, accu, entropy_b) of shape [T, num_splits] into global (max, accu, entropy_b sum).
+
+    The running maximum starts at -inf here; the reference kernel starts it at 0 (TR:421), which is the same number for any
+    row with a non-negative logit and wrong (underflow) for rows whose logits are all very negative.  The HIP path follows
+    this restatement, not that quirk.
+    """
+    gmax = maxes.max(dim=-1).values
+    scale = (maxes - gmax.unsqueeze(-1)).exp()
+    return gmax, (scale * accus).sum(-1), (scale * entropy_bs).sum(-1)
+
+
+def linear_cross_entropy_forward(
+    hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor, temperature: float = 1.0, vocab_per_split: int = 1024
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """efficient_entropy_forward, TR:614-803 (REDUCTION none, one rank): returns (logprobs, entropy, maximum, accumulate,
+    entropy_b), each [T].  hidden [T,H], weight [V,H]; the dot products accumulate in fp32 from the stored dtype (TR:339),
+    logits are scaled by 1/temperature (TR:346); labels matching no column contribute no label logit, and the adapter forces
+    their logprob to 0 (TR:1898-1905)."""
+    T, V = int(hidden.shape[0]), int(weight.shape[0])
+    rcp_t = 1.0 / temperature
+    acc_dtype = torch.float64 if hidden.dtype == torch.float64 else torch.float32
+    ms, ss, es = [], [], []
+    label_logit = torch.zeros(T, dtype=acc_dtype)
+    for v0 in range(0, V, vocab_per_split):
+        v1 = min(V, v0 + vocab_per_split)
+        z = torch.matmul(hidden.to(acc_dtype), weight[v0:v1].to(acc_dtype).t()) * rcp_t
+        m, s, e = split_statistics(z)
+        ms.append(m), ss.append(s), es.append(e)
+        own = (labels >= v0) & (labels < v1)
+        idx = own.nonzero(as_tuple=True)[0]
+        label_logit[idx] = z[idx, labels[idx] - v0]
+    gmax, gacc, geb = merge_split_statistics(torch.stack(ms, 1), torch.stack(ss, 1), torch.stack(es, 1))
+    entropy_b = geb / gacc  # TR:453
+    entropy = gacc.log() + gmax - entropy_b  # TR:459
+    logprobs = -(gmax + gacc.log() - label_logit)  # TR:463-467
+    in_vocab = (labels >= 0) & (labels < V)
+    logprobs = logprobs.masked_fill(~in_vocab, 0.0)  # TR:1898-1905
+    return logprobs, entropy, gmax, gacc, entropy_b
+
+
+def d_logits_formula(
+    logits: torch.Tensor,
+    maximum: torch.Tensor,
+    accumulate: torch.Tensor,
+    entropy_b: torch.Tensor,
+    labels: torch.Tensor,
+    dlogprobs: torch.Tensor,
+    dentropy: torch.Tensor,
+    rcp_temperature: float,
+    vocab_offset: int = 0,
+) -> torch.Tensor:
+    """TR:947-957.  ``logits`` are already scaled by 1/temperature and cover columns [vocab_offset, vocab_offset + n).
+
+    exp_logits = exp(z - max);  d = (-g) * (exp_logits/accu - onehot) + q * (-exp_logits/accu) * (z - entropy_b);  d *= 1/temperature.
+    """
+    p = (logits - maximum.unsqueeze(-1)).exp() / accumulate.unsqueeze(-1)
+    cols = torch.arange(logits.shape[-1]) + vocab_offset
+    onehot = (cols.unsqueeze(0) == labels.unsqueeze(-1)).to(logits.dtype)
+    d = (-dlogprobs).unsqueeze(-1) * (p - onehot)
+    d = d + dentropy.unsqueeze(-1) * (-p) * (logits - entropy_b.unsqueeze(-1))
+    return d * rcp_temperature
+
+
+def linear_cross_entropy_backward(
+    dlogprobs: torch.Tensor,
+    dentropy: torch.Tensor,
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    maximum: torch.Tensor,
+    accumulate: torch.Tensor,
+    entropy_b: torch.Tensor,
+    temperature: float = 1.0,
+    vocab_per_split: int = 9504,
+    round_d_logits_to: Optional[torch.dtype] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """efficient_entropy_backward with the default ``_Split_Dlogits_N`` method (TR:1689-1748): per vocab split, recompute the
+    logits, form d_logits (rounded to the hidden dtype, TR:1402-1538 stores it in that dtype), then
+    d_hidden += d_logits @ W_split and d_weight[split] = d_logits^T @ hidden.  Returns fp32 (or fp64) accumulators; the reference
+    returns them in the hidden dtype."""
+    T, H = int(hidden.shape[0]), int(hidden.shape[1])
+    V = int(weight.shape[0])
+    rcp_t = 1.0 / temperature
+    acc_dtype = torch.float64 if hidden.dtype == torch.float64 else torch.float32
+    round_to = hidden.dtype if round_d_logits_to is None else round_d_logits_to
+    d_hidden = torch.zeros((T, H), dtype=acc_dtype)
+    d_weight = torch.zeros((V, H), dtype=acc_dtype)
+    h = hidden.to(acc_dtype)
+    for v0 in range(0, V, vocab_per_split):
+        v1 = min(V, v0 + vocab_per_split)
+        w = weight[v0:v1].to(acc_dtype)
+        z = torch.matmul(h, w.t()) * rcp_t
+        d = d_logits_formula(z, maximum.to(acc_dtype), accumulate.to(acc_dtype), entropy_b.to(acc_dtype), labels,
+                             dlogprobs.to(acc_dtype), dentropy.to(acc_dtype), rcp_t, vocab_offset=v0)
+        d = d.to(round_to).to(acc_dtype)
+        d_hidden += torch.matmul(d, w)
+        d_weight[v0:v1] = torch.matmul(d.t(), h)
+    return d_hidden, d_weight
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# Callers one level up: target roll, packed sequences
+# ----------------------------------------------------------------------------------------------------------------------
+def from_parallel_hidden_to_logprobs(
+    hidden: torch.Tensor, weight: torch.Tensor, target: torch.Tensor, chunk_size: Optional[int] = None, temperature: float = 1.0
+) -> torch.Tensor:
+    """MU:713-770 at TP = CP = 1: weight / temperature (in the weight dtype, MU:739-740), targets rolled left by one
+    (MU:741), fused op, last column dropped (MU:770).  -> [B, S-1]."""
+    if temperature != 1.0:
+        weight = weight / temperature
+    target = target.roll(shifts=-1, dims=-1)
+    S = int(hidden.shape[1])
+    eff = chunk_size if (chunk_size is not None and chunk_size < S) else S
+    lp = fused_chunked_logprob_forward(hidden, weight, target, 0, int(weight.shape[0]), eff)
+    return lp[:, :-1]
+
+
+def packed_sequence_indices(cu_seqlens: torch.Tensor, total_tokens: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """MU:920-928: for every packed token its sequence index, offset inside the sequence, and the sequence lengths."""
+    cu = cu_seqlens.to(torch.long)
+    tok = torch.arange(total_tokens)
+    seq_idx = torch.searchsorted(cu[1:], tok, right=True)
+    seq_off = tok - cu[seq_idx]
+    return seq_idx, seq_off, cu[1:] - cu[:-1]
+
+
+def packed_rolled_targets(target: torch.Tensor, cu_seqlens: torch.Tensor) -> torch.Tensor:
+    """MU:810-815: per-sequence roll(-1) inside a packed [T] stream: next = (offset + 1) mod len."""
+    seq_idx, seq_off, seq_len = packed_sequence_indices(cu_seqlens, int(target.shape[0]))
+    nxt = torch.remainder(seq_off + 1, seq_len[seq_idx])
+    return target[cu_seqlens.to(torch.long)[seq_idx] + nxt]
+
+
+def packed_scatter_back(probs: torch.Tensor, cu_seqlens: torch.Tensor, batch_size: int, unpacked_seqlen: int) -> torch.Tensor:
+    """MU:851-883, the plain branch (no sub-sequences, no attention mask): token at (seq i, offset o) goes to out[i, o] for
+    o < len_i - 1 and o < unpacked_seqlen - 1; everything else stays 0."""
+    out = torch.zeros((batch_size, unpacked_seqlen - 1), dtype=probs.dtype)
+    seq_idx, seq_off, seq_len = packed_sequence_indices(cu_seqlens, int(probs.shape[0]))
+    valid = torch.clamp(seq_len - 1, min=0)
+    mask = (seq_off < valid[seq_idx]) & (seq_off < unpacked_seqlen - 1)
+    out[seq_idx[mask], seq_off[mask]] = probs[mask]
+    return out
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# Convenience used by the parity tests and the CPU baseline: one call = forward + backward of the whole path
+# ----------------------------------------------------------------------------------------------------------------------
+def reference_faithful_fwd_bwd(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    temperature: float,
+    dlogprobs: Optional[torch.Tensor],
+    chunk_size: int = 1024,
+    want_entropy: bool = True,
+):
+    """The reference's pure-torch path exactly as the trainer runs it on one rank (bf16 matmul, fp32 softmax, W / temperature
+    in the weight dtype): logprobs via MU:302-359, entropy metric via MU:1090-1121, backward via MU:361-428.
+    hidden [T,H], labels [T] already shifted.  Returns dict of tensors; gradients are w.r.t. the *scaled* weight W/temperature
+    multiplied back by 1/temperature (the chain rule autograd applies for MU:739-740)."""
+    w_scaled = weight / temperature if temperature != 1.0 else weight
+    h3 = hidden.unsqueeze(0)
+    y3 = labels.unsqueeze(0)
+    V = int(weight.shape[0])
+    out = {"logprobs": fused_chunked_logprob_forward(h3, w_scaled, y3, 0, V, chunk_size).squeeze(0)}
+    if want_entropy:
+        out["entropy"] = fused_entropy_from_hidden(h3, weight, chunk_size, temperature).squeeze(0)
+    if dlogprobs is not None:
+        gh, gw = fused_chunked_logprob_backward(h3, w_scaled, y3, 0, V, chunk_size, dlogprobs.unsqueeze(0))
+        out["d_hidden"] = gh.squeeze(0)
+        out["d_weight"] = gw / temperature
+    return out
+
+
+def exact_fwd_bwd(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    temperature: float,
+    dlogprobs: Optional[torch.Tensor] = None,
+    dentropy: Optional[torch.Tensor] = None,
+    dtype: torch.dtype = torch.float64,
+    vocab_per_split: int = 8192,
+):
+    """High-precision statement of the whole path (the verl formulas evaluated in ``dtype`` with no intermediate rounding).
+    This is the "fp32 reference" side of the gradient-cosine criterion; fp64 by default."""
+    h, w = hidden.to(dtype), weight.to(dtype)
+    lp, ent, mx, acc, eb = linear_cross_entropy_forward(h, w, labels, temperature, vocab_per_split)
+    out = {"logprobs": lp, "entropy": ent, "lse": mx + acc.log(), "pz": eb}
+    if dlogprobs is not None:
+        q = dentropy if dentropy is not None else torch.zeros_like(dlogprobs)
+        dh, dw = linear_cross_entropy_backward(dlogprobs, q, h, w, labels, mx, acc, eb, temperature, vocab_per_split,
+                                               round_d_logits_to=dtype)
+        out["d_hidden"], out["d_weight"] = dh, dw
+    return out

@@ -32,6 +32,10 @@ SIGNATURES = {
         [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, ctypes.c_float, _c_p, _c_p,
          ctypes.c_int, _c_i64, _c_p, ctypes.c_size_t, _c_p],
     ),
+    "skyrl_lmhead_num_kernel_kinds": (ctypes.c_int, []),
+    "skyrl_lmhead_kernel_name": (ctypes.c_char_p, [ctypes.c_int]),
+    "skyrl_lmhead_profile_begin": (_c_p, []),
+    "skyrl_lmhead_profile_end": (ctypes.c_int, [_c_p, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(_c_i64)]),
 }
 
 _lock = threading.Lock()
@@ -86,3 +90,28 @@ def check(status: int, what: str) -> None:
     if status < 0:
         raise ValueError(msg)
     raise LmHeadLibraryError(msg)
+
+
+class KernelProfile:
+    """Context manager around skyrl_lmhead_profile_begin/end: per-kernel HIP-event times of the calls made inside it.
+
+    ``with KernelProfile() as prof: ...`` then ``prof.results`` is ``{kernel name: (total_ms, launches)}``.
+    """
+
+    def __enter__(self):
+        self._lib = load()
+        self._handle = self._lib.skyrl_lmhead_profile_begin()
+        if not self._handle:
+            raise LmHeadLibraryError("a kernel profile is already open on this thread")
+        self.results = {}
+        return self
+
+    def __exit__(self, *exc):
+        n = self._lib.skyrl_lmhead_num_kernel_kinds()
+        ms = (ctypes.c_double * n)()
+        cnt = (_c_i64 * n)()
+        st = self._lib.skyrl_lmhead_profile_end(self._handle, ms, cnt)
+        if exc[0] is None:
+            check(st, "skyrl_lmhead_profile_end")
+        self.results = {self._lib.skyrl_lmhead_kernel_name(k).decode(): (float(ms[k]), int(cnt[k])) for k in range(n)}
+        return False

@@ -15,6 +15,8 @@
 #include <math.h>
 #include <stdint.h>
 
+#include <vector>
+
 #include "../../include/skyrl_lmhead.h"
 #include "gemm_core.hpp"
 
@@ -383,6 +385,35 @@ __global__ __launch_bounds__(256) void transpose_bf16(const uint16_t* __restrict
 // ------------------------------------------------------------------------------------------------------------
 // Host side
 // ------------------------------------------------------------------------------------------------------------
+// Optional per-kernel timing: while a profile is open on the calling thread every launch below is bracketed by a pair of
+// HIP events on the launch stream.  Closed profiles cost one thread-local load per launch.
+enum KernelKind { kFwdTiles = 0, kFwdMerge, kTranspose, kBwdDzTiles, kGemmDHidden, kGemmDWeight, kNumKernelKinds };
+const char* const kKernelNames[kNumKernelKinds] = {"lmhead_fwd_tiles", "lmhead_fwd_merge", "transpose_bf16",
+                                                   "lmhead_bwd_dz_tiles", "gemm_nt_store(dHidden)", "gemm_nt_store(dWeight)"};
+struct Profile {
+  struct Rec {
+    int kind;
+    hipEvent_t a, b;
+  };
+  std::vector<Rec> recs;
+};
+thread_local Profile* tl_profile = nullptr;
+
+struct Timed {
+  int kind;
+  hipStream_t s;
+  hipEvent_t a = nullptr, b = nullptr;
+  Timed(int k, hipStream_t st) : kind(k), s(st) {
+    if (tl_profile && hipEventCreate(&a) == hipSuccess && hipEventCreate(&b) == hipSuccess) (void)hipEventRecord(a, s);
+  }
+  ~Timed() {
+    if (tl_profile && a && b) {
+      (void)hipEventRecord(b, s);
+      tl_profile->recs.push_back({kind, a, b});
+    }
+  }
+};
+
 struct Carver {
   char* base;
   size_t off = 0;
@@ -437,10 +468,11 @@ BwdWorkspace carve_bwd(void* ws, int64_t T, int64_t H, int64_t V, int64_t vc) {
   return w;
 }
 
-hipError_t launch_gemm(hipStream_t s, const uint16_t* A, int64_t lda, int64_t a_rows, const uint16_t* B, int64_t ldb,
+hipError_t launch_gemm(int kind, hipStream_t s, const uint16_t* A, int64_t lda, int64_t a_rows, const uint16_t* B, int64_t ldb,
                        int64_t b_rows, int64_t nk, int64_t M, int64_t N, const float* Cin, float* Cf, uint16_t* Cb,
                        int64_t ldc) {
   const unsigned tiles = (unsigned)(((M + BM - 1) / BM) * ((N + BN - 1) / BN));
+  Timed timed(kind, s);
   hipLaunchKernelGGL(gemm_nt_store, dim3(tiles), dim3(NTHREADS), 0, s, A, (int)lda, (int)a_rows, B, (int)ldb, (int)b_rows,
                      (int)nk, (int)M, (int)N, Cin, Cf, Cb, (int)ldc);
   return hipGetLastError();
@@ -504,14 +536,18 @@ int skyrl_lmhead_fwd(const void* hidden, int64_t ld_hidden, const void* weight, 
   const uint16_t* Wp = (const uint16_t*)weight;
   const uint16_t* Hp = (const uint16_t*)hidden;
   const dim3 grid((unsigned)(tiles_m * tiles_n)), block(NTHREADS);
-  if (want_pz)
-    hipLaunchKernelGGL(lmhead_fwd_tiles<true>, grid, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)T, (int)H,
-                       (int)V, rcp_temperature, pmax, psum, ppz);
-  else
-    hipLaunchKernelGGL(lmhead_fwd_tiles<false>, grid, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)T, (int)H,
-                       (int)V, rcp_temperature, pmax, psum, ppz);
+  {
+    Timed timed(kFwdTiles, s);
+    if (want_pz)
+        hipLaunchKernelGGL(lmhead_fwd_tiles<true>, grid, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)T, (int)H,
+                         (int)V, rcp_temperature, pmax, psum, ppz);
+    else
+      hipLaunchKernelGGL(lmhead_fwd_tiles<false>, grid, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)T, (int)H,
+                         (int)V, rcp_temperature, pmax, psum, ppz);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
+  Timed timed(kFwdMerge, s);
   hipLaunchKernelGGL(lmhead_fwd_merge, dim3((unsigned)((T + 31) / 32)), dim3(256), 0, s, pmax, psum,
                      want_pz ? ppz : (float*)nullptr, (int)nparts, (int)T, Hp, (int)ld_hidden, Wp, (int)ld_weight, labels,
                      (int)H, (int)V, rcp_temperature, logprobs, entropy, row_lse, row_pz);
@@ -542,10 +578,16 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
   hipError_t e;
 
   // weight^T [H, Vpad] and hidden^T [H, Tpad], zero in the padding columns.
-  hipLaunchKernelGGL(transpose_bf16, dim3((unsigned)(Vpad / 64), (unsigned)(H / 64)), dim3(256), 0, s, Wp, (int)ld_weight,
-                     (int)V, (int)H, w.Wt, (int)Vpad, (int)Vpad);
-  hipLaunchKernelGGL(transpose_bf16, dim3((unsigned)(Tpad / 64), (unsigned)(H / 64)), dim3(256), 0, s, Hp, (int)ld_hidden,
-                     (int)T, (int)H, w.Ht, (int)Tpad, (int)Tpad);
+  {
+    Timed timed(kTranspose, s);
+    hipLaunchKernelGGL(transpose_bf16, dim3((unsigned)(Vpad / 64), (unsigned)(H / 64)), dim3(256), 0, s, Wp, (int)ld_weight,
+                       (int)V, (int)H, w.Wt, (int)Vpad, (int)Vpad);
+  }
+  {
+    Timed timed(kTranspose, s);
+    hipLaunchKernelGGL(transpose_bf16, dim3((unsigned)(Tpad / 64), (unsigned)(H / 64)), dim3(256), 0, s, Hp, (int)ld_hidden,
+                       (int)T, (int)H, w.Ht, (int)Tpad, (int)Tpad);
+  }
   if ((e = hipGetLastError()) != hipSuccess) return (int)e;
 
   const int tiles_t = (int)(Tpad / 256);
@@ -556,19 +598,22 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
     const int64_t vcw = (Vpad - vc0) < vc ? (Vpad - vc0) : vc;  // multiple of 256
     const int tiles_v = (int)(vcw / 256);
     const dim3 grid_dz((unsigned)(tiles_v * tiles_t)), block(NTHREADS);
-    if (dentropy)
-      hipLaunchKernelGGL(lmhead_bwd_dz_tiles<true>, grid_dz, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)T,
+    {
+      Timed timed(kBwdDzTiles, s);
+      if (dentropy)
+        hipLaunchKernelGGL(lmhead_bwd_dz_tiles<true>, grid_dz, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)T,
                          (int)H, (int)V, rcp_temperature, labels, row_lse, row_pz, dlogprobs, dentropy, (int)vc0, tiles_v,
                          tiles_t, w.D, (int)vcw, w.DT, (int)Tpad);
-    else
-      hipLaunchKernelGGL(lmhead_bwd_dz_tiles<false>, grid_dz, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)T,
-                         (int)H, (int)V, rcp_temperature, labels, row_lse, row_pz, dlogprobs, dentropy, (int)vc0, tiles_v,
-                         tiles_t, w.D, (int)vcw, w.DT, (int)Tpad);
+      else
+        hipLaunchKernelGGL(lmhead_bwd_dz_tiles<false>, grid_dz, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)T,
+                           (int)H, (int)V, rcp_temperature, labels, row_lse, row_pz, dlogprobs, dentropy, (int)vc0, tiles_v,
+                           tiles_t, w.D, (int)vcw, w.DT, (int)Tpad);
+    }
     if ((e = hipGetLastError()) != hipSuccess) return (int)e;
 
     // dHidden[T, H] (+)= D[T, vcw] . weight[vc0 : vc0 + vcw, :]    (B operand = weight^T rows, k offset vc0)
     const bool first = ci == 0, last = ci == nchunks - 1;
-    e = launch_gemm(s, w.D, vcw, Tpad, w.Wt + vc0, Vpad, H, vcw / BK, T, H,
+    e = launch_gemm(kGemmDHidden, s, w.D, vcw, Tpad, w.Wt + vc0, Vpad, H, vcw / BK, T, H,
                     first ? (const float*)nullptr : (const float*)w.dHacc, last ? (float*)nullptr : w.dHacc,
                     last ? (uint16_t*)d_hidden : (uint16_t*)nullptr, H);
     if (e != hipSuccess) return (int)e;
@@ -576,11 +621,46 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
     // dW[vc0 : vc0 + rows, :] (+)= D^T[vcw, Tpad] . hidden   (B operand = hidden^T rows)
     const int64_t rows = (V - vc0) < vcw ? (V - vc0) : vcw;
     float* dWc = d_weight + (size_t)vc0 * (size_t)H;
-    e = launch_gemm(s, w.DT, Tpad, vcw, w.Ht, Tpad, H, Tpad / BK, rows, H,
+    e = launch_gemm(kGemmDWeight, s, w.DT, Tpad, vcw, w.Ht, Tpad, H, Tpad / BK, rows, H,
                     accumulate_dw ? (const float*)dWc : (const float*)nullptr, dWc, (uint16_t*)nullptr, H);
     if (e != hipSuccess) return (int)e;
   }
   return SKYRL_LMHEAD_OK;
+}
+
+int skyrl_lmhead_num_kernel_kinds(void) { return kNumKernelKinds; }
+
+const char* skyrl_lmhead_kernel_name(int kind) {
+  return (kind >= 0 && kind < kNumKernelKinds) ? kKernelNames[kind] : "";
+}
+
+void* skyrl_lmhead_profile_begin(void) {
+  if (tl_profile) return nullptr;
+  tl_profile = new Profile();
+  return tl_profile;
+}
+
+int skyrl_lmhead_profile_end(void* handle, double* total_ms, int64_t* launches) {
+  if (!handle || handle != (void*)tl_profile || !total_ms || !launches) return SKYRL_LMHEAD_ERR_NULL;
+  Profile* p = tl_profile;
+  tl_profile = nullptr;
+  for (int k = 0; k < kNumKernelKinds; ++k) total_ms[k] = 0.0, launches[k] = 0;
+  int status = SKYRL_LMHEAD_OK;
+  for (auto& r : p->recs) {
+    hipError_t e = hipEventSynchronize(r.b);
+    float ms = 0.f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, r.a, r.b);
+    if (e == hipSuccess) {
+      total_ms[r.kind] += ms;
+      launches[r.kind] += 1;
+    } else if (status == SKYRL_LMHEAD_OK) {
+      status = (int)e;
+    }
+    (void)hipEventDestroy(r.a);
+    (void)hipEventDestroy(r.b);
+  }
+  delete p;
+  return status;
 }
 
 }  // extern "C"

@@ -1,0 +1,230 @@
+"""Host-side mirror of the reference's fused LM-head call sites, with ``"hip"`` as the backend.
+
+Same names, argument order and return shapes as ``skyrl/backends/skyrl_train/distributed/megatron/model_utils.py`` so a
+trainer can import these instead:
+
+* ``_fused_lm_head_logprob_apply``                       (reference :431-484)
+* ``from_parallel_hidden_to_logprobs``                   (:713-770)
+* ``from_parallel_hidden_to_logprobs_packed_sequences``  (:773-883)
+* ``_fused_vocab_parallel_entropy_from_hidden``          (:1090-1121)
+* ``_packed_sequence_indices``, ``_packed_subseq_row_indices_offsets_and_lens``  (:920-928, :886-917)
+
+Differences, all forced by the one-GPU scope: tensor/context-parallel groups must be ``None`` or of size 1, and the only
+backend is ``"hip"`` -- there is no fallback to another implementation when the HIP library is missing.
+
+Temperature: the reference divides the weight by the temperature in the weight's dtype and lets autograd chain the 1/T
+factor (:734-740).  Here the kernel scales the fp32 logits (as the vendored verl kernel does,
+fused_linear_logprob_triton.py:346, 957) and applies 1/T to both gradients itself, so no ``[V, H]`` temporary is made and
+the gradients are with respect to the unscaled weight -- the same quantities autograd yields in the reference.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+import torch.distributed as dist
+
+from . import ops
+from .fused_linear_logprob_hip import FusedLinearLogprobHip, _group_size, _require_single_shard, linear_cross_entropy
+
+FUSED_LM_HEAD_LOGPROB_BACKENDS = ("hip",)
+
+
+def validate_fused_backend(backend: str) -> str:
+    """Mirror of the config check at skyrl/train/config/config.py:1539-1543, with this package's backend list."""
+    if backend not in FUSED_LM_HEAD_LOGPROB_BACKENDS:
+        raise ValueError(
+            f"trainer.fused_lm_head_logprob_backend must be one of {FUSED_LM_HEAD_LOGPROB_BACKENDS}, got {backend!r} "
+            "(the 'torch' and 'triton' backends live in the SkyRL tree, not in this package)"
+        )
+    return backend
+
+
+def _fused_lm_head_logprob_apply(
+    backend: str,
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    target: torch.Tensor,
+    vocab_start_index: int,
+    vocab_end_index: int,
+    chunk_size: int,
+    tp_group: Optional[dist.ProcessGroup],
+    inference_only: bool,
+    temperature: float = 1.0,
+) -> torch.Tensor:
+    """Dispatch the fused LM-head token-logprob to the HIP backend; returns ``[B, S]`` fp32.
+
+    ``temperature`` is an extension over the reference signature (default 1.0 keeps it call-compatible): when it is not 1 the
+    op scales the logits inside the kernel instead of the caller scaling the weight.
+    """
+    validate_fused_backend(backend)
+    if temperature == 1.0:
+        return FusedLinearLogprobHip.apply(hidden, weight, target, vocab_start_index, vocab_end_index, chunk_size, tp_group,
+                                           inference_only)
+    _require_single_shard(tp_group, "_fused_lm_head_logprob_apply")
+    B, S, H = hidden.shape
+    target_mask = (target < vocab_start_index) | (target >= vocab_end_index)
+    labels = torch.where(target_mask, torch.iinfo(torch.int64).max, target - vocab_start_index).to(torch.int64)
+    hidden_c = hidden.to(weight.dtype)
+    if inference_only:
+        with torch.no_grad():
+            logprobs, _ = linear_cross_entropy(hidden_c, weight.contiguous(), labels, float(temperature), "none", None)
+    else:
+        logprobs, _ = linear_cross_entropy(hidden_c, weight.contiguous(), labels, float(temperature), "none", None)
+    return logprobs.reshape(B, S)
+
+
+def from_parallel_hidden_to_logprobs(
+    hidden: torch.Tensor,
+    lm_head_weight: torch.Tensor,
+    target: torch.Tensor,
+    vocab_start_index: int,
+    vocab_end_index: int,
+    tp_group: Optional[dist.ProcessGroup],
+    inference_only: bool = False,
+    cp_group: Optional[dist.ProcessGroup] = None,
+    chunk_size: Optional[int] = None,
+    temperature: float = 1.0,
+    fused_backend: str = "hip",
+) -> torch.Tensor:
+    """``hidden`` [B, S, H] + ``lm_head_weight`` [V, H] + token ids ``target`` [B, S] -> next-token logprobs [B, S-1]."""
+    if _group_size(cp_group) > 1:
+        raise NotImplementedError("context parallelism is outside the one-GPU scope of the HIP fused LM-head path")
+    target = target.roll(shifts=-1, dims=-1)
+    seq_len_local = hidden.shape[1]
+    eff_chunk = chunk_size if (chunk_size is not None and chunk_size < seq_len_local) else seq_len_local
+    logprobs = _fused_lm_head_logprob_apply(
+        fused_backend, hidden, lm_head_weight, target, vocab_start_index, vocab_end_index, eff_chunk, tp_group,
+        inference_only, temperature,
+    ).contiguous()
+    return logprobs[:, :-1]
+
+
+def _packed_sequence_indices(cu_seqlens_padded: torch.Tensor, total_tokens: int, device: torch.device):
+    cu = cu_seqlens_padded.to(device=device, dtype=torch.long)
+    token_indices = torch.arange(total_tokens, device=device)
+    seq_indices = torch.searchsorted(cu[1:], token_indices, right=True)
+    seq_offsets = token_indices - cu[seq_indices]
+    seq_lens_padded = cu[1:] - cu[:-1]
+    return cu, token_indices, seq_indices, seq_offsets, seq_lens_padded
+
+
+def _packed_subseq_row_indices_offsets_and_lens(cu_seqlens_padded: torch.Tensor, sub_seq_lengths, device: torch.device):
+    """Per-packed-segment (row, column offset, true length) for controller-side packing of several sequences per row."""
+    bounds = cu_seqlens_padded.detach().cpu().tolist()
+    padded = [bounds[i + 1] - bounds[i] for i in range(len(bounds) - 1)]
+    rows, offs, lens = [], [], []
+    seg = 0
+    for row, row_lens in enumerate(sub_seq_lengths):
+        col = 0
+        for n in row_lens:
+            if seg >= len(padded):
+                raise ValueError("sub_seq_lengths contains more sub-sequences than cu_seqlens_padded")
+            rows.append(row), offs.append(col), lens.append(int(n))
+            col += padded[seg]
+            seg += 1
+    if seg != len(padded):
+        raise ValueError(f"sub_seq_lengths describes {seg} sub-sequences, but cu_seqlens_padded describes {len(padded)}")
+    mk = lambda x: torch.tensor(x, dtype=torch.long, device=device)  # noqa: E731
+    return mk(rows), mk(offs), mk(lens)
+
+
+def from_parallel_hidden_to_logprobs_packed_sequences(
+    hidden: torch.Tensor,
+    lm_head_weight: torch.Tensor,
+    target: torch.Tensor,
+    cu_seqlens_padded: torch.Tensor,
+    unpacked_seqlen: int,
+    vocab_start_index: int,
+    vocab_end_index: int,
+    group: Optional[dist.ProcessGroup],
+    inference_only: bool = False,
+    cp_group: Optional[dist.ProcessGroup] = None,
+    chunk_size: Optional[int] = None,
+    attention_mask: Optional[torch.Tensor] = None,
+    sub_seq_lengths: Optional[list] = None,
+    temperature: float = 1.0,
+    fused_backend: str = "hip",
+) -> torch.Tensor:
+    """Packed variant: ``hidden`` [1, T, H], ``target`` [1, T], ``cu_seqlens_padded`` [n+1] -> [batch, unpacked_seqlen-1]."""
+    if _group_size(cp_group) > 1:
+        raise NotImplementedError("context parallelism is outside the one-GPU scope of the HIP fused LM-head path")
+    hidden = hidden.squeeze(0)
+    target = target.squeeze(0)
+    batch_size = len(sub_seq_lengths) if sub_seq_lengths is not None else cu_seqlens_padded.shape[0] - 1
+    if attention_mask is not None:
+        attention_mask = attention_mask.to(device=target.device, dtype=torch.bool)
+
+    cu, _, seq_indices, seq_offsets, seq_lens_padded = _packed_sequence_indices(cu_seqlens_padded, target.shape[0],
+                                                                                target.device)
+    next_offsets = torch.remainder(seq_offsets + 1, seq_lens_padded[seq_indices])
+    rolled_targets = target[cu[seq_indices] + next_offsets].unsqueeze(0)
+    hidden = hidden.unsqueeze(0)
+
+    seq_len_local = hidden.shape[1]
+    eff_chunk = chunk_size if (chunk_size is not None and chunk_size < seq_len_local) else seq_len_local
+    probs = _fused_lm_head_logprob_apply(
+        fused_backend, hidden, lm_head_weight, rolled_targets, vocab_start_index, vocab_end_index, eff_chunk, group,
+        inference_only, temperature,
+    ).contiguous().squeeze(0)
+    if probs.dim() != 1:
+        raise ValueError(f"Expected probs to be 1D after squeezing, but got shape {probs.shape}.")
+
+    out = torch.zeros((batch_size, unpacked_seqlen - 1), dtype=probs.dtype, device=probs.device)
+    if sub_seq_lengths is not None:
+        rows, row_offs, seq_lens = _packed_subseq_row_indices_offsets_and_lens(cu, sub_seq_lengths, probs.device)
+        valid = torch.clamp(seq_lens - 1, min=0)
+        packed_mask = seq_offsets < valid[seq_indices]
+        cols = row_offs[seq_indices[packed_mask]] + seq_offsets[packed_mask]
+        rws = rows[seq_indices[packed_mask]]
+        inb = cols < unpacked_seqlen - 1
+        out[rws[inb], cols[inb]] = probs[packed_mask][inb]
+        return out
+    if attention_mask is not None:
+        seq_lens = attention_mask.sum(dim=1, dtype=torch.long)
+        ordinals = attention_mask.to(torch.long).cumsum(dim=1)
+        output_mask = attention_mask[:, :-1] & (ordinals[:, :-1] < seq_lens.unsqueeze(1))
+        valid = torch.clamp(seq_lens - 1, min=0)
+        packed_mask = seq_offsets < valid[seq_indices]
+        out[output_mask] = probs[packed_mask]
+        return out
+    valid = torch.clamp(seq_lens_padded - 1, min=0)
+    packed_mask = (seq_offsets < valid[seq_indices]) & (seq_offsets < unpacked_seqlen - 1)
+    out[seq_indices[packed_mask], seq_offsets[packed_mask]] = probs[packed_mask]
+    return out
+
+
+def _fused_vocab_parallel_entropy_from_hidden(
+    hidden: torch.Tensor,
+    lm_head_weight: torch.Tensor,
+    tp_group: Optional[dist.ProcessGroup],
+    chunk_size: Optional[int] = None,
+    temperature: float = 1.0,
+) -> torch.Tensor:
+    """Per-token entropy [B, S] fp32 from ``hidden`` [B, S, H] + LM-head weight, no gradient (the entropy *metric*)."""
+    _require_single_shard(tp_group, "_fused_vocab_parallel_entropy_from_hidden")
+    B, S, H = hidden.shape
+    with torch.no_grad():
+        labels = torch.full((B * S,), torch.iinfo(torch.int64).max, dtype=torch.int64, device=hidden.device)
+        _, entropy, _, _ = ops.lmhead_fwd(hidden.reshape(B * S, H).to(lm_head_weight.dtype).contiguous(),
+                                          lm_head_weight.contiguous(), labels, 1.0 / float(temperature), True)
+    return entropy.reshape(B, S)
+
+
+def fused_logprobs_and_entropy_from_hidden(
+    hidden: torch.Tensor,
+    lm_head_weight: torch.Tensor,
+    target: torch.Tensor,
+    temperature: float = 1.0,
+):
+    """One pass for both outputs, both differentiable: ``(logprobs [B,S], entropy [B,S])`` for already-shifted ``target``.
+
+    The reference needs two LM-head GEMMs for this (logprob op + entropy op, megatron_model_wrapper.py:648-679 and :852-878);
+    the kernel produces both from one.  This is the entry the FSDP wrapper would use for ``compute_entropy=True`` with
+    ``entropy_requires_grad`` (workers/worker.py:976-986, 1058-1065).
+    """
+    B, S, H = hidden.shape
+    lp, ent = linear_cross_entropy(hidden.to(lm_head_weight.dtype), lm_head_weight.contiguous(), target.reshape(B, S),
+                                   float(temperature), "none", None)
+    return lp.reshape(B, S), ent.reshape(B, S)

@@ -1,0 +1,199 @@
+"""CPU-only checks of the boundary: the C-ABI library loads, exports every symbol the header declares, rejects bad arguments
+before touching a device, and the Python host layer mirrors the reference's interface and error behaviour.  No kernel is
+launched here."""
+
+import ctypes
+import inspect
+import os
+import re
+
+import pytest
+import torch
+
+from skyrl_amd import _lib, model_utils, ops
+from skyrl_amd.fused_linear_logprob_hip import FusedLinearLogprobHip, LinearCrossEntropy, linear_cross_entropy
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "skyrl_lmhead.h")
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(skyrl_lmhead_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = _declared_functions()
+    assert names == sorted(_lib.SIGNATURES), "ctypes table and header disagree"
+    for n in names:
+        assert getattr(lib, n) is not None
+    assert lib.skyrl_lmhead_version() == _lib.ABI_VERSION
+
+
+def test_library_is_in_tree_and_has_no_torch_dependency():
+    assert _lib.lib_path().startswith(ROOT)
+    out = os.popen(f"ldd {_lib.lib_path()}").read()
+    assert "libamdhip64" in out and "torch" not in out and "libc10" not in out
+
+
+def test_strerror_table():
+    for code in (0, -1, -2, -3, -4, -5):
+        assert _lib.strerror(code)
+    assert "unknown" in _lib.strerror(-99)
+
+
+def test_workspace_queries():
+    lib = _lib.load()
+    T, H, V = 16384, 3584, 152064
+    fwd = lib.skyrl_lmhead_fwd_workspace_bytes(T, H, V)
+    assert 3 * 4 * T * 2 * 594 <= fwd <= 3 * 4 * T * 2 * 594 + 4096
+    bwd = lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, 4096)
+    # weight^T + hidden^T + fp32 dHidden + two dz panels; nothing of size T*V
+    expect = 2 * H * V + 2 * H * T + 4 * T * H + 2 * 2 * T * 4096
+    assert expect <= bwd <= expect + 4096
+    assert bwd < 2 * T * V
+    assert lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, 100) == 0  # not a multiple of 256
+    assert lib.skyrl_lmhead_fwd_workspace_bytes(0, H, V) == 0
+
+
+def _call_fwd(lib, **kw):
+    a = dict(hidden=0x1000, ldh=128, weight=0x2000, ldw=128, labels=0x3000, T=4, H=128, V=16, rt=1.0, lp=0x4000, ent=None,
+             lse=None, pz=None, ws=0x10000, wsb=1 << 20, stream=None)
+    a.update(kw)
+    return lib.skyrl_lmhead_fwd(a["hidden"], a["ldh"], a["weight"], a["ldw"], a["labels"], a["T"], a["H"], a["V"], a["rt"],
+                                a["lp"], a["ent"], a["lse"], a["pz"], a["ws"], a["wsb"], a["stream"])
+
+
+def test_forward_argument_errors_are_reported_before_any_launch():
+    lib = _lib.load()
+    assert _call_fwd(lib, hidden=None) == -1
+    assert _call_fwd(lib, lp=None) == -1
+    assert _call_fwd(lib, H=100, ldh=104, ldw=104) == -2  # H not a multiple of 64
+    assert _call_fwd(lib, T=0) == -2
+    assert _call_fwd(lib, ldh=64) == -2  # leading dimension < H
+    assert _call_fwd(lib, hidden=0x1008) == -3
+    assert _call_fwd(lib, ldw=132) == -3
+    assert _call_fwd(lib, ws=None) == -4
+    assert _call_fwd(lib, wsb=16) == -4
+    assert _call_fwd(lib, rt=0.0) == -5
+    assert _call_fwd(lib, rt=float("inf")) == -5
+    assert _call_fwd(lib, rt=float("nan")) == -5
+
+
+def test_backward_argument_errors():
+    lib = _lib.load()
+
+    def call(**kw):
+        a = dict(hidden=0x1000, ldh=128, weight=0x2000, ldw=128, labels=0x3000, lse=0x4000, pz=None, g=0x5000, q=None, T=4,
+                 H=128, V=16, rt=1.0, dh=0x6000, dw=0x7000, acc=0, vc=0, ws=0x10000, wsb=1 << 30, stream=None)
+        a.update(kw)
+        return lib.skyrl_lmhead_bwd(a["hidden"], a["ldh"], a["weight"], a["ldw"], a["labels"], a["lse"], a["pz"], a["g"],
+                                    a["q"], a["T"], a["H"], a["V"], a["rt"], a["dh"], a["dw"], a["acc"], a["vc"], a["ws"],
+                                    a["wsb"], a["stream"])
+
+    assert call(lse=None) == -1
+    assert call(q=0x8000, pz=None) == -1  # an entropy gradient needs row_pz
+    assert call(dh=0x6004) == -3
+    assert call(vc=100) == -5
+    assert call(wsb=1024) == -4
+    assert call(H=96, ldh=96, ldw=96) == -2
+
+
+def test_status_to_exception_mapping():
+    with pytest.raises(ValueError, match="NULL"):
+        _lib.check(-1, "x")
+    with pytest.raises(_lib.LmHeadLibraryError):
+        _lib.check(1, "x")
+    _lib.check(0, "x")
+
+
+def test_ops_refuse_cpu_tensors_and_wrong_dtypes():
+    h = torch.zeros(4, 128, dtype=torch.bfloat16)
+    w = torch.zeros(16, 128, dtype=torch.bfloat16)
+    y = torch.zeros(4, dtype=torch.int64)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        ops.lmhead_fwd(h, w, y, 1.0, True)
+    with pytest.raises(TypeError, match="bf16"):
+        ops.lmhead_fwd(h.float(), w, y, 1.0, True)
+    with pytest.raises(TypeError, match="int64"):
+        ops.lmhead_fwd(h, w, y.int(), 1.0, True)
+    with pytest.raises(ValueError):
+        ops.lmhead_fwd(h, w[:, :64], y, 1.0, True)
+
+
+def test_fake_kernels_give_shapes_without_a_device():
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    with FakeTensorMode():
+        h = torch.empty(12, 128, dtype=torch.bfloat16)
+        w = torch.empty(40, 128, dtype=torch.bfloat16)
+        y = torch.empty(12, dtype=torch.int64)
+        lp, ent, lse, pz = torch.ops.skyrl_amd.lmhead_fwd(h, w, y, 1.0, True)
+        assert lp.shape == (12,) and ent.shape == (12,) and lp.dtype == torch.float32
+        lp, ent, lse, pz = torch.ops.skyrl_amd.lmhead_fwd(h, w, y, 1.0, False)
+        assert ent.numel() == 0 and pz.numel() == 0
+        dh, dw = torch.ops.skyrl_amd.lmhead_bwd(h, w, y, lse, None, lp, None, 1.0, 0)
+        assert dh.shape == (12, 128) and dh.dtype == torch.bfloat16 and dw.shape == (40, 128) and dw.dtype == torch.float32
+
+
+def test_signatures_mirror_the_reference():
+    # FusedLinearChunkedDistributedLogprob.forward / FusedLinearLogprobTriton.forward (model_utils.py:302-313)
+    assert list(inspect.signature(FusedLinearLogprobHip.forward).parameters) == [
+        "ctx", "hidden", "weight", "target", "vocab_start_index", "vocab_end_index", "chunk_size", "tp_group", "inference_only"]
+    # LinearCrossEntropy.forward (fused_linear_logprob_triton.py:1763-1775)
+    assert list(inspect.signature(LinearCrossEntropy.forward).parameters) == [
+        "ctx", "hidden", "weight", "labels", "temperature", "reduction", "dist_process_group"]
+    # model_utils.py:713-725
+    assert list(inspect.signature(model_utils.from_parallel_hidden_to_logprobs).parameters) == [
+        "hidden", "lm_head_weight", "target", "vocab_start_index", "vocab_end_index", "tp_group", "inference_only",
+        "cp_group", "chunk_size", "temperature", "fused_backend"]
+    # model_utils.py:773-789
+    assert list(inspect.signature(model_utils.from_parallel_hidden_to_logprobs_packed_sequences).parameters) == [
+        "hidden", "lm_head_weight", "target", "cu_seqlens_padded", "unpacked_seqlen", "vocab_start_index", "vocab_end_index",
+        "group", "inference_only", "cp_group", "chunk_size", "attention_mask", "sub_seq_lengths", "temperature",
+        "fused_backend"]
+    # model_utils.py:1090-1096
+    assert list(inspect.signature(model_utils._fused_vocab_parallel_entropy_from_hidden).parameters) == [
+        "hidden", "lm_head_weight", "tp_group", "chunk_size", "temperature"]
+    # model_utils.py:431-441 (+ one trailing optional argument)
+    assert list(inspect.signature(model_utils._fused_lm_head_logprob_apply).parameters)[:9] == [
+        "backend", "hidden", "weight", "target", "vocab_start_index", "vocab_end_index", "chunk_size", "tp_group",
+        "inference_only"]
+
+
+def test_linear_cross_entropy_argument_asserts():
+    h = torch.zeros(4, 128, dtype=torch.bfloat16)
+    w = torch.zeros(16, 128, dtype=torch.bfloat16)
+    y = torch.zeros(4, dtype=torch.int64)
+    with pytest.raises(AssertionError, match="temperature must be a float"):
+        linear_cross_entropy(h, w, y, 1, "none", None)
+    with pytest.raises(AssertionError, match="reduction must be a str"):
+        linear_cross_entropy(h, w, y, 1.0, 0, None)
+    with pytest.raises(ValueError, match="Invalid reduction"):
+        linear_cross_entropy(h, w, y, 1.0, "max", None)
+
+
+def test_backend_validation():
+    assert model_utils.validate_fused_backend("hip") == "hip"
+    for bad in ("torch", "triton", "cuda"):
+        with pytest.raises(ValueError):
+            model_utils.validate_fused_backend(bad)
+
+
+def test_packed_index_helpers_match_brute_force():
+    cu = torch.tensor([0, 4, 5, 12, 12, 20])
+    _, tok, si, so, sl = model_utils._packed_sequence_indices(cu, 20, torch.device("cpu"))
+    want_si, want_so = [], []
+    for i in range(len(cu) - 1):
+        for o in range(int(cu[i + 1] - cu[i])):
+            want_si.append(i), want_so.append(o)
+    assert si.tolist() == want_si and so.tolist() == want_so and sl.tolist() == [4, 1, 7, 0, 8]
+    rows, offs, lens = model_utils._packed_subseq_row_indices_offsets_and_lens(
+        torch.tensor([0, 4, 8, 16]), [[3, 4], [7]], torch.device("cpu"))
+    assert rows.tolist() == [0, 0, 1] and offs.tolist() == [0, 4, 0] and lens.tolist() == [3, 4, 7]
+    with pytest.raises(ValueError):
+        model_utils._packed_subseq_row_indices_offsets_and_lens(torch.tensor([0, 4, 8]), [[3], [4], [1]], torch.device("cpu"))
+    with pytest.raises(ValueError):
+        model_utils._packed_subseq_row_indices_offsets_and_lens(torch.tensor([0, 4, 8, 9]), [[3], [4]], torch.device("cpu"))
