@@ -5,13 +5,11 @@
 // backward logits recompute, dHidden and dW.  A workgroup of 8 wavefronts (2 along M x 4 along N) owns a
 // 256x256 tile of C; each wavefront owns 128x64 of it as 4x2 accumulators of v_mfma_f32_32x32x16_bf16.
 //
-// Data path: 16-byte global_load_lds (global -> LDS without a VGPR round trip) into a double-buffered,
-// XOR-swizzled LDS tile; ds_read_b128 fragments; MFMA with fp32 accumulation.
+// Data path: 16-byte global_load_lds (global -> LDS without a VGPR round trip) into a ring of XOR-swizzled LDS
+// stages; ds_read_b128 fragments; MFMA with fp32 accumulation.
 //
-// LDS tile layout (one operand, one stage): 256 rows x 64 k bf16 = 256 x 128 B.  The 16-byte chunk
-// (row, kc) lives at byte  row*128 + ((kc ^ (row & 7)) << 4).  Eight consecutive rows at the same kc then
-// fall into eight different 16-byte slots of a 128-byte line, so the fragment reads (lane -> row) sweep all
-// 32 banks instead of hammering four of them.
+// LDS tile layout (one operand, one stage): 256 rows x BK k bf16.  The 16-byte chunk (row, kc) lives at byte
+// row*ROW_BYTES + ((kc ^ swz(row)) << 4), see swz() below.
 //
 // Accumulator layout of v_mfma_f32_32x32x16 (lane l, register r in 0..15):
 //     m = (r >> 2) * 8 + (l >> 5) * 4 + (r & 3),   n = l & 31
@@ -21,6 +19,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
 
 namespace lmhead {
 
@@ -33,17 +33,48 @@ typedef __attribute__((ext_vector_type(2))) float f32x2;
 
 constexpr int BM = 256;            // tile rows (A rows)
 constexpr int BN = 256;            // tile cols (B rows)
-constexpr int BK = 64;             // k per pipeline stage
-constexpr int NTHREADS = 512;      // 8 wavefronts
-constexpr int WAVES_M = 2, WAVES_N = 4;
+#ifndef LMHEAD_BK
+#define LMHEAD_BK 64
+#endif
+#ifndef LMHEAD_NSTAGES
+#define LMHEAD_NSTAGES 2
+#endif
+constexpr int BK = LMHEAD_BK;      // k per pipeline stage (32 or 64)
+constexpr int NSTAGES = LMHEAD_NSTAGES;
+static_assert(BK == 32 || BK == 64, "BK must be 32 or 64");
+#ifndef LMHEAD_WAVES_N
+#define LMHEAD_WAVES_N 4
+#endif
+constexpr int WAVES_M = 2, WAVES_N = LMHEAD_WAVES_N;
+constexpr int NWAVES = WAVES_M * WAVES_N;
+constexpr int NTHREADS = 64 * NWAVES;
 constexpr int WM = BM / WAVES_M;   // 128
 constexpr int WN = BN / WAVES_N;   // 64
 constexpr int TM = WM / 32;        // 4 MFMA tiles along M per wave
 constexpr int TN = WN / 32;        // 2 MFMA tiles along N per wave
-constexpr int OPERAND_BYTES = BM * BK * 2;         // 32 KiB
-constexpr int STAGE_BYTES = 2 * OPERAND_BYTES;     // 64 KiB (A then B)
-constexpr int NSTAGES = 2;
+constexpr int KSTEPS = BK / 16;                    // MFMA k-steps per stage
+constexpr int ROW_BYTES = BK * 2;                  // one operand row inside a stage
+constexpr int CHUNKS_PER_ROW = ROW_BYTES / 16;     // 16-byte chunks per row
+constexpr int OPERAND_BYTES = BM * ROW_BYTES;      // 16 or 32 KiB
+constexpr int STAGE_BYTES = 2 * OPERAND_BYTES;     // A then B
+constexpr int GROUPS = OPERAND_BYTES / 1024;       // global_load_lds instructions (one wave each) per operand tile
+constexpr int LOADS_PER_TILE = 2 * GROUPS / NWAVES;  // per lane, both operands
 constexpr int LDS_BYTES = NSTAGES * STAGE_BYTES;   // 128 KiB of the CU's 160 KiB
+static_assert(LDS_BYTES <= 160 * 1024, "stages do not fit LDS");
+static_assert(GROUPS % NWAVES == 0, "operand tile must split evenly over the waves");
+#ifndef LMHEAD_SCHED
+#define LMHEAD_SCHED 1
+#endif
+#ifndef LMHEAD_ABL
+#define LMHEAD_ABL 0  // timing-only ablations (wrong results): 1 no global loads, 2 no fragment reads, 4 no barrier
+#endif
+
+// LDS on gfx950 has 64 banks of 4 bytes and serves a ds_read_b128 sixteen lanes (256 B) at a time.  Lanes 0..15 of a
+// fragment read touch 16 consecutive rows at one k-chunk.  XOR-ing the chunk index with a few row bits spreads those
+// sixteen reads over all sixteen 16-byte slots of a 256-byte window: with 128-byte rows (BK = 64) a window holds
+// 2 rows x 8 chunks and the key is (row >> 1) & 7; with 64-byte rows (BK = 32) it holds 4 rows x 4 chunks and the key
+// is (row >> 2) & 3.
+__device__ __forceinline__ int swz(int row) { return BK == 64 ? ((row >> 1) & 7) : ((row >> 2) & 3); }
 
 typedef f32x16 acc_t[TM][TN];
 
@@ -54,21 +85,37 @@ struct Operand {
   int rows;             // total valid rows; rows past the end are clamped (their results are masked later)
 };
 
-// Issue the global->LDS copies of one 256 x 64 operand tile (4 x 16 B per lane).
-// One instruction of one wave fills 64 consecutive 16-byte chunks = 8 LDS rows; the lane picks the global
-// chunk whose swizzled home is its LDS slot.
+// Issue the global->LDS copies of one 256 x BK operand tile (16 B per lane and instruction).
+// One instruction of one wave fills 64 consecutive 16-byte chunks of LDS; the lane picks the global chunk whose
+// swizzled home is its LDS slot.
 __device__ __forceinline__ void issue_operand_loads(const Operand& op, int k0, char* lds_operand, int wave, int lane) {
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int grp = j * 8 + wave;          // 32 groups of 64 chunks
+  for (int j = 0; j < GROUPS / NWAVES; ++j) {
+    const int grp = j * NWAVES + wave;
     const int p = grp * 64 + lane;         // chunk slot in LDS
-    const int row = p >> 3;
-    const int kc = (p & 7) ^ (row & 7);    // global chunk that lives in this slot
+    const int row = p / CHUNKS_PER_ROW;
+    const int kc = (p % CHUNKS_PER_ROW) ^ swz(row);  // global chunk that lives in this slot
     int grow = op.row0 + row;
     grow = grow < op.rows ? grow : op.rows - 1;
     const uint16_t* src = op.ptr + (size_t)grow * (size_t)op.ld + (size_t)(k0 + kc * 8);
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                      (__attribute__((address_space(3))) void*)(lds_operand + grp * 1024), 16, 0, 0);
+  }
+}
+
+// Wait until at most N of this lane's global->LDS copies are still in flight and all of its LDS reads have returned,
+// then meet the rest of the workgroup.  The "memory" clobber keeps the compiler from moving LDS accesses across it.
+template <int N>
+__device__ __forceinline__ void wait_copies_and_barrier() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+__device__ __forceinline__ void wait_copies_and_barrier(int tiles_in_flight) {
+  switch (tiles_in_flight) {
+    case 0: wait_copies_and_barrier<0>(); break;
+    case 1: wait_copies_and_barrier<1 * LOADS_PER_TILE>(); break;
+    case 2: wait_copies_and_barrier<(NSTAGES > 3 ? 2 : 0) * LOADS_PER_TILE>(); break;
+    default: wait_copies_and_barrier<(NSTAGES > 4 ? 3 : 0) * LOADS_PER_TILE>(); break;
   }
 }
 
@@ -81,8 +128,28 @@ __device__ __forceinline__ void zero_acc(acc_t& acc) {
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 }
 
-// acc += A[a.row0 : +256, k_begin : k_begin + nk*64] * B[b.row0 : +256, same k]^T
+__device__ __forceinline__ void read_frags(const char* stage, const int (&a_off)[TM], const int (&b_off)[TN], int kc_sw,
+                                           bf16x8 (&af)[TM], bf16x8 (&bfr)[TN]) {
+#pragma unroll
+  for (int i = 0; i < TM; ++i) af[i] = *(const bf16x8*)(stage + a_off[i] + kc_sw);
+#pragma unroll
+  for (int j = 0; j < TN; ++j) bfr[j] = *(const bf16x8*)(stage + b_off[j] + kc_sw);
+}
+
+__device__ __forceinline__ void mfma_step(const bf16x8 (&af)[TM], const bf16x8 (&bfr)[TN], acc_t& acc) {
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+}
+
+// acc += A[a.row0 : +256, k_begin : k_begin + nk*BK] * B[b.row0 : +256, same k]^T
 // Every thread of the workgroup must call this with identical arguments (it contains barriers).
+//
+// Pipeline: global->LDS copies run NSTAGES-1 k-tiles ahead through a ring of NSTAGES LDS stages; LDS->register
+// fragment reads run one 16-k step ahead (two fragment sets).  The one barrier per k-tile sits between the last
+// fragment read of a tile and the MFMAs that consume it, so the matrix pipe has a full step of work queued while
+// the copies of a later tile are issued and the first fragments of the next tile come back from LDS.
 __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int k_begin, int nk, char* lds, acc_t& acc) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -90,46 +157,76 @@ __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int
   const int wm = wave / WAVES_N;
   const int wn = wave % WAVES_N;
 
-  // Per-lane fragment addresses inside an operand tile (k-step 0); k-step s XORs in (2*s) << 4 ... the
-  // swizzle is (kc ^ (row & 7)) << 4 with kc = 2*s + (lane >> 5), and row & 7 == lane & 7 for every tile.
+  // Per-lane fragment addresses inside a stage; k-step s XORs in the swizzled chunk (2*s + lane/32).
   const int lrow = lane & 31;
-  const int sw = lane & 7;
+  const int sw = swz(lrow);  // every fragment row is lrow plus a multiple of 32, so the swizzle depends on the lane only
   const int khalf = lane >> 5;
   int a_off[TM], b_off[TN];
 #pragma unroll
-  for (int i = 0; i < TM; ++i) a_off[i] = (wm * WM + i * 32 + lrow) * 128;
+  for (int i = 0; i < TM; ++i) a_off[i] = (wm * WM + i * 32 + lrow) * ROW_BYTES;
 #pragma unroll
-  for (int j = 0; j < TN; ++j) b_off[j] = OPERAND_BYTES + (wn * WN + j * 32 + lrow) * 128;
+  for (int j = 0; j < TN; ++j) b_off[j] = OPERAND_BYTES + (wn * WN + j * 32 + lrow) * ROW_BYTES;
+  int kc_sw[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) kc_sw[ks] = ((ks * 2 + khalf) ^ sw) << 4;
 
-  issue_operand_loads(a, k_begin, lds, wave, lane);
-  issue_operand_loads(b, k_begin, lds + OPERAND_BYTES, wave, lane);
+  bf16x8 af[2][TM], bfr[2][TN];
 
-  for (int kt = 0; kt < nk; ++kt) {
-    char* cur = lds + (kt & 1) * STAGE_BYTES;
-    char* nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
-    // Tile kt has landed in every wave's share of LDS, and every wave has finished reading the other stage.
-    __syncthreads();
-    if (kt + 1 < nk) {
-      const int k0 = k_begin + (kt + 1) * BK;
-      issue_operand_loads(a, k0, nxt, wave, lane);
-      issue_operand_loads(b, k0, nxt + OPERAND_BYTES, wave, lane);
+  // Prologue: fill the ring (tiles 0 .. NSTAGES-1), wait for tile 0.
+  const int pre = nk < NSTAGES ? nk : NSTAGES;
+  for (int t = 0; t < pre; ++t) {
+    issue_operand_loads(a, k_begin + t * BK, lds + t * STAGE_BYTES, wave, lane);
+    issue_operand_loads(b, k_begin + t * BK, lds + t * STAGE_BYTES + OPERAND_BYTES, wave, lane);
+  }
+  wait_copies_and_barrier(pre - 1);
+  read_frags(lds, a_off, b_off, kc_sw[0], af[0], bfr[0]);
+
+  int stage = 0;  // ring slot of tile kt
+  for (int kt = 0; kt + 1 < nk; ++kt) {
+    char* cur = lds + stage * STAGE_BYTES;
+    const int next_stage = stage + 1 == NSTAGES ? 0 : stage + 1;
+    char* nxt = lds + next_stage * STAGE_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      if (LMHEAD_ABL & 2) {
+      } else if (ks + 1 < KSTEPS) {
+        read_frags(cur, a_off, b_off, kc_sw[ks + 1], af[(ks + 1) & 1], bfr[(ks + 1) & 1]);
+      } else {
+        // Tiles kt+1 .. min(nk-1, kt+NSTAGES-1) have been issued; all but tile kt+1 may stay in flight.  After the
+        // barrier every wave's copies of tile kt+1 have landed and every wave is done reading tile kt, whose stage
+        // the copies of tile kt+NSTAGES may now overwrite.
+        const int last_issued = nk - 1 < kt + NSTAGES - 1 ? nk - 1 : kt + NSTAGES - 1;
+        wait_copies_and_barrier(last_issued - (kt + 1));
+        if (kt + NSTAGES < nk && !(LMHEAD_ABL & 1)) {
+          const int k0 = k_begin + (kt + NSTAGES) * BK;
+          issue_operand_loads(a, k0, cur, wave, lane);
+          issue_operand_loads(b, k0, cur + OPERAND_BYTES, wave, lane);
+        }
+        read_frags(nxt, a_off, b_off, kc_sw[0], af[(ks + 1) & 1], bfr[(ks + 1) & 1]);
+      }
+      mfma_step(af[ks & 1], bfr[ks & 1], acc);
+#if LMHEAD_SCHED == 1
+      // one LDS read behind each of the first MFMAs of the step
+#pragma unroll
+      for (int x = 0; x < TM + TN; ++x) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - TM - TN, 0);
+#endif
     }
+    stage = next_stage;
+  }
+  {  // last tile: nothing left to prefetch
+    char* cur = lds + stage * STAGE_BYTES;
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
-      const int kc_sw = ((ks * 2 + khalf) ^ sw) << 4;
-      bf16x8 af[TM], bfr[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i) af[i] = *(const bf16x8*)(cur + a_off[i] + kc_sw);
-#pragma unroll
-      for (int j = 0; j < TN; ++j) bfr[j] = *(const bf16x8*)(cur + b_off[j] + kc_sw);
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      if (ks + 1 < KSTEPS) read_frags(cur, a_off, b_off, kc_sw[ks + 1], af[(ks + 1) & 1], bfr[(ks + 1) & 1]);
+      mfma_step(af[ks & 1], bfr[ks & 1], acc);
     }
   }
   // The caller may reuse LDS (or start another mainloop) only after all waves are done reading.
-  __syncthreads();
+  wait_copies_and_barrier<0>();
 }
 
 // Workgroup id -> tile coordinates.

@@ -294,24 +294,44 @@ __global__ __launch_bounds__(NTHREADS) void lmhead_bwd_dz_tiles(
 
 // ------------------------------------------------------------------------------------------------------------
 // Plain NT GEMM with an fp32 / bf16 store epilogue:  C[M,N] (+)= A[M,K] . B[N,K]^T.
-//   load_c     add the existing fp32 C before storing (accumulation across vocab chunks / micro-batches)
-//   Cf != 0    store fp32;   Cb != 0  store bf16 (round-to-nearest-even)
+//   Cin != 0   add the existing fp32 C before storing (accumulation across vocab chunks / micro-batches)
+//   Cf  != 0   store fp32;   Cb != 0  store bf16 (round-to-nearest-even)
+// One launch carries up to two independent problems (workgroups [0, tiles0) work on p0, the rest on p1): the dHidden
+// and dWeight products of a vocab chunk have no dependency on each other, and together they fill the 256 CUs in whole
+// rounds where each alone leaves a partial last round.
 // ------------------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(NTHREADS) void gemm_nt_store(const uint16_t* __restrict__ A, int lda, int a_rows,
-                                                          const uint16_t* __restrict__ B, int ldb, int b_rows, int nk,
-                                                          int M, int N, const float* __restrict__ Cin, float* __restrict__ Cf,
-                                                          uint16_t* __restrict__ Cb, int ldc) {
+struct GemmArgs {
+  const uint16_t* A;
+  int lda, a_rows;
+  const uint16_t* B;
+  int ldb, b_rows;
+  int nk, M, N;
+  const float* Cin;
+  float* Cf;
+  uint16_t* Cb;
+  int ldc;
+};
+
+__global__ __launch_bounds__(NTHREADS) void gemm_nt_store(const GemmArgs p0, const GemmArgs p1, int tiles0) {
   __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
+  const bool second = (int)blockIdx.x >= tiles0;
+  const GemmArgs& p = second ? p1 : p0;
+  const int bid = second ? (int)blockIdx.x - tiles0 : (int)blockIdx.x;
+  const int M = p.M, N = p.N;
   const int tiles_m = (M + BM - 1) / BM;
   const int tiles_n = (N + BN - 1) / BN;
   int tm, tn;
-  tile_coords(blockIdx.x, tiles_m, tiles_n, kGroupM, tm, tn);
-  Operand a{A, lda, tm * BM, a_rows};
-  Operand b{B, ldb, tn * BN, b_rows};
+  tile_coords(bid, tiles_m, tiles_n, kGroupM, tm, tn);
+  Operand a{p.A, p.lda, tm * BM, p.a_rows};
+  Operand b{p.B, p.ldb, tn * BN, p.b_rows};
   acc_t acc;
   zero_acc(acc);
-  mainloop(a, b, 0, nk, lds, acc);
+  mainloop(a, b, 0, p.nk, lds, acc);
 
+  const float* __restrict__ Cin = p.Cin;
+  float* __restrict__ Cf = p.Cf;
+  uint16_t* __restrict__ Cb = p.Cb;
+  const int ldc = p.ldc;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int lrow = lane & 31, khalf = lane >> 5;
@@ -387,9 +407,9 @@ __global__ __launch_bounds__(256) void transpose_bf16(const uint16_t* __restrict
 // ------------------------------------------------------------------------------------------------------------
 // Optional per-kernel timing: while a profile is open on the calling thread every launch below is bracketed by a pair of
 // HIP events on the launch stream.  Closed profiles cost one thread-local load per launch.
-enum KernelKind { kFwdTiles = 0, kFwdMerge, kTranspose, kBwdDzTiles, kGemmDHidden, kGemmDWeight, kNumKernelKinds };
+enum KernelKind { kFwdTiles = 0, kFwdMerge, kTranspose, kBwdDzTiles, kGemmGrad, kNumKernelKinds };
 const char* const kKernelNames[kNumKernelKinds] = {"lmhead_fwd_tiles", "lmhead_fwd_merge", "transpose_bf16",
-                                                   "lmhead_bwd_dz_tiles", "gemm_nt_store(dHidden)", "gemm_nt_store(dWeight)"};
+                                                   "lmhead_bwd_dz_tiles", "gemm_nt_store"};
 struct Profile {
   struct Rec {
     int kind;
@@ -468,13 +488,17 @@ BwdWorkspace carve_bwd(void* ws, int64_t T, int64_t H, int64_t V, int64_t vc) {
   return w;
 }
 
-hipError_t launch_gemm(int kind, hipStream_t s, const uint16_t* A, int64_t lda, int64_t a_rows, const uint16_t* B, int64_t ldb,
-                       int64_t b_rows, int64_t nk, int64_t M, int64_t N, const float* Cin, float* Cf, uint16_t* Cb,
-                       int64_t ldc) {
-  const unsigned tiles = (unsigned)(((M + BM - 1) / BM) * ((N + BN - 1) / BN));
+GemmArgs make_gemm(const uint16_t* A, int64_t lda, int64_t a_rows, const uint16_t* B, int64_t ldb, int64_t b_rows, int64_t nk,
+                   int64_t M, int64_t N, const float* Cin, float* Cf, uint16_t* Cb, int64_t ldc) {
+  return GemmArgs{A, (int)lda, (int)a_rows, B, (int)ldb, (int)b_rows, (int)nk, (int)M, (int)N, Cin, Cf, Cb, (int)ldc};
+}
+
+unsigned gemm_tiles(const GemmArgs& g) { return (unsigned)(((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN)); }
+
+hipError_t launch_gemm_pair(int kind, hipStream_t s, const GemmArgs& p0, const GemmArgs& p1) {
+  const unsigned t0 = gemm_tiles(p0), t1 = gemm_tiles(p1);
   Timed timed(kind, s);
-  hipLaunchKernelGGL(gemm_nt_store, dim3(tiles), dim3(NTHREADS), 0, s, A, (int)lda, (int)a_rows, B, (int)ldb, (int)b_rows,
-                     (int)nk, (int)M, (int)N, Cin, Cf, Cb, (int)ldc);
+  hipLaunchKernelGGL(gemm_nt_store, dim3(t0 + t1), dim3(NTHREADS), 0, s, p0, p1, (int)t0);
   return hipGetLastError();
 }
 
@@ -612,17 +636,16 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
     if ((e = hipGetLastError()) != hipSuccess) return (int)e;
 
     // dHidden[T, H] (+)= D[T, vcw] . weight[vc0 : vc0 + vcw, :]    (B operand = weight^T rows, k offset vc0)
+    // dW[vc0 : vc0 + rows, :] (+)= D^T[vcw, Tpad] . hidden          (B operand = hidden^T rows)
     const bool first = ci == 0, last = ci == nchunks - 1;
-    e = launch_gemm(kGemmDHidden, s, w.D, vcw, Tpad, w.Wt + vc0, Vpad, H, vcw / BK, T, H,
-                    first ? (const float*)nullptr : (const float*)w.dHacc, last ? (float*)nullptr : w.dHacc,
-                    last ? (uint16_t*)d_hidden : (uint16_t*)nullptr, H);
-    if (e != hipSuccess) return (int)e;
-
-    // dW[vc0 : vc0 + rows, :] (+)= D^T[vcw, Tpad] . hidden   (B operand = hidden^T rows)
     const int64_t rows = (V - vc0) < vcw ? (V - vc0) : vcw;
     float* dWc = d_weight + (size_t)vc0 * (size_t)H;
-    e = launch_gemm(kGemmDWeight, s, w.DT, Tpad, vcw, w.Ht, Tpad, H, Tpad / BK, rows, H,
-                    accumulate_dw ? (const float*)dWc : (const float*)nullptr, dWc, (uint16_t*)nullptr, H);
+    const GemmArgs gh = make_gemm(w.D, vcw, Tpad, w.Wt + vc0, Vpad, H, vcw / BK, T, H,
+                                  first ? (const float*)nullptr : (const float*)w.dHacc, last ? (float*)nullptr : w.dHacc,
+                                  last ? (uint16_t*)d_hidden : (uint16_t*)nullptr, H);
+    const GemmArgs gw = make_gemm(w.DT, Tpad, vcw, w.Ht, Tpad, H, Tpad / BK, rows, H,
+                                  accumulate_dw ? (const float*)dWc : (const float*)nullptr, dWc, (uint16_t*)nullptr, H);
+    e = launch_gemm_pair(kGemmGrad, s, gh, gw);
     if (e != hipSuccess) return (int)e;
   }
   return SKYRL_LMHEAD_OK;
