@@ -31,9 +31,10 @@ if ROOT not in sys.path:
 PEAK_BF16_DENSE_FLOPS = 2.5e15  # MI355X dense bf16 MFMA
 METRIC = "fused LM-head fwd+bwd tokens/sec on 1 MI355X; % bf16 MFMA peak"
 
-# HBM bytes per gemm_nt_store launch from `rocprofv3 --pmc` (FETCH_SIZE, then WRITE_SIZE) scaled by a copy kernel of known size;
-# None until measured for the workload.  Keyed by config name.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {}
+# Bytes beyond L2 per gemm_nt_store launch from two `rocprofv3 --pmc` passes (FETCH_SIZE, then WRITE_SIZE), each scaled by what
+# the same counter reads for the 1 GiB copy of --copy-probe (x2048 and x1024 bytes per count).  Not measurable live; None for
+# workloads that have not been profiled.  Keyed by config name.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"qwen2.5-7b-fwdbwd": 8172173164}
 
 
 def cpu_baseline(cfg, sample_tokens: int):
@@ -75,6 +76,9 @@ def main() -> int:
     ap.add_argument("--vocab-chunk", type=int, default=0)
     ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one plain 1 GiB device-to-device copy (a kernel of known HBM traffic) so that rocprofv3 "
+                         "--pmc FETCH_SIZE / WRITE_SIZE readings of the same run can be scaled to bytes")
     args = ap.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -128,6 +132,13 @@ def main() -> int:
                                       g.data_ptr(), ptr(q), T, H, V, rcp_t, d_hidden.data_ptr(), d_weight.data_ptr(), 0,
                                       args.vocab_chunk, ws_b.data_ptr(), ws_b.numel(), stream)
             _lib.check(st, "skyrl_lmhead_bwd")
+
+    if args.copy_probe:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # 1 GiB read + 1 GiB written
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step()
