@@ -5,7 +5,7 @@
 // backward logits recompute, dHidden and dW.  A workgroup of 8 wavefronts (2 along M x 4 along N) owns a
 // 256x256 tile of C; each wavefront owns 128x64 of it as 4x2 accumulators of v_mfma_f32_32x32x16_bf16.
 //
-// Data path: 16-byte global_load_lds (global -> LDS without a VGPR round trip) into a ring of XOR-swizzled LDS
+// Data path: 16-byte global_load_lds (global -> LDS without a VGPR round trip) into two XOR-swizzled LDS
 // stages; ds_read_b128 fragments; MFMA with fp32 accumulation.
 //
 // LDS tile layout (one operand, one stage): 256 rows x BK k bf16.  The 16-byte chunk (row, kc) lives at byte
@@ -33,15 +33,8 @@ typedef __attribute__((ext_vector_type(2))) float f32x2;
 
 constexpr int BM = 256;            // tile rows (A rows)
 constexpr int BN = 256;            // tile cols (B rows)
-#ifndef LMHEAD_BK
-#define LMHEAD_BK 64
-#endif
-#ifndef LMHEAD_NSTAGES
-#define LMHEAD_NSTAGES 2
-#endif
-constexpr int BK = LMHEAD_BK;      // k per pipeline stage (32 or 64)
-constexpr int NSTAGES = LMHEAD_NSTAGES;
-static_assert(BK == 32 || BK == 64, "BK must be 32 or 64");
+constexpr int BK = 64;             // k per pipeline stage: 128-byte rows keep the direct-to-LDS copies at full rate
+constexpr int NSTAGES = 2;         // two 64 KiB stages; a third does not fit the CU's 160 KiB
 #ifndef LMHEAD_WAVES_N
 #define LMHEAD_WAVES_N 4
 #endif
@@ -61,12 +54,11 @@ constexpr int GROUPS = OPERAND_BYTES / 1024;       // global_load_lds instructio
 constexpr int LOADS_PER_TILE = 2 * GROUPS / NWAVES;  // per lane, both operands
 constexpr int LDS_BYTES = NSTAGES * STAGE_BYTES;   // 128 KiB of the CU's 160 KiB
 static_assert(LDS_BYTES <= 160 * 1024, "stages do not fit LDS");
-static_assert(GROUPS % NWAVES == 0, "operand tile must split evenly over the waves");
 #ifndef LMHEAD_SCHED
 #define LMHEAD_SCHED 1
 #endif
 #ifndef LMHEAD_ABL
-#define LMHEAD_ABL 0  // timing-only ablations (wrong results): 1 no global loads, 2 no fragment reads, 4 no barrier
+#define LMHEAD_ABL 0  // timing-only ablations (wrong results): 1 no global loads, 2 no fragment reads, 8 wait one tile late
 #endif
 
 // LDS on gfx950 has 64 banks of 4 bytes and serves a ds_read_b128 sixteen lanes (256 B) at a time.  Lanes 0..15 of a
@@ -110,15 +102,6 @@ __device__ __forceinline__ void wait_copies_and_barrier() {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
 }
-__device__ __forceinline__ void wait_copies_and_barrier(int tiles_in_flight) {
-  switch (tiles_in_flight) {
-    case 0: wait_copies_and_barrier<0>(); break;
-    case 1: wait_copies_and_barrier<1 * LOADS_PER_TILE>(); break;
-    case 2: wait_copies_and_barrier<(NSTAGES > 3 ? 2 : 0) * LOADS_PER_TILE>(); break;
-    default: wait_copies_and_barrier<(NSTAGES > 4 ? 3 : 0) * LOADS_PER_TILE>(); break;
-  }
-}
-
 __device__ __forceinline__ void zero_acc(acc_t& acc) {
 #pragma unroll
   for (int i = 0; i < TM; ++i)
@@ -146,10 +129,10 @@ __device__ __forceinline__ void mfma_step(const bf16x8 (&af)[TM], const bf16x8 (
 // acc += A[a.row0 : +256, k_begin : k_begin + nk*BK] * B[b.row0 : +256, same k]^T
 // Every thread of the workgroup must call this with identical arguments (it contains barriers).
 //
-// Pipeline: global->LDS copies run NSTAGES-1 k-tiles ahead through a ring of NSTAGES LDS stages; LDS->register
-// fragment reads run one 16-k step ahead (two fragment sets).  The one barrier per k-tile sits between the last
-// fragment read of a tile and the MFMAs that consume it, so the matrix pipe has a full step of work queued while
-// the copies of a later tile are issued and the first fragments of the next tile come back from LDS.
+// Pipeline: global->LDS copies run one k-tile ahead (two LDS stages); LDS->register fragment reads run one 16-k step
+// ahead (two fragment sets).  The one barrier per k-tile sits between the last fragment read of a tile and the MFMAs
+// that consume it, so the matrix pipe has a full step of work queued while the copies of tile kt+2 are issued and the
+// first fragments of tile kt+1 come back from LDS.
 __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int k_begin, int nk, char* lds, acc_t& acc) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -172,33 +155,34 @@ __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int
 
   bf16x8 af[2][TM], bfr[2][TN];
 
-  // Prologue: fill the ring (tiles 0 .. NSTAGES-1), wait for tile 0.
-  const int pre = nk < NSTAGES ? nk : NSTAGES;
-  for (int t = 0; t < pre; ++t) {
-    issue_operand_loads(a, k_begin + t * BK, lds + t * STAGE_BYTES, wave, lane);
-    issue_operand_loads(b, k_begin + t * BK, lds + t * STAGE_BYTES + OPERAND_BYTES, wave, lane);
+  // Prologue: tiles 0 and 1 in flight, wait for tile 0.
+  issue_operand_loads(a, k_begin, lds, wave, lane);
+  issue_operand_loads(b, k_begin, lds + OPERAND_BYTES, wave, lane);
+  if (nk > 1) {
+    issue_operand_loads(a, k_begin + BK, lds + STAGE_BYTES, wave, lane);
+    issue_operand_loads(b, k_begin + BK, lds + STAGE_BYTES + OPERAND_BYTES, wave, lane);
+    wait_copies_and_barrier<LOADS_PER_TILE>();
+  } else {
+    wait_copies_and_barrier<0>();
   }
-  wait_copies_and_barrier(pre - 1);
   read_frags(lds, a_off, b_off, kc_sw[0], af[0], bfr[0]);
 
-  int stage = 0;  // ring slot of tile kt
-  for (int kt = 0; kt + 1 < nk; ++kt) {
-    char* cur = lds + stage * STAGE_BYTES;
-    const int next_stage = stage + 1 == NSTAGES ? 0 : stage + 1;
-    char* nxt = lds + next_stage * STAGE_BYTES;
+  // Three copies of the tile step (steady state, second-to-last, last) instead of conditions inside one loop body: a
+  // branch that joins a path with outstanding LDS reads makes the compiler wait for all of them.
+  auto tile_step = [&](int kt, auto has_next, auto load_next2) {
+    char* cur = lds + (kt & 1) * STAGE_BYTES;
+    char* nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       if (LMHEAD_ABL & 2) {
       } else if (ks + 1 < KSTEPS) {
         read_frags(cur, a_off, b_off, kc_sw[ks + 1], af[(ks + 1) & 1], bfr[(ks + 1) & 1]);
-      } else {
-        // Tiles kt+1 .. min(nk-1, kt+NSTAGES-1) have been issued; all but tile kt+1 may stay in flight.  After the
-        // barrier every wave's copies of tile kt+1 have landed and every wave is done reading tile kt, whose stage
-        // the copies of tile kt+NSTAGES may now overwrite.
-        const int last_issued = nk - 1 < kt + NSTAGES - 1 ? nk - 1 : kt + NSTAGES - 1;
-        wait_copies_and_barrier(last_issued - (kt + 1));
-        if (kt + NSTAGES < nk && !(LMHEAD_ABL & 1)) {
-          const int k0 = k_begin + (kt + NSTAGES) * BK;
+      } else if (has_next) {
+        // All of this wave's reads of `cur` are complete and its copies into `nxt` have landed; after the barrier that
+        // holds for every wave, so `cur` may be overwritten (tile kt+2) and `nxt` may be read.
+        if (LMHEAD_ABL & 8) wait_copies_and_barrier<LOADS_PER_TILE>(); else wait_copies_and_barrier<0>();
+        if (load_next2 && !(LMHEAD_ABL & 1)) {
+          const int k0 = k_begin + (kt + 2) * BK;
           issue_operand_loads(a, k0, cur, wave, lane);
           issue_operand_loads(b, k0, cur + OPERAND_BYTES, wave, lane);
         }
@@ -207,24 +191,24 @@ __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int
       mfma_step(af[ks & 1], bfr[ks & 1], acc);
 #if LMHEAD_SCHED == 1
       // one LDS read behind each of the first MFMAs of the step
+      if (ks + 1 < KSTEPS || has_next) {
 #pragma unroll
-      for (int x = 0; x < TM + TN; ++x) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        for (int x = 0; x < TM + TN; ++x) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - TM - TN, 0);
       }
-      __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - TM - TN, 0);
 #endif
     }
-    stage = next_stage;
+  };
+  int kt = 0;
+  for (; kt + 2 < nk; ++kt) tile_step(kt, std::true_type{}, std::true_type{});
+  if (kt + 1 < nk) {
+    tile_step(kt, std::true_type{}, std::false_type{});
+    ++kt;
   }
-  {  // last tile: nothing left to prefetch
-    char* cur = lds + stage * STAGE_BYTES;
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-      if (ks + 1 < KSTEPS) read_frags(cur, a_off, b_off, kc_sw[ks + 1], af[(ks + 1) & 1], bfr[(ks + 1) & 1]);
-      mfma_step(af[ks & 1], bfr[ks & 1], acc);
-    }
-  }
+  tile_step(kt, std::false_type{}, std::false_type{});
   // The caller may reuse LDS (or start another mainloop) only after all waves are done reading.
   wait_copies_and_barrier<0>();
 }
