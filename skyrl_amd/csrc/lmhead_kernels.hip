@@ -89,6 +89,7 @@ __global__ __launch_bounds__(NTHREADS) void lmhead_fwd_tiles(const uint16_t* __r
   Operand b{Hd, ldh, tn * BN, T};
   acc_t acc;
   zero_acc(acc);
+  prefetch_first_tiles(a, b, 0, H / BK, lds);
   mainloop(a, b, 0, H / BK, lds, acc);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -230,6 +231,7 @@ __global__ __launch_bounds__(NTHREADS) void lmhead_bwd_dz_tiles(
   Operand b{Hd, ldh, tn * BN, T};
   acc_t acc;
   zero_acc(acc);
+  prefetch_first_tiles(a, b, 0, H / BK, lds);
   mainloop(a, b, 0, H / BK, lds, acc);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -326,6 +328,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_nt_store(const GemmArgs p0, con
   Operand b{p.B, p.ldb, tn * BN, p.b_rows};
   acc_t acc;
   zero_acc(acc);
+  prefetch_first_tiles(a, b, 0, p.nk, lds);
   mainloop(a, b, 0, p.nk, lds, acc);
 
   const float* __restrict__ Cin = p.Cin;
