@@ -9,8 +9,8 @@ log-probabilities and the entropy).  The step goes through the C ABI (``skyrl_lm
 as the torch custom ops call it.  One JSON line is printed:
 
   value / unit   tokens per second of forward + backward (whole job; one GPU)
-  roofline       the dominant kernel (the gradient GEMM ``gemm_nt_store``, 4*T*V*H of the 8*T*V*H flop) against the dense bf16
-                 MFMA peak of 2.5 PFLOP/s; its time is measured live with HIP events on the launch stream
+  roofline       the dominant kernel (``lmhead_bwd_chunk``: logits recompute + dHidden + dWeight, 6*T*V*H of the 8*T*V*H flop)
+                 against the dense bf16 MFMA peak of 2.5 PFLOP/s; its time is measured live with HIP events on the launch stream
   step_roofline  the whole step (8*T*V*H algorithmic flop / step time) against the same peak
   kernels        live HIP-event time per kernel and step
   cpu_baseline   the CPU restatement of the reference's torch implementation, timed on this host on a bounded sample
@@ -31,10 +31,10 @@ if ROOT not in sys.path:
 PEAK_BF16_DENSE_FLOPS = 2.5e15  # MI355X dense bf16 MFMA
 METRIC = "fused LM-head fwd+bwd tokens/sec on 1 MI355X; % bf16 MFMA peak"
 
-# Bytes beyond L2 per gemm_nt_store launch from two `rocprofv3 --pmc` passes (FETCH_SIZE, then WRITE_SIZE), each scaled by what
+# Bytes beyond L2 per lmhead_bwd_chunk launch from two `rocprofv3 --pmc` passes (FETCH_SIZE, then WRITE_SIZE), each scaled by what
 # the same counter reads for the 1 GiB copy of --copy-probe (x2048 and x1024 bytes per count).  Not measurable live; None for
 # workloads that have not been profiled.  Keyed by config name.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"qwen2.5-7b-fwdbwd": 8172173164}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {}
 
 
 def cpu_baseline(cfg, sample_tokens: int):
@@ -162,11 +162,13 @@ def main() -> int:
                      "unit": "TFLOP/s"}
     step_roofline["frac"] = step_roofline["achieved"] / step_roofline["peak"]
 
-    # Dominant kernel.  With a backward pass it is gemm_nt_store (dHidden and dWeight launches, 2*T*V*H flop each in total);
-    # forward-only workloads are all lmhead_fwd_tiles.
+    # Dominant kernel: lmhead_bwd_chunk with a backward pass; forward-only workloads are all lmhead_fwd_tiles.
     if cfg.backward:
-        k = kernels["gemm_nt_store"]  # one launch per vocab chunk carries that chunk's dHidden and dWeight products
-        dom_name, dom_ms, dom_launches, dom_flop = "gemm_nt_store", k["ms_per_step"], k["launches_per_step"], 4.0 * T * V * H
+        # lmhead_bwd_chunk: every backward launch (per vocab chunk one with the dz tiles, one with the gradient GEMM tiles);
+        # over a step the launches add up to the logits recompute, dHidden and dWeight = 6*T*V*H flop.
+        ks = [kernels[n] for n in ("lmhead_bwd_chunk[dz]", "lmhead_bwd_chunk[gemm]")]  # the same kernel, two kinds of launch
+        dom_name, dom_flop = "lmhead_bwd_chunk", 6.0 * T * V * H
+        dom_ms, dom_launches = sum(k["ms_per_step"] for k in ks), sum(k["launches_per_step"] for k in ks)
     else:
         k = kernels["lmhead_fwd_tiles"]
         dom_name, dom_ms, dom_launches, dom_flop = "lmhead_fwd_tiles", k["ms_per_step"], k["launches_per_step"], 2.0 * T * V * H

@@ -8,9 +8,9 @@
 //                      fp32 dot product hidden[t] . weight[label], writes logprob / entropy / lse / pz.
 // Backward (6*T*V*H flop), looped over vocab chunks of `vocab_chunk` columns:
 //   transpose_bf16     weight^T and hidden^T once per call, so that every contraction is K-contiguous.
-//   lmhead_bwd_dz_tiles recomputes a logits tile and forms dz in registers; writes it (bf16) row-major and
-//                      transposed into two chunk-sized panels.
-//   gemm_nt_store      dHidden (+)= dz . weight   and   dW[chunk] = dz^T . hidden, fp32 accumulation.
+//   lmhead_bwd_chunk   dz tiles: recompute a logits tile and form dz in registers; write it (bf16) row-major and
+//                      transposed into two chunk-sized panels.  GEMM tiles: dHidden (+)= dz . weight and
+//                      dW[chunk] = dz^T . hidden, fp32 accumulation.
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdint.h>
@@ -26,7 +26,13 @@ namespace {
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
-constexpr int kGroupM = 8;
+#ifndef LMHEAD_GROUP_M
+#define LMHEAD_GROUP_M 8
+#endif
+constexpr int kGroupM = LMHEAD_GROUP_M;
+// Scratch matrices get 64 extra elements (128 B) per row: with a power-of-two row pitch (T' = 16384 -> 32 KiB) the 256 rows of
+// an operand tile would all start in the same L2 channel and set.
+constexpr int kLdPad = 64;
 
 __host__ __device__ inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
@@ -217,15 +223,40 @@ __global__ __launch_bounds__(256) void lmhead_fwd_merge(const float* __restrict_
 // written as  p * (c0 + c1*x) + onehot*g/temperature  with x the raw dot product.
 // Out-of-range labels get no one-hot term but keep -p*g (model_utils.py:405-411).
 // ------------------------------------------------------------------------------------------------------------
+struct DzArgs {
+  const uint16_t* W;
+  int ldw;
+  const uint16_t* Hd;
+  int ldh;
+  int T, H, V;
+  float rcp_temp;
+  const int64_t* labels;
+  const float* row_lse;
+  const float* row_pz;
+  const float* dlogprobs;
+  const float* dentropy;
+  int vc0, tiles_m, tiles_n;  // first vocab row of the chunk; tiles of the chunk panel along vocab and tokens
+  uint16_t* D;                // [tiles_n * 256, ldd]  dz, token-major
+  int ldd;
+  uint16_t* DT;               // [tiles_m * 256, lddt] dz, vocab-major
+  int lddt;
+};
+
 template <bool ENTGRAD>
-__global__ __launch_bounds__(NTHREADS) void lmhead_bwd_dz_tiles(
-    const uint16_t* __restrict__ W, int ldw, const uint16_t* __restrict__ Hd, int ldh, int T, int H, int V, float rcp_temp,
-    const int64_t* __restrict__ labels, const float* __restrict__ row_lse, const float* __restrict__ row_pz,
-    const float* __restrict__ dlogprobs, const float* __restrict__ dentropy, int vc0, int tiles_m, int tiles_n,
-    uint16_t* __restrict__ D, int ldd, uint16_t* __restrict__ DT, int lddt) {
-  __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
+__device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
+  const uint16_t* __restrict__ W = z.W;
+  const uint16_t* __restrict__ Hd = z.Hd;
+  const int ldw = z.ldw, ldh = z.ldh, T = z.T, H = z.H, V = z.V, vc0 = z.vc0, ldd = z.ldd, lddt = z.lddt;
+  const float rcp_temp = z.rcp_temp;
+  const int64_t* __restrict__ labels = z.labels;
+  const float* __restrict__ row_lse = z.row_lse;
+  const float* __restrict__ row_pz = z.row_pz;
+  const float* __restrict__ dlogprobs = z.dlogprobs;
+  const float* __restrict__ dentropy = z.dentropy;
+  uint16_t* __restrict__ D = z.D;
+  uint16_t* __restrict__ DT = z.DT;
   int tm, tn;
-  tile_coords(blockIdx.x, tiles_m, tiles_n, kGroupM, tm, tn);
+  tile_coords(id, z.tiles_m, z.tiles_n, kGroupM, tm, tn);
 
   Operand a{W, ldw, vc0 + tm * BM, V};
   Operand b{Hd, ldh, tn * BN, T};
@@ -314,11 +345,10 @@ struct GemmArgs {
   int ldc;
 };
 
-__global__ __launch_bounds__(NTHREADS) void gemm_nt_store(const GemmArgs p0, const GemmArgs p1, int tiles0) {
-  __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
-  const bool second = (int)blockIdx.x >= tiles0;
+__device__ __forceinline__ void gemm_tile(const GemmArgs& p0, const GemmArgs& p1, int tiles0, int id, char* lds) {
+  const bool second = id >= tiles0;
   const GemmArgs& p = second ? p1 : p0;
-  const int bid = second ? (int)blockIdx.x - tiles0 : (int)blockIdx.x;
+  const int bid = second ? id - tiles0 : id;
   const int M = p.M, N = p.N;
   const int tiles_m = (M + BM - 1) / BM;
   const int tiles_n = (N + BN - 1) / BN;
@@ -359,6 +389,17 @@ __global__ __launch_bounds__(NTHREADS) void gemm_nt_store(const GemmArgs p0, con
         }
       }
   }
+}
+
+// One kernel for both kinds of backward tile: workgroups [0, gemm_tiles) run gradient GEMM tiles, the rest dz tiles.
+// The host launches it twice per vocab chunk: dz tiles only (gemm_tiles == 0), then the two GEMMs (grid == gemm_tiles).
+template <bool ENTGRAD>
+__global__ __launch_bounds__(NTHREADS) void lmhead_bwd_chunk(const DzArgs z, const GemmArgs p0, const GemmArgs p1, int tiles0,
+                                                             int gemm_tiles) {
+  __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
+  const int id = blockIdx.x;
+  if (id < gemm_tiles) gemm_tile(p0, p1, tiles0, id, lds);
+  else dz_tile<ENTGRAD>(z, id - gemm_tiles, lds);
 }
 
 // dst[c, r] = src[r, c] for r < R, c < C;  dst[c, r] = 0 for R <= r < Rpad.  bf16 bits, 64 x 64 tiles.
@@ -410,9 +451,9 @@ __global__ __launch_bounds__(256) void transpose_bf16(const uint16_t* __restrict
 // ------------------------------------------------------------------------------------------------------------
 // Optional per-kernel timing: while a profile is open on the calling thread every launch below is bracketed by a pair of
 // HIP events on the launch stream.  Closed profiles cost one thread-local load per launch.
-enum KernelKind { kFwdTiles = 0, kFwdMerge, kTranspose, kBwdDzTiles, kGemmGrad, kNumKernelKinds };
+enum KernelKind { kFwdTiles = 0, kFwdMerge, kTranspose, kBwdChunkDz, kBwdChunkGemm, kNumKernelKinds };
 const char* const kKernelNames[kNumKernelKinds] = {"lmhead_fwd_tiles", "lmhead_fwd_merge", "transpose_bf16",
-                                                   "lmhead_bwd_dz_tiles", "gemm_nt_store"};
+                                                   "lmhead_bwd_chunk[dz]", "lmhead_bwd_chunk[gemm]"};
 struct Profile {
   struct Rec {
     int kind;
@@ -482,11 +523,11 @@ BwdWorkspace carve_bwd(void* ws, int64_t T, int64_t H, int64_t V, int64_t vc) {
   const int64_t Tpad = round_up(T, 256), Vpad = round_up(V, 256);
   Carver c(ws);
   BwdWorkspace w;
-  w.Wt = c.take<uint16_t>((size_t)H * Vpad);
-  w.Ht = c.take<uint16_t>((size_t)H * Tpad);
+  w.Wt = c.take<uint16_t>((size_t)H * (Vpad + kLdPad));
+  w.Ht = c.take<uint16_t>((size_t)H * (Tpad + kLdPad));
   w.dHacc = c.take<float>((size_t)T * H);
-  w.D = c.take<uint16_t>((size_t)Tpad * vc);
-  w.DT = c.take<uint16_t>((size_t)vc * Tpad);
+  w.D = c.take<uint16_t>((size_t)Tpad * (vc + kLdPad));
+  w.DT = c.take<uint16_t>((size_t)vc * (Tpad + kLdPad));
   w.bytes = (size_t)round_up((int64_t)c.off, 256);
   return w;
 }
@@ -498,10 +539,17 @@ GemmArgs make_gemm(const uint16_t* A, int64_t lda, int64_t a_rows, const uint16_
 
 unsigned gemm_tiles(const GemmArgs& g) { return (unsigned)(((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN)); }
 
-hipError_t launch_gemm_pair(int kind, hipStream_t s, const GemmArgs& p0, const GemmArgs& p1) {
-  const unsigned t0 = gemm_tiles(p0), t1 = gemm_tiles(p1);
-  Timed timed(kind, s);
-  hipLaunchKernelGGL(gemm_nt_store, dim3(t0 + t1), dim3(NTHREADS), 0, s, p0, p1, (int)t0);
+// gemm == false: dz tiles only; dz_tiles == 0: GEMM tiles only.
+hipError_t launch_bwd_chunk(hipStream_t s, bool entgrad, const DzArgs& z, unsigned dz_tiles, bool gemm, const GemmArgs& p0,
+                            const GemmArgs& p1) {
+  const unsigned t0 = gemm ? gemm_tiles(p0) : 0, t1 = gemm ? gemm_tiles(p1) : 0;
+  Timed timed(gemm ? kBwdChunkGemm : kBwdChunkDz, s);
+  if (entgrad)
+    hipLaunchKernelGGL(lmhead_bwd_chunk<true>, dim3(t0 + t1 + dz_tiles), dim3(NTHREADS), 0, s, z, p0, p1, (int)t0,
+                       (int)(t0 + t1));
+  else
+    hipLaunchKernelGGL(lmhead_bwd_chunk<false>, dim3(t0 + t1 + dz_tiles), dim3(NTHREADS), 0, s, z, p0, p1, (int)t0,
+                       (int)(t0 + t1));
   return hipGetLastError();
 }
 
@@ -608,47 +656,43 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
   {
     Timed timed(kTranspose, s);
     hipLaunchKernelGGL(transpose_bf16, dim3((unsigned)(Vpad / 64), (unsigned)(H / 64)), dim3(256), 0, s, Wp, (int)ld_weight,
-                       (int)V, (int)H, w.Wt, (int)Vpad, (int)Vpad);
+                       (int)V, (int)H, w.Wt, (int)(Vpad + kLdPad), (int)Vpad);
   }
   {
     Timed timed(kTranspose, s);
     hipLaunchKernelGGL(transpose_bf16, dim3((unsigned)(Tpad / 64), (unsigned)(H / 64)), dim3(256), 0, s, Hp, (int)ld_hidden,
-                       (int)T, (int)H, w.Ht, (int)Tpad, (int)Tpad);
+                       (int)T, (int)H, w.Ht, (int)(Tpad + kLdPad), (int)Tpad);
   }
   if ((e = hipGetLastError()) != hipSuccess) return (int)e;
 
   const int tiles_t = (int)(Tpad / 256);
-  const int tiles_h = (int)((H + 255) / 256);
   const int64_t nchunks = (Vpad + vc - 1) / vc;
+  auto chunk_width = [&](int64_t ci) { return (Vpad - ci * vc) < vc ? (Vpad - ci * vc) : vc; };  // multiple of 256
+  auto dz_args = [&](int64_t ci) {
+    const int64_t vc0 = ci * vc, vcw = chunk_width(ci);
+    return DzArgs{Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)T, (int)H, (int)V, rcp_temperature, labels, row_lse, row_pz,
+                  dlogprobs, dentropy, (int)vc0, (int)(vcw / 256), tiles_t, w.D, (int)(vcw + kLdPad), w.DT,
+                  (int)(Tpad + kLdPad)};
+  };
+  const GemmArgs none{};
   for (int64_t ci = 0; ci < nchunks; ++ci) {
-    const int64_t vc0 = ci * vc;
-    const int64_t vcw = (Vpad - vc0) < vc ? (Vpad - vc0) : vc;  // multiple of 256
-    const int tiles_v = (int)(vcw / 256);
-    const dim3 grid_dz((unsigned)(tiles_v * tiles_t)), block(NTHREADS);
-    {
-      Timed timed(kBwdDzTiles, s);
-      if (dentropy)
-        hipLaunchKernelGGL(lmhead_bwd_dz_tiles<true>, grid_dz, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)T,
-                         (int)H, (int)V, rcp_temperature, labels, row_lse, row_pz, dlogprobs, dentropy, (int)vc0, tiles_v,
-                         tiles_t, w.D, (int)vcw, w.DT, (int)Tpad);
-      else
-        hipLaunchKernelGGL(lmhead_bwd_dz_tiles<false>, grid_dz, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)T,
-                           (int)H, (int)V, rcp_temperature, labels, row_lse, row_pz, dlogprobs, dentropy, (int)vc0, tiles_v,
-                           tiles_t, w.D, (int)vcw, w.DT, (int)Tpad);
-    }
-    if ((e = hipGetLastError()) != hipSuccess) return (int)e;
-
+    // dz panels of this chunk, then the two gradient GEMMs that consume them (one launch, they are independent).
+    // Carrying the next chunk's dz tiles in the GEMM launch (to fill its tail) was measured: no gain at the default chunk
+    // width, and it needs a second pair of panels.
+    e = launch_bwd_chunk(s, dentropy != nullptr, dz_args(ci), (unsigned)(chunk_width(ci) / 256 * tiles_t), false, none, none);
+    if (e != hipSuccess) return (int)e;
+    const int64_t vc0 = ci * vc, vcw = chunk_width(ci);
     // dHidden[T, H] (+)= D[T, vcw] . weight[vc0 : vc0 + vcw, :]    (B operand = weight^T rows, k offset vc0)
     // dW[vc0 : vc0 + rows, :] (+)= D^T[vcw, Tpad] . hidden          (B operand = hidden^T rows)
     const bool first = ci == 0, last = ci == nchunks - 1;
     const int64_t rows = (V - vc0) < vcw ? (V - vc0) : vcw;
     float* dWc = d_weight + (size_t)vc0 * (size_t)H;
-    const GemmArgs gh = make_gemm(w.D, vcw, Tpad, w.Wt + vc0, Vpad, H, vcw / BK, T, H,
+    const GemmArgs gh = make_gemm(w.D, vcw + kLdPad, Tpad, w.Wt + vc0, Vpad + kLdPad, H, vcw / BK, T, H,
                                   first ? (const float*)nullptr : (const float*)w.dHacc, last ? (float*)nullptr : w.dHacc,
                                   last ? (uint16_t*)d_hidden : (uint16_t*)nullptr, H);
-    const GemmArgs gw = make_gemm(w.DT, Tpad, vcw, w.Ht, Tpad, H, Tpad / BK, rows, H,
+    const GemmArgs gw = make_gemm(w.DT, Tpad + kLdPad, vcw, w.Ht, Tpad + kLdPad, H, Tpad / BK, rows, H,
                                   accumulate_dw ? (const float*)dWc : (const float*)nullptr, dWc, (uint16_t*)nullptr, H);
-    e = launch_gemm_pair(kGemmGrad, s, gh, gw);
+    e = launch_bwd_chunk(s, dentropy != nullptr, DzArgs{}, 0, true, gh, gw);
     if (e != hipSuccess) return (int)e;
   }
   return SKYRL_LMHEAD_OK;

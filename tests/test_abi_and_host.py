@@ -52,7 +52,7 @@ def test_workspace_queries():
     bwd = lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, 4096)
     # weight^T + hidden^T + fp32 dHidden + two dz panels; nothing of size T*V
     expect = 2 * H * V + 2 * H * T + 4 * T * H + 2 * 2 * T * 4096
-    assert expect <= bwd <= expect + 4096
+    assert expect <= bwd <= expect + (8 << 20)  # + 128 B of row padding per scratch row
     assert bwd < 2 * T * V
     assert lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, 100) == 0  # not a multiple of 256
     assert lib.skyrl_lmhead_fwd_workspace_bytes(0, H, V) == 0
