@@ -270,56 +270,99 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
   const int lrow = lane & 31, khalf = lane >> 5;
   const int vloc_base = tm * BM + wm * WM;    // first vocab row of this wave inside the chunk panel
   const int vbase = vc0 + vloc_base;          // ... and in the full vocab
+  const int tbase = tn * BN + wn * WN;        // first token of this wave (always inside the padded panels)
   const bool full = vbase + WM <= V;
   const float scale2 = rcp_temp * kLog2e;
+
+  // The wave's 128 x 128 dz block leaves through LDS so that both panels are written with 16-byte stores.  A lane holds
+  // four consecutive vocab rows of one token, which is an 8-byte piece of a D row; for D^T the four lanes of a quad
+  // (four consecutive tokens) first transpose their 4 x 4 block in registers (DPP + byte permute).  The block goes in
+  // two halves of 64 tokens; mainloop() left LDS free and every wave uses a private region, so no barrier is needed
+  // (LDS operations of one wave execute in order).
+  constexpr int kTokRow = WM * 2 + 16;            // D staging: 64 token rows x (128 vocab x 2 B + pad)
+  constexpr int kVocRow = 64 * 2 + 16;            // D^T staging: 128 vocab rows x (64 tokens x 2 B + pad)
+  constexpr int kStageD = 64 * kTokRow, kStageDT = WM * kVocRow;
+  static_assert(NWAVES * (kStageD + kStageDT) <= LDS_BYTES, "dz staging does not fit LDS");
+  char* stage_d = lds + wave * (kStageD + kStageDT);
+  char* stage_dt = stage_d + kStageD;
+  const int q4 = lane & 3;
+  const uint32_t sel1 = (q4 & 1) ? 0x03020706u : 0x05040100u;
+  const bool upper = (q4 & 2) != 0;
+
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int t = tn * BN + wn * WN + j * 32 + lrow;  // < tiles_n * 256 = padded T: always inside the panels
-    const bool valid = t < T;
-    const float g = valid ? dlogprobs[t] : 0.f;
-    const float q = (ENTGRAD && valid) ? dentropy[t] : 0.f;
-    const float lse2 = valid ? row_lse[t] * kLog2e : INFINITY;
-    const float pz = (ENTGRAD && valid) ? row_pz[t] : 0.f;
-    const int64_t y = valid ? labels[t] : (int64_t)-1;
-    const int64_t yrel64 = y - (int64_t)vbase;
-    const int yrel = (y >= 0 && y < (int64_t)V && yrel64 >= 0 && yrel64 < WM) ? (int)yrel64 : -1;
-    const float gs = g * rcp_temp;
-    const float c0 = -(g - q * pz) * rcp_temp;
-    const float c1 = -q * rcp_temp * rcp_temp;
+  for (int half = 0; half < 2; ++half) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      float d[16];
+    for (int jj = 0; jj < 2; ++jj) {
+      const int j = half * 2 + jj;
+      const int t = tbase + j * 32 + lrow;
+      const bool valid = t < T;
+      const float g = valid ? dlogprobs[t] : 0.f;
+      const float q = (ENTGRAD && valid) ? dentropy[t] : 0.f;
+      const float lse2 = valid ? row_lse[t] * kLog2e : INFINITY;
+      const float pz = (ENTGRAD && valid) ? row_pz[t] : 0.f;
+      const int64_t y = valid ? labels[t] : (int64_t)-1;
+      const int64_t yrel64 = y - (int64_t)vbase;
+      const int yrel = (y >= 0 && y < (int64_t)V && yrel64 >= 0 && yrel64 < WM) ? (int)yrel64 : -1;
+      const float gs = g * rcp_temp;
+      const float c0 = -(g - q * pz) * rcp_temp;
+      const float c1 = -q * rcp_temp * rcp_temp;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float x = acc[i][j][r];
-        const float p = __builtin_amdgcn_exp2f(fmaf(x, scale2, -lse2));
-        d[r] = ENTGRAD ? p * fmaf(c1, x, c0) : p * c0;
-      }
-      const int rel = yrel - i * 32;
-      const bool hit = (yrel >= 0) && ((unsigned)rel < 32u);
-      if (__any(hit)) {
+      for (int i = 0; i < TM; ++i) {
+        float d[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int row_r = (r >> 2) * 8 + khalf * 4 + (r & 3);
-          if (hit && rel == row_r) d[r] += gs;
+          const float x = acc[i][j][r];
+          const float p = __builtin_amdgcn_exp2f(fmaf(x, scale2, -lse2));
+          d[r] = ENTGRAD ? p * fmaf(c1, x, c0) : p * c0;
+        }
+        const int rel = yrel - i * 32;
+        const bool hit = (yrel >= 0) && ((unsigned)rel < 32u);
+        if (__any(hit)) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int row_r = (r >> 2) * 8 + khalf * 4 + (r & 3);
+            if (hit && rel == row_r) d[r] += gs;
+          }
+        }
+        if (!full) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int v = vbase + i * 32 + (r >> 2) * 8 + khalf * 4 + (r & 3);
+            if (v >= V) d[r] = 0.f;
+          }
+        }
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+          const int vl = i * 32 + rg * 8 + khalf * 4;  // vocab row inside the wave block; this lane holds vl .. vl+3
+          f32x4 v4 = {d[rg * 4 + 0], d[rg * 4 + 1], d[rg * 4 + 2], d[rg * 4 + 3]};
+          const bf16x4 b4 = __builtin_convertvector(v4, bf16x4);
+          uint32_t w0 = ((const uint32_t*)&b4)[0], w1 = ((const uint32_t*)&b4)[1];
+          *(uint2*)(stage_d + (jj * 32 + lrow) * kTokRow + vl * 2) = make_uint2(w0, w1);
+          // 4 x 4 transpose inside the quad: afterwards lane q4 holds vocab row vl + q4 for the quad's four tokens
+          const uint32_t p0 = (uint32_t)__builtin_amdgcn_mov_dpp((int)w0, 0xB1, 0xF, 0xF, true);  // lane ^ 1
+          const uint32_t p1 = (uint32_t)__builtin_amdgcn_mov_dpp((int)w1, 0xB1, 0xF, 0xF, true);
+          w0 = __builtin_amdgcn_perm(p0, w0, sel1);
+          w1 = __builtin_amdgcn_perm(p1, w1, sel1);
+          const uint32_t send = upper ? w0 : w1;
+          const uint32_t recv = (uint32_t)__builtin_amdgcn_mov_dpp((int)send, 0x4E, 0xF, 0xF, true);  // lane ^ 2
+          const uint32_t t0 = upper ? recv : w0, t1 = upper ? w1 : recv;
+          *(uint2*)(stage_dt + (vl + q4) * kVocRow + (jj * 32 + (lrow & ~3)) * 2) = make_uint2(t0, t1);
         }
       }
-      if (!full) {
+    }
+    // 64 tokens x 128 vocab staged both ways: 1024 16-byte pieces each, 16 per lane.
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int v = vbase + i * 32 + (r >> 2) * 8 + khalf * 4 + (r & 3);
-          if (v >= V) d[r] = 0.f;
-        }
+    for (int it = 0; it < 16; ++it) {
+      const int idx = it * 64 + lane;
+      {
+        const int n = idx >> 4, c = idx & 15;  // token row, 8-vocab piece
+        const uint4 v = *(const uint4*)(stage_d + n * kTokRow + c * 16);
+        *(uint4*)(D + (size_t)(tbase + half * 64 + n) * (size_t)ldd + vloc_base + c * 8) = v;
       }
-#pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        const int vl = vloc_base + i * 32 + rg * 8 + khalf * 4;
-        f32x4 v4 = {d[rg * 4 + 0], d[rg * 4 + 1], d[rg * 4 + 2], d[rg * 4 + 3]};
-        const bf16x4 b4 = __builtin_convertvector(v4, bf16x4);
-        *(bf16x4*)(D + (size_t)t * (size_t)ldd + vl) = b4;
-        const uint16_t* bits = (const uint16_t*)&b4;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) DT[(size_t)(vl + k) * (size_t)lddt + t] = bits[k];
+      {
+        const int vr = idx >> 3, c = idx & 7;  // vocab row, 8-token piece
+        const uint4 v = *(const uint4*)(stage_dt + vr * kVocRow + c * 16);
+        *(uint4*)(DT + (size_t)(vloc_base + vr) * (size_t)lddt + tbase + half * 64 + c * 8) = v;
       }
     }
   }
