@@ -27,7 +27,7 @@ namespace {
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 #ifndef LMHEAD_GROUP_M
-#define LMHEAD_GROUP_M 8
+#define LMHEAD_GROUP_M 4  // measured best of 2, 4, 6, 8, 16, 32 on both passes
 #endif
 constexpr int kGroupM = LMHEAD_GROUP_M;
 // Scratch matrices get 64 extra elements (128 B) per row: with a power-of-two row pitch (T' = 16384 -> 32 KiB) the 256 rows of
@@ -43,41 +43,43 @@ __host__ __device__ inline int64_t round_up(int64_t x, int64_t m) { return (x + 
 // The label-logit gather of that kernel (:364-385) is done in lmhead_fwd_merge instead.
 // ------------------------------------------------------------------------------------------------------------
 template <bool ENTROPY, bool MASKED>
-__device__ __forceinline__ void fwd_tile_stats(acc_t& acc, int j, int vbase, int V, float scale2, int khalf, float& m_out,
+__device__ __forceinline__ void fwd_tile_stats(const acc_t& acc, int j, int vbase, int V, float scale2, int khalf, float& m_out,
                                                float& s_out, float& e_out) {
+  // Two read-only passes over the accumulators (they live in AGPRs; writing scaled values back would cost a move each
+  // way).  scale2 > 0, so the maximum commutes with the scaling, and sum z*p = scale2 * sum x*p.
   float mx = -INFINITY;
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      float z2 = acc[i][j][r] * scale2;
+      float x = acc[i][j][r];
       if (MASKED) {
         const int v = vbase + i * 32 + (r >> 2) * 8 + khalf * 4 + (r & 3);
-        if (v >= V) z2 = -INFINITY;
+        if (v >= V) x = -INFINITY;
       }
-      acc[i][j][r] = z2;
-      mx = fmaxf(mx, z2);
+      mx = fmaxf(mx, x);
     }
   mx = fmaxf(mx, shfl_xor32(mx));  // finite: the wave has at least one row below V
+  const float m2 = mx * scale2;
   float s = 0.f, e = 0.f;
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const float z2 = acc[i][j][r];
-      const float p = __builtin_amdgcn_exp2f(z2 - mx);
-      s += p;
-      if (ENTROPY) {
-        float zz = z2;
-        if (MASKED) zz = (z2 == -INFINITY) ? 0.f : z2;
-        e = fmaf(zz, p, e);
+      const float x = acc[i][j][r];
+      float p = __builtin_amdgcn_exp2f(fmaf(x, scale2, -m2));
+      if (MASKED) {
+        const int v = vbase + i * 32 + (r >> 2) * 8 + khalf * 4 + (r & 3);
+        if (v >= V) p = 0.f;
       }
+      s += p;
+      if (ENTROPY) e = fmaf(x, p, e);
     }
   s += shfl_xor32(s);
   if (ENTROPY) e += shfl_xor32(e);
-  m_out = mx * kLn2;
+  m_out = m2 * kLn2;
   s_out = s;
-  e_out = e * kLn2;
+  e_out = e * scale2 * kLn2;
 }
 
 template <bool ENTROPY>
@@ -258,13 +260,6 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
   int tm, tn;
   tile_coords(id, z.tiles_m, z.tiles_n, kGroupM, tm, tn);
 
-  Operand a{W, ldw, vc0 + tm * BM, V};
-  Operand b{Hd, ldh, tn * BN, T};
-  acc_t acc;
-  zero_acc(acc);
-  prefetch_first_tiles(a, b, 0, H / BK, lds);
-  mainloop(a, b, 0, H / BK, lds, acc);
-
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int lrow = lane & 31, khalf = lane >> 5;
@@ -273,6 +268,32 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
   const int tbase = tn * BN + wn * WN;        // first token of this wave (always inside the padded panels)
   const bool full = vbase + WM <= V;
   const float scale2 = rcp_temp * kLog2e;
+
+  // Per-token inputs of the epilogue, loaded before the mainloop so that their latency is not paid after it.
+  float gs_[TN], c0_[TN], c1_[TN], lse2_[TN];
+  int yrel_[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int t = tbase + j * 32 + lrow;
+    const bool valid = t < T;
+    const float g = valid ? dlogprobs[t] : 0.f;
+    const float q = (ENTGRAD && valid) ? dentropy[t] : 0.f;
+    lse2_[j] = valid ? row_lse[t] * kLog2e : INFINITY;
+    const float pz = (ENTGRAD && valid) ? row_pz[t] : 0.f;
+    const int64_t y = valid ? labels[t] : (int64_t)-1;
+    const int64_t yrel64 = y - (int64_t)vbase;
+    yrel_[j] = (y >= 0 && y < (int64_t)V && yrel64 >= 0 && yrel64 < WM) ? (int)yrel64 : -1;
+    gs_[j] = g * rcp_temp;
+    c0_[j] = -(g - q * pz) * rcp_temp;
+    c1_[j] = -q * rcp_temp * rcp_temp;
+  }
+
+  Operand a{W, ldw, vc0 + tm * BM, V};
+  Operand b{Hd, ldh, tn * BN, T};
+  acc_t acc;
+  zero_acc(acc);
+  prefetch_first_tiles(a, b, 0, H / BK, lds);
+  mainloop(a, b, 0, H / BK, lds, acc);
 
   // The wave's 128 x 128 dz block leaves through LDS so that both panels are written with 16-byte stores.  A lane holds
   // four consecutive vocab rows of one token, which is an 8-byte piece of a D row; for D^T the four lanes of a quad
@@ -294,18 +315,8 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
 #pragma unroll
     for (int jj = 0; jj < 2; ++jj) {
       const int j = half * 2 + jj;
-      const int t = tbase + j * 32 + lrow;
-      const bool valid = t < T;
-      const float g = valid ? dlogprobs[t] : 0.f;
-      const float q = (ENTGRAD && valid) ? dentropy[t] : 0.f;
-      const float lse2 = valid ? row_lse[t] * kLog2e : INFINITY;
-      const float pz = (ENTGRAD && valid) ? row_pz[t] : 0.f;
-      const int64_t y = valid ? labels[t] : (int64_t)-1;
-      const int64_t yrel64 = y - (int64_t)vbase;
-      const int yrel = (y >= 0 && y < (int64_t)V && yrel64 >= 0 && yrel64 < WM) ? (int)yrel64 : -1;
-      const float gs = g * rcp_temp;
-      const float c0 = -(g - q * pz) * rcp_temp;
-      const float c1 = -q * rcp_temp * rcp_temp;
+      const float gs = gs_[j], c0 = c0_[j], c1 = c1_[j], lse2 = lse2_[j];
+      const int yrel = yrel_[j];
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
         float d[16];
