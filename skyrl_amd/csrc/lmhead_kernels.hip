@@ -397,6 +397,12 @@ struct GemmArgs {
   float* Cf;
   uint16_t* Cb;
   int ldc;
+  // Partial sums carried from launch to launch (dHidden across vocab chunks) live in "accumulator order": tile by tile,
+  // wave by wave, each lane's 16 registers of an MFMA block contiguous.  Reading and writing them is 16 bytes per lane
+  // and 4 KiB contiguous per wave instruction group -- a quarter of the instructions of the row-major form, where a
+  // lane's values sit a row apart (measured: the row-major read-modify-write cost 6 % of the backward pass).
+  const float* Pin;
+  float* Pout;
 };
 
 __device__ __forceinline__ void gemm_tile(const GemmArgs& p0, const GemmArgs& p1, int tiles0, int id, char* lds) {
@@ -422,6 +428,33 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p0, const GemmArgs& p1
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int lrow = lane & 31, khalf = lane >> 5;
+
+  if (p.Pin || p.Pout) {
+    const size_t base = ((size_t)(tm * tiles_n + tn) * NWAVES + wave) * (TM * TN * 64 * 16) + (size_t)lane * 16;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const size_t off = base + (size_t)(i * TN + j) * (64 * 16);
+        if (p.Pin) {
+          const f32x4* src = (const f32x4*)(p.Pin + off);
+#pragma unroll
+          for (int r4 = 0; r4 < 4; ++r4) {
+            const f32x4 v = src[r4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) acc[i][j][r4 * 4 + k] += v[k];
+          }
+        }
+        if (p.Pout) {
+          f32x4* dst = (f32x4*)(p.Pout + off);
+#pragma unroll
+          for (int r4 = 0; r4 < 4; ++r4)
+            dst[r4] = f32x4{acc[i][j][r4 * 4], acc[i][j][r4 * 4 + 1], acc[i][j][r4 * 4 + 2], acc[i][j][r4 * 4 + 3]};
+        }
+      }
+  }
+  if (!Cf && !Cb) return;
+
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int n = tn * BN + wn * WN + j * 32 + lrow;
@@ -579,7 +612,7 @@ BwdWorkspace carve_bwd(void* ws, int64_t T, int64_t H, int64_t V, int64_t vc) {
   BwdWorkspace w;
   w.Wt = c.take<uint16_t>((size_t)H * (Vpad + kLdPad));
   w.Ht = c.take<uint16_t>((size_t)H * (Tpad + kLdPad));
-  w.dHacc = c.take<float>((size_t)T * H);
+  w.dHacc = c.take<float>((size_t)Tpad * round_up(H, 256));  // accumulator order, whole tiles
   w.D = c.take<uint16_t>((size_t)Tpad * (vc + kLdPad));
   w.DT = c.take<uint16_t>((size_t)vc * (Tpad + kLdPad));
   w.bytes = (size_t)round_up((int64_t)c.off, 256);
@@ -587,8 +620,9 @@ BwdWorkspace carve_bwd(void* ws, int64_t T, int64_t H, int64_t V, int64_t vc) {
 }
 
 GemmArgs make_gemm(const uint16_t* A, int64_t lda, int64_t a_rows, const uint16_t* B, int64_t ldb, int64_t b_rows, int64_t nk,
-                   int64_t M, int64_t N, const float* Cin, float* Cf, uint16_t* Cb, int64_t ldc) {
-  return GemmArgs{A, (int)lda, (int)a_rows, B, (int)ldb, (int)b_rows, (int)nk, (int)M, (int)N, Cin, Cf, Cb, (int)ldc};
+                   int64_t M, int64_t N, const float* Cin, float* Cf, uint16_t* Cb, int64_t ldc, const float* Pin = nullptr,
+                   float* Pout = nullptr) {
+  return GemmArgs{A, (int)lda, (int)a_rows, B, (int)ldb, (int)b_rows, (int)nk, (int)M, (int)N, Cin, Cf, Cb, (int)ldc, Pin, Pout};
 }
 
 unsigned gemm_tiles(const GemmArgs& g) { return (unsigned)(((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN)); }
@@ -741,9 +775,9 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
     const bool first = ci == 0, last = ci == nchunks - 1;
     const int64_t rows = (V - vc0) < vcw ? (V - vc0) : vcw;
     float* dWc = d_weight + (size_t)vc0 * (size_t)H;
-    const GemmArgs gh = make_gemm(w.D, vcw + kLdPad, Tpad, w.Wt + vc0, Vpad + kLdPad, H, vcw / BK, T, H,
-                                  first ? (const float*)nullptr : (const float*)w.dHacc, last ? (float*)nullptr : w.dHacc,
-                                  last ? (uint16_t*)d_hidden : (uint16_t*)nullptr, H);
+    const GemmArgs gh = make_gemm(w.D, vcw + kLdPad, Tpad, w.Wt + vc0, Vpad + kLdPad, H, vcw / BK, T, H, nullptr, nullptr,
+                                  last ? (uint16_t*)d_hidden : (uint16_t*)nullptr, H,
+                                  first ? (const float*)nullptr : (const float*)w.dHacc, last ? (float*)nullptr : w.dHacc);
     const GemmArgs gw = make_gemm(w.DT, Tpad + kLdPad, vcw, w.Ht, Tpad + kLdPad, H, Tpad / BK, rows, H,
                                   accumulate_dw ? (const float*)dWc : (const float*)nullptr, dWc, (uint16_t*)nullptr, H);
     e = launch_bwd_chunk(s, dentropy != nullptr, DzArgs{}, 0, true, gh, gw);
