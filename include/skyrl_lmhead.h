@@ -40,7 +40,7 @@ extern "C" {
 
 #define SKYRL_LMHEAD_OK 0
 #define SKYRL_LMHEAD_ERR_NULL (-1)      /* a required pointer is NULL */
-#define SKYRL_LMHEAD_ERR_SHAPE (-2)     /* T, V < 1, H not a positive multiple of 64, or a leading dimension < H */
+#define SKYRL_LMHEAD_ERR_SHAPE (-2)     /* T, V < 1, H not a positive multiple of 64, a leading dimension < H, or an operand of 4 GiB or more */
 #define SKYRL_LMHEAD_ERR_ALIGN (-3)     /* a pointer is not 16-byte aligned or a leading dimension is not a multiple of 8 */
 #define SKYRL_LMHEAD_ERR_WORKSPACE (-4) /* workspace is NULL or smaller than the matching *_workspace_bytes() */
 #define SKYRL_LMHEAD_ERR_ARG (-5)       /* rcp_temperature not finite and positive, or vocab_chunk not a multiple of 256 */

@@ -586,6 +586,10 @@ int check_common(const void* hidden, int64_t ldh, const void* weight, int64_t ld
   if (T < 1 || V < 1 || H < BK || H % BK != 0 || ldh < H || ldw < H) return SKYRL_LMHEAD_ERR_SHAPE;
   if (T > (int64_t)1 << 30 || V > (int64_t)1 << 30 || ldh > (int64_t)1 << 30 || ldw > (int64_t)1 << 30)
     return SKYRL_LMHEAD_ERR_SHAPE;
+  // The copy plan addresses an operand with 32-bit byte offsets: each operand (and each backward scratch matrix, which is
+  // never larger than these two transposed) must stay below 4 GiB.
+  const int64_t kMaxBytes = (int64_t)1 << 32;
+  if (T * ldh * 2 >= kMaxBytes || V * ldw * 2 >= kMaxBytes) return SKYRL_LMHEAD_ERR_SHAPE;
   if (!aligned16(hidden) || !aligned16(weight) || ((uintptr_t)labels & 7u) || ldh % 8 != 0 || ldw % 8 != 0)
     return SKYRL_LMHEAD_ERR_ALIGN;
   if (!(rcp_temperature > 0.f) || !isfinite(rcp_temperature)) return SKYRL_LMHEAD_ERR_ARG;
@@ -731,6 +735,10 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
   const int64_t Tpad = round_up(T, 256), Vpad = round_up(V, 256);
   int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(T, V);
   if (vc > Vpad) vc = Vpad;
+  // 32-bit byte offsets inside the scratch matrices as well (weight^T, hidden^T, the two dz panels)
+  if (H * (Vpad + kLdPad) * 2 >= ((int64_t)1 << 32) || H * (Tpad + kLdPad) * 2 >= ((int64_t)1 << 32) ||
+      Tpad * (vc + kLdPad) * 2 >= ((int64_t)1 << 32) || vc * (Tpad + kLdPad) * 2 >= ((int64_t)1 << 32))
+    return SKYRL_LMHEAD_ERR_SHAPE;
   if (!workspace || workspace_bytes < skyrl_lmhead_bwd_workspace_bytes(T, H, V, vc)) return SKYRL_LMHEAD_ERR_WORKSPACE;
   if ((uintptr_t)workspace & 255u) return SKYRL_LMHEAD_ERR_ALIGN;
 

@@ -73,6 +73,7 @@ def test_forward_argument_errors_are_reported_before_any_launch():
     assert _call_fwd(lib, H=100, ldh=104, ldw=104) == -2  # H not a multiple of 64
     assert _call_fwd(lib, T=0) == -2
     assert _call_fwd(lib, ldh=64) == -2  # leading dimension < H
+    assert _call_fwd(lib, V=300000, H=8192, ldh=8192, ldw=8192, wsb=1 << 40) == -2  # weight of 4 GiB or more
     assert _call_fwd(lib, hidden=0x1008) == -3
     assert _call_fwd(lib, ldw=132) == -3
     assert _call_fwd(lib, ws=None) == -4
