@@ -124,11 +124,14 @@ __global__ __launch_bounds__(NTHREADS) void lmhead_fwd_tiles(const uint16_t* __r
 }
 
 // ------------------------------------------------------------------------------------------------------------
-// Forward merge.  32 tokens per workgroup of 256 threads.
+// Forward merge.  8 tokens per workgroup of 256 threads (32 threads per token).
 // Merge algebra as in efficient_entropy_triton_kernel_epilogue (fused_linear_logprob_triton.py:417-467) except that
 // the running max starts at -inf (that kernel starts it at 0, which loses rows whose logits are all << 0).
 // Out-of-range labels give logprob 0 (model_utils.py:337; fused_linear_logprob_triton.py:1898-1905).
 // ------------------------------------------------------------------------------------------------------------
+constexpr int kMergeTokens = 8;
+constexpr int kMergeGroups = 256 / kMergeTokens;  // partial groups per token
+
 __global__ __launch_bounds__(256) void lmhead_fwd_merge(const float* __restrict__ part_max, const float* __restrict__ part_sum,
                                                         const float* __restrict__ part_pz, int nparts, int T,
                                                         const uint16_t* __restrict__ Hd, int ldh,
@@ -136,15 +139,15 @@ __global__ __launch_bounds__(256) void lmhead_fwd_merge(const float* __restrict_
                                                         const int64_t* __restrict__ labels, int H, int V, float rcp_temp,
                                                         float* __restrict__ logprobs, float* __restrict__ entropy,
                                                         float* __restrict__ row_lse, float* __restrict__ row_pz) {
-  __shared__ float sm_m[8][32], sm_s[8][32], sm_e[8][32];
-  __shared__ float sm_lse[32], sm_pz[32];
+  __shared__ float sm_m[kMergeGroups][kMergeTokens], sm_s[kMergeGroups][kMergeTokens], sm_e[kMergeGroups][kMergeTokens];
+  __shared__ float sm_lse[kMergeTokens], sm_pz[kMergeTokens];
   const int tid = threadIdx.x;
   {
-    const int tl = tid & 31, grp = tid >> 5;
-    const int t = blockIdx.x * 32 + tl;
+    const int tl = tid % kMergeTokens, grp = tid / kMergeTokens;
+    const int t = blockIdx.x * kMergeTokens + tl;
     float M = -INFINITY, S = 0.f, E = 0.f;
     if (t < T) {
-      for (int p = grp; p < nparts; p += 8) {
+      for (int p = grp; p < nparts; p += kMergeGroups) {
         const size_t idx = (size_t)p * (size_t)T + t;
         const float m = part_max[idx];
         if (m > -INFINITY) {
@@ -164,11 +167,9 @@ __global__ __launch_bounds__(256) void lmhead_fwd_merge(const float* __restrict_
     __syncthreads();
     if (grp == 0) {
       float Mg = -INFINITY;
-#pragma unroll
-      for (int g = 0; g < 8; ++g) Mg = fmaxf(Mg, sm_m[g][tl]);
+      for (int g = 0; g < kMergeGroups; ++g) Mg = fmaxf(Mg, sm_m[g][tl]);
       float Sg = 0.f, Eg = 0.f;
-#pragma unroll
-      for (int g = 0; g < 8; ++g) {
+      for (int g = 0; g < kMergeGroups; ++g) {
         const float m = sm_m[g][tl];
         if (m > -INFINITY) {
           const float c = expf(m - Mg);
@@ -181,9 +182,9 @@ __global__ __launch_bounds__(256) void lmhead_fwd_merge(const float* __restrict_
     }
     __syncthreads();
   }
-  // Label logit: 8 lanes per token, 16-byte loads, fp32 accumulation.
-  const int tl = tid >> 3, sub = tid & 7;
-  const int t = blockIdx.x * 32 + tl;
+  // Label logit: 32 lanes per token, 16-byte loads, fp32 accumulation.
+  const int tl = tid / kMergeGroups, sub = tid % kMergeGroups;
+  const int t = blockIdx.x * kMergeTokens + tl;
   float dot = 0.f;
   bool has_label = false;
   if (t < T) {
@@ -192,7 +193,7 @@ __global__ __launch_bounds__(256) void lmhead_fwd_merge(const float* __restrict_
     if (has_label) {
       const uint16_t* hp = Hd + (size_t)t * (size_t)ldh;
       const uint16_t* wp = W + (size_t)y * (size_t)ldw;
-      for (int c = sub * 8; c < H; c += 64) {
+      for (int c = sub * 8; c < H; c += kMergeGroups * 8) {
         const uint4 hv = *(const uint4*)(hp + c);
         const uint4 wv = *(const uint4*)(wp + c);
         const uint32_t hh[4] = {hv.x, hv.y, hv.z, hv.w};
@@ -205,9 +206,8 @@ __global__ __launch_bounds__(256) void lmhead_fwd_merge(const float* __restrict_
       }
     }
   }
-  dot += __shfl_xor(dot, 1, 64);
-  dot += __shfl_xor(dot, 2, 64);
-  dot += __shfl_xor(dot, 4, 64);
+#pragma unroll
+  for (int o = 1; o < kMergeGroups; o <<= 1) dot += __shfl_xor(dot, o, 64);
   if (sub == 0 && t < T) {
     const float lse = sm_lse[tl], pz = sm_pz[tl];
     logprobs[t] = has_label ? dot * rcp_temp - lse : 0.f;
@@ -715,7 +715,7 @@ int skyrl_lmhead_fwd(const void* hidden, int64_t ld_hidden, const void* weight, 
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
   Timed timed(kFwdMerge, s);
-  hipLaunchKernelGGL(lmhead_fwd_merge, dim3((unsigned)((T + 31) / 32)), dim3(256), 0, s, pmax, psum,
+  hipLaunchKernelGGL(lmhead_fwd_merge, dim3((unsigned)((T + kMergeTokens - 1) / kMergeTokens)), dim3(256), 0, s, pmax, psum,
                      want_pz ? ppz : (float*)nullptr, (int)nparts, (int)T, Hp, (int)ld_hidden, Wp, (int)ld_weight, labels,
                      (int)H, (int)V, rcp_temperature, logprobs, entropy, row_lse, row_pz);
   e = hipGetLastError();

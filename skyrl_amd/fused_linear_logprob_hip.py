@@ -95,8 +95,8 @@ class LinearCrossEntropy(torch.autograd.Function):
         else:
             g = (dlogprobs.to(torch.float32) / T).expand(T).contiguous()
         q = None if dentropy is None else dentropy.reshape(-1).to(torch.float32).contiguous()
-        d_hidden, d_weight = ops.lmhead_bwd(hidden2, weight, labels1, row_lse, row_pz if q is not None else None, g, q,
-                                            ctx.rcp_t, 0)
+        d_hidden, d_weight = ops.lmhead_bwd_active_rows(hidden2, weight, labels1, row_lse, row_pz if q is not None else None,
+                                                        g, q, ctx.rcp_t, 0)
         return d_hidden.view(ctx.original_hidden_shape), d_weight.to(weight.dtype), None, None, None, None
 
 
@@ -148,7 +148,7 @@ class FusedLinearLogprobHip(torch.autograd.Function):
             g = torch.zeros(B * S, dtype=torch.float32, device=hidden_2d.device)
         else:
             g = grad_output.reshape(-1).to(torch.float32).contiguous()
-        d_hidden, d_weight = ops.lmhead_bwd(hidden_2d, weight_c, labels, row_lse, None, g, None, 1.0, 0)
+        d_hidden, d_weight = ops.lmhead_bwd_active_rows(hidden_2d, weight_c, labels, row_lse, None, g, None, 1.0, 0)
         # grad_hidden in the hidden dtype, grad_weight in the weight dtype (model_utils.py:381, 428).
         return (d_hidden.reshape(B, S, H).to(ctx.hidden_dtype), d_weight.to(weight_c.dtype), None, None, None, None, None,
                 None)

@@ -248,6 +248,33 @@ def test_backward_is_linear_in_upstream_grads_and_deterministic(cuda_device):
     assert torch.equal(lp, lp2)
 
 
+def test_backward_skips_rows_without_upstream_gradient(cuda_device):
+    # the masked configurations (prompt tokens carry no gradient): compacted and dense backward agree, masked rows are exactly 0
+    cfg = SMALL_TWINS["qwen2.5-1.5b-fwdbwd"]
+    d = make_inputs(cfg)
+    dev = cuda_device
+    h, w, y, g = (d[k].to(dev) for k in ("hidden", "weight", "labels", "dlogprobs"))
+    lp, _, lse, _ = ops.lmhead_fwd(h, w, y, 1.0, False)
+    dense = ops.lmhead_bwd(h, w, y, lse, None, g, None, 1.0, 0)
+    compact = ops.lmhead_bwd_active_rows(h, w, y, lse, None, g, None, 1.0, 0)
+    masked = (d["mask"] == 0).to(dev)
+    assert masked.float().mean().item() == pytest.approx(0.5)
+    assert compact[0][masked].abs().max().item() == 0.0
+    assert rel_l2(compact[0].float(), dense[0].float()) < 2e-2 and rel_l2(compact[1], dense[1]) < 1e-3
+    ex = O.exact_fwd_bwd(d["hidden"], d["weight"], d["labels"], 1.0, d["dlogprobs"], None)
+    assert cos(compact[0], ex["d_hidden"]) >= GRAD_COS and cos(compact[1], ex["d_weight"]) >= GRAD_COS
+    # all-zero upstream gradient: zeros, no kernel launched
+    z = ops.lmhead_bwd_active_rows(h, w, y, lse, None, torch.zeros_like(g), None, 1.0, 0)
+    assert z[0].abs().max().item() == 0.0 and z[1].abs().max().item() == 0.0
+    # through autograd (FusedLinearLogprobHip uses the compacting path)
+    B, S = cfg.n_seqs, cfg.T // cfg.n_seqs
+    hd = d["hidden"].reshape(B, S, cfg.H).to(dev).requires_grad_(True)
+    wd = w.clone().requires_grad_(True)
+    out = FusedLinearLogprobHip.apply(hd, wd, d["labels"].reshape(B, S).to(dev), 0, cfg.V, S, None, False)
+    (out * g.reshape(B, S)).sum().backward()
+    assert cos(hd.grad.reshape(-1, cfg.H), ex["d_hidden"]) >= GRAD_COS and cos(wd.grad, ex["d_weight"]) >= GRAD_COS
+
+
 def test_c_abi_called_directly(cuda_device):
     """No torch op wrapper in between: raw pointers into the exported symbols."""
     lib = _lib.load()
