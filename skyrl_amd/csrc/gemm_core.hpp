@@ -3,29 +3,35 @@
 // All contractions on the path are brought into one form, C[M,N] = A[M,K] * B[N,K]^T with A and B bf16, row-major and
 // K-contiguous, so one software-pipelined mainloop serves the forward logits GEMM, the backward logits recompute,
 // dHidden and dW.  A workgroup of 4 wavefronts (2 x 2, one per SIMD) owns a 256 x 256 tile of C; each wavefront owns
-// 128 x 128 of it as 4 x 4 accumulators of v_mfma_f32_32x32x16_bf16 (256 accumulator registers, in AGPRs).
+// 128 x 128 of it as 8 x 8 accumulators of v_mfma_f32_16x16x32_bf16 (256 accumulator registers, in AGPRs).
 //
 // What bounds the loop (measured on the MI355X):
+//   * with random operands the matrix pipe is power-limited, not issue-limited: a loop of nothing but MFMAs on
+//     N(0,1) data sustains 1.69-1.84 PFLOP/s with v_mfma_f32_32x32x16_bf16 and 2.08-2.10 PFLOP/s with
+//     v_mfma_f32_16x16x32_bf16 (both 2.46-2.49 on zeros), so the 16 x 16 x 32 shape is used although it needs twice
+//     the MFMA instructions;
 //   * a CU takes at most ~32 B/clk from L2, through global_load_lds as well as through ordinary loads; a 64 KiB k-tile
 //     (256 + 256 rows x 64 k) therefore needs >= 2048 clk, exactly the MFMA time of a 256 x 256 x 64 tile: the copy
 //     path, not the matrix pipe, is the resource that must never idle;
 //   * every LDS read cycle steals about half a cycle from the direct-to-LDS copies, so LDS is read as little as
-//     possible: 128 x 128 wave tiles need 8 fragment reads per 16 MFMAs (128 x 64 tiles need 12);
+//     possible: 128 x 128 wave tiles need 16 fragment reads per 32-k step (128 x 64 tiles need 24);
 //   * the copy unit takes one 1 KiB copy about every 34 clk for the whole CU and a wave that issues into a full queue
 //     stalls -- with one wave per SIMD that stalls the matrix pipe -- so a lane's 16 copies per k-tile are spread
-//     evenly over its 64 MFMAs.
+//     evenly over its 128 MFMAs.
 //
 // Data path: 16-byte global_load_lds (global -> LDS without a VGPR round trip) into a ring of five 32 KiB operand
-// slots (2.5 k-tiles, all of the CU's 160 KiB); ds_read_b128 fragments two 16-k steps ahead; MFMA, fp32 accumulation.
+// slots (2.5 k-tiles, all of the CU's 160 KiB); ds_read_b128 fragments one 32-k step ahead; MFMA, fp32 accumulation.
 //
 // LDS operand slot: 256 rows x 64 k bf16 = 256 x 128 B.  The 16-byte chunk (row, kc) lives at byte
 // row*128 + ((kc ^ swz(row)) << 4), see swz() below.
 //
-// Accumulator layout of v_mfma_f32_32x32x16 (lane l, register r in 0..15):
-//     m = (r >> 2) * 8 + (l >> 5) * 4 + (r & 3),   n = l & 31
-// i.e. a lane holds one column n and 16 rows m.  The kernels put the *vocab* index on M and the *token* index on N, so
-// every per-token quantity (running max, sum-exp, upstream grads) is a per-lane scalar and the vocab reduction is an
-// in-register loop plus one lane^32 exchange.
+// Operand layout of v_mfma_f32_16x16x32 (lane l): row (A) or column (B) l & 15, the eight k values (l >> 4) * 8 .. + 7,
+// i.e. one 16-byte LDS chunk per lane.  Accumulator layout (lane l, register r in 0..3):
+//     m = (l >> 4) * 4 + r,   n = l & 15
+// i.e. a lane holds one column n and four consecutive rows m.  The kernels put the *vocab* index on M and the *token*
+// index on N, so every per-token quantity (running max, sum-exp, upstream grads) is a per-lane scalar and the vocab
+// reduction is an in-register loop plus the lane^16 and lane^32 exchanges; a lane's four values are an 8-byte piece
+// of a bf16 row (16 bytes of an fp32 row) along M.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -47,26 +53,27 @@ constexpr int NWAVES = WAVES_M * WAVES_N;
 constexpr int NTHREADS = 64 * NWAVES;
 constexpr int WM = BM / WAVES_M;   // 128
 constexpr int WN = BN / WAVES_N;   // 128
-constexpr int TM = WM / 32;        // 4 MFMA tiles along M per wave
-constexpr int TN = WN / 32;        // 4 MFMA tiles along N per wave
-constexpr int KSTEPS = BK / 16;                    // MFMA k-steps per k-tile
+constexpr int MT = 16;             // MFMA tile edge
+constexpr int TM = WM / MT;        // 8 MFMA tiles along M per wave
+constexpr int TN = WN / MT;        // 8 MFMA tiles along N per wave
+constexpr int KSTEPS = BK / 32;                    // MFMA k-steps per k-tile
 constexpr int ROW_BYTES = BK * 2;                  // one operand row inside a slot
 constexpr int OPERAND_BYTES = BM * ROW_BYTES;      // 32 KiB
 constexpr int RING_SLOTS = 5;
 constexpr int LDS_BYTES = RING_SLOTS * OPERAND_BYTES;  // 160 KiB: the whole LDS of a CU
 constexpr int COPIES_PER_OPERAND = OPERAND_BYTES / 1024 / NWAVES;  // 8 global_load_lds per lane per operand tile
-static_assert(KSTEPS == 4 && TM == 4 && TN == 4 && COPIES_PER_OPERAND == 8, "the schedule below is written for these");
+static_assert(KSTEPS == 2 && TM == 8 && TN == 8 && COPIES_PER_OPERAND == 8, "the schedule below is written for these");
 #ifndef LMHEAD_ABL
 #define LMHEAD_ABL 0  // timing-only ablations (wrong results): 1 no copies in the loop, 2 no fragment reads in the loop
 #endif
 
-// LDS on gfx950 has 64 banks of 4 bytes and serves a ds_read_b128 sixteen lanes (256 B) at a time.  Lanes 0..15 of a
-// fragment read touch 16 consecutive rows at one k-chunk.  XOR-ing the chunk index with (row >> 1) & 7 spreads those
+// LDS on gfx950 has 64 banks of 4 bytes and serves a ds_read_b128 sixteen lanes (256 B) at a time.  Sixteen consecutive
+// lanes of a fragment read touch 16 consecutive rows at one k-chunk.  XOR-ing the chunk index with (row >> 1) & 7 spreads those
 // sixteen reads over all sixteen 16-byte slots of a 256-byte window (2 rows x 8 chunks): conflict-free, 256 B/clk
 // measured; the obvious key row & 7 reaches 159 B/clk.
 __device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
 
-typedef f32x16 acc_t[TM][TN];
+typedef f32x4 acc_t[TM][TN];
 
 struct Operand {
   const uint16_t* ptr;  // bf16 bits, row-major, K contiguous
@@ -85,13 +92,22 @@ __device__ __forceinline__ void wait_copies_and_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
+// One MFMA, accumulating in place in AGPRs.  Written as inline assembly because the register allocator, given 64
+// separate four-register accumulators through the builtin, rotates them through the loop (MFMA destination != source)
+// and repairs the permutation with hundreds of v_accvgpr moves per iteration.  The compiler does not know this is an
+// MFMA, so the two hazards it would otherwise pad are handled by construction: an accumulator is reused only after
+// 63 other MFMAs, and mainloop() ends with explicit wait states before anything reads the accumulators.
+__device__ __forceinline__ void mfma_16x16x32(f32x4& c, const bf16x8& a, const bf16x8& b) {
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+
 __device__ __forceinline__ void zero_acc(acc_t& acc) {
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 }
 
 // Per-lane plan of the global->LDS copies of one output tile: which global 16-byte chunk lands in which LDS chunk.
@@ -154,63 +170,63 @@ __device__ __forceinline__ void prefetch_first_tiles(const Operand& a, const Ope
 // reading LDS, and all ring slots are free.
 //
 // Ring: A(t) sits in slot 2t mod 5, B(t) in slot (2t+1) mod 5.  While k-tile kt is consumed, A(kt+1) and B(kt+1) are
-// ready or landing and A(kt+2) is being issued.  Per k-tile (four 16-k steps of 16 MFMAs):
-//   steps 0, 1:  copies of A(kt+2) into the slot that held B(kt-1)          (freed by the barrier of iteration kt-1)
-//   step 2:      barrier -- all fragment reads of tile kt have returned, this wave's copies of tile kt+1 have landed --
-//                then the first half of B(kt+2) into the slot that held A(kt); step 3: the second half
-//   every step:  the eight fragment reads of the step two ahead ride behind its first eight MFMAs (four register sets),
-//                one copy behind every fourth MFMA; sched_barrier pins that order.
+// ready or landing and A(kt+2) is being issued.  Per k-tile (two 32-k steps of 64 MFMAs):
+//   step 0:      copies of A(kt+2) into the slot that held B(kt-1)          (freed by the barrier of iteration kt-1);
+//                fragment reads of step 1
+//   step 1:      barrier -- all fragment reads of tile kt have returned, this wave's copies of tile kt+1 have landed --
+//                then B(kt+2) into the slot that held A(kt); fragment reads of step 0 of tile kt+1
+//   every step:  the sixteen fragment reads of the next step ride behind every second MFMA of its first half (two
+//                register sets), one copy behind every eighth MFMA; sched_barrier pins that order.
+// MFMA order inside a step is a serpentine over the 8 x 8 accumulators (the B fragment is kept where the A fragment
+// changes): fewer operand toggles, measurably less power.
 __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int k_begin, int nk, char* lds, acc_t& acc) {
   CopyPlan p;
   make_plan(p, a, b, k_begin);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-  const int lrow = lane & 31;
-  const int xsw = ((lane >> 5) ^ swz(lrow)) << 4;  // chunk offset of k-step 0; k-step s is xsw ^ (s << 5)
+  const int lrow = lane & 15;
+  const int xsw = ((lane >> 4) ^ swz(lrow)) << 4;  // chunk offset of k-step 0; k-step 1 is xsw ^ 64
   const int a_base = (wm * WM + lrow) * ROW_BYTES;
   const int b_base = (wn * WN + lrow) * ROW_BYTES;
   auto wrap = [](int x) { return x >= RING_SLOTS ? x - RING_SLOTS : x; };
 
-  bf16x8 af[4][TM], bfr[4][TN];
-  // Fragment x of a 16-k step: x < TM is the A fragment of MFMA row x, otherwise the B fragment of MFMA column x - TM.
+  bf16x8 af[2][TM], bfr[2][TN];
+  // Fragment x of a 32-k step: x < TM is the A fragment of MFMA row x, otherwise the B fragment of MFMA column x - TM.
   auto read_one = [&](int slot_a, int slot_b, int ks, int set, int x) {
     if (x < TM)
-      af[set][x] = *(const bf16x8*)(lds + slot_a * OPERAND_BYTES + a_base + (xsw ^ (ks << 5)) + x * 32 * ROW_BYTES);
+      af[set][x] = *(const bf16x8*)(lds + slot_a * OPERAND_BYTES + a_base + (xsw ^ (ks << 6)) + x * MT * ROW_BYTES);
     else
-      bfr[set][x - TM] = *(const bf16x8*)(lds + slot_b * OPERAND_BYTES + b_base + (xsw ^ (ks << 5)) + (x - TM) * 32 * ROW_BYTES);
+      bfr[set][x - TM] = *(const bf16x8*)(lds + slot_b * OPERAND_BYTES + b_base + (xsw ^ (ks << 6)) + (x - TM) * MT * ROW_BYTES);
   };
 
   if (nk > 1) wait_copies_and_barrier<2 * COPIES_PER_OPERAND>(); else wait_copies_and_barrier<0>();  // tile 0 has landed
 #pragma unroll
   for (int x = 0; x < TM + TN; ++x) read_one(0, 1, 0, 0, x);
-#pragma unroll
-  for (int x = 0; x < TM + TN; ++x) read_one(0, 1, 1, 1, x);
 
   int s = 0;  // ring slot of A(kt)
   // Three copies of the tile step (steady state, second-to-last, last) instead of conditions inside one loop body: a
   // branch that joins a path with outstanding LDS reads makes the compiler wait for all of them.
   auto tile_step = [&](int kt, auto has_next, auto load2) {
     const int sa = s, sb = wrap(s + 1), na = wrap(s + 2), nb = wrap(s + 3), fa = wrap(s + 4);
-    constexpr int HALF = COPIES_PER_OPERAND / 2;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
-      if (ks == 2 && has_next) {
+      if (ks == 1 && has_next) {
         if (load2) wait_copies_and_barrier<COPIES_PER_OPERAND>();  // A(kt+2) may still be in flight
         else wait_copies_and_barrier<0>();
       }
 #pragma unroll
       for (int x = 0; x < TM * TN; ++x) {
-        const int i = x / TN, j = x % TN;
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks][i], bfr[ks][j], acc[i][j], 0, 0, 0);
+        const int i = x / TN, j = (i & 1) ? TN - 1 - x % TN : x % TN;
+        mfma_16x16x32(acc[i][j], af[ks][i], bfr[ks][j]);
         __builtin_amdgcn_sched_barrier(0);
-        if (x < TM + TN && !(LMHEAD_ABL & 2)) {
-          if (ks < 2) read_one(sa, sb, ks + 2, ks + 2, x);
-          else if (has_next) read_one(na, nb, ks - 2, ks - 2, x);
+        if (x % 2 == 0 && x < 2 * (TM + TN) && !(LMHEAD_ABL & 2)) {
+          if (ks == 0) read_one(sa, sb, 1, 1, x / 2);
+          else if (has_next) read_one(na, nb, 0, 0, x / 2);
         }
-        if (load2 && x % 4 == 0 && !(LMHEAD_ABL & 1)) {
-          if (ks < 2) copy_part(p.a_bytes, p.a_src, kt + 2, fa, ks * HALF + x / 4, 1, lds);
-          else copy_part(p.b_bytes, p.b_src, kt + 2, sa, (ks - 2) * HALF + x / 4, 1, lds);
+        if (load2 && x % 8 == 4 && !(LMHEAD_ABL & 1)) {
+          if (ks == 0) copy_part(p.a_bytes, p.a_src, kt + 2, fa, x / 8, 1, lds);
+          else copy_part(p.b_bytes, p.b_src, kt + 2, sa, x / 8, 1, lds);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -227,6 +243,16 @@ __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int
   }
   tile_step(kt, no, no);
   wait_copies_and_barrier<0>();
+  // The hardware does not interlock an accumulator read (v_accvgpr_read) against an MFMA still in flight, and the
+  // compiler does not know that the inline assembly is one: left alone it copies an accumulator to a VGPR right
+  // behind the MFMA that wrote it last and gets the old value.  So: 32 wait states behind the last MFMA, then every
+  // accumulator passes through an empty volatile asm -- a new value as far as the compiler can tell, so whatever
+  // reads it is placed after this point.
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) asm volatile("" : "+a"(acc[i][j]));
 }
 
 // Work item id -> tile coordinates.
@@ -251,6 +277,14 @@ __device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, in
   tm = m_first + (in_band - tn * gm);
 }
 
-__device__ __forceinline__ float shfl_xor32(float v) { return __shfl_xor(v, 32, 64); }
+// Sum / maximum over the four lanes (l, l^16, l^32, l^48) that hold the same accumulator column.
+__device__ __forceinline__ float col_sum(float v) {
+  v += __shfl_xor(v, 16, 64);
+  return v + __shfl_xor(v, 32, 64);
+}
+__device__ __forceinline__ float col_max(float v) {
+  v = fmaxf(v, __shfl_xor(v, 16, 64));
+  return fmaxf(v, __shfl_xor(v, 32, 64));
+}
 
 }  // namespace lmhead

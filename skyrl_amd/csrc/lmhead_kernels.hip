@@ -43,7 +43,7 @@ __host__ __device__ inline int64_t round_up(int64_t x, int64_t m) { return (x + 
 // The label-logit gather of that kernel (:364-385) is done in lmhead_fwd_merge instead.
 // ------------------------------------------------------------------------------------------------------------
 template <bool ENTROPY, bool MASKED>
-__device__ __forceinline__ void fwd_tile_stats(const acc_t& acc, int j, int vbase, int V, float scale2, int khalf, float& m_out,
+__device__ __forceinline__ void fwd_tile_stats(const acc_t& acc, int j, int vbase, int V, float scale2, int kq, float& m_out,
                                                float& s_out, float& e_out) {
   // Two read-only passes over the accumulators (they live in AGPRs; writing scaled values back would cost a move each
   // way).  scale2 > 0, so the maximum commutes with the scaling, and sum z*p = scale2 * sum x*p.
@@ -51,32 +51,32 @@ __device__ __forceinline__ void fwd_tile_stats(const acc_t& acc, int j, int vbas
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
+    for (int r = 0; r < 4; ++r) {
       float x = acc[i][j][r];
       if (MASKED) {
-        const int v = vbase + i * 32 + (r >> 2) * 8 + khalf * 4 + (r & 3);
+        const int v = vbase + i * MT + kq * 4 + r;
         if (v >= V) x = -INFINITY;
       }
       mx = fmaxf(mx, x);
     }
-  mx = fmaxf(mx, shfl_xor32(mx));  // finite: the wave has at least one row below V
+  mx = col_max(mx);  // finite: the wave has at least one row below V
   const float m2 = mx * scale2;
   float s = 0.f, e = 0.f;
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
+    for (int r = 0; r < 4; ++r) {
       const float x = acc[i][j][r];
       float p = __builtin_amdgcn_exp2f(fmaf(x, scale2, -m2));
       if (MASKED) {
-        const int v = vbase + i * 32 + (r >> 2) * 8 + khalf * 4 + (r & 3);
+        const int v = vbase + i * MT + kq * 4 + r;
         if (v >= V) p = 0.f;
       }
       s += p;
       if (ENTROPY) e = fmaf(x, p, e);
     }
-  s += shfl_xor32(s);
-  if (ENTROPY) e += shfl_xor32(e);
+  s = col_sum(s);
+  if (ENTROPY) e = col_sum(e);
   m_out = m2 * kLn2;
   s_out = s;
   e_out = e * scale2 * kLn2;
@@ -102,20 +102,20 @@ __global__ __launch_bounds__(NTHREADS) void lmhead_fwd_tiles(const uint16_t* __r
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-  const int lrow = lane & 31, khalf = lane >> 5;
+  const int lrow = lane & 15, kq = lane >> 4;
   const int vbase = tm * BM + wm * WM;
   const size_t part = (size_t)(tm * WAVES_M + wm) * (size_t)T;
   const float scale2 = rcp_temp * kLog2e;
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
-    const int t = tn * BN + wn * WN + j * 32 + lrow;
+    const int t = tn * BN + wn * WN + j * MT + lrow;
     float m = -INFINITY, s = 0.f, e = 0.f;
     if (vbase + WM <= V) {
-      fwd_tile_stats<ENTROPY, false>(acc, j, vbase, V, scale2, khalf, m, s, e);
+      fwd_tile_stats<ENTROPY, false>(acc, j, vbase, V, scale2, kq, m, s, e);
     } else if (vbase < V) {
-      fwd_tile_stats<ENTROPY, true>(acc, j, vbase, V, scale2, khalf, m, s, e);
+      fwd_tile_stats<ENTROPY, true>(acc, j, vbase, V, scale2, kq, m, s, e);
     }
-    if (khalf == 0 && t < T) {
+    if (kq == 0 && t < T) {
       part_max[part + t] = m;
       part_sum[part + t] = s;
       if (ENTROPY) part_pz[part + t] = e;
@@ -262,7 +262,7 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-  const int lrow = lane & 31, khalf = lane >> 5;
+  const int lrow = lane & 15, kq = lane >> 4;
   const int vloc_base = tm * BM + wm * WM;    // first vocab row of this wave inside the chunk panel
   const int vbase = vc0 + vloc_base;          // ... and in the full vocab
   const int tbase = tn * BN + wn * WN;        // first token of this wave (always inside the padded panels)
@@ -274,7 +274,7 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
   int yrel_[TN];
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
-    const int t = tbase + j * 32 + lrow;
+    const int t = tbase + j * MT + lrow;
     const bool valid = t < T;
     const float g = valid ? dlogprobs[t] : 0.f;
     const float q = (ENTGRAD && valid) ? dentropy[t] : 0.f;
@@ -309,56 +309,49 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
   const int q4 = lane & 3;
   const uint32_t sel1 = (q4 & 1) ? 0x03020706u : 0x05040100u;
   const bool upper = (q4 & 2) != 0;
+  constexpr int JH = TN / 2;  // column tiles per half
 
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
 #pragma unroll
-    for (int jj = 0; jj < 2; ++jj) {
-      const int j = half * 2 + jj;
+    for (int jj = 0; jj < JH; ++jj) {
+      const int j = half * JH + jj;
       const float gs = gs_[j], c0 = c0_[j], c1 = c1_[j], lse2 = lse2_[j];
       const int yrel = yrel_[j];
+      const bool any_label = __any(yrel >= 0);  // some token of this column tile has its label inside the wave's rows
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
-        float d[16];
+        float d[4];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
+        for (int r = 0; r < 4; ++r) {
           const float x = acc[i][j][r];
           const float p = __builtin_amdgcn_exp2f(fmaf(x, scale2, -lse2));
           d[r] = ENTGRAD ? p * fmaf(c1, x, c0) : p * c0;
         }
-        const int rel = yrel - i * 32;
-        const bool hit = (yrel >= 0) && ((unsigned)rel < 32u);
-        if (__any(hit)) {
+        const int vl = i * MT + kq * 4;  // vocab row inside the wave block; this lane holds vl .. vl+3
+        if (any_label) {
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int row_r = (r >> 2) * 8 + khalf * 4 + (r & 3);
-            if (hit && rel == row_r) d[r] += gs;
-          }
+          for (int r = 0; r < 4; ++r)
+            if (yrel == vl + r) d[r] += gs;
         }
         if (!full) {
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int v = vbase + i * 32 + (r >> 2) * 8 + khalf * 4 + (r & 3);
-            if (v >= V) d[r] = 0.f;
-          }
+          for (int r = 0; r < 4; ++r)
+            if (vbase + vl + r >= V) d[r] = 0.f;
         }
-#pragma unroll
-        for (int rg = 0; rg < 4; ++rg) {
-          const int vl = i * 32 + rg * 8 + khalf * 4;  // vocab row inside the wave block; this lane holds vl .. vl+3
-          f32x4 v4 = {d[rg * 4 + 0], d[rg * 4 + 1], d[rg * 4 + 2], d[rg * 4 + 3]};
-          const bf16x4 b4 = __builtin_convertvector(v4, bf16x4);
-          uint32_t w0 = ((const uint32_t*)&b4)[0], w1 = ((const uint32_t*)&b4)[1];
-          *(uint2*)(stage_d + (jj * 32 + lrow) * kTokRow + vl * 2) = make_uint2(w0, w1);
-          // 4 x 4 transpose inside the quad: afterwards lane q4 holds vocab row vl + q4 for the quad's four tokens
-          const uint32_t p0 = (uint32_t)__builtin_amdgcn_mov_dpp((int)w0, 0xB1, 0xF, 0xF, true);  // lane ^ 1
-          const uint32_t p1 = (uint32_t)__builtin_amdgcn_mov_dpp((int)w1, 0xB1, 0xF, 0xF, true);
-          w0 = __builtin_amdgcn_perm(p0, w0, sel1);
-          w1 = __builtin_amdgcn_perm(p1, w1, sel1);
-          const uint32_t send = upper ? w0 : w1;
-          const uint32_t recv = (uint32_t)__builtin_amdgcn_mov_dpp((int)send, 0x4E, 0xF, 0xF, true);  // lane ^ 2
-          const uint32_t t0 = upper ? recv : w0, t1 = upper ? w1 : recv;
-          *(uint2*)(stage_dt + (vl + q4) * kVocRow + (jj * 32 + (lrow & ~3)) * 2) = make_uint2(t0, t1);
-        }
+        f32x4 v4 = {d[0], d[1], d[2], d[3]};
+        const bf16x4 b4 = __builtin_convertvector(v4, bf16x4);
+        uint32_t w0 = ((const uint32_t*)&b4)[0], w1 = ((const uint32_t*)&b4)[1];
+        *(uint2*)(stage_d + (jj * MT + lrow) * kTokRow + vl * 2) = make_uint2(w0, w1);
+        // 4 x 4 transpose inside the quad: afterwards lane q4 holds vocab row vl + q4 for the quad's four tokens
+        const uint32_t p0 = (uint32_t)__builtin_amdgcn_mov_dpp((int)w0, 0xB1, 0xF, 0xF, true);  // lane ^ 1
+        const uint32_t p1 = (uint32_t)__builtin_amdgcn_mov_dpp((int)w1, 0xB1, 0xF, 0xF, true);
+        w0 = __builtin_amdgcn_perm(p0, w0, sel1);
+        w1 = __builtin_amdgcn_perm(p1, w1, sel1);
+        const uint32_t send = upper ? w0 : w1;
+        const uint32_t recv = (uint32_t)__builtin_amdgcn_mov_dpp((int)send, 0x4E, 0xF, 0xF, true);  // lane ^ 2
+        const uint32_t t0 = upper ? recv : w0, t1 = upper ? w1 : recv;
+        *(uint2*)(stage_dt + (vl + q4) * kVocRow + (jj * MT + (lrow & ~3)) * 2) = make_uint2(t0, t1);
       }
     }
     // 64 tokens x 128 vocab staged both ways: 1024 16-byte pieces each, 16 per lane.
@@ -380,8 +373,10 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
 }
 
 // ------------------------------------------------------------------------------------------------------------
-// Plain NT GEMM with an fp32 / bf16 store epilogue:  C[M,N] (+)= A[M,K] . B[N,K]^T.
-//   Cin != 0   add the existing fp32 C before storing (accumulation across vocab chunks / micro-batches)
+// Plain NT GEMM with an fp32 / bf16 store epilogue:  C[N,M] (+)= B[N,K] . A[M,K]^T, i.e. C[n][m] = sum_k A[m][k] B[n][k]:
+// the MFMA M axis (rows of A) runs along the contiguous dimension of C, because a lane's four accumulator values are
+// consecutive along M -- one 16-byte fp32 (8-byte bf16) store.  M must be a multiple of 4.
+//   Cin != 0   add the existing fp32 C before storing (accumulation across micro-batches)
 //   Cf  != 0   store fp32;   Cb != 0  store bf16 (round-to-nearest-even)
 // One launch carries up to two independent problems (workgroups [0, tiles0) work on p0, the rest on p1): the dHidden
 // and dWeight products of a vocab chunk have no dependency on each other, and together they fill the 256 CUs in whole
@@ -398,9 +393,8 @@ struct GemmArgs {
   uint16_t* Cb;
   int ldc;
   // Partial sums carried from launch to launch (dHidden across vocab chunks) live in "accumulator order": tile by tile,
-  // wave by wave, each lane's 16 registers of an MFMA block contiguous.  Reading and writing them is 16 bytes per lane
-  // and 4 KiB contiguous per wave instruction group -- a quarter of the instructions of the row-major form, where a
-  // lane's values sit a row apart (measured: the row-major read-modify-write cost 6 % of the backward pass).
+  // wave by wave, MFMA block by MFMA block, each lane's 4 registers contiguous.  Reading and writing them is 16 bytes
+  // per lane and 1 KiB contiguous per wave instruction, with no address arithmetic beyond a constant offset.
   const float* Pin;
   float* Pout;
 };
@@ -427,54 +421,39 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p0, const GemmArgs& p1
   const int ldc = p.ldc;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-  const int lrow = lane & 31, khalf = lane >> 5;
+  const int lrow = lane & 15, kq = lane >> 4;
 
   if (p.Pin || p.Pout) {
-    const size_t base = ((size_t)(tm * tiles_n + tn) * NWAVES + wave) * (TM * TN * 64 * 16) + (size_t)lane * 16;
+    const size_t base = ((size_t)(tm * tiles_n + tn) * NWAVES + wave) * (TM * TN * 64 * 4) + (size_t)lane * 4;
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
-        const size_t off = base + (size_t)(i * TN + j) * (64 * 16);
-        if (p.Pin) {
-          const f32x4* src = (const f32x4*)(p.Pin + off);
-#pragma unroll
-          for (int r4 = 0; r4 < 4; ++r4) {
-            const f32x4 v = src[r4];
-#pragma unroll
-            for (int k = 0; k < 4; ++k) acc[i][j][r4 * 4 + k] += v[k];
-          }
-        }
-        if (p.Pout) {
-          f32x4* dst = (f32x4*)(p.Pout + off);
-#pragma unroll
-          for (int r4 = 0; r4 < 4; ++r4)
-            dst[r4] = f32x4{acc[i][j][r4 * 4], acc[i][j][r4 * 4 + 1], acc[i][j][r4 * 4 + 2], acc[i][j][r4 * 4 + 3]};
-        }
+        const size_t off = base + (size_t)(i * TN + j) * (64 * 4);
+        if (p.Pin) acc[i][j] += *(const f32x4*)(p.Pin + off);
+        if (p.Pout) *(f32x4*)(p.Pout + off) = acc[i][j];
       }
   }
   if (!Cf && !Cb) return;
 
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
-    const int n = tn * BN + wn * WN + j * 32 + lrow;
+    const int n = tn * BN + wn * WN + j * MT + lrow;
     if (n >= N) continue;
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = tm * BM + wm * WM + i * 32 + (r >> 2) * 8 + khalf * 4 + (r & 3);
-        if (m < M) {
-          const size_t idx = (size_t)m * (size_t)ldc + n;
-          float v = acc[i][j][r];
-          if (Cin) v += Cin[idx];
-          if (Cf) Cf[idx] = v;
-          if (Cb) {
-            const __bf16 bv = (__bf16)v;
-            Cb[idx] = *(const uint16_t*)&bv;
-          }
+    for (int i = 0; i < TM; ++i) {
+      const int m = tm * BM + wm * WM + i * MT + kq * 4;  // this lane holds m .. m+3
+      if (m < M) {
+        const size_t idx = (size_t)n * (size_t)ldc + m;
+        f32x4 v = acc[i][j];
+        if (Cin) v += *(const f32x4*)(Cin + idx);
+        if (Cf) *(f32x4*)(Cf + idx) = v;
+        if (Cb) {
+          const bf16x4 b4 = __builtin_convertvector(v, bf16x4);
+          *(uint2*)(Cb + idx) = *(const uint2*)&b4;
         }
       }
+    }
   }
 }
 
@@ -778,15 +757,15 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
     e = launch_bwd_chunk(s, dentropy != nullptr, dz_args(ci), (unsigned)(chunk_width(ci) / 256 * tiles_t), false, none, none);
     if (e != hipSuccess) return (int)e;
     const int64_t vc0 = ci * vc, vcw = chunk_width(ci);
-    // dHidden[T, H] (+)= D[T, vcw] . weight[vc0 : vc0 + vcw, :]    (B operand = weight^T rows, k offset vc0)
-    // dW[vc0 : vc0 + rows, :] (+)= D^T[vcw, Tpad] . hidden          (B operand = hidden^T rows)
+    // dHidden[t, h] (+)= sum_v D[t, v] . weight^T[h, vc0 + v]        (A = weight^T rows at k offset vc0, B = D rows)
+    // dW[vc0 + v, h]  (+)= sum_t D^T[v, t] . hidden^T[h, t]           (A = hidden^T rows, B = D^T rows)
     const bool first = ci == 0, last = ci == nchunks - 1;
     const int64_t rows = (V - vc0) < vcw ? (V - vc0) : vcw;
     float* dWc = d_weight + (size_t)vc0 * (size_t)H;
-    const GemmArgs gh = make_gemm(w.D, vcw + kLdPad, Tpad, w.Wt + vc0, Vpad + kLdPad, H, vcw / BK, T, H, nullptr, nullptr,
+    const GemmArgs gh = make_gemm(w.Wt + vc0, Vpad + kLdPad, H, w.D, vcw + kLdPad, Tpad, vcw / BK, H, T, nullptr, nullptr,
                                   last ? (uint16_t*)d_hidden : (uint16_t*)nullptr, H,
                                   first ? (const float*)nullptr : (const float*)w.dHacc, last ? (float*)nullptr : w.dHacc);
-    const GemmArgs gw = make_gemm(w.DT, Tpad + kLdPad, vcw, w.Ht, Tpad + kLdPad, H, Tpad / BK, rows, H,
+    const GemmArgs gw = make_gemm(w.Ht, Tpad + kLdPad, H, w.DT, Tpad + kLdPad, vcw, Tpad / BK, H, rows,
                                   accumulate_dw ? (const float*)dWc : (const float*)nullptr, dWc, (uint16_t*)nullptr, H);
     e = launch_bwd_chunk(s, dentropy != nullptr, DzArgs{}, 0, true, gh, gw);
     if (e != hipSuccess) return (int)e;
