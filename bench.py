@@ -14,6 +14,9 @@ as the torch custom ops call it.  One JSON line is printed:
   step_roofline  the whole step (8*T*V*H algorithmic flop / step time) against the same peak
   kernels        live HIP-event time per kernel and step
   cpu_baseline   the CPU restatement of the reference's torch implementation, timed on this host on a bounded sample
+  mfma_probe     what the matrix pipe of this GPU sustains with the mainloop's MFMA sequence alone (operands in registers, no
+                 memory access), on N(0,1) operands and on zeros: with random operands the chip is power-limited well below
+                 the published peak, which bounds every bf16 kernel on this benchmark's data
 """
 
 from __future__ import annotations
@@ -67,6 +70,32 @@ def cpu_baseline(cfg, sample_tokens: int):
     }
 
 
+def mfma_probe(lib, dev):
+    """Pure-MFMA rate (TFLOP/s) of the GEMM mainloop's instruction sequence on random and on zero operands."""
+    import torch
+
+    from skyrl_amd import _lib
+
+    wgs, iters = 256, 50000
+    flop = 4.0 * wgs * iters * 128 * 16384
+    sink = torch.empty(256 * wgs, dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    out = {"mfma": "v_mfma_f32_16x16x32_bf16", "workgroups": wgs}
+    gen = torch.Generator().manual_seed(7)
+    for name in ("random", "zero"):
+        ops_ = (torch.randn(65536, generator=gen) if name == "random" else torch.zeros(65536)).to(torch.bfloat16).to(dev)
+        ms = []
+        for it in (iters // 10, iters, iters):  # short warm-up, then two timed launches
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            _lib.check(lib.skyrl_lmhead_mfma_probe(ops_.data_ptr(), wgs, it, sink.data_ptr(), stream), "skyrl_lmhead_mfma_probe")
+            e1.record()
+            torch.cuda.synchronize()
+            ms.append(e0.elapsed_time(e1))
+        out[f"{name}_operands_tflops"] = flop / (min(ms[1:]) * 1e-3) / 1e12
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -76,6 +105,7 @@ def main() -> int:
     ap.add_argument("--vocab-chunk", type=int, default=0)
     ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-mfma-probe", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain 1 GiB device-to-device copy (a kernel of known HBM traffic) so that rocprofv3 "
                          "--pmc FETCH_SIZE / WRITE_SIZE readings of the same run can be scaled to bytes")
@@ -214,6 +244,8 @@ def main() -> int:
         "step_roofline": step_roofline,
         "kernels": kernels,
     }
+    if not args.no_mfma_probe:
+        out["mfma_probe"] = mfma_probe(lib, dev)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_sample_tokens)
     print(json.dumps(out))

@@ -93,6 +93,16 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
                      void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * Measurement aid for benchmarks (no counterpart in the reference): what the matrix pipe sustains on a given kind of
+ * data.  Launches `workgroups` workgroups of 4 wavefronts; each wavefront loads 32 operand fragments once from
+ * `operands` (bf16, 32 fragments x 256 lanes x 8 values = 128 KiB) and then issues iters x 128 v_mfma_f32_16x16x32_bf16
+ * in the order of the GEMM mainloop, with no memory access in the loop: 4 * workgroups * iters * 128 * 16384 flop.
+ * `sink` receives 256 * workgroups floats.  On an MI355X the rate depends on the operand values (power): zeros run at the
+ * published peak, N(0,1) operands well below it.
+ */
+int skyrl_lmhead_mfma_probe(const void* operands, int workgroups, int iters, float* sink, void* stream);
+
+/*
  * Per-kernel timing for benchmarks (no counterpart in the reference, which times whole calls from Python with
  * torch.cuda.synchronize, skyrl/benchmarks/bench_fused_linear_logprob.py:96-101).
  * skyrl_lmhead_profile_begin() opens a profile on the calling thread and returns its handle (NULL if one is already open):

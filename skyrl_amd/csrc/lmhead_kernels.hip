@@ -468,6 +468,40 @@ __global__ __launch_bounds__(NTHREADS) void lmhead_bwd_chunk(const DzArgs z, con
   else dz_tile<ENTGRAD>(z, id - gemm_tiles, lds);
 }
 
+// Measurement aid: the mainloop's MFMA sequence (two 32-k steps of 64 MFMAs, same order, accumulators in AGPRs) with
+// register-resident operands and nothing else in the loop -- what the matrix pipe sustains on a given kind of data.
+__global__ __launch_bounds__(NTHREADS) void mfma_probe(const bf16x8* __restrict__ operands, int iters, float* __restrict__ sink) {
+  bf16x8 af[2][TM], bfr[2][TN];
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      af[s][i] = operands[((s * TM + i) * 2 + 0) * NTHREADS + threadIdx.x];
+      bfr[s][i] = operands[((s * TM + i) * 2 + 1) * NTHREADS + threadIdx.x];
+    }
+  acc_t acc;
+  zero_acc(acc);
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks)
+#pragma unroll
+      for (int x = 0; x < TM * TN; ++x) {
+        const int i = x / TN, j = (i & 1) ? TN - 1 - x % TN : x % TN;
+        mfma_16x16x32(acc[i][j], af[ks][i], bfr[ks][j]);
+      }
+  }
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      asm volatile("" : "+a"(acc[i][j]));
+      sum += acc[i][j][0] + acc[i][j][1] + acc[i][j][2] + acc[i][j][3];
+    }
+  sink[blockIdx.x * NTHREADS + threadIdx.x] = sum;
+}
+
 // dst[c, r] = src[r, c] for r < R, c < C;  dst[c, r] = 0 for R <= r < Rpad.  bf16 bits, 64 x 64 tiles.
 __global__ __launch_bounds__(256) void transpose_bf16(const uint16_t* __restrict__ src, int lds_src, int R, int C,
                                                       uint16_t* __restrict__ dst, int ld_dst, int Rpad) {
@@ -628,7 +662,7 @@ hipError_t launch_bwd_chunk(hipStream_t s, bool entgrad, const DzArgs& z, unsign
 
 extern "C" {
 
-int skyrl_lmhead_version(void) { return 1; }
+int skyrl_lmhead_version(void) { return 2; }
 
 const char* skyrl_lmhead_strerror(int status) {
   switch (status) {
@@ -771,6 +805,15 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
     if (e != hipSuccess) return (int)e;
   }
   return SKYRL_LMHEAD_OK;
+}
+
+int skyrl_lmhead_mfma_probe(const void* operands, int workgroups, int iters, float* sink, void* stream) {
+  if (!operands || !sink) return SKYRL_LMHEAD_ERR_NULL;
+  if (workgroups < 1 || workgroups > 65536 || iters < 1) return SKYRL_LMHEAD_ERR_ARG;
+  if (!aligned16(operands)) return SKYRL_LMHEAD_ERR_ALIGN;
+  hipLaunchKernelGGL(mfma_probe, dim3((unsigned)workgroups), dim3(NTHREADS), 0, (hipStream_t)stream, (const bf16x8*)operands, iters,
+                     sink);
+  return (int)hipGetLastError();
 }
 
 int skyrl_lmhead_num_kernel_kinds(void) { return kNumKernelKinds; }

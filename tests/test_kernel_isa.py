@@ -1,0 +1,98 @@
+"""Checks on the generated gfx950 code of the MFMA kernels (no GPU needed: hipcc cross-compiles to assembly).
+
+The mainloop issues its MFMAs as inline assembly (``gemm_core.hpp: mfma_16x16x32``), so the compiler neither pads the
+MFMA -> accumulator-read hazard nor knows that the accumulators must stay where they are.  These tests read the assembly of
+every kernel that contains MFMAs and check the three properties the source relies on:
+
+* every ``v_accvgpr_read`` comes after the explicit wait states that follow the last MFMA before it;
+* every MFMA accumulates in place, in AGPRs (no rotation of accumulators through the loop);
+* the steady-state loop (the block with MFMAs and global->LDS copies) has no scratch (spill) traffic and no accumulator moves.
+"""
+
+from __future__ import annotations
+
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+from skyrl_amd.csrc import build as B
+
+pytestmark = pytest.mark.skipif(
+    not (shutil.which("hipcc") or os.path.exists("/opt/rocm/bin/hipcc")), reason="hipcc not available"
+)
+
+
+@pytest.fixture(scope="module")
+def kernels(tmp_path_factory):
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    out = tmp_path_factory.mktemp("isa") / "lmhead.s"
+    flags = [f for f in B.HIPCC_FLAGS if f not in ("-shared", "-fPIC")]
+    cmd = [hipcc, *flags, "-S", "--cuda-device-only", "-o", str(out), os.path.join(B.HERE, B.SOURCES[0])]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    text = out.read_text()
+    found = {}
+    for m in re.finditer(r"^(_Z\w+):", text, re.M):
+        name = m.group(1)
+        end = text.find(".end_amdhsa_kernel", m.end())
+        nxt = text.find("\n_Z", m.end())
+        body = text[m.end(): end if end != -1 else None]
+        if nxt != -1 and nxt < end:
+            continue  # a device function label, not a kernel body
+        lines = [ln.strip() for ln in body.split("\n") if ln.strip() and not ln.strip().startswith(";")]
+        if any(ln.startswith("v_mfma") for ln in lines):
+            found[name] = lines
+    return found
+
+
+def test_mfma_kernels_found(kernels):
+    names = " ".join(kernels)
+    for expect in ("lmhead_fwd_tiles", "lmhead_bwd_chunk", "mfma_probe"):
+        assert expect in names, f"no MFMA kernel named *{expect}* in the assembly: {list(kernels)}"
+
+
+def test_accumulator_reads_follow_the_wait_states(kernels):
+    for name, lines in kernels.items():
+        waited = False
+        for ln in lines:
+            if ln.startswith("v_mfma"):
+                waited = False
+            elif ln.startswith("s_nop 15"):
+                waited = True
+            elif ln.startswith("v_accvgpr_read"):
+                assert waited, f"{name}: '{ln}' is not behind the wait states that follow the last MFMA"
+
+
+def test_mfma_accumulates_in_place_in_agprs(kernels):
+    pat = re.compile(r"v_mfma_f32_16x16x32_bf16 (a\[\d+:\d+\]), v\[\d+:\d+\], v\[\d+:\d+\], (a\[\d+:\d+\])$")
+    for name, lines in kernels.items():
+        for ln in lines:
+            if ln.startswith("v_mfma"):
+                m = pat.match(ln)
+                assert m and m.group(1) == m.group(2), f"{name}: unexpected MFMA form '{ln}'"
+
+
+def test_steady_state_loop_is_clean(kernels):
+    for name, lines in kernels.items():
+        # split into basic blocks at labels
+        blocks, cur = [], []
+        for ln in lines:
+            if re.match(r"^\.LBB\w+:", ln):
+                blocks.append(cur)
+                cur = []
+            cur.append(ln)
+        blocks.append(cur)
+        matched = 0
+        for b in blocks:
+            n_mfma = sum(ln.startswith("v_mfma") for ln in b)
+            n_copy = sum(ln.startswith("global_load_lds") for ln in b)
+            if n_mfma >= 128 and n_copy >= 16:  # the steady-state k-tile step
+                matched += 1
+                bad = [ln for ln in b if ln.startswith(("scratch_", "v_accvgpr_"))]
+                assert not bad, f"{name}: steady-state loop has spill / accumulator traffic: {bad[:4]}"
+                assert n_mfma == 128 and n_copy == 16, f"{name}: loop body has {n_mfma} MFMAs, {n_copy} copies"
+        if any(ln.startswith("global_load_lds") for ln in lines):
+            assert matched >= 1, f"{name}: no steady-state loop block recognised"
