@@ -138,12 +138,12 @@ __device__ __forceinline__ void make_plan(CopyPlan& p, const Operand& a, const O
   p.b_bytes = (const char*)b.ptr + (size_t)k_begin * 2;
 }
 
-// Copies j0 .. j0+n-1 (of COPIES_PER_OPERAND) of k-tile t of one operand into ring slot `slot`.
-__device__ __forceinline__ void copy_part(const char* bytes, const uint32_t (&src)[COPIES_PER_OPERAND], int t, int slot,
+// Copies j0 .. j0+n-1 (of COPIES_PER_OPERAND) of k-tile t of one operand into the ring slot at byte offset `slot_off`.
+__device__ __forceinline__ void copy_part(const char* bytes, const uint32_t (&src)[COPIES_PER_OPERAND], int t, int slot_off,
                                           int j0, int n, char* lds) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const char* g = bytes + (size_t)t * (BK * 2);
-  char* dst = lds + slot * OPERAND_BYTES + wave * 1024;
+  char* dst = lds + slot_off + wave * 1024;
 #pragma unroll
   for (int j = j0; j < j0 + n; ++j)
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(g + src[j]),
@@ -156,11 +156,11 @@ __device__ __forceinline__ void copy_part(const char* bytes, const uint32_t (&sr
 __device__ __forceinline__ void prefetch_first_tiles(const Operand& a, const Operand& b, int k_begin, int nk, char* lds) {
   CopyPlan p;  // rebuilt by mainloop(): keeping it in registers across an epilogue costs more than recomputing it
   make_plan(p, a, b, k_begin);
-  copy_part(p.a_bytes, p.a_src, 0, 0, 0, COPIES_PER_OPERAND, lds);
-  copy_part(p.b_bytes, p.b_src, 0, 1, 0, COPIES_PER_OPERAND, lds);
+  copy_part(p.a_bytes, p.a_src, 0, 0 * OPERAND_BYTES, 0, COPIES_PER_OPERAND, lds);
+  copy_part(p.b_bytes, p.b_src, 0, 1 * OPERAND_BYTES, 0, COPIES_PER_OPERAND, lds);
   if (nk > 1) {
-    copy_part(p.a_bytes, p.a_src, 1, 2, 0, COPIES_PER_OPERAND, lds);
-    copy_part(p.b_bytes, p.b_src, 1, 3, 0, COPIES_PER_OPERAND, lds);
+    copy_part(p.a_bytes, p.a_src, 1, 2 * OPERAND_BYTES, 0, COPIES_PER_OPERAND, lds);
+    copy_part(p.b_bytes, p.b_src, 1, 3 * OPERAND_BYTES, 0, COPIES_PER_OPERAND, lds);
   }
 }
 
@@ -187,28 +187,37 @@ __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int lrow = lane & 15;
   const int xsw = ((lane >> 4) ^ swz(lrow)) << 4;  // chunk offset of k-step 0; k-step 1 is xsw ^ 64
-  const int a_base = (wm * WM + lrow) * ROW_BYTES;
-  const int b_base = (wn * WN + lrow) * ROW_BYTES;
-  auto wrap = [](int x) { return x >= RING_SLOTS ? x - RING_SLOTS : x; };
+  // Per-lane fragment addresses inside a slot, for k-step 0 and 1 of the A and of the B operand.
+  const int a_off0 = (wm * WM + lrow) * ROW_BYTES + xsw, a_off1 = (wm * WM + lrow) * ROW_BYTES + (xsw ^ 64);
+  const int b_off0 = (wn * WN + lrow) * ROW_BYTES + xsw, b_off1 = (wn * WN + lrow) * ROW_BYTES + (xsw ^ 64);
 
   bf16x8 af[2][TM], bfr[2][TN];
   // Fragment x of a 32-k step: x < TM is the A fragment of MFMA row x, otherwise the B fragment of MFMA column x - TM.
-  auto read_one = [&](int slot_a, int slot_b, int ks, int set, int x) {
-    if (x < TM)
-      af[set][x] = *(const bf16x8*)(lds + slot_a * OPERAND_BYTES + a_base + (xsw ^ (ks << 6)) + x * MT * ROW_BYTES);
-    else
-      bfr[set][x - TM] = *(const bf16x8*)(lds + slot_b * OPERAND_BYTES + b_base + (xsw ^ (ks << 6)) + (x - TM) * MT * ROW_BYTES);
+  auto read_one = [&](const char* pa, const char* pb, int set, int x) {
+    if (x < TM) af[set][x] = *(const bf16x8*)(pa + x * MT * ROW_BYTES);
+    else bfr[set][x - TM] = *(const bf16x8*)(pb + (x - TM) * MT * ROW_BYTES);
   };
 
   if (nk > 1) wait_copies_and_barrier<2 * COPIES_PER_OPERAND>(); else wait_copies_and_barrier<0>();  // tile 0 has landed
 #pragma unroll
-  for (int x = 0; x < TM + TN; ++x) read_one(0, 1, 0, 0, x);
+  for (int x = 0; x < TM + TN; ++x) read_one(lds + a_off0, lds + OPERAND_BYTES + b_off0, 0, x);
 
-  int s = 0;  // ring slot of A(kt)
+  // Ring state, as byte offsets of the slots in the order A(kt), B(kt), A(kt+1), B(kt+1), free.  Advancing one k-tile
+  // rotates the five values by two places, so no arithmetic is needed; the fragment addresses of the next k-tile are
+  // formed in the shadow of MFMAs in the middle of a step, not at the top of the loop where nothing would hide them.
+  int o0 = 0, o1 = OPERAND_BYTES, o2 = 2 * OPERAND_BYTES, o3 = 3 * OPERAND_BYTES, o4 = 4 * OPERAND_BYTES;
+  int ra1 = o0 + a_off1, rb1 = o1 + b_off1;  // step-0 reads: k-step 1 of this k-tile (byte offsets into lds)
+  int ra0 = o2 + a_off0, rb0 = o3 + b_off0;  // step-1 reads: k-step 0 of the next k-tile
+  // An add the compiler cannot move: it would otherwise collect these at the top of the loop body.
+  auto pinned_add = [](int slot_off, int lane_off) {
+    int r;
+    asm volatile("v_add_u32_e32 %0, %1, %2" : "=v"(r) : "s"(slot_off), "v"(lane_off));
+    return r;
+  };
   // Three copies of the tile step (steady state, second-to-last, last) instead of conditions inside one loop body: a
   // branch that joins a path with outstanding LDS reads makes the compiler wait for all of them.
   auto tile_step = [&](int kt, auto has_next, auto load2) {
-    const int sa = s, sb = wrap(s + 1), na = wrap(s + 2), nb = wrap(s + 3), fa = wrap(s + 4);
+    int nra1 = ra1, nrb1 = rb1, nra0 = ra0, nrb0 = rb0;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       if (ks == 1 && has_next) {
@@ -221,17 +230,25 @@ __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int
         mfma_16x16x32(acc[i][j], af[ks][i], bfr[ks][j]);
         __builtin_amdgcn_sched_barrier(0);
         if (x % 2 == 0 && x < 2 * (TM + TN) && !(LMHEAD_ABL & 2)) {
-          if (ks == 0) read_one(sa, sb, 1, 1, x / 2);
-          else if (has_next) read_one(na, nb, 0, 0, x / 2);
+          if (ks == 0) read_one(lds + ra1, lds + rb1, 1, x / 2);
+          else if (has_next) read_one(lds + ra0, lds + rb0, 0, x / 2);
         }
         if (load2 && x % 8 == 4 && !(LMHEAD_ABL & 1)) {
-          if (ks == 0) copy_part(p.a_bytes, p.a_src, kt + 2, fa, x / 8, 1, lds);
-          else copy_part(p.b_bytes, p.b_src, kt + 2, sa, x / 8, 1, lds);
+          if (ks == 0) copy_part(p.a_bytes, p.a_src, kt + 2, o4, x / 8, 1, lds);
+          else copy_part(p.b_bytes, p.b_src, kt + 2, o0, x / 8, 1, lds);
+        }
+        if (has_next) {  // next k-tile's fragment addresses, one per MFMA shadow, after this step's reads are issued
+          if (ks == 0 && x == 41) nra1 = pinned_add(o2, a_off1);
+          if (ks == 0 && x == 43) nrb1 = pinned_add(o3, b_off1);
+          if (ks == 1 && x == 41) nra0 = pinned_add(o4, a_off0);
+          if (ks == 1 && x == 43) nrb0 = pinned_add(o0, b_off0);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    s = wrap(s + 2);
+    ra1 = nra1, rb1 = nrb1, ra0 = nra0, rb0 = nrb0;
+    const int t0 = o0, t1 = o1;
+    o0 = o2, o1 = o3, o2 = o4, o3 = t0, o4 = t1;
   };
   std::true_type yes;
   std::false_type no;
