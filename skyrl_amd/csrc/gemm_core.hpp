@@ -253,11 +253,6 @@ __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int
   std::true_type yes;
   std::false_type no;
   int kt = 0;
-  // Five k-tiles bring the ring back to where it started: unrolled by five the rotation costs no moves.
-  for (; kt + 2 + (RING_SLOTS - 1) < nk; kt += RING_SLOTS) {
-#pragma unroll
-    for (int u = 0; u < RING_SLOTS; ++u) tile_step(kt + u, yes, yes);
-  }
   for (; kt + 2 < nk; ++kt) tile_step(kt, yes, yes);
   if (kt + 1 < nk) {
     tile_step(kt, yes, no);
