@@ -106,6 +106,10 @@ def main() -> int:
     ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-mfma-probe", action="store_true")
+    ap.add_argument("--skip-masked-rows", action="store_true",
+                    help="run the backward pass through skyrl_amd.ops.lmhead_bwd_active_rows, which drops the tokens whose "
+                         "upstream gradients are zero (the configurations with a response mask); value stays tokens/s over "
+                         "all T tokens, the roofline figures count the flop actually executed")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain 1 GiB device-to-device copy (a kernel of known HBM traffic) so that rocprofv3 "
                          "--pmc FETCH_SIZE / WRITE_SIZE readings of the same run can be scaled to bytes")
@@ -151,12 +155,18 @@ def main() -> int:
     stream = torch.cuda.current_stream(dev).cuda_stream
     ptr = lambda t: None if t is None else t.data_ptr()  # noqa: E731
 
+    skip = bool(args.skip_masked_rows and cfg.backward)
+    t_active = int(((g != 0) | ((q != 0) if q is not None else False)).sum().item()) if skip else T
+
     def step():
         st = lib.skyrl_lmhead_fwd(hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), labels.data_ptr(),
                                   T, H, V, rcp_t, logprobs.data_ptr(), ptr(entropy), row_lse.data_ptr(), ptr(row_pz),
                                   ws_f.data_ptr(), ws_f.numel(), stream)
         _lib.check(st, "skyrl_lmhead_fwd")
-        if cfg.backward:
+        if skip:
+            ops.lmhead_bwd_active_rows(hidden, weight, labels, row_lse, row_pz if q is not None else None, g, q, rcp_t,
+                                       args.vocab_chunk)
+        elif cfg.backward:
             st = lib.skyrl_lmhead_bwd(hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0),
                                       labels.data_ptr(), row_lse.data_ptr(), ptr(row_pz) if q is not None else None,
                                       g.data_ptr(), ptr(q), T, H, V, rcp_t, d_hidden.data_ptr(), d_weight.data_ptr(), 0,
@@ -187,7 +197,8 @@ def main() -> int:
 
     kernels = {k: {"ms_per_step": ms / args.steps, "launches_per_step": n / args.steps, "avg_launch_ms": ms / n}
                for k, (ms, n) in prof.results.items() if n}
-    step_flop = cfg.total_flop
+    # Executed flop: forward over all T tokens, backward over the tokens that were not dropped.
+    step_flop = cfg.total_flop if not skip else 2.0 * T * V * H + 6.0 * t_active * V * H
     step_roofline = {"bound": "mfma", "achieved": step_flop / (ms_per_step * 1e-3) / 1e12, "peak": PEAK_BF16_DENSE_FLOPS / 1e12,
                      "unit": "TFLOP/s"}
     step_roofline["frac"] = step_roofline["achieved"] / step_roofline["peak"]
@@ -197,7 +208,7 @@ def main() -> int:
         # lmhead_bwd_chunk: every backward launch (per vocab chunk one with the dz tiles, one with the gradient GEMM tiles);
         # over a step the launches add up to the logits recompute, dHidden and dWeight = 6*T*V*H flop.
         ks = [kernels[n] for n in ("lmhead_bwd_chunk[dz]", "lmhead_bwd_chunk[gemm]")]  # the same kernel, two kinds of launch
-        dom_name, dom_flop = "lmhead_bwd_chunk", 6.0 * T * V * H
+        dom_name, dom_flop = "lmhead_bwd_chunk", 6.0 * t_active * V * H
         dom_ms, dom_launches = sum(k["ms_per_step"] for k in ks), sum(k["launches_per_step"] for k in ks)
     else:
         k = kernels["lmhead_fwd_tiles"]
@@ -235,6 +246,7 @@ def main() -> int:
                         f"{', entropy with upstream grad' if cfg.entropy_grad else (', entropy' if cfg.entropy else '')}",
             "T": T, "H": H, "V": V, "temperature": cfg.temperature,
             "vocab_chunk": args.vocab_chunk or "library default",
+            "backward_tokens": t_active,
             "device": torch.cuda.get_device_name(0),
             "compute_units": torch.cuda.get_device_properties(0).multi_processor_count,
         },

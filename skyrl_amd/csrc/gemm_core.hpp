@@ -63,9 +63,6 @@ constexpr int RING_SLOTS = 5;
 constexpr int LDS_BYTES = RING_SLOTS * OPERAND_BYTES;  // 160 KiB: the whole LDS of a CU
 constexpr int COPIES_PER_OPERAND = OPERAND_BYTES / 1024 / NWAVES;  // 8 global_load_lds per lane per operand tile
 static_assert(KSTEPS == 2 && TM == 8 && TN == 8 && COPIES_PER_OPERAND == 8, "the schedule below is written for these");
-#ifndef LMHEAD_ABL
-#define LMHEAD_ABL 0  // timing-only ablations (wrong results): 1 no copies in the loop, 2 no fragment reads in the loop
-#endif
 
 // LDS on gfx950 has 64 banks of 4 bytes and serves a ds_read_b128 sixteen lanes (256 B) at a time.  Sixteen consecutive
 // lanes of a fragment read touch 16 consecutive rows at one k-chunk.  XOR-ing the chunk index with (row >> 1) & 7 spreads those
@@ -229,11 +226,11 @@ __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int
         const int i = x / TN, j = (i & 1) ? TN - 1 - x % TN : x % TN;
         mfma_16x16x32(acc[i][j], af[ks][i], bfr[ks][j]);
         __builtin_amdgcn_sched_barrier(0);
-        if (x % 2 == 0 && x < 2 * (TM + TN) && !(LMHEAD_ABL & 2)) {
+        if (x % 2 == 0 && x < 2 * (TM + TN)) {
           if (ks == 0) read_one(lds + ra1, lds + rb1, 1, x / 2);
           else if (has_next) read_one(lds + ra0, lds + rb0, 0, x / 2);
         }
-        if (load2 && x % 8 == 4 && !(LMHEAD_ABL & 1)) {
+        if (load2 && x % 8 == 4) {
           if (ks == 0) copy_part(p.a_bytes, p.a_src, kt + 2, o4, x / 8, 1, lds);
           else copy_part(p.b_bytes, p.b_src, kt + 2, o0, x / 8, 1, lds);
         }
