@@ -102,6 +102,15 @@ def test_backward_argument_errors():
     assert call(H=96, ldh=96, ldw=96) == -2
 
 
+def test_mfma_probe_argument_errors():
+    lib = _lib.load()
+    assert lib.skyrl_lmhead_mfma_probe(None, 256, 10, 0x2000, None) == -1
+    assert lib.skyrl_lmhead_mfma_probe(0x1000, 256, 10, None, None) == -1
+    assert lib.skyrl_lmhead_mfma_probe(0x1000, 0, 10, 0x2000, None) == -5
+    assert lib.skyrl_lmhead_mfma_probe(0x1000, 256, 0, 0x2000, None) == -5
+    assert lib.skyrl_lmhead_mfma_probe(0x1008, 256, 10, 0x2000, None) == -3
+
+
 def test_status_to_exception_mapping():
     with pytest.raises(ValueError, match="NULL"):
         _lib.check(-1, "x")

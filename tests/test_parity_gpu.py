@@ -308,6 +308,30 @@ def test_c_abi_called_directly(cuda_device):
 # ---------------------------------------------------------------------------------------------------------------------
 # the reference's call signatures
 # ---------------------------------------------------------------------------------------------------------------------
+def test_mfma_probe_sums_exactly(cuda_device):
+    """The measurement kernel runs the mainloop's MFMA sequence on caller-given operands: with small integers the sum of
+    every wavefront's accumulators has a closed form, sum_k (sum_m A[m,k]) (sum_n B[n,k]) per pair of fragments."""
+    lib = _lib.load()
+    gen = torch.Generator().manual_seed(3)
+    ops_cpu = torch.randint(-3, 4, (2, 8, 2, 256, 8), generator=gen).to(torch.float32)  # [k-step, fragment, A/B, thread, 8 k]
+    dev_ops = ops_cpu.to(torch.bfloat16).to(cuda_device).contiguous()
+    wgs, iters = 3, 5
+    sink = torch.empty(256 * wgs, dtype=torch.float32, device=cuda_device)
+    st = lib.skyrl_lmhead_mfma_probe(dev_ops.data_ptr(), wgs, iters, sink.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    _lib.check(st, "skyrl_lmhead_mfma_probe")
+    torch.cuda.synchronize()
+    got = sink.view(wgs, 4, 64).sum(-1).double().cpu()  # per workgroup and wavefront
+    want = torch.zeros(4, dtype=torch.float64)
+    for w in range(4):
+        frag = ops_cpu[:, :, :, 64 * w:64 * (w + 1), :].double()             # [2, 8, 2, 64 lanes, 8]
+        # lane l holds row l & 15 and the k values (l >> 4) * 8 .. + 7: sum over the 16 rows -> [2, 8, 2, 32 k]
+        colsum = frag.view(2, 8, 2, 4, 16, 8).sum(4).reshape(2, 8, 2, 32)
+        a, b = colsum[:, :, 0].sum(1), colsum[:, :, 1].sum(1)                 # sums over the 8 A / 8 B fragments: [2, 32]
+        want[w] = iters * (a * b).sum()
+    for g in range(wgs):
+        assert torch.equal(got[g], want), f"workgroup {g}: {got[g].tolist()} vs {want.tolist()}"
+
+
 @pytest.mark.parametrize("oov", [False, True])
 @pytest.mark.parametrize("chunk", [1, 7, 64, 512])
 def test_fused_linear_logprob_apply_matches_reference_statement(oov, chunk, cuda_device):
