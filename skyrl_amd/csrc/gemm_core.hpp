@@ -105,6 +105,14 @@ __device__ __forceinline__ void zero_acc(acc_t& acc) {
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+  // The other hazard the compiler cannot see: an MFMA must not read an accumulator within a few cycles of the
+  // v_accvgpr_write that set it.  Wait states here, and every accumulator passes through an empty volatile asm so that
+  // the writes are placed before them.
+  asm volatile("s_nop 7" ::: "memory");
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) asm volatile("" : "+a"(acc[i][j]));
 }
 
 // Per-lane plan of the global->LDS copies of one output tile: which global 16-byte chunk lands in which LDS chunk.

@@ -2,9 +2,10 @@
 
 The mainloop issues its MFMAs as inline assembly (``gemm_core.hpp: mfma_16x16x32``), so the compiler neither pads the
 MFMA -> accumulator-read hazard nor knows that the accumulators must stay where they are.  These tests read the assembly of
-every kernel that contains MFMAs and check the three properties the source relies on:
+every kernel that contains MFMAs and check the properties the source relies on:
 
-* every ``v_accvgpr_read`` comes after the explicit wait states that follow the last MFMA before it;
+* every ``v_accvgpr_read`` comes after the explicit wait states that follow the last MFMA before it, and no
+  ``v_accvgpr_write`` sits right in front of an MFMA;
 * every MFMA accumulates in place, in AGPRs (no rotation of accumulators through the loop);
 * the steady-state loop (the block with MFMAs and global->LDS copies) has no scratch (spill) traffic and no accumulator moves.
 """
@@ -64,6 +65,14 @@ def test_accumulator_reads_follow_the_wait_states(kernels):
                 waited = True
             elif ln.startswith("v_accvgpr_read"):
                 assert waited, f"{name}: '{ln}' is not behind the wait states that follow the last MFMA"
+
+
+def test_no_accumulator_write_right_before_an_mfma(kernels):
+    for name, lines in kernels.items():
+        for k, ln in enumerate(lines):
+            if ln.startswith("v_mfma"):
+                near = [p for p in lines[max(0, k - 3):k] if p.startswith("v_accvgpr_write")]
+                assert not near, f"{name}: {near[0]} within three instructions of '{ln}'"
 
 
 def test_mfma_accumulates_in_place_in_agprs(kernels):
