@@ -93,6 +93,24 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
                      void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * The consumer one step after the log-probabilities: PPO policy loss ("regular" and "dual_clip") and its gradient with
+ * respect to the log-probabilities in one pass -- what ppo_policy_loss computes with elementwise torch kernels plus
+ * autograd (skyrl/backends/skyrl_train/utils/ppo_utils.py:555-588, with safe_exp_delta / masked_mean of
+ * skyrl/backends/skyrl_train/utils/torch_utils.py:180-192 and reduce_loss of ppo_utils.py:1145-1149):
+ *     ratio = exp(clamp(logprobs - old_logprobs, -20, 20))
+ *     loss  = -min(ratio * A, clamp(ratio, 1 - eps_clip_low, 1 + eps_clip_high) * A)
+ *     dual_clip != 0:  loss = A < 0 ? min(-A * clip_ratio_c, loss) : loss
+ * All arrays fp32 [T].  loss_mask and loss_weight may be NULL (= 1); loss_weight is any factor of the loss that does not
+ * depend on logprobs (the off-policy importance ratio).  out3 = { sum loss*mask*weight, sum [clipped]*mask, sum mask }
+ * (clip_ratio of the reference = out3[1] / max(out3[2], 1)).  dlogprobs (may be NULL) receives
+ * d out3[0] / d logprobs, i.e. the upstream gradient skyrl_lmhead_bwd takes when the loss is that sum.
+ */
+int skyrl_ppo_policy_loss(const float* logprobs, const float* old_logprobs, const float* advantages,
+                          const float* loss_mask, const float* loss_weight, int64_t T,
+                          float eps_clip_low, float eps_clip_high, float clip_ratio_c, int dual_clip,
+                          float* out3, float* dlogprobs, void* stream);
+
+/*
  * Measurement aid for benchmarks (no counterpart in the reference): what the matrix pipe sustains on a given kind of
  * data.  Launches `workgroups` workgroups of 4 wavefronts; each wavefront loads 32 operand fragments once from
  * `operands` (bf16, 32 fragments x 256 lanes x 8 values = 128 KiB) and then issues iters x 128 v_mfma_f32_16x16x32_bf16

@@ -20,6 +20,9 @@ What pins each function (all in ``tests/test_oracle.py``; none of them re-types 
   * out-of-vocabulary targets: forward 0 / backward keeps -p*g, by construction of an autograd twin whose target logit is
     multiplied by the in-vocabulary mask.
   * packed-sequence roll and scatter-back: a per-sequence Python loop.
+  * PPO policy loss: hand-computed cases on both sides of every branch (unclipped, clipped high / low for either sign of
+    the advantage, dual-clip active / inactive, the +-20 clamp of the log-ratio), fp64 central finite differences of the
+    loss for the gradient autograd derives from it, and the masked-mean definition of clip_ratio counted by hand.
 No function is left "parity unpinned".
 """
 
@@ -347,3 +350,39 @@ def exact_fwd_bwd(
                                                round_d_logits_to=dtype)
         out["d_hidden"], out["d_weight"] = dh, dw
     return out
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# The consumer one step after the log-probabilities: PPO policy loss
+# ----------------------------------------------------------------------------------------------------------------------
+def ppo_policy_loss(
+    log_probs: torch.Tensor,
+    old_log_probs: torch.Tensor,
+    advantages: torch.Tensor,
+    eps_clip_low: float,
+    eps_clip_high: float,
+    clip_ratio_c: float = 3.0,
+    dual_clip: bool = False,
+    loss_mask: Optional[torch.Tensor] = None,
+    loss_weight: Optional[torch.Tensor] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """skyrl/backends/skyrl_train/utils/ppo_utils.py:555-588 ("regular" and "dual_clip"), with safe_exp_delta and masked_mean of
+    skyrl/backends/skyrl_train/utils/torch_utils.py:180-192 and reduce_loss of ppo_utils.py:1145-1149.  ``loss_weight`` stands
+    for the importance ratio apply_off_policy_correction multiplies in (off_policy_correction_utils.py:383-384).  Returns
+    ``(loss, clip_ratio)``; the gradient is whatever autograd derives from these torch ops, as in the reference."""
+    ratio = torch.clamp(log_probs - old_log_probs, -20.0, 20.0).exp()                    # safe_exp_delta, clip=20
+    surr1 = ratio * advantages
+    surr2 = ratio.clamp(1 - eps_clip_low, 1 + eps_clip_high) * advantages
+    loss = -torch.min(surr1, surr2)
+    clipped = (-surr2 > -surr1).to(log_probs.dtype)
+    if loss_mask is None:
+        clip_ratio = clipped.mean()                                                      # masked_mean without a mask
+    else:
+        clip_ratio = (clipped * loss_mask).sum() / loss_mask.sum().clamp(min=1.0)
+    if dual_clip:
+        pg_losses3 = -advantages * clip_ratio_c
+        loss = torch.where(advantages < 0, torch.min(pg_losses3, loss), loss)
+    if loss_weight is not None:
+        loss = loss * loss_weight
+    loss = (loss * loss_mask).sum() if loss_mask is not None else loss.sum()            # reduce_loss
+    return loss, clip_ratio.detach()

@@ -11,7 +11,7 @@ import os
 import threading
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libskyrl_lmhead.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _c_i64 = ctypes.c_int64
 _c_p = ctypes.c_void_p
@@ -31,6 +31,10 @@ SIGNATURES = {
         ctypes.c_int,
         [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, ctypes.c_float, _c_p, _c_p,
          ctypes.c_int, _c_i64, _c_p, ctypes.c_size_t, _c_p],
+    ),
+    "skyrl_ppo_policy_loss": (
+        ctypes.c_int,
+        [_c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_int, _c_p, _c_p, _c_p],
     ),
     "skyrl_lmhead_mfma_probe": (ctypes.c_int, [_c_p, ctypes.c_int, ctypes.c_int, _c_p, _c_p]),
     "skyrl_lmhead_num_kernel_kinds": (ctypes.c_int, []),

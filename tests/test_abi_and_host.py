@@ -20,7 +20,7 @@ HEADER = os.path.join(ROOT, "include", "skyrl_lmhead.h")
 def _declared_functions():
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(skyrl_lmhead_\w+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(skyrl_(?:lmhead|ppo)_\w+)\s*\(", text)))
 
 
 def test_library_exports_every_declared_symbol():
@@ -109,6 +109,34 @@ def test_mfma_probe_argument_errors():
     assert lib.skyrl_lmhead_mfma_probe(0x1000, 0, 10, 0x2000, None) == -5
     assert lib.skyrl_lmhead_mfma_probe(0x1000, 256, 0, 0x2000, None) == -5
     assert lib.skyrl_lmhead_mfma_probe(0x1008, 256, 10, 0x2000, None) == -3
+
+
+def test_ppo_policy_loss_argument_errors():
+    lib = _lib.load()
+    call = lambda **kw: lib.skyrl_ppo_policy_loss(*[{**dict(lp=0x1000, old=0x2000, adv=0x3000, mask=None, w=None, T=8, lo=0.2,  # noqa: E731
+                                                        hi=0.2, c=3.0, dual=0, out=0x4000, g=None, stream=None), **kw}[k]
+                                                     for k in ("lp", "old", "adv", "mask", "w", "T", "lo", "hi", "c", "dual", "out", "g",
+                                                               "stream")])
+    assert call(lp=None) == -1
+    assert call(out=None) == -1
+    assert call(T=0) == -2
+    assert call(lo=float("nan")) == -5
+    assert call(dual=1, c=float("inf")) == -5
+
+
+def test_ppo_policy_loss_mirror_contract():
+    from types import SimpleNamespace
+
+    from skyrl_amd.policy_loss import ppo_policy_loss
+
+    x = torch.zeros(2, 4)
+    cfg = SimpleNamespace(policy_loss_type="regular", eps_clip_low=0.2, eps_clip_high=0.2, clip_ratio_c=3.0)
+    with pytest.raises(AssertionError):
+        ppo_policy_loss(x, x, x, SimpleNamespace(policy_loss_type="gspo", eps_clip_low=0.2, eps_clip_high=0.2))
+    with pytest.raises(NotImplementedError):
+        ppo_policy_loss(x, x, x, cfg, rollout_logprobs=x)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        ppo_policy_loss(x, x, x, cfg)
 
 
 def test_status_to_exception_mapping():

@@ -333,3 +333,77 @@ def test_packed_roll_and_scatter_back_brute_force():
             if o < L - 1:
                 ref[i, o] = probs[cu[i] + o]
     assert torch.equal(out, ref)
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# PPO policy loss
+# ----------------------------------------------------------------------------------------------------------------------
+def _ppo(lp, old, adv, **kw):
+    lp = torch.tensor(lp, dtype=torch.float64, requires_grad=True)
+    loss, clip = O.ppo_policy_loss(lp, torch.tensor(old, dtype=torch.float64), torch.tensor(adv, dtype=torch.float64), 0.2, 0.2, **kw)
+    loss.backward()
+    return loss.item(), clip.item(), lp.grad.tolist()
+
+
+def test_ppo_loss_hand_computed_branches():
+    ln2, ln4, lnhalf = math.log(2.0), math.log(4.0), math.log(0.5)
+    # ratio 1: nothing clips; loss = -A, gradient -A (both branches of the min agree)
+    loss, clip, g = _ppo([0.3], [0.3], [1.5])
+    assert loss == pytest.approx(-1.5) and clip == 0.0 and g == pytest.approx([-1.5])
+    # ratio 2, A > 0: the clipped branch 1.2*A is the smaller one -> loss -1.2*A, no gradient, counted as clipped
+    loss, clip, g = _ppo([ln2], [0.0], [2.0])
+    assert loss == pytest.approx(-2.4) and clip == 1.0 and g == pytest.approx([0.0])
+    # ratio 2, A < 0: the unclipped branch 2*A is the smaller one -> loss -2*A = 4, gradient -ratio*A = 4, not clipped
+    loss, clip, g = _ppo([ln2], [0.0], [-2.0])
+    assert loss == pytest.approx(4.0) and clip == 0.0 and g == pytest.approx([4.0])
+    # ratio 0.5, A < 0: clipped low, 0.8*A < 0.5*A -> loss 1.6, no gradient
+    loss, clip, g = _ppo([lnhalf], [0.0], [-2.0])
+    assert loss == pytest.approx(1.6) and clip == 1.0 and g == pytest.approx([0.0])
+    # ratio 0.5, A > 0: unclipped branch is smaller -> loss -1, gradient -ratio*A = -1
+    loss, clip, g = _ppo([lnhalf], [0.0], [2.0])
+    assert loss == pytest.approx(-1.0) and clip == 0.0 and g == pytest.approx([-1.0])
+    # dual clip, A < 0: ratio 2 stays below c = 3 (unchanged), ratio 4 is capped at -A*c = 6 with no gradient
+    loss, clip, g = _ppo([ln2], [0.0], [-2.0], dual_clip=True, clip_ratio_c=3.0)
+    assert loss == pytest.approx(4.0) and g == pytest.approx([4.0])
+    loss, clip, g = _ppo([ln4], [0.0], [-2.0], dual_clip=True, clip_ratio_c=3.0)
+    assert loss == pytest.approx(6.0) and g == pytest.approx([0.0])
+    # dual clip leaves A > 0 alone
+    loss, clip, g = _ppo([lnhalf], [0.0], [2.0], dual_clip=True, clip_ratio_c=3.0)
+    assert loss == pytest.approx(-1.0) and g == pytest.approx([-1.0])
+    # the log-ratio is clamped to +-20 before exp: ratio e^20, and no gradient passes the clamp
+    loss, clip, g = _ppo([25.0], [0.0], [-1.0])
+    assert loss == pytest.approx(math.exp(20.0)) and g == pytest.approx([0.0])
+
+
+def test_ppo_loss_mask_weight_and_clip_ratio_by_hand():
+    lp = [math.log(2.0), 0.0, math.log(2.0), math.log(0.5)]
+    adv = [1.0, 1.0, 1.0, -1.0]
+    mask = torch.tensor([1.0, 1.0, 0.0, 1.0], dtype=torch.float64)
+    weight = torch.tensor([0.5, 2.0, 7.0, 1.0], dtype=torch.float64)
+    loss, clip, g = _ppo(lp, [0.0] * 4, adv, loss_mask=mask, loss_weight=weight)
+    # tokens: clipped (-1.2 * 0.5), unclipped (-1 * 2), masked out, clipped low (0.8 * 1)
+    assert loss == pytest.approx(-0.6 - 2.0 + 0.8)
+    assert clip == pytest.approx(2.0 / 3.0)  # two of the three unmasked tokens are clipped
+    assert g == pytest.approx([0.0, -2.0, 0.0, 0.0])
+    _, clip_all, _ = _ppo(lp, [0.0] * 4, adv)
+    assert clip_all == pytest.approx(3.0 / 4.0)  # without a mask: plain mean
+
+
+@pytest.mark.parametrize("dual", [False, True])
+def test_ppo_loss_gradient_matches_finite_differences(dual):
+    gen = torch.Generator().manual_seed(11)
+    n = 64
+    lp = torch.randn(n, generator=gen, dtype=torch.float64) * 0.4
+    old = torch.randn(n, generator=gen, dtype=torch.float64) * 0.4
+    adv = torch.randn(n, generator=gen, dtype=torch.float64)
+    mask = (torch.rand(n, generator=gen) > 0.3).double()
+    w = torch.rand(n, generator=gen, dtype=torch.float64) + 0.5
+    f = lambda x: O.ppo_policy_loss(x, old, adv, 0.2, 0.28, 3.0, dual, mask, w)[0]  # noqa: E731
+    x = lp.clone().requires_grad_(True)
+    f(x).backward()
+    eps = 1e-6
+    for i in range(n):
+        d = torch.zeros(n, dtype=torch.float64)
+        d[i] = eps
+        fd = (f(lp + d) - f(lp - d)).item() / (2 * eps)
+        assert x.grad[i].item() == pytest.approx(fd, abs=1e-6), f"token {i}"

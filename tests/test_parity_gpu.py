@@ -308,6 +308,74 @@ def test_c_abi_called_directly(cuda_device):
 # ---------------------------------------------------------------------------------------------------------------------
 # the reference's call signatures
 # ---------------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("loss_type", ["regular", "dual_clip"])
+@pytest.mark.parametrize("masked", [False, True])
+def test_ppo_policy_loss_matches_oracle(loss_type, masked, cuda_device):
+    from types import SimpleNamespace
+
+    from skyrl_amd.policy_loss import ppo_policy_loss
+
+    gen = torch.Generator().manual_seed(5)
+    B, S = 6, 517
+    lp = (torch.randn(B, S, generator=gen) * 0.5 - 2.0)
+    old = lp + torch.randn(B, S, generator=gen) * 0.3
+    old[0, :4] = lp[0, :4]                       # exact ties of the two surrogates
+    old[1, 0], old[1, 1] = lp[1, 0] - 30.0, lp[1, 1] + 30.0  # beyond the +-20 clamp
+    adv = torch.randn(B, S, generator=gen)
+    mask = (torch.rand(B, S, generator=gen) > 0.4).float() if masked else None
+    weight = (torch.rand(B, S, generator=gen) + 0.5) if masked else None
+    cfg = SimpleNamespace(policy_loss_type=loss_type, eps_clip_low=0.2, eps_clip_high=0.28, clip_ratio_c=3.0)
+
+    ref_lp = lp.double().requires_grad_(True)
+    ref_loss, ref_clip = O.ppo_policy_loss(ref_lp, old.double(), adv.double(), 0.2, 0.28, 3.0, loss_type == "dual_clip",
+                                           None if mask is None else mask.double(), None if weight is None else weight.double())
+    ref_loss.backward()
+
+    dlp = lp.to(cuda_device).requires_grad_(True)
+    to = lambda t: None if t is None else t.to(cuda_device)  # noqa: E731
+    loss, metrics = ppo_policy_loss(dlp, to(old), to(adv), cfg, to(mask), loss_weight=to(weight))
+    loss.backward()
+    assert loss.dtype == torch.float32 and isinstance(metrics["clip_ratio"], float)
+    # fp32 sum of ~3000 terms, one of them about e^20 (the clamped log-ratio): a relative bound
+    assert abs(loss.item() - ref_loss.item()) <= 5e-6 * max(abs(ref_loss.item()), 1e3)
+    assert metrics["clip_ratio"] == pytest.approx(ref_clip.item(), abs=1e-6)
+    err = (dlp.grad.double().cpu() - ref_lp.grad).abs().max().item()
+    assert err <= 1e-5 * max(1.0, ref_lp.grad.abs().max().item()), f"gradient max abs err {err}"
+    # scaling the loss scales the gradient; metrics without a host synchronisation come back as tensors
+    dlp2 = lp.to(cuda_device).requires_grad_(True)
+    loss2, m2 = ppo_policy_loss(dlp2, to(old), to(adv), cfg, to(mask), loss_weight=to(weight), sync_metrics=False)
+    (loss2 * 3.0).backward()
+    assert torch.equal(dlp2.grad, dlp.grad * 3.0) and torch.is_tensor(m2["clip_ratio"])
+
+
+def test_policy_loss_feeds_the_fused_backward(cuda_device):
+    """log-probabilities from the fused forward -> PPO loss -> backward through the fused LM head, against the oracle chain."""
+    from types import SimpleNamespace
+
+    from skyrl_amd.policy_loss import ppo_policy_loss
+
+    gen = torch.Generator().manual_seed(9)
+    T, H, V = 384, 128, 1000
+    hidden = torch.randn(T, H, generator=gen).bfloat16()
+    weight = (torch.randn(V, H, generator=gen) * 3 / H ** 0.5).bfloat16()
+    labels = torch.randint(0, V, (T,), generator=gen)
+    adv = torch.randn(T, generator=gen)
+    mask = (torch.rand(T, generator=gen) > 0.5).float()
+    cfg = SimpleNamespace(policy_loss_type="regular", eps_clip_low=0.2, eps_clip_high=0.2)
+
+    h64, w64 = hidden.double().requires_grad_(True), weight.double().requires_grad_(True)
+    ref_lp = torch.log_softmax(h64 @ w64.t(), -1).gather(-1, labels[:, None])[:, 0]
+    old = (ref_lp.detach() + torch.randn(T, generator=gen).double() * 0.3).float()
+    O.ppo_policy_loss(ref_lp, old.double(), adv.double(), 0.2, 0.2, loss_mask=mask.double())[0].backward()
+
+    dh = hidden.to(cuda_device).requires_grad_(True)
+    dw = weight.to(cuda_device).requires_grad_(True)
+    lp = FusedLinearLogprobHip.apply(dh[None], dw, labels.to(cuda_device)[None], 0, V, 1024, None, False)[0]
+    loss, _ = ppo_policy_loss(lp, old.to(cuda_device), adv.to(cuda_device), cfg, mask.to(cuda_device))
+    loss.backward()
+    assert cos(dh.grad.float(), h64.grad) >= GRAD_COS and cos(dw.grad.float(), w64.grad) >= GRAD_COS
+
+
 def test_mfma_probe_sums_exactly(cuda_device):
     """The measurement kernel runs the mainloop's MFMA sequence on caller-given operands: with small integers the sum of
     every wavefront's accumulators has a closed form, sum_k (sum_m A[m,k]) (sum_n B[n,k]) per pair of fragments."""
