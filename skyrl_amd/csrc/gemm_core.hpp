@@ -7,7 +7,7 @@
 //
 // What bounds the loop (measured on the MI355X):
 //   * with random operands the matrix pipe is power-limited, not issue-limited: a loop of nothing but MFMAs on
-//     N(0,1) data sustains 1.69-1.84 PFLOP/s with v_mfma_f32_32x32x16_bf16 and 2.08-2.10 PFLOP/s with
+//     N(0,1) data sustains 1.69-1.84 PFLOP/s with v_mfma_f32_32x32x16_bf16 and 2.00-2.10 PFLOP/s with
 //     v_mfma_f32_16x16x32_bf16 (both 2.46-2.49 on zeros), so the 16 x 16 x 32 shape is used although it needs twice
 //     the MFMA instructions;
 //   * a CU takes at most ~32 B/clk from L2, through global_load_lds as well as through ordinary loads; a 64 KiB k-tile
