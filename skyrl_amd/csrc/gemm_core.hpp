@@ -299,14 +299,30 @@ __device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, in
   tm = m_first + (in_band - tn * gm);
 }
 
-// Sum / maximum over the four lanes (l, l^16, l^32, l^48) that hold the same accumulator column.
+// Sum / maximum over the four lanes (l, l^16, l^32, l^48) that hold the same accumulator column, result in all four.
+// v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even rows of its second, and
+// v_permlane32_swap the upper half of the first with the lower half of the second: fed the same value twice, the two
+// results hold the two partners' values side by side in every lane.  Plain VALU operations -- the ds_bpermute form costs
+// an LDS round trip per step, and the statistics epilogue has six of these chains per 16 tokens.
+__device__ __forceinline__ void swap16(float v, float& a, float& b) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  a = __uint_as_float(r[0]), b = __uint_as_float(r[1]);
+}
+__device__ __forceinline__ void swap32(float v, float& a, float& b) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  a = __uint_as_float(r[0]), b = __uint_as_float(r[1]);
+}
 __device__ __forceinline__ float col_sum(float v) {
-  v += __shfl_xor(v, 16, 64);
-  return v + __shfl_xor(v, 32, 64);
+  float a, b;
+  swap16(v, a, b);
+  swap32(a + b, a, b);
+  return a + b;
 }
 __device__ __forceinline__ float col_max(float v) {
-  v = fmaxf(v, __shfl_xor(v, 16, 64));
-  return fmaxf(v, __shfl_xor(v, 32, 64));
+  float a, b;
+  swap16(v, a, b);
+  swap32(fmaxf(a, b), a, b);
+  return fmaxf(a, b);
 }
 
 }  // namespace lmhead

@@ -75,6 +75,13 @@ def test_no_accumulator_write_right_before_an_mfma(kernels):
                 assert not near, f"{name}: {near[0]} within three instructions of '{ln}'"
 
 
+def test_no_packed_fp32_arithmetic(kernels):
+    """The build switches the packed fp32 instructions off (``-packed-fp32-ops``); none may appear in the MFMA kernels."""
+    for name, lines in kernels.items():
+        bad = [ln for ln in lines if ln.startswith(("v_pk_add_f32", "v_pk_mul_f32", "v_pk_fma_f32"))]
+        assert not bad, f"{name}: {bad[:3]}"
+
+
 def test_mfma_accumulates_in_place_in_agprs(kernels):
     pat = re.compile(r"v_mfma_f32_16x16x32_bf16 (a\[\d+:\d+\]), v\[\d+:\d+\], v\[\d+:\d+\], (a\[\d+:\d+\])$")
     for name, lines in kernels.items():
