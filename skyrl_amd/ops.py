@@ -79,6 +79,8 @@ def lmhead_fwd(
     dev = _require_device(hidden, weight, labels)
     lib = _lib.load()
     f32 = dict(dtype=torch.float32, device=dev)
+    if T == 0:  # an empty micro-batch: nothing to launch
+        return torch.empty(0, **f32), torch.empty(0, **f32), torch.empty(0, **f32), torch.empty(0, **f32)
     logprobs = torch.empty(T, **f32)
     row_lse = torch.empty(T, **f32)
     entropy = torch.empty(T if want_entropy else 0, **f32)
@@ -121,6 +123,8 @@ def lmhead_bwd(
     dev = _require_device(hidden, weight, labels, row_lse, dlogprobs)
     lib = _lib.load()
     d_hidden = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    if T == 0:  # an empty micro-batch contributes a zero weight gradient
+        return d_hidden, torch.zeros((V, H), dtype=torch.float32, device=dev)
     d_weight = torch.empty((V, H), dtype=torch.float32, device=dev)
     _bwd_into(lib, hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk, d_hidden,
               d_weight, False)

@@ -55,6 +55,8 @@ def ppo_policy_loss_terms(
             continue
         if t.dtype != torch.float32 or t.dim() != 1 or t.numel() != n or not t.is_contiguous():
             raise ValueError(f"{name} must be a contiguous fp32 vector of {n} elements, got {t.dtype} {tuple(t.shape)}")
+    if n == 0:
+        return torch.zeros(3, dtype=torch.float32, device=dev), torch.empty(0, dtype=torch.float32, device=dev)
     sums = torch.empty(3, dtype=torch.float32, device=dev)
     grad = torch.empty(n, dtype=torch.float32, device=dev)
     ptr = lambda t: None if t is None else t.data_ptr()  # noqa: E731

@@ -175,6 +175,27 @@ def test_zero_weight_known_answer(cuda_device):
     torch.testing.assert_close(out["entropy"], torch.full((T,), math.log(V)), atol=1e-5, rtol=0)
 
 
+def test_empty_micro_batch(cuda_device):
+    """Zero tokens: empty outputs, a zero weight gradient, no launch (the C ABI itself rejects T < 1)."""
+    from types import SimpleNamespace
+
+    from skyrl_amd.policy_loss import ppo_policy_loss
+
+    H, V = 128, 512
+    hidden = torch.zeros(1, 0, H, dtype=torch.bfloat16, device=cuda_device, requires_grad=True)
+    weight = torch.randn(V, H, device=cuda_device).bfloat16().requires_grad_(True)
+    target = torch.zeros(1, 0, dtype=torch.int64, device=cuda_device)
+    lp = FusedLinearLogprobHip.apply(hidden, weight, target, 0, V, 1024, None, False)
+    assert lp.shape == (1, 0) and lp.dtype == torch.float32
+    cfg = SimpleNamespace(policy_loss_type="regular", eps_clip_low=0.2, eps_clip_high=0.2)
+    loss, metrics = ppo_policy_loss(lp, torch.zeros_like(lp), torch.zeros_like(lp), cfg, torch.zeros_like(lp))
+    assert loss.item() == 0.0 and metrics["clip_ratio"] == 0.0
+    loss.backward()
+    assert hidden.grad.shape == hidden.shape and float(weight.grad.abs().max()) == 0.0
+    lp2, ent2 = linear_cross_entropy(hidden.detach()[0], weight.detach(), target[0], 1.0, "none")
+    assert lp2.numel() == 0 and ent2.numel() == 0
+
+
 def test_extreme_logits(cuda_device):
     # one dominant logit -> logprob, entropy -> 0; all logits very negative -> the split merge must not underflow
     T, H, V = 40, 64, 700
