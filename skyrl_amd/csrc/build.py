@@ -27,6 +27,7 @@ HIPCC_FLAGS = [
     "-Xclang",
     "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    "-Wno-inline-asm",  # the copy instruction names M0 as clobbered; clang warns that M0 is a reserved register
 ]
 
 

@@ -144,15 +144,21 @@ __device__ __forceinline__ void make_plan(CopyPlan& p, const Operand& a, const O
 }
 
 // Copies j0 .. j0+n-1 (of COPIES_PER_OPERAND) of k-tile t of one operand into the ring slot at byte offset `slot_off`.
+// Written as assembly to get the "SGPR base + 32-bit VGPR offset" address form: through the builtin the compiler keeps
+// sixteen 64-bit per-lane addresses and spends a 64-bit VALU add per copy, and with one wave per SIMD an MFMA leaves
+// room for only three other instructions before the matrix pipe runs dry.  M0 (the LDS destination of the copy) is
+// written immediately before every use and nothing else in these kernels reads it.
 __device__ __forceinline__ void copy_part(const char* bytes, const uint32_t (&src)[COPIES_PER_OPERAND], int t, int slot_off,
                                           int j0, int n, char* lds) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const char* g = bytes + (size_t)t * (BK * 2);
-  char* dst = lds + slot_off + wave * 1024;
+  const char* g = bytes + (size_t)t * (BK * 2);  // wave-uniform
+  const uint32_t dst = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds + slot_off + wave * 1024;
 #pragma unroll
   for (int j = j0; j < j0 + n; ++j)
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(g + src[j]),
-                                     (__attribute__((address_space(3))) void*)(dst + j * NWAVES * 1024), 16, 0, 0);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(dst + j * NWAVES * 1024), "v"(src[j]), "s"(g)
+                 : "memory", "m0");
 }
 
 // Put the first k-tiles of an output tile in flight: A(0) B(0) A(1) B(1) into slots 0..3.  All five slots must be free
@@ -181,7 +187,7 @@ __device__ __forceinline__ void prefetch_first_tiles(const Operand& a, const Ope
 //   step 1:      barrier -- all fragment reads of tile kt have returned, this wave's copies of tile kt+1 have landed --
 //                then B(kt+2) into the slot that held A(kt); fragment reads of step 0 of tile kt+1
 //   every step:  the sixteen fragment reads of the next step ride behind every second MFMA of its first half (two
-//                register sets), one copy behind every eighth MFMA; sched_barrier pins that order.
+//                register sets), one copy behind every eighth MFMA, in a gap without a read; sched_barrier pins that order.
 // MFMA order inside a step is a serpentine over the 8 x 8 accumulators (the B fragment is kept where the A fragment
 // changes): fewer operand toggles, measurably less power.
 __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int k_begin, int nk, char* lds, acc_t& acc) {
@@ -238,7 +244,7 @@ __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int
           if (ks == 0) read_one(lds + ra1, lds + rb1, 1, x / 2);
           else if (has_next) read_one(lds + ra0, lds + rb0, 0, x / 2);
         }
-        if (load2 && x % 8 == 4) {
+        if (load2 && x % 8 == 5) {  // an MFMA gap that carries no fragment read
           if (ks == 0) copy_part(p.a_bytes, p.a_src, kt + 2, o4, x / 8, 1, lds);
           else copy_part(p.b_bytes, p.b_src, kt + 2, o0, x / 8, 1, lds);
         }

@@ -75,6 +75,18 @@ def test_no_accumulator_write_right_before_an_mfma(kernels):
                 assert not near, f"{name}: {near[0]} within three instructions of '{ln}'"
 
 
+def test_every_lds_copy_sets_m0_first(kernels):
+    """global_load_lds takes its LDS destination from M0: each one must be preceded, within a few instructions and with no
+    other copy in between, by a write of M0."""
+    for name, lines in kernels.items():
+        for k, ln in enumerate(lines):
+            if ln.startswith("global_load_lds"):
+                window = lines[max(0, k - 4):k]
+                writes = [i for i, p in enumerate(window) if re.match(r"s_(mov_b32|add_i32|add_u32) m0,", p)]
+                assert writes, f"{name}: no M0 write right before '{ln}': {window}"
+                assert not any(p.startswith("global_load_lds") for p in window[writes[-1]:]), f"{name}: stale M0 before '{ln}'"
+
+
 def test_no_packed_fp32_arithmetic(kernels):
     """The build switches the packed fp32 instructions off (``-packed-fp32-ops``); none may appear in the MFMA kernels."""
     for name, lines in kernels.items():
