@@ -143,22 +143,28 @@ __device__ __forceinline__ void make_plan(CopyPlan& p, const Operand& a, const O
   p.b_bytes = (const char*)b.ptr + (size_t)k_begin * 2;
 }
 
-// Copies j0 .. j0+n-1 (of COPIES_PER_OPERAND) of k-tile t of one operand into the ring slot at byte offset `slot_off`.
+// Copies j0 .. j0+n-1 (of COPIES_PER_OPERAND) of k-tile t of one operand into a ring slot; `slot_wave_addr` is the LDS
+// address of the slot plus this wave's share of a 4 KiB copy group (wave_copy_base() + slot offset).
 // Written as assembly to get the "SGPR base + 32-bit VGPR offset" address form: through the builtin the compiler keeps
 // sixteen 64-bit per-lane addresses and spends a 64-bit VALU add per copy, and with one wave per SIMD an MFMA leaves
 // room for only three other instructions before the matrix pipe runs dry.  M0 (the LDS destination of the copy) is
 // written immediately before every use and nothing else in these kernels reads it.
-__device__ __forceinline__ void copy_part(const char* bytes, const uint32_t (&src)[COPIES_PER_OPERAND], int t, int slot_off,
-                                          int j0, int n, char* lds) {
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+__device__ __forceinline__ void copy_part(const char* bytes, const uint32_t (&src)[COPIES_PER_OPERAND], int t,
+                                          uint32_t slot_wave_addr, int j0, int n) {
   const char* g = bytes + (size_t)t * (BK * 2);  // wave-uniform
-  const uint32_t dst = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds + slot_off + wave * 1024;
 #pragma unroll
   for (int j = j0; j < j0 + n; ++j)
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+    asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3"
                  :
-                 : "s"(dst + j * NWAVES * 1024), "v"(src[j]), "s"(g)
-                 : "memory", "m0");
+                 : "s"(slot_wave_addr), "n"(j * NWAVES * 1024), "v"(src[j]), "s"(g)
+                 : "memory", "m0", "scc");
+}
+
+// LDS address of this wave's first 1 KiB copy destination inside ring slot 0 (wave-uniform, kept in an SGPR); slot k
+// is k * OPERAND_BYTES further.
+__device__ __forceinline__ uint32_t wave_copy_base(char* lds) {
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds + wave * 1024u;
 }
 
 // Put the first k-tiles of an output tile in flight: A(0) B(0) A(1) B(1) into slots 0..3.  All five slots must be free
@@ -167,11 +173,12 @@ __device__ __forceinline__ void copy_part(const char* bytes, const uint32_t (&sr
 __device__ __forceinline__ void prefetch_first_tiles(const Operand& a, const Operand& b, int k_begin, int nk, char* lds) {
   CopyPlan p;  // rebuilt by mainloop(): keeping it in registers across an epilogue costs more than recomputing it
   make_plan(p, a, b, k_begin);
-  copy_part(p.a_bytes, p.a_src, 0, 0 * OPERAND_BYTES, 0, COPIES_PER_OPERAND, lds);
-  copy_part(p.b_bytes, p.b_src, 0, 1 * OPERAND_BYTES, 0, COPIES_PER_OPERAND, lds);
+  const uint32_t w0 = wave_copy_base(lds);
+  copy_part(p.a_bytes, p.a_src, 0, w0 + 0 * OPERAND_BYTES, 0, COPIES_PER_OPERAND);
+  copy_part(p.b_bytes, p.b_src, 0, w0 + 1 * OPERAND_BYTES, 0, COPIES_PER_OPERAND);
   if (nk > 1) {
-    copy_part(p.a_bytes, p.a_src, 1, 2 * OPERAND_BYTES, 0, COPIES_PER_OPERAND, lds);
-    copy_part(p.b_bytes, p.b_src, 1, 3 * OPERAND_BYTES, 0, COPIES_PER_OPERAND, lds);
+    copy_part(p.a_bytes, p.a_src, 1, w0 + 2 * OPERAND_BYTES, 0, COPIES_PER_OPERAND);
+    copy_part(p.b_bytes, p.b_src, 1, w0 + 3 * OPERAND_BYTES, 0, COPIES_PER_OPERAND);
   }
 }
 
@@ -199,36 +206,41 @@ __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int
   const int lrow = lane & 15;
   const int xsw = ((lane >> 4) ^ swz(lrow)) << 4;  // chunk offset of k-step 0; k-step 1 is xsw ^ 64
   // Per-lane fragment addresses inside a slot, for k-step 0 and 1 of the A and of the B operand.
-  const int a_off0 = (wm * WM + lrow) * ROW_BYTES + xsw, a_off1 = (wm * WM + lrow) * ROW_BYTES + (xsw ^ 64);
-  const int b_off0 = (wn * WN + lrow) * ROW_BYTES + xsw, b_off1 = (wn * WN + lrow) * ROW_BYTES + (xsw ^ 64);
+  // The ring state below carries LDS addresses that already include this wave's copy offset (what the copies need, with
+  // no further arithmetic); the per-lane fragment offsets are taken relative to it.
+  const uint32_t w0 = wave_copy_base(lds);
+  const int rel = -(wave * 1024);
+  const int a_off0 = (wm * WM + lrow) * ROW_BYTES + xsw + rel, a_off1 = (wm * WM + lrow) * ROW_BYTES + (xsw ^ 64) + rel;
+  const int b_off0 = (wn * WN + lrow) * ROW_BYTES + xsw + rel, b_off1 = (wn * WN + lrow) * ROW_BYTES + (xsw ^ 64) + rel;
+  typedef const __attribute__((address_space(3))) bf16x8* frag_ptr;
 
   bf16x8 af[2][TM], bfr[2][TN];
   // Fragment x of a 32-k step: x < TM is the A fragment of MFMA row x, otherwise the B fragment of MFMA column x - TM.
-  auto read_one = [&](const char* pa, const char* pb, int set, int x) {
-    if (x < TM) af[set][x] = *(const bf16x8*)(pa + x * MT * ROW_BYTES);
-    else bfr[set][x - TM] = *(const bf16x8*)(pb + (x - TM) * MT * ROW_BYTES);
+  auto read_one = [&](uint32_t pa, uint32_t pb, int set, int x) {  // pa, pb: LDS addresses of fragment 0
+    if (x < TM) af[set][x] = *(frag_ptr)(uintptr_t)(pa + x * MT * ROW_BYTES);
+    else bfr[set][x - TM] = *(frag_ptr)(uintptr_t)(pb + (x - TM) * MT * ROW_BYTES);
   };
 
   if (nk > 1) wait_copies_and_barrier<2 * COPIES_PER_OPERAND>(); else wait_copies_and_barrier<0>();  // tile 0 has landed
 #pragma unroll
-  for (int x = 0; x < TM + TN; ++x) read_one(lds + a_off0, lds + OPERAND_BYTES + b_off0, 0, x);
+  for (int x = 0; x < TM + TN; ++x) read_one(w0 + a_off0, w0 + OPERAND_BYTES + b_off0, 0, x);
 
   // Ring state, as byte offsets of the slots in the order A(kt), B(kt), A(kt+1), B(kt+1), free.  Advancing one k-tile
   // rotates the five values by two places, so no arithmetic is needed; the fragment addresses of the next k-tile are
   // formed in the shadow of MFMAs in the middle of a step, not at the top of the loop where nothing would hide them.
-  int o0 = 0, o1 = OPERAND_BYTES, o2 = 2 * OPERAND_BYTES, o3 = 3 * OPERAND_BYTES, o4 = 4 * OPERAND_BYTES;
-  int ra1 = o0 + a_off1, rb1 = o1 + b_off1;  // step-0 reads: k-step 1 of this k-tile (byte offsets into lds)
-  int ra0 = o2 + a_off0, rb0 = o3 + b_off0;  // step-1 reads: k-step 0 of the next k-tile
+  uint32_t o0 = w0, o1 = w0 + OPERAND_BYTES, o2 = w0 + 2 * OPERAND_BYTES, o3 = w0 + 3 * OPERAND_BYTES, o4 = w0 + 4 * OPERAND_BYTES;
+  uint32_t ra1 = o0 + a_off1, rb1 = o1 + b_off1;  // step-0 reads: k-step 1 of this k-tile (LDS addresses)
+  uint32_t ra0 = o2 + a_off0, rb0 = o3 + b_off0;  // step-1 reads: k-step 0 of the next k-tile
   // An add the compiler cannot move: it would otherwise collect these at the top of the loop body.
-  auto pinned_add = [](int slot_off, int lane_off) {
-    int r;
+  auto pinned_add = [](uint32_t slot_off, int lane_off) {
+    uint32_t r;
     asm volatile("v_add_u32_e32 %0, %1, %2" : "=v"(r) : "s"(slot_off), "v"(lane_off));
     return r;
   };
   // Three copies of the tile step (steady state, second-to-last, last) instead of conditions inside one loop body: a
   // branch that joins a path with outstanding LDS reads makes the compiler wait for all of them.
   auto tile_step = [&](int kt, auto has_next, auto load2) {
-    int nra1 = ra1, nrb1 = rb1, nra0 = ra0, nrb0 = rb0;
+    uint32_t nra1 = ra1, nrb1 = rb1, nra0 = ra0, nrb0 = rb0;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       if (ks == 1 && has_next) {
@@ -241,12 +253,12 @@ __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int
         mfma_16x16x32(acc[i][j], af[ks][i], bfr[ks][j]);
         __builtin_amdgcn_sched_barrier(0);
         if (x % 2 == 0 && x < 2 * (TM + TN)) {
-          if (ks == 0) read_one(lds + ra1, lds + rb1, 1, x / 2);
-          else if (has_next) read_one(lds + ra0, lds + rb0, 0, x / 2);
+          if (ks == 0) read_one(ra1, rb1, 1, x / 2);
+          else if (has_next) read_one(ra0, rb0, 0, x / 2);
         }
         if (load2 && x % 8 == 5) {  // an MFMA gap that carries no fragment read
-          if (ks == 0) copy_part(p.a_bytes, p.a_src, kt + 2, o4, x / 8, 1, lds);
-          else copy_part(p.b_bytes, p.b_src, kt + 2, o0, x / 8, 1, lds);
+          if (ks == 0) copy_part(p.a_bytes, p.a_src, kt + 2, o4, x / 8, 1);
+          else copy_part(p.b_bytes, p.b_src, kt + 2, o0, x / 8, 1);
         }
         if (has_next) {  // next k-tile's fragment addresses, one per MFMA shadow, after this step's reads are issued
           if (ks == 0 && x == 41) nra1 = pinned_add(o2, a_off1);
@@ -258,7 +270,7 @@ __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int
       }
     }
     ra1 = nra1, rb1 = nrb1, ra0 = nra0, rb0 = nrb0;
-    const int t0 = o0, t1 = o1;
+    const uint32_t t0 = o0, t1 = o1;
     o0 = o2, o1 = o3, o2 = o4, o3 = t0, o4 = t1;
   };
   std::true_type yes;
