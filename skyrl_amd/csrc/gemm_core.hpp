@@ -143,15 +143,15 @@ __device__ __forceinline__ void make_plan(CopyPlan& p, const Operand& a, const O
   p.b_bytes = (const char*)b.ptr + (size_t)k_begin * 2;
 }
 
-// Copies j0 .. j0+n-1 (of COPIES_PER_OPERAND) of k-tile t of one operand into a ring slot; `slot_wave_addr` is the LDS
-// address of the slot plus this wave's share of a 4 KiB copy group (wave_copy_base() + slot offset).
+// Copies j0 .. j0+n-1 (of COPIES_PER_OPERAND) of one k-tile of one operand into a ring slot.  `g` is the wave-uniform
+// address of the operand at that k-tile (base + k offset); `slot_wave_addr` is the LDS address of the slot plus this wave's
+// share of a 4 KiB copy group (wave_copy_base() + slot offset).
 // Written as assembly to get the "SGPR base + 32-bit VGPR offset" address form: through the builtin the compiler keeps
 // sixteen 64-bit per-lane addresses and spends a 64-bit VALU add per copy, and with one wave per SIMD an MFMA leaves
 // room for only three other instructions before the matrix pipe runs dry.  M0 (the LDS destination of the copy) is
 // written immediately before every use and nothing else in these kernels reads it.
-__device__ __forceinline__ void copy_part(const char* bytes, const uint32_t (&src)[COPIES_PER_OPERAND], int t,
+__device__ __forceinline__ void copy_part(const char* g, const uint32_t (&src)[COPIES_PER_OPERAND],
                                           uint32_t slot_wave_addr, int j0, int n) {
-  const char* g = bytes + (size_t)t * (BK * 2);  // wave-uniform
 #pragma unroll
   for (int j = j0; j < j0 + n; ++j)
     asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3"
@@ -174,11 +174,11 @@ __device__ __forceinline__ void prefetch_first_tiles(const Operand& a, const Ope
   CopyPlan p;  // rebuilt by mainloop(): keeping it in registers across an epilogue costs more than recomputing it
   make_plan(p, a, b, k_begin);
   const uint32_t w0 = wave_copy_base(lds);
-  copy_part(p.a_bytes, p.a_src, 0, w0 + 0 * OPERAND_BYTES, 0, COPIES_PER_OPERAND);
-  copy_part(p.b_bytes, p.b_src, 0, w0 + 1 * OPERAND_BYTES, 0, COPIES_PER_OPERAND);
+  copy_part(p.a_bytes, p.a_src, w0 + 0 * OPERAND_BYTES, 0, COPIES_PER_OPERAND);
+  copy_part(p.b_bytes, p.b_src, w0 + 1 * OPERAND_BYTES, 0, COPIES_PER_OPERAND);
   if (nk > 1) {
-    copy_part(p.a_bytes, p.a_src, 1, w0 + 2 * OPERAND_BYTES, 0, COPIES_PER_OPERAND);
-    copy_part(p.b_bytes, p.b_src, 1, w0 + 3 * OPERAND_BYTES, 0, COPIES_PER_OPERAND);
+    copy_part(p.a_bytes + BK * 2, p.a_src, w0 + 2 * OPERAND_BYTES, 0, COPIES_PER_OPERAND);
+    copy_part(p.b_bytes + BK * 2, p.b_src, w0 + 3 * OPERAND_BYTES, 0, COPIES_PER_OPERAND);
   }
 }
 
@@ -237,9 +237,14 @@ __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int
     asm volatile("v_add_u32_e32 %0, %1, %2" : "=v"(r) : "s"(slot_off), "v"(lane_off));
     return r;
   };
+  // Source addresses of the k-tile being copied (two ahead of the one being consumed).  They advance in an MFMA shadow
+  // right behind the last copy that uses them -- the empty asm keeps the compiler from gathering the increments at the
+  // end of the loop body, where every instruction is a bubble.
+  const char* ga = p.a_bytes + 2 * (BK * 2);
+  const char* gb = p.b_bytes + 2 * (BK * 2);
   // Three copies of the tile step (steady state, second-to-last, last) instead of conditions inside one loop body: a
   // branch that joins a path with outstanding LDS reads makes the compiler wait for all of them.
-  auto tile_step = [&](int kt, auto has_next, auto load2) {
+  auto tile_step = [&](auto has_next, auto load2) {
     uint32_t nra1 = ra1, nrb1 = rb1, nra0 = ra0, nrb0 = rb0;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
@@ -257,8 +262,17 @@ __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int
           else if (has_next) read_one(ra0, rb0, 0, x / 2);
         }
         if (load2 && x % 8 == 5) {  // an MFMA gap that carries no fragment read
-          if (ks == 0) copy_part(p.a_bytes, p.a_src, kt + 2, o4, x / 8, 1);
-          else copy_part(p.b_bytes, p.b_src, kt + 2, o0, x / 8, 1);
+          if (ks == 0) copy_part(ga, p.a_src, o4, x / 8, 1);
+          else copy_part(gb, p.b_src, o0, x / 8, 1);
+        }
+        if (load2 && x == 62) {
+          if (ks == 0) {
+            ga += BK * 2;
+            asm volatile("" : "+s"(ga));
+          } else {
+            gb += BK * 2;
+            asm volatile("" : "+s"(gb));
+          }
         }
         if (has_next) {  // next k-tile's fragment addresses, one per MFMA shadow, after this step's reads are issued
           if (ks == 0 && x == 41) nra1 = pinned_add(o2, a_off1);
@@ -276,12 +290,9 @@ __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int
   std::true_type yes;
   std::false_type no;
   int kt = 0;
-  for (; kt + 2 < nk; ++kt) tile_step(kt, yes, yes);
-  if (kt + 1 < nk) {
-    tile_step(kt, yes, no);
-    ++kt;
-  }
-  tile_step(kt, no, no);
+  for (; kt + 2 < nk; ++kt) tile_step(yes, yes);
+  if (kt + 1 < nk) tile_step(yes, no);
+  tile_step(no, no);
   wait_copies_and_barrier<0>();
   // The hardware does not interlock an accumulator read (v_accvgpr_read) against an MFMA still in flight, and the
   // compiler does not know that the inline assembly is one: left alone it copies an accumulator to a VGPR right
