@@ -39,11 +39,11 @@ extern "C" {
 #endif
 
 #define SKYRL_LMHEAD_OK 0
-#define SKYRL_LMHEAD_ERR_NULL (-1)      /* a required pointer is NULL */
-#define SKYRL_LMHEAD_ERR_SHAPE (-2)     /* T, V < 1, H not a positive multiple of 64, a leading dimension < H, or an operand of 4 GiB or more */
+#define SKYRL_LMHEAD_ERR_NULL (-1)      /* a required pointer is NULL, or only some of seg_row / seg_col / seg_len are given */
+#define SKYRL_LMHEAD_ERR_SHAPE (-2)     /* T, V < 1, H not a positive multiple of 64, a leading dimension < H, an operand of 4 GiB or more, a negative count */
 #define SKYRL_LMHEAD_ERR_ALIGN (-3)     /* a pointer is not 16-byte aligned or a leading dimension is not a multiple of 8 */
 #define SKYRL_LMHEAD_ERR_WORKSPACE (-4) /* workspace is NULL or smaller than the matching *_workspace_bytes() */
-#define SKYRL_LMHEAD_ERR_ARG (-5)       /* rcp_temperature not finite and positive, or vocab_chunk not a multiple of 256 */
+#define SKYRL_LMHEAD_ERR_ARG (-5)       /* rcp_temperature not finite and positive, vocab_chunk not a multiple of 256, or both sub-sequence arrays and a mask */
 
 /* ABI version of this header (bumped on any signature change). */
 int skyrl_lmhead_version(void);
@@ -109,6 +109,39 @@ int skyrl_ppo_policy_loss(const float* logprobs, const float* old_logprobs, cons
                           const float* loss_mask, const float* loss_weight, int64_t T,
                           float eps_clip_low, float eps_clip_high, float clip_ratio_c, int dual_clip,
                           float* out3, float* dlogprobs, void* stream);
+
+/*
+ * Packed-sequence front end: the label of every token of a packed [T] stream is its successor inside its own sequence,
+ *     labels[t] = tokens[cu[s] + (t - cu[s] + 1) mod (cu[s+1] - cu[s])],   s = the sequence with cu[s] <= t < cu[s+1]
+ * (next_offsets / rolled_targets_full of from_parallel_hidden_to_logprobs_packed_sequences,
+ * skyrl/backends/skyrl_train/distributed/megatron/model_utils.py:810-815, with _packed_sequence_indices, :920-928).
+ * tokens, labels int64 [T]; cu_seqlens int64 [num_seqs + 1], non-decreasing, cu_seqlens[0] = 0.  Tokens at or beyond
+ * cu_seqlens[num_seqs] (the reference indexes out of range there) get INT64_MAX, the "not in this shard" label.
+ */
+int skyrl_packed_next_token_labels(const int64_t* tokens, const int64_t* cu_seqlens, int64_t num_seqs, int64_t T,
+                                   int64_t* labels, void* stream);
+
+/*
+ * Packed-sequence back end: packed per-token values fp32 [T] -> out fp32 [rows, cols] (cols = unpacked_seqlen - 1), every
+ * element of out written (0 where no token lands); the three branches of model_utils.py:851-883.  Token t of sequence s,
+ * offset o = t - cu[s]:
+ *   plain (seg_* and attention_mask NULL; :880-883):  out[s, o]                        for o < cu[s+1] - cu[s] - 1
+ *   sub-sequences (seg_row, seg_col, seg_len int64 [num_seqs], all three; :859-871):
+ *                                                     out[seg_row[s], seg_col[s] + o]  for o < seg_len[s] - 1
+ *   attention mask (uint8 [rows, cols + 1], rows == num_seqs; :873-878): the j-th non-zero column of row s takes token
+ *     cu[s] + j, for every non-zero column but the last of the row.  This is the reference's
+ *     out[output_mask] = probs[packed_mask] whenever each packed segment holds at least its row's real tokens minus one
+ *     (otherwise the reference raises a shape error; here the tokens that do not exist read as 0).
+ * Destinations outside [rows, cols] are dropped, as the reference's in-bounds masks do.  T = 0 and rows * cols = 0 are
+ * valid (the pointer of an empty array may then be NULL).
+ * skyrl_packed_gather_grad is the adjoint: d_packed[t] = d_out[destination of t], 0 for tokens without one.
+ */
+int skyrl_packed_scatter_logprobs(const float* packed, const int64_t* cu_seqlens, int64_t num_seqs, int64_t T,
+                                  const int64_t* seg_row, const int64_t* seg_col, const int64_t* seg_len,
+                                  const uint8_t* attention_mask, int64_t rows, int64_t cols, float* out, void* stream);
+int skyrl_packed_gather_grad(const float* d_out, const int64_t* cu_seqlens, int64_t num_seqs, int64_t T,
+                             const int64_t* seg_row, const int64_t* seg_col, const int64_t* seg_len,
+                             const uint8_t* attention_mask, int64_t rows, int64_t cols, float* d_packed, void* stream);
 
 /*
  * Measurement aid for benchmarks (no counterpart in the reference): what the matrix pipe sustains on a given kind of

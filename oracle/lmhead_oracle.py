@@ -19,7 +19,9 @@ What pins each function (all in ``tests/test_oracle.py``; none of them re-types 
     linearity in (g, q), the reference's tolerances (test_fused_linear_logprob.py:89-95).
   * out-of-vocabulary targets: forward 0 / backward keeps -p*g, by construction of an autograd twin whose target logit is
     multiplied by the in-vocabulary mask.
-  * packed-sequence roll and scatter-back: a per-sequence Python loop.
+  * packed-sequence roll and scatter-back (plain, sub-sequence and attention-mask layouts): per-sequence Python loops that
+    place each token by hand, over ragged cases with length-1 and empty sequences, padded segments, left- and
+    interior-padded masks and outputs narrower than a row's content.
   * PPO policy loss: hand-computed cases on both sides of every branch (unclipped, clipped high / low for either sign of
     the advantage, dual-clip active / inactive, the +-20 clamp of the log-ratio), fp64 central finite differences of the
     loss for the gradient autograd derives from it, and the masked-mean definition of clip_ratio counted by hand.
@@ -288,11 +290,59 @@ def packed_rolled_targets(target: torch.Tensor, cu_seqlens: torch.Tensor) -> tor
     return target[cu_seqlens.to(torch.long)[seq_idx] + nxt]
 
 
-def packed_scatter_back(probs: torch.Tensor, cu_seqlens: torch.Tensor, batch_size: int, unpacked_seqlen: int) -> torch.Tensor:
-    """MU:851-883, the plain branch (no sub-sequences, no attention mask): token at (seq i, offset o) goes to out[i, o] for
-    o < len_i - 1 and o < unpacked_seqlen - 1; everything else stays 0."""
+def packed_subseq_rows_offsets_lens(cu_seqlens: torch.Tensor, sub_seq_lengths: Sequence[Sequence[int]]):
+    """MU:886-917: with several sequences packed per output row, segment k (in stream order) belongs to the row that lists
+    it, starts at the column where the *padded* lengths of the row's earlier segments end, and has the listed true length."""
+    bounds = [int(x) for x in cu_seqlens.tolist()]
+    padded = [bounds[i + 1] - bounds[i] for i in range(len(bounds) - 1)]
+    rows, offs, lens = [], [], []
+    k = 0
+    for r, row_lens in enumerate(sub_seq_lengths):
+        col = 0
+        for n in row_lens:
+            if k >= len(padded):
+                raise ValueError("sub_seq_lengths contains more sub-sequences than cu_seqlens_padded")
+            rows.append(r)
+            offs.append(col)
+            lens.append(int(n))
+            col += padded[k]
+            k += 1
+    if k != len(padded):
+        raise ValueError(f"sub_seq_lengths describes {k} sub-sequences, but cu_seqlens_padded describes {len(padded)}")
+    return torch.tensor(rows, dtype=torch.long), torch.tensor(offs, dtype=torch.long), torch.tensor(lens, dtype=torch.long)
+
+
+def packed_scatter_back(
+    probs: torch.Tensor,
+    cu_seqlens: torch.Tensor,
+    batch_size: int,
+    unpacked_seqlen: int,
+    sub_seq_lengths: Optional[Sequence[Sequence[int]]] = None,
+    attention_mask: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """MU:851-883, all three branches.  Plain: token at (seq i, offset o) goes to out[i, o] for o < len_i - 1 and
+    o < unpacked_seqlen - 1.  Sub-sequences (MU:859-871): to out[row_i, col_i + o] for o < true_len_i - 1, column in bounds.
+    Attention mask (MU:873-878): the positions of ``mask[:, :-1]`` that hold a real token other than the row's last one
+    receive, in row-major order, the tokens with o < real_len_i - 1.  Everything else stays 0."""
     out = torch.zeros((batch_size, unpacked_seqlen - 1), dtype=probs.dtype)
     seq_idx, seq_off, seq_len = packed_sequence_indices(cu_seqlens, int(probs.shape[0]))
+    if sub_seq_lengths is not None:
+        rows, offs, lens = packed_subseq_rows_offsets_lens(cu_seqlens, sub_seq_lengths)
+        valid = torch.clamp(lens - 1, min=0)
+        mask = seq_off < valid[seq_idx]
+        cols = offs[seq_idx[mask]] + seq_off[mask]
+        rws = rows[seq_idx[mask]]
+        inb = cols < unpacked_seqlen - 1
+        out[rws[inb], cols[inb]] = probs[mask][inb]
+        return out
+    if attention_mask is not None:
+        am = attention_mask.to(torch.bool)
+        real = am.sum(dim=1, dtype=torch.long)
+        ordinal = am.to(torch.long).cumsum(dim=1)
+        out_mask = am[:, :-1] & (ordinal[:, :-1] < real.unsqueeze(1))
+        valid = torch.clamp(real - 1, min=0)
+        out[out_mask] = probs[seq_off < valid[seq_idx]]
+        return out
     valid = torch.clamp(seq_len - 1, min=0)
     mask = (seq_off < valid[seq_idx]) & (seq_off < unpacked_seqlen - 1)
     out[seq_idx[mask], seq_off[mask]] = probs[mask]

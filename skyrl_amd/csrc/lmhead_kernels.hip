@@ -730,16 +730,20 @@ hipError_t launch_bwd_chunk(hipStream_t s, bool entgrad, const DzArgs& z, unsign
 
 extern "C" {
 
-int skyrl_lmhead_version(void) { return 3; }
+int skyrl_lmhead_version(void) { return 4; }
 
 const char* skyrl_lmhead_strerror(int status) {
   switch (status) {
     case SKYRL_LMHEAD_OK: return "ok";
-    case SKYRL_LMHEAD_ERR_NULL: return "a required pointer is NULL";
-    case SKYRL_LMHEAD_ERR_SHAPE: return "bad shape: need T >= 1, V >= 1, H a positive multiple of 64, leading dimensions >= H";
+    case SKYRL_LMHEAD_ERR_NULL: return "a required pointer is NULL (or only some of seg_row, seg_col, seg_len are given)";
+    case SKYRL_LMHEAD_ERR_SHAPE:
+      return "bad shape: need T >= 1, V >= 1, H a positive multiple of 64, leading dimensions >= H, every matrix under 4 GiB; "
+             "packed-sequence calls: counts >= 0, rows == num_seqs with an attention mask";
     case SKYRL_LMHEAD_ERR_ALIGN: return "bad alignment: pointers must be 16-byte aligned, leading dimensions multiples of 8";
     case SKYRL_LMHEAD_ERR_WORKSPACE: return "workspace is NULL or too small";
-    case SKYRL_LMHEAD_ERR_ARG: return "bad argument: rcp_temperature must be finite and > 0, vocab_chunk a multiple of 256";
+    case SKYRL_LMHEAD_ERR_ARG:
+      return "bad argument: rcp_temperature must be finite and > 0, vocab_chunk a multiple of 256; packed-sequence calls take "
+             "sub-sequence arrays or an attention mask, not both";
     default: break;
   }
   if (status > 0) return hipGetErrorString((hipError_t)status);

@@ -9,6 +9,10 @@ trainer can import these instead:
 * ``_fused_vocab_parallel_entropy_from_hidden``          (:1090-1121)
 * ``_packed_sequence_indices``, ``_packed_subseq_row_indices_offsets_and_lens``  (:920-928, :886-917)
 
+The packed variant prepares its labels and scatters its result back with one HIP kernel each (``skyrl_amd/packed.py``)
+instead of the reference's torch index arithmetic; ``_packed_sequence_indices`` is kept as the host-side statement of that
+arithmetic.
+
 Differences, all forced by the one-GPU scope: tensor/context-parallel groups must be ``None`` or of size 1, and the only
 backend is ``"hip"`` -- there is no fallback to another implementation when the HIP library is missing.
 
@@ -27,6 +31,7 @@ import torch.distributed as dist
 
 from . import ops
 from .fused_linear_logprob_hip import FusedLinearLogprobHip, _group_size, _require_single_shard, linear_cross_entropy
+from .packed import packed_next_token_labels, packed_scatter_logprobs
 
 FUSED_LM_HEAD_LOGPROB_BACKENDS = ("hip",)
 
@@ -156,10 +161,9 @@ def from_parallel_hidden_to_logprobs_packed_sequences(
     if attention_mask is not None:
         attention_mask = attention_mask.to(device=target.device, dtype=torch.bool)
 
-    cu, _, seq_indices, seq_offsets, seq_lens_padded = _packed_sequence_indices(cu_seqlens_padded, target.shape[0],
-                                                                                target.device)
-    next_offsets = torch.remainder(seq_offsets + 1, seq_lens_padded[seq_indices])
-    rolled_targets = target[cu[seq_indices] + next_offsets].unsqueeze(0)
+    # Labels: every token's successor inside its own sequence, one kernel (reference: index arithmetic, :810-815).
+    cu = cu_seqlens_padded.to(device=target.device, dtype=torch.long)
+    rolled_targets = packed_next_token_labels(target.to(torch.long).contiguous(), cu).unsqueeze(0)
     hidden = hidden.unsqueeze(0)
 
     seq_len_local = hidden.shape[1]
@@ -171,28 +175,14 @@ def from_parallel_hidden_to_logprobs_packed_sequences(
     if probs.dim() != 1:
         raise ValueError(f"Expected probs to be 1D after squeezing, but got shape {probs.shape}.")
 
-    out = torch.zeros((batch_size, unpacked_seqlen - 1), dtype=probs.dtype, device=probs.device)
+    # Scatter-back to [batch, unpacked_seqlen - 1], one kernel per direction (reference: boolean-mask indexing, :851-883).
+    cols = unpacked_seqlen - 1
     if sub_seq_lengths is not None:
         rows, row_offs, seq_lens = _packed_subseq_row_indices_offsets_and_lens(cu, sub_seq_lengths, probs.device)
-        valid = torch.clamp(seq_lens - 1, min=0)
-        packed_mask = seq_offsets < valid[seq_indices]
-        cols = row_offs[seq_indices[packed_mask]] + seq_offsets[packed_mask]
-        rws = rows[seq_indices[packed_mask]]
-        inb = cols < unpacked_seqlen - 1
-        out[rws[inb], cols[inb]] = probs[packed_mask][inb]
-        return out
+        return packed_scatter_logprobs(probs, cu, batch_size, cols, seg_row=rows, seg_col=row_offs, seg_len=seq_lens)
     if attention_mask is not None:
-        seq_lens = attention_mask.sum(dim=1, dtype=torch.long)
-        ordinals = attention_mask.to(torch.long).cumsum(dim=1)
-        output_mask = attention_mask[:, :-1] & (ordinals[:, :-1] < seq_lens.unsqueeze(1))
-        valid = torch.clamp(seq_lens - 1, min=0)
-        packed_mask = seq_offsets < valid[seq_indices]
-        out[output_mask] = probs[packed_mask]
-        return out
-    valid = torch.clamp(seq_lens_padded - 1, min=0)
-    packed_mask = (seq_offsets < valid[seq_indices]) & (seq_offsets < unpacked_seqlen - 1)
-    out[seq_indices[packed_mask], seq_offsets[packed_mask]] = probs[packed_mask]
-    return out
+        return packed_scatter_logprobs(probs, cu, batch_size, cols, attention_mask=attention_mask)
+    return packed_scatter_logprobs(probs, cu, batch_size, cols)
 
 
 def _fused_vocab_parallel_entropy_from_hidden(

@@ -335,6 +335,57 @@ def test_packed_roll_and_scatter_back_brute_force():
     assert torch.equal(out, ref)
 
 
+def test_packed_roll_skips_empty_sequences():
+    cu = torch.tensor([0, 0, 3, 3, 4, 9])
+    target = torch.arange(50, 59)
+    want = torch.cat([target[0:3].roll(-1), target[3:4], target[4:9].roll(-1)])
+    assert torch.equal(O.packed_rolled_targets(target, cu), want)
+
+
+def test_packed_scatter_back_sub_sequences_brute_force():
+    # Two output rows; row 0 holds segments of true lengths 3 and 4 padded to 4 and 6, row 1 one segment of 5 padded to 8.
+    sub = [[3, 4], [5]]
+    cu = torch.tensor([0, 4, 10, 18])
+    probs = torch.arange(18, dtype=torch.float32) + 1
+    for L in (12, 8, 6):
+        out = O.packed_scatter_back(probs, cu, 2, L, sub_seq_lengths=sub)
+        ref = torch.zeros(2, L - 1)
+        placements = [(0, 0, 0, 3), (0, 4, 4, 4), (1, 0, 10, 5)]  # (row, first column, first packed token, true length)
+        for row, col0, tok0, n in placements:
+            for o in range(n - 1):
+                if col0 + o < L - 1:
+                    ref[row, col0 + o] = probs[tok0 + o]
+        assert torch.equal(out, ref), L
+    with pytest.raises(ValueError):
+        O.packed_scatter_back(probs, cu, 2, 12, sub_seq_lengths=[[3], [5]])
+    with pytest.raises(ValueError):
+        O.packed_scatter_back(probs, cu, 2, 12, sub_seq_lengths=[[3, 4], [5, 1]])
+
+
+def test_packed_scatter_back_attention_mask_brute_force():
+    # Rows with left padding, interior padding, a single real token, no real token, and a real token in the last column.
+    am = torch.tensor([
+        [0, 0, 1, 1, 1, 1, 0, 0],
+        [1, 0, 1, 1, 0, 1, 1, 0],
+        [0, 0, 0, 1, 0, 0, 0, 0],
+        [0, 0, 0, 0, 0, 0, 0, 0],
+        [1, 1, 1, 0, 0, 0, 0, 1],
+    ])
+    real = am.sum(1).tolist()
+    padded = [6, 5, 2, 1, 4]  # packed segments may be longer than the real lengths
+    cu = torch.tensor([0] + list(torch.tensor(padded).cumsum(0)))
+    T = int(cu[-1])
+    probs = torch.arange(T, dtype=torch.float32) + 1
+    out = O.packed_scatter_back(probs, cu, 5, 8, attention_mask=am)
+    ref = torch.zeros(5, 7)
+    for b in range(5):
+        positions = [c for c in range(8) if am[b, c]]
+        for j, c in enumerate(positions[:-1]):  # every real token but the last of its row
+            ref[b, c] = probs[cu[b] + j]
+    assert torch.equal(out, ref)
+    assert [int((ref[b] != 0).sum()) for b in range(5)] == [max(n - 1, 0) for n in real]
+
+
 # ----------------------------------------------------------------------------------------------------------------------
 # PPO policy loss
 # ----------------------------------------------------------------------------------------------------------------------

@@ -518,6 +518,164 @@ def test_wrappers_roll_packing_entropy(cuda_device):
     assert cos(hd.grad.reshape(-1, H), ex["d_hidden"]) >= GRAD_COS and cos(wd.grad, ex["d_weight"]) >= GRAD_COS
 
 
+# ---------------------------------------------------------------------------------------------------------------------
+# packed-sequence label preparation and scatter-back: integer / index work, bit-exact against the oracle
+# ---------------------------------------------------------------------------------------------------------------------
+def _ragged_cu(n, max_len, seed, empties=True):
+    gen = torch.Generator().manual_seed(seed)
+    lens = torch.randint(0 if empties else 1, max_len + 1, (n,), generator=gen)
+    lens[torch.randint(0, n, (1,), generator=gen)] = 1
+    if int(lens.sum()) == 0:
+        lens[0] = 3
+    return torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)]), lens
+
+
+@pytest.mark.parametrize("n,max_len,seed", [(1, 1, 0), (4, 17, 1), (37, 300, 2), (700, 50, 3), (3, 40000, 4)])
+def test_packed_next_token_labels_bit_exact(cuda_device, n, max_len, seed):
+    from skyrl_amd.packed import packed_next_token_labels
+    cu, _ = _ragged_cu(n, max_len, seed)
+    T = int(cu[-1])
+    tokens = torch.randint(0, 1 << 40, (T,), generator=torch.Generator().manual_seed(seed))
+    got = packed_next_token_labels(tokens.to(cuda_device), cu.to(cuda_device))
+    assert got.dtype == torch.int64 and torch.equal(got.cpu(), O.packed_rolled_targets(tokens, cu))
+    # a stream longer than cu_seqlens describes: the excess tokens have no sequence and get the "no target" label
+    longer = torch.cat([tokens, tokens[:5]])
+    got = packed_next_token_labels(longer.to(cuda_device), cu.to(cuda_device)).cpu()
+    assert torch.equal(got[:T], O.packed_rolled_targets(tokens, cu)) and bool((got[T:] == SENTINEL).all())
+
+
+@pytest.mark.parametrize("n,max_len,L,seed", [(1, 1, 2, 0), (4, 17, 9, 1), (37, 300, 301, 2), (700, 50, 33, 3), (5, 3000, 2500, 4)])
+def test_packed_scatter_plain_and_adjoint_bit_exact(cuda_device, n, max_len, L, seed):
+    from skyrl_amd.packed import packed_scatter_logprobs
+    cu, _ = _ragged_cu(n, max_len, seed)
+    T = int(cu[-1])
+    gen = torch.Generator().manual_seed(seed)
+    probs = torch.randn(T, generator=gen)
+    pd = probs.to(cuda_device).requires_grad_(True)
+    out = packed_scatter_logprobs(pd, cu.to(cuda_device), n, L - 1)
+    want = O.packed_scatter_back(probs, cu, n, L)
+    assert torch.equal(out.detach().cpu(), want)
+    # adjoint: <scatter(p), G> = <p, gather(G)> with both sides exact sums of selected products
+    G = torch.randn(n, L - 1, generator=gen)
+    out.backward(G.to(cuda_device))
+    idx, off, lens = O.packed_sequence_indices(cu, T)
+    keep = (off < (lens - 1).clamp(min=0)[idx]) & (off < L - 1)
+    want_grad = torch.where(keep, G[idx.clamp(max=n - 1), off.clamp(max=L - 2)], torch.zeros(()))
+    assert torch.equal(pd.grad.cpu(), want_grad)
+
+
+def test_packed_scatter_sub_sequences_bit_exact(cuda_device):
+    from skyrl_amd.packed import packed_scatter_logprobs
+    gen = torch.Generator().manual_seed(9)
+    sub, padded = [], []
+    for r in range(23):
+        k = int(torch.randint(1, 5, (1,), generator=gen))
+        row = [int(x) for x in torch.randint(1, 40, (k,), generator=gen)]
+        sub.append(row)
+        padded += [n + int(torch.randint(0, 4, (1,), generator=gen)) for n in row]
+    cu = torch.cat([torch.zeros(1, dtype=torch.long), torch.tensor(padded).cumsum(0)])
+    T = int(cu[-1])
+    probs = torch.randn(T, generator=gen)
+    rows, offs, lens = model_utils._packed_subseq_row_indices_offsets_and_lens(cu, sub, torch.device("cpu"))
+    r2, o2, l2 = O.packed_subseq_rows_offsets_lens(cu, sub)
+    assert torch.equal(rows, r2) and torch.equal(offs, o2) and torch.equal(lens, l2)
+    for L in (200, 61, 17):
+        pd = probs.to(cuda_device).requires_grad_(True)
+        out = packed_scatter_logprobs(pd, cu.to(cuda_device), len(sub), L - 1, seg_row=rows, seg_col=offs, seg_len=lens)
+        want = O.packed_scatter_back(probs, cu, len(sub), L, sub_seq_lengths=sub)
+        assert torch.equal(out.detach().cpu(), want), L
+        G = torch.randn(len(sub), L - 1, generator=gen)
+        out.backward(G.to(cuda_device))
+        pr = probs.clone().requires_grad_(True)  # the oracle's scatter is differentiable torch indexing: autograd is its adjoint
+        O.packed_scatter_back(pr, cu, len(sub), L, sub_seq_lengths=sub).backward(G)
+        assert torch.equal(pd.grad.cpu(), pr.grad), L
+
+
+@pytest.mark.parametrize("rows,L,seed", [(1, 2, 0), (5, 8, 1), (19, 257, 2), (7, 1500, 3)])
+def test_packed_scatter_attention_mask_bit_exact(cuda_device, rows, L, seed):
+    from skyrl_amd.packed import packed_scatter_logprobs
+    gen = torch.Generator().manual_seed(seed)
+    am = torch.rand(rows, L, generator=gen) < 0.7
+    am[0] = False          # a row without tokens
+    if rows > 1:
+        am[1] = True       # a full row: its last real token sits in the last column
+    if rows > 2:
+        am[2] = False
+        am[2, L // 2] = True  # a single real token
+    real = am.sum(1)
+    padded = real + torch.randint(0, 3, (rows,), generator=gen)
+    cu = torch.cat([torch.zeros(1, dtype=torch.long), padded.cumsum(0)])
+    T = int(cu[-1])
+    probs = torch.randn(max(T, 1), generator=gen)[:T]
+    pd = probs.to(cuda_device).requires_grad_(True)
+    out = packed_scatter_logprobs(pd, cu.to(cuda_device), rows, L - 1, attention_mask=am.to(cuda_device))
+    want = O.packed_scatter_back(probs, cu, rows, L, attention_mask=am)
+    assert torch.equal(out.detach().cpu(), want)
+    G = torch.randn(rows, L - 1, generator=gen)
+    out.backward(G.to(cuda_device))
+    pr = probs.clone().requires_grad_(True)
+    O.packed_scatter_back(pr, cu, rows, L, attention_mask=am).backward(G)
+    assert torch.equal(pd.grad.cpu(), pr.grad)
+
+
+def test_packed_wrapper_all_layouts_with_gradient(cuda_device):
+    """from_parallel_hidden_to_logprobs_packed_sequences end to end (labels kernel -> LM head -> scatter kernel), the three
+    layouts against the oracle's statement of the same pipeline, and the gradient through scatter + LM head."""
+    dev = cuda_device
+    H, V, t = 128, 515, 0.8
+    gen = torch.Generator().manual_seed(52)
+    true_lens = [9, 1, 17, 13, 6]
+    padded = [10, 2, 17, 16, 6]
+    cu = torch.cat([torch.zeros(1, dtype=torch.long), torch.tensor(padded).cumsum(0)])
+    T = int(cu[-1])
+    hidden = torch.randn(1, T, H, generator=gen).to(torch.bfloat16)
+    weight = (torch.randn(V, H, generator=gen) * 3 / H**0.5).to(torch.bfloat16)
+    tokens = torch.randint(0, V, (1, T), generator=gen)
+    rolled = O.packed_rolled_targets(tokens[0], cu)
+    probs = O.fused_chunked_logprob_forward(hidden.float(), weight.float() / t, rolled[None], 0, V, 8)[0]
+    L = 20
+    am = torch.zeros(len(true_lens), L, dtype=torch.bool)
+    for b, n in enumerate(true_lens):
+        am[b, L - n:] = True  # left padded rows
+    sub = [[9, 1], [17], [13, 6]]
+    cases = {
+        "plain": (dict(), O.packed_scatter_back(probs, cu, len(padded), L)),
+        "mask": (dict(attention_mask=am.to(dev)), O.packed_scatter_back(probs, cu, len(padded), L, attention_mask=am)),
+        "sub": (dict(sub_seq_lengths=sub), O.packed_scatter_back(probs, cu, len(sub), 30, sub_seq_lengths=sub)),
+    }
+    for name, (kw, want) in cases.items():
+        hd = hidden.to(dev).requires_grad_(True)
+        wd = weight.to(dev).requires_grad_(True)
+        got = model_utils.from_parallel_hidden_to_logprobs_packed_sequences(
+            hd, wd, tokens.to(dev), cu.to(dev), want.shape[1] + 1, 0, V, None, temperature=t, **kw)
+        assert got.shape == want.shape, name
+        torch.testing.assert_close(got.detach().cpu(), want, atol=2e-3, rtol=1e-4, msg=name)
+        assert torch.equal(got.detach().cpu() == 0, want == 0), name
+        G = torch.randn(want.shape, generator=gen)
+        (got * G.to(dev)).sum().backward()
+        # upstream gradient per packed token = the oracle scatter's adjoint applied to G
+        pr = probs.clone().requires_grad_(True)
+        O.packed_scatter_back(pr, cu, want.shape[0], want.shape[1] + 1, **{k: (v.cpu() if torch.is_tensor(v) else v)
+                                                                          for k, v in kw.items()}).backward(G)
+        ex = O.exact_fwd_bwd(hidden[0], weight, rolled, t, pr.grad.double(), None)
+        assert cos(hd.grad[0], ex["d_hidden"]) >= GRAD_COS and cos(wd.grad, ex["d_weight"]) >= GRAD_COS, name
+
+
+def test_packed_argument_errors(cuda_device):
+    lib = _lib.load()
+    x = torch.zeros(8, dtype=torch.float32, device=cuda_device)
+    i = torch.zeros(8, dtype=torch.int64, device=cuda_device)
+    m = torch.zeros(8, dtype=torch.uint8, device=cuda_device)
+    p = lambda t: t.data_ptr()  # noqa: E731
+    assert lib.skyrl_packed_next_token_labels(None, p(i), 1, 4, p(i), None) == -1
+    assert lib.skyrl_packed_next_token_labels(p(i), p(i), -1, 4, p(i), None) == -2
+    assert lib.skyrl_packed_scatter_logprobs(p(x), p(i), 1, 4, p(i), None, None, None, 1, 4, p(x), None) == -1
+    assert lib.skyrl_packed_scatter_logprobs(p(x), p(i), 1, 4, p(i), p(i), p(i), p(m), 1, 4, p(x), None) == -5
+    assert lib.skyrl_packed_scatter_logprobs(p(x), p(i), 2, 4, None, None, None, p(m), 1, 4, p(x), None) == -2
+    assert lib.skyrl_packed_gather_grad(p(x), p(i), 1, 4, None, None, None, None, 1, -1, p(x), None) == -2
+    torch.cuda.synchronize()
+
+
 def test_opcheck_registration(cuda_device):
     T, H, V = 64, 64, 300
     hidden, weight, labels, _, _ = _rand(T, H, V, seed=2)
