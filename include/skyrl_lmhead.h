@@ -93,22 +93,60 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
                      void* workspace, size_t workspace_bytes, void* stream);
 
 /*
- * The consumer one step after the log-probabilities: PPO policy loss ("regular" and "dual_clip") and its gradient with
- * respect to the log-probabilities in one pass -- what ppo_policy_loss computes with elementwise torch kernels plus
- * autograd (skyrl/backends/skyrl_train/utils/ppo_utils.py:555-588, with safe_exp_delta / masked_mean of
- * skyrl/backends/skyrl_train/utils/torch_utils.py:180-192 and reduce_loss of ppo_utils.py:1145-1149):
+ * The consumer one step after the log-probabilities: the policy loss and its gradient with respect to the
+ * log-probabilities in one pass -- what the reference computes with elementwise torch kernels plus autograd
+ * (skyrl/backends/skyrl_train/utils/ppo_utils.py; safe_exp_delta / masked_mean of
+ * skyrl/backends/skyrl_train/utils/torch_utils.py:180-192; reduce_loss of ppo_utils.py:1145-1149).  loss_type:
+ *   REGULAR, DUAL_CLIP (ppo_policy_loss, ppo_utils.py:555-588):
  *     ratio = exp(clamp(logprobs - old_logprobs, -20, 20))
  *     loss  = -min(ratio * A, clamp(ratio, 1 - eps_clip_low, 1 + eps_clip_high) * A)
- *     dual_clip != 0:  loss = A < 0 ? min(-A * clip_ratio_c, loss) : loss
+ *     DUAL_CLIP:  loss = A < 0 ? min(-A * clip_ratio_c, loss) : loss
+ *     out3[1] = sum [clipped] * mask            (clip_ratio of the reference = out3[1] / max(out3[2], 1))
+ *   CROSS_ENTROPY (cross_entropy_loss, ppo_utils.py:1056-1092):  loss = -logprobs; old_logprobs and advantages are not
+ *     read and may be NULL; out3[1] = 0
+ *   IMPORTANCE_SAMPLING (importance_sampling_loss, ppo_utils.py:1095-1142):  loss = -exp(logprobs - old_logprobs) * A;
+ *     out3[1] = sum exp(logprobs - old_logprobs) * mask     (importance_ratio of the reference = out3[1] / out3[2])
  * All arrays fp32 [T].  loss_mask and loss_weight may be NULL (= 1); loss_weight is any factor of the loss that does not
- * depend on logprobs (the off-policy importance ratio).  out3 = { sum loss*mask*weight, sum [clipped]*mask, sum mask }
- * (clip_ratio of the reference = out3[1] / max(out3[2], 1)).  dlogprobs (may be NULL) receives
- * d out3[0] / d logprobs, i.e. the upstream gradient skyrl_lmhead_bwd takes when the loss is that sum.
+ * depend on logprobs (the off-policy importance ratio).  out3 = { sum loss*mask*weight, (see above), sum mask }.
+ * dlogprobs (may be NULL) receives d out3[0] / d logprobs, i.e. the upstream gradient skyrl_lmhead_bwd takes when the
+ * loss is that sum.  The eps / clip_ratio_c arguments are ignored by the loss types that do not clip.
  */
+#define SKYRL_POLICY_LOSS_REGULAR 0
+#define SKYRL_POLICY_LOSS_DUAL_CLIP 1
+#define SKYRL_POLICY_LOSS_CROSS_ENTROPY 2
+#define SKYRL_POLICY_LOSS_IMPORTANCE_SAMPLING 3
 int skyrl_ppo_policy_loss(const float* logprobs, const float* old_logprobs, const float* advantages,
                           const float* loss_mask, const float* loss_weight, int64_t T,
-                          float eps_clip_low, float eps_clip_high, float clip_ratio_c, int dual_clip,
+                          float eps_clip_low, float eps_clip_high, float clip_ratio_c, int loss_type,
                           float* out3, float* dlogprobs, void* stream);
+
+/*
+ * Approximate KL divergence to a base policy per token (compute_approx_kl, ppo_utils.py:88-126), reduced as the trainer
+ * reduces it for the KL loss term (workers/worker.py:1071-1077: masked_mean over dim -1, then the mean over rows), with
+ * d = logprobs - base_logprobs:
+ *     K1: d        ABS: |d|        K2: d^2 / 2        K3: k = clamp(-d, -20, 20); clamp(exp(k) - k - 1, -10, 10)
+ *     kld[b,s]    = mask != 0 ? value * mask : 0                              (optional output, [rows, cols])
+ *     row_mean[b] = sum_s kld[b,s] * mask[b,s] / max(sum_s mask[b,s], 1)      (required output, [rows])
+ *     mean[0]     = sum_b row_mean[b] / rows                                  (required output)
+ * logprobs, base_logprobs fp32 [rows, cols]; loss_mask fp32 [rows, cols] or NULL (= 1, plain means).
+ * grad_mode 0: dlogprobs not written; 1: dlogprobs = d kld / d logprobs elementwise; 2: dlogprobs = d mean[0] / d logprobs.
+ * Derivatives follow torch: clamp passes the gradient on its closed interval, |.| has derivative 0 at 0.
+ */
+#define SKYRL_KL_K1 0
+#define SKYRL_KL_ABS 1
+#define SKYRL_KL_K2 2
+#define SKYRL_KL_K3 3
+int skyrl_approx_kl(const float* logprobs, const float* base_logprobs, const float* loss_mask, int64_t rows, int64_t cols,
+                    int estimator, float* kld, float* row_mean, float* mean, int grad_mode, float* dlogprobs, void* stream);
+
+/*
+ * masked_mean (torch_utils.py:180-184) per row of values fp32 [rows, cols]:
+ *     means[b] = sum_s values * mask / max(sum_s mask, 1)          (mask NULL: the plain mean)
+ * and, when dvalues is not NULL, dvalues[b,s] = d means[b] / d values[b,s] = mask / max(sum_s mask, 1).
+ * The global form (dim=None, e.g. the entropy term of workers/worker.py:1062) is rows = 1, cols = the element count.
+ */
+int skyrl_masked_mean(const float* values, const float* mask, int64_t rows, int64_t cols, float* means, float* dvalues,
+                      void* stream);
 
 /*
  * Packed-sequence front end: the label of every token of a packed [T] stream is its successor inside its own sequence,

@@ -25,6 +25,11 @@ What pins each function (all in ``tests/test_oracle.py``; none of them re-types 
   * PPO policy loss: hand-computed cases on both sides of every branch (unclipped, clipped high / low for either sign of
     the advantage, dual-clip active / inactive, the +-20 clamp of the log-ratio), fp64 central finite differences of the
     loss for the gradient autograd derives from it, and the masked-mean definition of clip_ratio counted by hand.
+  * cross-entropy and importance-sampling losses, masked_mean: values worked out by hand on small inputs.
+  * approximate KL: hand values at d = 0, ln 2, -1 and in both clamps; the identities the estimators are built on --
+    under x ~ p the expectation of k1 and of k3 is KL(p || q) exactly, summed by brute force over a small alphabet and
+    compared with ``torch.nn.functional.kl_div`` -- and k3 ~ k2 for small differences; the trainer's reduction against a
+    per-row Python loop.
 No function is left "parity unpinned".
 """
 
@@ -436,3 +441,55 @@ def ppo_policy_loss(
         loss = loss * loss_weight
     loss = (loss * loss_mask).sum() if loss_mask is not None else loss.sum()            # reduce_loss
     return loss, clip_ratio.detach()
+
+
+def cross_entropy_loss(log_probs: torch.Tensor, loss_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """ppo_utils.py:1056-1092: the negative log-likelihood, reduced by reduce_loss (:1145-1149)."""
+    loss = -log_probs
+    return (loss * loss_mask).sum() if loss_mask is not None else loss.sum()
+
+
+def importance_sampling_loss(
+    log_probs: torch.Tensor, old_log_probs: torch.Tensor, advantages: torch.Tensor, loss_mask: Optional[torch.Tensor] = None
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """ppo_utils.py:1095-1142: ``(loss, mean importance ratio)``; neither the log-ratio nor the mask count is clamped."""
+    ratio = torch.exp(log_probs - old_log_probs)
+    elementwise = -(ratio * advantages)
+    if loss_mask is not None:
+        return (elementwise * loss_mask).sum(), ((ratio * loss_mask).sum() / loss_mask.sum()).detach()
+    return elementwise.sum(), ratio.mean().detach()
+
+
+def masked_mean(tensor: torch.Tensor, mask: Optional[torch.Tensor], dim: Optional[int] = None) -> torch.Tensor:
+    """skyrl/backends/skyrl_train/utils/torch_utils.py:180-184."""
+    if mask is None:
+        return tensor.mean(dim=dim) if dim is not None else tensor.mean()
+    if dim is None:
+        return (tensor * mask).sum() / mask.sum().clamp(min=1.0)
+    return (tensor * mask).sum(dim=dim) / mask.sum(dim=dim).clamp(min=1.0)
+
+
+def compute_approx_kl(
+    log_probs: torch.Tensor, log_probs_base: torch.Tensor, loss_mask: Optional[torch.Tensor] = None, kl_estimator_type: str = "k3"
+) -> torch.Tensor:
+    """ppo_utils.py:88-126: the k1 / abs / k2 / k3 estimators of KL(policy || base) per token; masked positions are set to 0
+    by ``where`` rather than by the product alone."""
+    if kl_estimator_type == "k1":
+        kld = log_probs - log_probs_base
+    elif kl_estimator_type == "abs":
+        kld = (log_probs - log_probs_base).abs()
+    elif kl_estimator_type == "k2":
+        kld = 0.5 * (log_probs - log_probs_base).square()
+    elif kl_estimator_type == "k3":
+        kl = torch.clamp(log_probs_base - log_probs, min=-20, max=20)
+        kld = torch.clamp(torch.exp(kl) - kl - 1, min=-10, max=10)
+    else:
+        raise ValueError(f"Invalid KL estimator type: {kl_estimator_type}")
+    if loss_mask is not None:
+        kld = torch.where(loss_mask.bool(), kld * loss_mask, torch.zeros((), dtype=kld.dtype))
+    return kld
+
+
+def approx_kl_loss(log_probs, log_probs_base, loss_mask=None, kl_estimator_type: str = "k3") -> torch.Tensor:
+    """The KL loss term as the trainer reduces it (skyrl/backends/skyrl_train/workers/worker.py:1071-1077)."""
+    return masked_mean(compute_approx_kl(log_probs, log_probs_base, loss_mask, kl_estimator_type), loss_mask, dim=-1).mean()

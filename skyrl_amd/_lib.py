@@ -36,6 +36,8 @@ SIGNATURES = {
         ctypes.c_int,
         [_c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_int, _c_p, _c_p, _c_p],
     ),
+    "skyrl_approx_kl": (ctypes.c_int, [_c_p, _c_p, _c_p, _c_i64, _c_i64, ctypes.c_int, _c_p, _c_p, _c_p, ctypes.c_int, _c_p, _c_p]),
+    "skyrl_masked_mean": (ctypes.c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_p, _c_p, _c_p]),
     "skyrl_packed_next_token_labels": (ctypes.c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_p, _c_p]),
     "skyrl_packed_scatter_logprobs": (
         ctypes.c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_p, _c_p]),

@@ -502,74 +502,6 @@ __global__ __launch_bounds__(NTHREADS) void mfma_probe(const bf16x8* __restrict_
   sink[blockIdx.x * NTHREADS + threadIdx.x] = sum;
 }
 
-// ------------------------------------------------------------------------------------------------------------
-// PPO policy loss on the log-probabilities the forward pass produced, and its gradient, in one pass: what
-// ppo_policy_loss does with a chain of elementwise torch kernels and autograd
-// (skyrl/backends/skyrl_train/utils/ppo_utils.py:555-588; safe_exp_delta and masked_mean,
-// skyrl/backends/skyrl_train/utils/torch_utils.py:180-192; reduce_loss, ppo_utils.py:1145-1149).
-//     ratio = exp(clamp(lp - old, -20, 20));  surr1 = ratio * A;  surr2 = clamp(ratio, 1 - lo, 1 + hi) * A
-//     loss  = -min(surr1, surr2);   dual clip: loss = A < 0 ? min(-A * c, loss) : loss
-//     out   = { sum loss * mask * weight,  sum [surr2 < surr1] * mask,  sum mask }
-//     g     = d(sum loss * mask * weight) / d lp      (min and clamp differentiate as torch does: ties of min split
-//             evenly, clamp passes the gradient on its closed interval)
-// `weight` carries whatever multiplies the loss without depending on lp (the off-policy importance ratio).
-// One workgroup: the data is a few hundred KiB, and a fixed reduction order keeps the sums bit-reproducible.
-// ------------------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(1024) void ppo_policy_loss_kernel(const float* __restrict__ lp, const float* __restrict__ old,
-                                                               const float* __restrict__ adv, const float* __restrict__ mask,
-                                                               const float* __restrict__ weight, int64_t T, float eps_low,
-                                                               float eps_high, float clip_c, int dual, float* __restrict__ out,
-                                                               float* __restrict__ g) {
-  __shared__ float red[3][16];
-  float s_loss = 0.f, s_clip = 0.f, s_mask = 0.f;
-  const float lo = 1.f - eps_low, hi = 1.f + eps_high;
-  for (int64_t t = threadIdx.x; t < T; t += blockDim.x) {
-    const float delta = lp[t] - old[t];
-    const float dc = fminf(fmaxf(delta, -20.f), 20.f);
-    const float ratio = expf(dc);
-    const float A = adv[t];
-    const float d_ratio = (delta >= -20.f && delta <= 20.f) ? ratio : 0.f;  // d ratio / d lp
-    const float surr1 = ratio * A;
-    const float rc = fminf(fmaxf(ratio, lo), hi);
-    const float surr2 = rc * A;
-    const float d1 = d_ratio * A;
-    const float d2 = (ratio >= lo && ratio <= hi) ? d_ratio * A : 0.f;
-    float loss = -fminf(surr1, surr2);
-    float dloss = surr1 < surr2 ? -d1 : (surr1 > surr2 ? -d2 : -0.5f * (d1 + d2));
-    const float clipped = surr2 < surr1 ? 1.f : 0.f;
-    if (dual && A < 0.f) {
-      const float pg3 = -A * clip_c;
-      if (pg3 < loss) {
-        loss = pg3;
-        dloss = 0.f;
-      } else if (pg3 == loss) {
-        dloss *= 0.5f;
-      }
-    }
-    const float m = mask ? mask[t] : 1.f;
-    const float w = weight ? m * weight[t] : m;
-    s_loss += loss * w;
-    s_clip += clipped * m;
-    s_mask += m;
-    if (g) g[t] = dloss * w;
-  }
-  // wave reduction, then across the 16 waves
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    s_loss += __shfl_xor(s_loss, off, 64);
-    s_clip += __shfl_xor(s_clip, off, 64);
-    s_mask += __shfl_xor(s_mask, off, 64);
-  }
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  if (lane == 0) red[0][wave] = s_loss, red[1][wave] = s_clip, red[2][wave] = s_mask;
-  __syncthreads();
-  if (threadIdx.x < 3) {
-    float v = 0.f;
-    for (int k = 0; k < (int)(blockDim.x >> 6); ++k) v += red[threadIdx.x][k];
-    out[threadIdx.x] = v;
-  }
-}
-
 // dst[c, r] = src[r, c] for r < R, c < C;  dst[c, r] = 0 for R <= r < Rpad.  bf16 bits, 64 x 64 tiles.
 __global__ __launch_bounds__(256) void transpose_bf16(const uint16_t* __restrict__ src, int lds_src, int R, int C,
                                                       uint16_t* __restrict__ dst, int ld_dst, int Rpad) {
@@ -877,18 +809,6 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
     if (e != hipSuccess) return (int)e;
   }
   return SKYRL_LMHEAD_OK;
-}
-
-int skyrl_ppo_policy_loss(const float* logprobs, const float* old_logprobs, const float* advantages, const float* loss_mask,
-                          const float* loss_weight, int64_t T, float eps_clip_low, float eps_clip_high, float clip_ratio_c,
-                          int dual_clip, float* out3, float* dlogprobs, void* stream) {
-  if (!logprobs || !old_logprobs || !advantages || !out3) return SKYRL_LMHEAD_ERR_NULL;
-  if (T < 1) return SKYRL_LMHEAD_ERR_SHAPE;
-  if (!std::isfinite(eps_clip_low) || !std::isfinite(eps_clip_high) || (dual_clip && !std::isfinite(clip_ratio_c)))
-    return SKYRL_LMHEAD_ERR_ARG;
-  hipLaunchKernelGGL(ppo_policy_loss_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, logprobs, old_logprobs, advantages,
-                     loss_mask, loss_weight, T, eps_clip_low, eps_clip_high, clip_ratio_c, dual_clip ? 1 : 0, out3, dlogprobs);
-  return (int)hipGetLastError();
 }
 
 int skyrl_lmhead_mfma_probe(const void* operands, int workgroups, int iters, float* sink, void* stream) {

@@ -1,0 +1,259 @@
+// The consumers one step after the LM head: per-token losses on the [B, S] log-probabilities and entropies, each with its
+// gradient in the same pass, so that the upstream gradient of the LM-head backward is ready without a chain of elementwise
+// kernels and without a host synchronisation.  All of it is a few hundred KiB of fp32 per micro-batch: HBM-bound,
+// latency-dominated work; the kernels use fixed reduction orders so that every sum is bit-reproducible.
+//
+// Reference (paths under skyrl/backends/skyrl_train/utils/):
+//   ppo_policy_loss            ppo_utils.py:555-588      (policy loss types "regular", "dual_clip")
+//   cross_entropy_loss         ppo_utils.py:1056-1092
+//   importance_sampling_loss   ppo_utils.py:1095-1142
+//   reduce_loss                ppo_utils.py:1145-1149
+//   compute_approx_kl          ppo_utils.py:88-126
+//   masked_mean, safe_exp_delta   torch_utils.py:180-192
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdint.h>
+
+#include <cmath>
+
+#include "../../include/skyrl_lmhead.h"
+
+namespace {
+
+// ------------------------------------------------------------------------------------------------------------
+// Policy loss and its gradient in one pass.
+//   regular / dual clip (ppo_utils.py:555-588):
+//     ratio = exp(clamp(lp - old, -20, 20));  surr1 = ratio * A;  surr2 = clamp(ratio, 1 - lo, 1 + hi) * A
+//     loss  = -min(surr1, surr2);   dual clip: loss = A < 0 ? min(-A * c, loss) : loss
+//     out   = { sum loss * mask * weight,  sum [surr2 < surr1] * mask,  sum mask }
+//   cross entropy (:1056-1092):        loss = -lp;                         out[1] = 0
+//   importance sampling (:1095-1142):  loss = -exp(lp - old) * A (no clamp);   out[1] = sum exp(lp - old) * mask
+//     g     = d(sum loss * mask * weight) / d lp      (min and clamp differentiate as torch does: ties of min split
+//             evenly, clamp passes the gradient on its closed interval)
+// `weight` carries whatever multiplies the loss without depending on lp (the off-policy importance ratio).
+// One workgroup: the data is a few hundred KiB, and a fixed reduction order keeps the sums bit-reproducible.
+// ------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void policy_loss_kernel(const float* __restrict__ lp, const float* __restrict__ old,
+                                                           const float* __restrict__ adv, const float* __restrict__ mask,
+                                                           const float* __restrict__ weight, int64_t T, float eps_low,
+                                                           float eps_high, float clip_c, int type, float* __restrict__ out,
+                                                           float* __restrict__ g) {
+  __shared__ float red[3][16];
+  float s_loss = 0.f, s_clip = 0.f, s_mask = 0.f;
+  const float lo = 1.f - eps_low, hi = 1.f + eps_high;
+  for (int64_t t = threadIdx.x; t < T; t += blockDim.x) {
+    float loss, dloss, stat;
+    if (type == SKYRL_POLICY_LOSS_CROSS_ENTROPY) {
+      loss = -lp[t];
+      dloss = -1.f;
+      stat = 0.f;
+    } else if (type == SKYRL_POLICY_LOSS_IMPORTANCE_SAMPLING) {
+      const float ratio = expf(lp[t] - old[t]);
+      loss = -(ratio * adv[t]);
+      dloss = loss;
+      stat = ratio;
+    } else {
+      const float delta = lp[t] - old[t];
+      const float dc = fminf(fmaxf(delta, -20.f), 20.f);
+      const float ratio = expf(dc);
+      const float A = adv[t];
+      const float d_ratio = (delta >= -20.f && delta <= 20.f) ? ratio : 0.f;  // d ratio / d lp
+      const float surr1 = ratio * A;
+      const float rc = fminf(fmaxf(ratio, lo), hi);
+      const float surr2 = rc * A;
+      const float d1 = d_ratio * A;
+      const float d2 = (ratio >= lo && ratio <= hi) ? d_ratio * A : 0.f;
+      loss = -fminf(surr1, surr2);
+      dloss = surr1 < surr2 ? -d1 : (surr1 > surr2 ? -d2 : -0.5f * (d1 + d2));
+      stat = surr2 < surr1 ? 1.f : 0.f;
+      if (type == SKYRL_POLICY_LOSS_DUAL_CLIP && A < 0.f) {
+        const float pg3 = -A * clip_c;
+        if (pg3 < loss) {
+          loss = pg3;
+          dloss = 0.f;
+        } else if (pg3 == loss) {
+          dloss *= 0.5f;
+        }
+      }
+    }
+    const float m = mask ? mask[t] : 1.f;
+    const float w = weight ? m * weight[t] : m;
+    s_loss += loss * w;
+    s_clip += stat * m;
+    s_mask += m;
+    if (g) g[t] = dloss * w;
+  }
+  // wave reduction, then across the 16 waves
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    s_loss += __shfl_xor(s_loss, off, 64);
+    s_clip += __shfl_xor(s_clip, off, 64);
+    s_mask += __shfl_xor(s_mask, off, 64);
+  }
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (lane == 0) red[0][wave] = s_loss, red[1][wave] = s_clip, red[2][wave] = s_mask;
+  __syncthreads();
+  if (threadIdx.x < 3) {
+    float v = 0.f;
+    for (int k = 0; k < (int)(blockDim.x >> 6); ++k) v += red[threadIdx.x][k];
+    out[threadIdx.x] = v;
+  }
+}
+
+constexpr int kRowThreads = 256;
+
+// Sum of one value per thread over the workgroup, in a fixed order; every thread receives it.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  __syncthreads();  // red may still be read from an earlier call
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float s = 0.f;
+  for (int k = 0; k < kRowThreads / 64; ++k) s += red[k];
+  return s;
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// Approximate KL between the policy and a base policy, per token (ppo_utils.py:88-126), reduced the way the trainer
+// reduces it (workers/worker.py:1071-1077): masked mean over each row, then the mean over rows.
+//   k1: d;  abs: |d|;  k2: d^2 / 2   with d = lp - base
+//   k3: k = clamp(base - lp, -20, 20);  kld = clamp(exp(k) - k - 1, -10, 10)
+//   kld_masked = mask != 0 ? kld * mask : 0            (the value compute_approx_kl returns)
+//   row_mean_b = sum_s kld_masked * mask / max(sum_s mask, 1)      (masked_mean multiplies by the mask once more)
+// One workgroup per row: mask sum, then values, row sum and gradient in a second sweep.  GRAD: 0 none, 1 the elementwise
+// derivative d kld_masked / d lp, 2 the derivative of mean_b row_mean_b.
+// ------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kRowThreads) void approx_kl_rows_kernel(const float* __restrict__ lp, const float* __restrict__ base,
+                                                                     const float* __restrict__ mask, int64_t rows, int64_t cols,
+                                                                     int estimator, int grad_mode, float* __restrict__ kld_out,
+                                                                     float* __restrict__ row_mean, float* __restrict__ g) {
+  __shared__ float red[kRowThreads / 64];
+  const int64_t row0 = (int64_t)blockIdx.x * cols;
+  float denom = (float)cols;
+  if (mask) {
+    float ms = 0.f;
+    for (int64_t c = threadIdx.x; c < cols; c += kRowThreads) ms += mask[row0 + c];
+    denom = fmaxf(block_sum(ms, red), 1.f);
+  }
+  const float gscale = 1.f / (denom * (float)rows);
+  float acc = 0.f;
+  for (int64_t c = threadIdx.x; c < cols; c += kRowThreads) {
+    const float d = lp[row0 + c] - base[row0 + c];
+    float kld, dk;
+    if (estimator == SKYRL_KL_K1) {
+      kld = d;
+      dk = 1.f;
+    } else if (estimator == SKYRL_KL_ABS) {
+      kld = fabsf(d);
+      dk = d > 0.f ? 1.f : (d < 0.f ? -1.f : 0.f);
+    } else if (estimator == SKYRL_KL_K2) {
+      kld = 0.5f * d * d;
+      dk = d;
+    } else {
+      const float kraw = base[row0 + c] - lp[row0 + c];
+      const float k = fminf(fmaxf(kraw, -20.f), 20.f);
+      const float ratio = expf(k);
+      const float v = ratio - k - 1.f;
+      kld = fminf(fmaxf(v, -10.f), 10.f);
+      const bool open = kraw >= -20.f && kraw <= 20.f && v >= -10.f && v <= 10.f;
+      dk = open ? 1.f - ratio : 0.f;  // d/d lp of exp(k) - k - 1 with k = base - lp
+    }
+    float m = 1.f;
+    if (mask) {
+      m = mask[row0 + c];
+      if (m != 0.f) {
+        kld *= m;
+        dk *= m;
+      } else {
+        kld = 0.f;
+        dk = 0.f;
+      }
+    }
+    if (kld_out) kld_out[row0 + c] = kld;
+    acc += mask ? kld * m : kld;
+    if (grad_mode == 1) g[row0 + c] = dk;
+    if (grad_mode == 2) g[row0 + c] = (mask ? dk * m : dk) * gscale;
+  }
+  const float total = block_sum(acc, red);
+  if (threadIdx.x == 0) row_mean[blockIdx.x] = total / denom;
+}
+
+// out[0] = sum_i v[i] * scale, one workgroup, fixed order.
+__global__ __launch_bounds__(kRowThreads) void scaled_sum_kernel(const float* __restrict__ v, int64_t n, float scale,
+                                                                 float* __restrict__ out) {
+  __shared__ float red[kRowThreads / 64];
+  float acc = 0.f;
+  for (int64_t i = threadIdx.x; i < n; i += kRowThreads) acc += v[i];
+  const float total = block_sum(acc, red);
+  if (threadIdx.x == 0) out[0] = total * scale;
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// masked_mean (torch_utils.py:180-184).  Per row: means[b] = sum_s v * mask / max(sum_s mask, 1) (mask NULL: plain mean),
+// dvalues = d means[b] / d v = mask / max(sum mask, 1).  The global form is the same kernel on one row of rows * cols.
+// ------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kRowThreads) void masked_mean_rows_kernel(const float* __restrict__ v, const float* __restrict__ mask,
+                                                                       int64_t cols, float* __restrict__ means,
+                                                                       float* __restrict__ dv) {
+  __shared__ float red[kRowThreads / 64];
+  const int64_t row0 = (int64_t)blockIdx.x * cols;
+  float sv = 0.f, sm = 0.f;
+  for (int64_t c = threadIdx.x; c < cols; c += kRowThreads) {
+    const float m = mask ? mask[row0 + c] : 1.f;
+    sv += v[row0 + c] * m;
+    sm += m;
+  }
+  const float total = block_sum(sv, red);
+  const float denom = mask ? fmaxf(block_sum(sm, red), 1.f) : (float)cols;
+  if (threadIdx.x == 0) means[blockIdx.x] = total / denom;
+  if (dv) {
+    const float r = 1.f / denom;
+    for (int64_t c = threadIdx.x; c < cols; c += kRowThreads) dv[row0 + c] = mask ? mask[row0 + c] * r : r;
+  }
+}
+
+bool finite(float x) { return std::isfinite(x); }
+
+}  // namespace
+
+extern "C" {
+
+int skyrl_ppo_policy_loss(const float* logprobs, const float* old_logprobs, const float* advantages, const float* loss_mask,
+                          const float* loss_weight, int64_t T, float eps_clip_low, float eps_clip_high, float clip_ratio_c,
+                          int loss_type, float* out3, float* dlogprobs, void* stream) {
+  if (loss_type < SKYRL_POLICY_LOSS_REGULAR || loss_type > SKYRL_POLICY_LOSS_IMPORTANCE_SAMPLING) return SKYRL_LMHEAD_ERR_ARG;
+  const bool needs_old = loss_type != SKYRL_POLICY_LOSS_CROSS_ENTROPY;
+  if (!logprobs || !out3 || (needs_old && (!old_logprobs || !advantages))) return SKYRL_LMHEAD_ERR_NULL;
+  if (T < 1) return SKYRL_LMHEAD_ERR_SHAPE;
+  const bool clips = loss_type == SKYRL_POLICY_LOSS_REGULAR || loss_type == SKYRL_POLICY_LOSS_DUAL_CLIP;
+  if (clips && (!finite(eps_clip_low) || !finite(eps_clip_high))) return SKYRL_LMHEAD_ERR_ARG;
+  if (loss_type == SKYRL_POLICY_LOSS_DUAL_CLIP && !finite(clip_ratio_c)) return SKYRL_LMHEAD_ERR_ARG;
+  hipLaunchKernelGGL(policy_loss_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, logprobs, old_logprobs, advantages,
+                     loss_mask, loss_weight, T, eps_clip_low, eps_clip_high, clip_ratio_c, loss_type, out3, dlogprobs);
+  return (int)hipGetLastError();
+}
+
+int skyrl_approx_kl(const float* logprobs, const float* base_logprobs, const float* loss_mask, int64_t rows, int64_t cols,
+                    int estimator, float* kld, float* row_mean, float* mean, int grad_mode, float* dlogprobs, void* stream) {
+  if (!logprobs || !base_logprobs || !row_mean || !mean) return SKYRL_LMHEAD_ERR_NULL;
+  if (grad_mode < 0 || grad_mode > 2 || estimator < SKYRL_KL_K1 || estimator > SKYRL_KL_K3) return SKYRL_LMHEAD_ERR_ARG;
+  if (grad_mode != 0 && !dlogprobs) return SKYRL_LMHEAD_ERR_NULL;
+  if (rows < 1 || cols < 1 || rows >= (int64_t(1) << 31)) return SKYRL_LMHEAD_ERR_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(approx_kl_rows_kernel, dim3((unsigned)rows), dim3(kRowThreads), 0, s, logprobs, base_logprobs, loss_mask,
+                     rows, cols, estimator, grad_mode, kld, row_mean, dlogprobs);
+  hipLaunchKernelGGL(scaled_sum_kernel, dim3(1), dim3(kRowThreads), 0, s, row_mean, rows, 1.f / (float)rows, mean);
+  return (int)hipGetLastError();
+}
+
+int skyrl_masked_mean(const float* values, const float* mask, int64_t rows, int64_t cols, float* means, float* dvalues,
+                      void* stream) {
+  if (!values || !means) return SKYRL_LMHEAD_ERR_NULL;
+  if (rows < 1 || cols < 1 || rows >= (int64_t(1) << 31)) return SKYRL_LMHEAD_ERR_SHAPE;
+  hipLaunchKernelGGL(masked_mean_rows_kernel, dim3((unsigned)rows), dim3(kRowThreads), 0, (hipStream_t)stream, values, mask, cols,
+                     means, dvalues);
+  return (int)hipGetLastError();
+}
+
+}  // extern "C"

@@ -1,16 +1,24 @@
-"""PPO policy loss on the fused path's log-probabilities: loss, clip statistics and d loss / d log-probs in one HIP kernel.
+"""Losses on the fused path's log-probabilities and entropies: value, statistics and gradient from one HIP kernel each.
 
-Mirrors ``ppo_policy_loss`` of the reference (skyrl/backends/skyrl_train/utils/ppo_utils.py:555-588; policy loss types
-"regular" and "dual_clip"): the same positional arguments, the same ``(loss, {"clip_ratio": ...})`` result, the loss reduced
-as ``reduce_loss`` does (masked sum, ppo_utils.py:1145-1149; the reference folds the kind of mean into the advantages
-beforehand, ppo_utils.py:1152-1181).  The reference computes it with about fifteen elementwise torch kernels and lets
-autograd derive the gradient; here one kernel produces the loss sum, the clip counts and the gradient, so the upstream
-gradient of ``skyrl_lmhead_bwd`` is ready without another pass over the ``[B, S]`` tensors and, with
-``sync_metrics=False``, without a host synchronisation.
+Mirrors of the reference's functions (skyrl/backends/skyrl_train/utils/ppo_utils.py unless noted), same positional arguments
+and results:
+
+* ``ppo_policy_loss``           :555-588  (policy loss types "regular" and "dual_clip") -> ``(loss, {"clip_ratio": ...})``
+* ``cross_entropy_loss``        :1056-1092 -> ``(loss, {"clip_ratio": 0.0})``
+* ``importance_sampling_loss``  :1095-1142 -> ``(loss, {"importance_ratio": ...})``
+* ``compute_approx_kl``         :88-126    -> per-token KL estimate ``[B, S]``
+* ``masked_mean``               torch_utils.py:180-184
+
+plus ``approx_kl_loss``, the reduction the trainer applies to the KL estimate (``masked_mean(kl, mask, dim=-1).mean()``,
+workers/worker.py:1071-1077) fused with the estimate and its gradient.  The losses are reduced as ``reduce_loss`` does
+(masked sum, :1145-1149; the reference folds the kind of mean into the advantages beforehand, :1152-1181).  The reference
+computes each with a chain of elementwise torch kernels and lets autograd derive the gradient; here one kernel produces
+value, statistics and gradient, so the upstream gradient of ``skyrl_lmhead_bwd`` is ready without another pass over the
+``[B, S]`` tensors and, with ``sync_metrics=False``, without a host synchronisation.
 
 Off-policy correction (``apply_off_policy_correction``, off_policy_correction_utils.py:351-385) multiplies the per-token
 loss by an importance ratio that does not depend on the policy's log-probabilities: pass that ratio as ``loss_weight``.
-Computing it from ``rollout_logprobs`` is outside this module, so ``rollout_logprobs`` must be ``None``.
+Computing it from ``rollout_logprobs`` is outside this module, so ``ppo_policy_loss`` needs ``rollout_logprobs=None``.
 """
 
 from __future__ import annotations
@@ -22,7 +30,11 @@ import torch
 from . import _lib
 from .ops import _require_device
 
-__all__ = ["ppo_policy_loss", "ppo_policy_loss_terms"]
+__all__ = ["ppo_policy_loss", "cross_entropy_loss", "importance_sampling_loss", "compute_approx_kl", "approx_kl_loss",
+           "masked_mean", "ppo_policy_loss_terms"]
+
+LOSS_REGULAR, LOSS_DUAL_CLIP, LOSS_CROSS_ENTROPY, LOSS_IMPORTANCE_SAMPLING = 0, 1, 2, 3
+KL_ESTIMATORS = {"k1": 0, "abs": 1, "k2": 2, "k3": 3}
 
 
 def _flat_f32(name: str, t: Optional[torch.Tensor], numel: int) -> Optional[torch.Tensor]:
@@ -36,18 +48,22 @@ def _flat_f32(name: str, t: Optional[torch.Tensor], numel: int) -> Optional[torc
 @torch.library.custom_op("skyrl_amd::ppo_policy_loss", mutates_args=())
 def ppo_policy_loss_terms(
     log_probs: torch.Tensor,
-    old_log_probs: torch.Tensor,
-    advantages: torch.Tensor,
+    old_log_probs: Optional[torch.Tensor],
+    advantages: Optional[torch.Tensor],
     loss_mask: Optional[torch.Tensor],
     loss_weight: Optional[torch.Tensor],
     eps_clip_low: float,
     eps_clip_high: float,
     clip_ratio_c: float,
-    dual_clip: bool,
+    loss_type: int,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
-    """``(sums, grad)``: sums = [sum loss*mask*weight, sum clipped*mask, sum mask] (fp32 [3]); grad = d sums[0] / d log_probs
-    (fp32, flat).  All inputs are flat contiguous fp32 tensors of one length."""
-    dev = _require_device(log_probs, old_log_probs, advantages)
+    """``(sums, grad)``: sums = [sum loss*mask*weight, statistic, sum mask] (fp32 [3]; the statistic is the number of clipped
+    tokens, or the sum of importance ratios for LOSS_IMPORTANCE_SAMPLING); grad = d sums[0] / d log_probs (fp32, flat).
+    All inputs are flat contiguous fp32 tensors of one length; LOSS_CROSS_ENTROPY reads neither old_log_probs nor
+    advantages."""
+    dev = _require_device(log_probs)
+    if loss_type != LOSS_CROSS_ENTROPY and (old_log_probs is None or advantages is None):
+        raise ValueError("this loss type needs old_log_probs and advantages")
     n = log_probs.numel()
     for name, t in (("log_probs", log_probs), ("old_log_probs", old_log_probs), ("advantages", advantages),
                     ("loss_mask", loss_mask), ("loss_weight", loss_weight)):
@@ -62,26 +78,26 @@ def ppo_policy_loss_terms(
     ptr = lambda t: None if t is None else t.data_ptr()  # noqa: E731
     with torch.cuda.device(dev):
         st = _lib.load().skyrl_ppo_policy_loss(
-            log_probs.data_ptr(), old_log_probs.data_ptr(), advantages.data_ptr(), ptr(loss_mask), ptr(loss_weight), n,
-            float(eps_clip_low), float(eps_clip_high), float(clip_ratio_c), int(bool(dual_clip)), sums.data_ptr(),
+            log_probs.data_ptr(), ptr(old_log_probs), ptr(advantages), ptr(loss_mask), ptr(loss_weight), n,
+            float(eps_clip_low), float(eps_clip_high), float(clip_ratio_c), int(loss_type), sums.data_ptr(),
             grad.data_ptr(), torch.cuda.current_stream(dev).cuda_stream)
     _lib.check(st, "skyrl_ppo_policy_loss")
     return sums, grad
 
 
 @ppo_policy_loss_terms.register_fake
-def _(log_probs, old_log_probs, advantages, loss_mask, loss_weight, eps_clip_low, eps_clip_high, clip_ratio_c, dual_clip):
+def _(log_probs, old_log_probs, advantages, loss_mask, loss_weight, eps_clip_low, eps_clip_high, clip_ratio_c, loss_type):
     return log_probs.new_empty(3, dtype=torch.float32), log_probs.new_empty(log_probs.numel(), dtype=torch.float32)
 
 
 class _PolicyLoss(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, log_probs, old_log_probs, advantages, loss_mask, loss_weight, eps_low, eps_high, clip_c, dual):
+    def forward(ctx, log_probs, old_log_probs, advantages, loss_mask, loss_weight, eps_low, eps_high, clip_c, loss_type):
         n = log_probs.numel()
         sums, grad = ppo_policy_loss_terms(
             _flat_f32("log_probs", log_probs, n), _flat_f32("old_log_probs", old_log_probs, n),
             _flat_f32("advantages", advantages, n), _flat_f32("loss_mask", loss_mask, n),
-            _flat_f32("loss_weight", loss_weight, n), eps_low, eps_high, clip_c, dual)
+            _flat_f32("loss_weight", loss_weight, n), eps_low, eps_high, clip_c, loss_type)
         ctx.save_for_backward(grad)
         ctx.shape, ctx.dtype = log_probs.shape, log_probs.dtype
         ctx.mark_non_differentiable(sums)
@@ -119,6 +135,187 @@ def ppo_policy_loss(
     dual = loss_type == "dual_clip"
     loss, sums = _PolicyLoss.apply(log_probs, old_log_probs, advantages, loss_mask, loss_weight, float(config.eps_clip_low),
                                    float(config.eps_clip_high), float(getattr(config, "clip_ratio_c", 0.0)) if dual else 0.0,
-                                   dual)
+                                   LOSS_DUAL_CLIP if dual else LOSS_REGULAR)
     clip_ratio = sums[1] / sums[2].clamp(min=1.0)
     return loss, {"clip_ratio": clip_ratio.item() if sync_metrics else clip_ratio}
+
+
+def cross_entropy_loss(
+    log_probs: torch.Tensor,
+    old_log_probs: Optional[torch.Tensor],
+    advantages: Optional[torch.Tensor],
+    config: Any,
+    loss_mask: Optional[torch.Tensor] = None,
+    rollout_logprobs: Optional[torch.Tensor] = None,
+) -> Tuple[torch.Tensor, Dict[str, Any]]:
+    """Supervised negative log-likelihood, ``-(log_probs * loss_mask).sum()`` (reference ``cross_entropy_loss``,
+    ppo_utils.py:1056-1092); ``old_log_probs``, ``advantages``, ``config`` and ``rollout_logprobs`` are ignored as there."""
+    loss, _ = _PolicyLoss.apply(log_probs, None, None, loss_mask, None, 0.0, 0.0, 0.0, LOSS_CROSS_ENTROPY)
+    return loss, {"clip_ratio": 0.0}
+
+
+def importance_sampling_loss(
+    log_probs: torch.Tensor,
+    old_log_probs: torch.Tensor,
+    advantages: torch.Tensor,
+    config: Any,
+    loss_mask: Optional[torch.Tensor] = None,
+    rollout_logprobs: Optional[torch.Tensor] = None,
+    *,
+    sync_metrics: bool = True,
+) -> Tuple[torch.Tensor, Dict[str, Any]]:
+    """``-(exp(log_probs - old_log_probs) * advantages * loss_mask).sum()`` and the masked mean importance ratio (reference
+    ``importance_sampling_loss``, ppo_utils.py:1095-1142; no clamp of the log-ratio, no clamp of the mask count)."""
+    loss, sums = _PolicyLoss.apply(log_probs, old_log_probs, advantages, loss_mask, None, 0.0, 0.0, 0.0,
+                                   LOSS_IMPORTANCE_SAMPLING)
+    ratio = sums[1] / sums[2]
+    return loss, {"importance_ratio": ratio.item() if sync_metrics else ratio}
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# approximate KL and masked mean
+# ----------------------------------------------------------------------------------------------------------------------
+def _rows_cols(t: torch.Tensor) -> Tuple[int, int]:
+    if t.dim() == 0:
+        return 1, 1
+    cols = t.shape[-1]
+    return (t.numel() // cols if cols else 0), cols
+
+
+def _same_f32(name: str, t: Optional[torch.Tensor], like: torch.Tensor) -> Optional[torch.Tensor]:
+    if t is None:
+        return None
+    if t.shape != like.shape:
+        raise ValueError(f"{name} has shape {tuple(t.shape)}, expected {tuple(like.shape)}")
+    return t.detach().to(torch.float32).contiguous()
+
+
+@torch.library.custom_op("skyrl_amd::approx_kl", mutates_args=())
+def _approx_kl(log_probs: torch.Tensor, log_probs_base: torch.Tensor, loss_mask: Optional[torch.Tensor], estimator: int,
+               grad_mode: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``(kld, row_mean, mean, grad)`` for contiguous fp32 ``[rows, cols]`` inputs; grad_mode 1: elementwise derivative of
+    kld, 2: derivative of ``mean``; 0: grad is empty."""
+    dev = _require_device(log_probs, log_probs_base)
+    rows, cols = log_probs.shape
+    kld = torch.empty_like(log_probs)
+    row_mean = torch.empty(rows, dtype=torch.float32, device=dev)
+    mean = torch.empty((), dtype=torch.float32, device=dev)
+    grad = torch.empty_like(log_probs) if grad_mode else torch.empty(0, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        st = _lib.load().skyrl_approx_kl(
+            log_probs.data_ptr(), log_probs_base.data_ptr(), None if loss_mask is None else loss_mask.data_ptr(), rows, cols,
+            int(estimator), kld.data_ptr(), row_mean.data_ptr(), mean.data_ptr(), int(grad_mode),
+            grad.data_ptr() if grad_mode else None, torch.cuda.current_stream(dev).cuda_stream)
+    _lib.check(st, "skyrl_approx_kl")
+    return kld, row_mean, mean, grad
+
+
+@_approx_kl.register_fake
+def _(log_probs, log_probs_base, loss_mask, estimator, grad_mode):
+    rows = log_probs.shape[0]
+    return (torch.empty_like(log_probs), log_probs.new_empty(rows), log_probs.new_empty(()),
+            torch.empty_like(log_probs) if grad_mode else log_probs.new_empty(0))
+
+
+def _kl_operands(log_probs, log_probs_base, loss_mask, kl_estimator_type):
+    if kl_estimator_type not in KL_ESTIMATORS:
+        raise ValueError(f"Invalid KL estimator type: {kl_estimator_type}")
+    if log_probs.numel() == 0:
+        raise ValueError("log_probs is empty")
+    rows, cols = _rows_cols(log_probs)
+    lp = log_probs.detach().to(torch.float32).contiguous().reshape(rows, cols)
+    base = _same_f32("log_probs_base", log_probs_base, log_probs).reshape(rows, cols)
+    mask = _same_f32("loss_mask", loss_mask, log_probs)
+    return lp, base, None if mask is None else mask.reshape(rows, cols), KL_ESTIMATORS[kl_estimator_type]
+
+
+class _ApproxKL(torch.autograd.Function):
+    """grad_mode 1: returns the per-token estimate; grad_mode 2: returns the trainer's scalar reduction of it."""
+
+    @staticmethod
+    def forward(ctx, log_probs, log_probs_base, loss_mask, kl_estimator_type, grad_mode):
+        lp, base, mask, est = _kl_operands(log_probs, log_probs_base, loss_mask, kl_estimator_type)
+        kld, _, mean, grad = _approx_kl(lp, base, mask, est, grad_mode)
+        ctx.save_for_backward(grad)
+        ctx.shape, ctx.dtype = log_probs.shape, log_probs.dtype
+        return kld.reshape(log_probs.shape) if grad_mode == 1 else mean
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        (grad,) = ctx.saved_tensors
+        d = grad.reshape(ctx.shape) * grad_out  # only the dependence on log_probs is tracked, as the trainer needs it
+        return d.to(ctx.dtype), None, None, None, None
+
+
+def compute_approx_kl(
+    log_probs: torch.Tensor,
+    log_probs_base: torch.Tensor,
+    loss_mask: Optional[torch.Tensor] = None,
+    kl_estimator_type: str = "k3",
+) -> torch.Tensor:
+    """Per-token KL estimate, same contract as the reference's ``compute_approx_kl`` (ppo_utils.py:88-126): estimators
+    ``k1``, ``abs``, ``k2``, ``k3``; masked positions are exactly 0.  fp32 result of the shape of ``log_probs``;
+    differentiable with respect to ``log_probs`` (the base policy's log-probabilities are treated as constants)."""
+    return _ApproxKL.apply(log_probs, log_probs_base, loss_mask, kl_estimator_type, 1)
+
+
+def approx_kl_loss(
+    log_probs: torch.Tensor,
+    log_probs_base: torch.Tensor,
+    loss_mask: Optional[torch.Tensor] = None,
+    kl_estimator_type: str = "k3",
+) -> torch.Tensor:
+    """``masked_mean(compute_approx_kl(...), loss_mask, dim=-1).mean()`` -- the KL loss term of the trainer
+    (workers/worker.py:1071-1077) -- from one kernel, with its gradient with respect to ``log_probs``."""
+    return _ApproxKL.apply(log_probs, log_probs_base, loss_mask, kl_estimator_type, 2)
+
+
+@torch.library.custom_op("skyrl_amd::masked_mean", mutates_args=())
+def _masked_mean(values: torch.Tensor, mask: Optional[torch.Tensor], want_grad: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``(means [rows], dvalues [rows, cols] or empty)`` for contiguous fp32 ``[rows, cols]`` inputs."""
+    dev = _require_device(values)
+    rows, cols = values.shape
+    means = torch.empty(rows, dtype=torch.float32, device=dev)
+    dv = torch.empty_like(values) if want_grad else torch.empty(0, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        st = _lib.load().skyrl_masked_mean(values.data_ptr(), None if mask is None else mask.data_ptr(), rows, cols,
+                                           means.data_ptr(), dv.data_ptr() if want_grad else None,
+                                           torch.cuda.current_stream(dev).cuda_stream)
+    _lib.check(st, "skyrl_masked_mean")
+    return means, dv
+
+
+@_masked_mean.register_fake
+def _(values, mask, want_grad):
+    return values.new_empty(values.shape[0]), torch.empty_like(values) if want_grad else values.new_empty(0)
+
+
+class _MaskedMean(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, tensor, mask, rows, cols, out_shape):
+        v = tensor.detach().to(torch.float32).contiguous().reshape(rows, cols)
+        m = None if mask is None else mask.detach().to(torch.float32).expand_as(tensor).contiguous().reshape(rows, cols)
+        means, dv = _masked_mean(v, m, bool(ctx.needs_input_grad[0]))
+        ctx.save_for_backward(dv)
+        ctx.shape, ctx.dtype, ctx.rows = tensor.shape, tensor.dtype, rows
+        return means.reshape(out_shape)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        (dv,) = ctx.saved_tensors
+        d = dv * grad_out.reshape(ctx.rows, 1).to(torch.float32)
+        return d.reshape(ctx.shape).to(ctx.dtype), None, None, None, None
+
+
+def masked_mean(tensor: torch.Tensor, mask: Optional[torch.Tensor], dim: Optional[int] = None) -> torch.Tensor:
+    """``(tensor * mask).sum(dim) / mask.sum(dim).clamp(min=1)``; ``mask=None``: the plain mean (reference ``masked_mean``,
+    torch_utils.py:180-184).  ``dim`` is ``None`` (everything) or the last dimension; fp32 result; differentiable with respect
+    to ``tensor``."""
+    if tensor.numel() == 0:
+        raise ValueError("masked_mean of an empty tensor")
+    if dim is None:
+        return _MaskedMean.apply(tensor, mask, 1, tensor.numel(), ())
+    if dim not in (-1, tensor.dim() - 1):
+        raise NotImplementedError("masked_mean reduces everything (dim=None) or the last dimension")
+    rows, cols = _rows_cols(tensor)
+    return _MaskedMean.apply(tensor, mask, rows, cols, tensor.shape[:-1])

@@ -458,3 +458,90 @@ def test_ppo_loss_gradient_matches_finite_differences(dual):
         d[i] = eps
         fd = (f(lp + d) - f(lp - d)).item() / (2 * eps)
         assert x.grad[i].item() == pytest.approx(fd, abs=1e-6), f"token {i}"
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# the other per-token losses: cross entropy, importance sampling, approximate KL, masked mean
+# ----------------------------------------------------------------------------------------------------------------------
+def test_cross_entropy_and_importance_sampling_by_hand():
+    lp = torch.tensor([-1.0, -2.0, -0.5, -3.0], dtype=torch.float64)
+    mask = torch.tensor([1.0, 0.0, 1.0, 1.0], dtype=torch.float64)
+    assert O.cross_entropy_loss(lp).item() == pytest.approx(6.5)
+    assert O.cross_entropy_loss(lp, mask).item() == pytest.approx(4.5)
+    old = lp - torch.tensor([math.log(2.0), 0.0, math.log(0.5), math.log(3.0)], dtype=torch.float64)   # ratios 2, 1, 1/2, 3
+    adv = torch.tensor([1.0, -1.0, 4.0, -2.0], dtype=torch.float64)
+    loss, ratio = O.importance_sampling_loss(lp, old, adv)
+    assert loss.item() == pytest.approx(-(2 - 1 + 2 - 6)) and ratio.item() == pytest.approx(6.5 / 4)
+    loss, ratio = O.importance_sampling_loss(lp, old, adv, mask)
+    assert loss.item() == pytest.approx(-(2 + 2 - 6)) and ratio.item() == pytest.approx(5.5 / 3)
+    # no clamp of the log-ratio: a difference of 30 gives e^30, which safe_exp_delta would have cut at e^20
+    big, _ = O.importance_sampling_loss(torch.tensor([0.0]), torch.tensor([-30.0]), torch.tensor([1.0]))
+    assert big.item() == pytest.approx(-math.exp(30.0), rel=1e-6)
+
+
+def test_masked_mean_by_hand():
+    t = torch.tensor([[1.0, 2.0, 3.0], [4.0, 5.0, 6.0]])
+    m = torch.tensor([[1.0, 0.0, 1.0], [0.0, 0.0, 0.0]])
+    assert O.masked_mean(t, None).item() == pytest.approx(3.5)
+    assert O.masked_mean(t, m).item() == pytest.approx(2.0)
+    assert O.masked_mean(t, None, dim=-1).tolist() == pytest.approx([2.0, 5.0])
+    assert O.masked_mean(t, m, dim=-1).tolist() == pytest.approx([2.0, 0.0])       # an all-masked row: 0 / clamp(0, 1)
+    half = torch.tensor([[0.5, 0.5, 0.0], [0.25, 0.0, 0.0]])                        # fractional weights, count below 1
+    assert O.masked_mean(t, half, dim=-1).tolist() == pytest.approx([1.5, 1.0])
+
+
+def test_approx_kl_hand_values_and_clamps():
+    base = torch.zeros(6, dtype=torch.float64)
+    # base - lp = k:            0      ln 2             -1      25 (clamped to 20)  -25 (clamped)   2
+    lp = torch.tensor([0.0, -math.log(2.0), 1.0, -25.0, 25.0, -2.0], dtype=torch.float64)
+    k3 = O.compute_approx_kl(lp, base, None, "k3").tolist()
+    assert k3[0] == 0.0
+    assert k3[1] == pytest.approx(1.0 - math.log(2.0))
+    assert k3[2] == pytest.approx(math.exp(-1.0))
+    assert k3[3] == 10.0                                                      # e^20 - 21 cut by the outer clamp
+    assert k3[4] == 10.0                                                      # e^-20 + 19 cut by the outer clamp
+    assert k3[5] == pytest.approx(math.exp(2.0) - 3.0)
+    assert O.compute_approx_kl(torch.tensor([-3.0]), torch.tensor([0.0]), None, "k3").item() == 10.0   # e^3 - 4 = 16.1
+    assert O.compute_approx_kl(lp, base, None, "k1").tolist() == lp.tolist()
+    assert O.compute_approx_kl(lp, base, None, "abs").tolist() == lp.abs().tolist()
+    assert O.compute_approx_kl(lp, base, None, "k2").tolist() == pytest.approx((0.5 * lp * lp).tolist())
+    with pytest.raises(ValueError):
+        O.compute_approx_kl(lp, base, None, "k4")
+    # masked positions are exactly zero even where the value is not finite
+    m = torch.tensor([1.0, 0.0, 2.0, 0.0, 1.0, 0.0], dtype=torch.float64)
+    lp_nan = lp.clone()
+    lp_nan[1] = float("nan")
+    out = O.compute_approx_kl(lp_nan, base, m, "k1")
+    assert out.tolist() == [0.0, 0.0, 2.0, 0.0, 25.0, 0.0]
+
+
+def test_approx_kl_estimators_are_unbiased_for_the_true_kl():
+    gen = torch.Generator().manual_seed(3)
+    # spreads small enough that no term reaches the clamps (|log ratio| < 20, value < 10)
+    logp = torch.log_softmax(0.5 * torch.randn(50, dtype=torch.float64, generator=gen), 0)
+    logq = torch.log_softmax(0.5 * torch.randn(50, dtype=torch.float64, generator=gen), 0)
+    assert float((logq - logp).abs().max()) < 3.0
+    true_kl = torch.nn.functional.kl_div(logq, logp, reduction="sum", log_target=True)   # KL(p || q)
+    p = logp.exp()
+    assert float((p * O.compute_approx_kl(logp, logq, None, "k1")).sum()) == pytest.approx(float(true_kl), rel=1e-12)
+    assert float((p * O.compute_approx_kl(logp, logq, None, "k3")).sum()) == pytest.approx(float(true_kl), rel=1e-12)
+    # second order: k3 and k2 agree for nearby distributions
+    near = logp + 1e-4 * torch.randn(50, dtype=torch.float64, generator=gen)
+    k2, k3 = O.compute_approx_kl(logp, near, None, "k2"), O.compute_approx_kl(logp, near, None, "k3")
+    torch.testing.assert_close(k3, k2, rtol=1e-3, atol=1e-14)
+
+
+def test_approx_kl_loss_reduction_brute_force():
+    gen = torch.Generator().manual_seed(4)
+    lp = torch.randn(3, 7, dtype=torch.float64, generator=gen)
+    base = torch.randn(3, 7, dtype=torch.float64, generator=gen)
+    mask = (torch.rand(3, 7, generator=gen) < 0.6).double()
+    mask[2] = 0
+    got = O.approx_kl_loss(lp, base, mask, "k2").item()
+    rows = []
+    for b in range(3):
+        vals = [0.5 * (lp[b, s] - base[b, s]).item() ** 2 for s in range(7) if mask[b, s] > 0]
+        rows.append(sum(vals) / max(len(vals), 1))
+    assert got == pytest.approx(sum(rows) / 3)
+    got = O.approx_kl_loss(lp, base, None, "abs").item()
+    assert got == pytest.approx(float((lp - base).abs().mean()))

@@ -397,6 +397,129 @@ def test_policy_loss_feeds_the_fused_backward(cuda_device):
     assert cos(dh.grad.float(), h64.grad) >= GRAD_COS and cos(dw.grad.float(), w64.grad) >= GRAD_COS
 
 
+@pytest.mark.parametrize("masked", [False, True])
+def test_cross_entropy_and_importance_sampling_losses_match_oracle(masked, cuda_device):
+    from skyrl_amd.policy_loss import cross_entropy_loss, importance_sampling_loss
+
+    gen = torch.Generator().manual_seed(15)
+    B, S = 5, 333
+    lp = torch.randn(B, S, generator=gen) * 0.5 - 2.0
+    old = lp + torch.randn(B, S, generator=gen) * 0.3
+    old[0, 0] = lp[0, 0] - 23.0                    # no clamp in this loss: a ratio of e^23
+    adv = torch.randn(B, S, generator=gen)
+    mask = (torch.rand(B, S, generator=gen) > 0.4).float() if masked else None
+    to = lambda t: None if t is None else t.to(cuda_device)  # noqa: E731
+    m64 = None if mask is None else mask.double()
+
+    ref_lp = lp.double().requires_grad_(True)
+    ref = O.cross_entropy_loss(ref_lp, m64)
+    ref.backward()
+    dlp = lp.to(cuda_device).requires_grad_(True)
+    loss, metrics = cross_entropy_loss(dlp, None, None, None, to(mask))
+    loss.backward()
+    assert metrics == {"clip_ratio": 0.0} and loss.item() == pytest.approx(ref.item(), rel=2e-6)
+    assert torch.equal(dlp.grad.cpu().double(), ref_lp.grad)
+
+    ref_lp = lp.double().requires_grad_(True)
+    ref, ref_ratio = O.importance_sampling_loss(ref_lp, old.double(), adv.double(), m64)
+    ref.backward()
+    dlp = lp.to(cuda_device).requires_grad_(True)
+    loss, metrics = importance_sampling_loss(dlp, to(old), to(adv), None, to(mask))
+    loss.backward()
+    assert abs(loss.item() - ref.item()) <= 5e-6 * max(abs(ref.item()), float((lp - old).exp().abs().max()))
+    assert metrics["importance_ratio"] == pytest.approx(ref_ratio.item(), rel=1e-5)
+    err = (dlp.grad.double().cpu() - ref_lp.grad).abs()
+    assert bool((err <= 1e-5 * ref_lp.grad.abs().clamp(min=1.0)).all())
+
+
+@pytest.mark.parametrize("estimator", ["k1", "abs", "k2", "k3"])
+@pytest.mark.parametrize("masked", [False, True])
+def test_approx_kl_matches_oracle(estimator, masked, cuda_device):
+    from skyrl_amd.policy_loss import approx_kl_loss, compute_approx_kl
+
+    gen = torch.Generator().manual_seed(16)
+    B, S = 7, 600
+    lp = torch.randn(B, S, generator=gen) * 0.5 - 2.0
+    base = lp + torch.randn(B, S, generator=gen) * 0.4
+    base[0, 0], base[0, 1] = lp[0, 0] + 25.0, lp[0, 1] - 25.0   # inner clamp on both sides
+    base[0, 2] = lp[0, 2] + 3.0                                 # outer clamp: e^3 - 4 > 10
+    base[0, 3] = lp[0, 3]                                       # zero difference (|.| has derivative 0 there)
+    mask = None
+    if masked:
+        mask = (torch.rand(B, S, generator=gen) > 0.4).float()
+        mask[1] = 0                                             # a row without loss tokens
+        mask[2, :10] = 0.5                                      # fractional weights
+        mask[0, :4] = 1
+    to = lambda t: None if t is None else t.to(cuda_device)  # noqa: E731
+    m64 = None if mask is None else mask.double()
+
+    # per-token values and their elementwise gradient
+    ref_lp = lp.double().requires_grad_(True)
+    ref = O.compute_approx_kl(ref_lp, base.double(), m64, estimator)
+    G = torch.randn(B, S, generator=gen)
+    (ref * G.double()).sum().backward()
+    dlp = lp.to(cuda_device).requires_grad_(True)
+    got = compute_approx_kl(dlp, to(base), to(mask), estimator)
+    (got * G.to(cuda_device)).sum().backward()
+    assert got.dtype == torch.float32 and got.shape == (B, S)
+    torch.testing.assert_close(got.detach().cpu().double(), ref.detach(), rtol=2e-5, atol=2e-6)
+    if masked:
+        assert bool((got.detach().cpu()[mask == 0] == 0).all())
+    torch.testing.assert_close(dlp.grad.cpu().double(), ref_lp.grad, rtol=2e-5, atol=2e-6)
+
+    # the trainer's reduction and its gradient
+    ref_lp = lp.double().requires_grad_(True)
+    ref = O.approx_kl_loss(ref_lp, base.double(), m64, estimator)
+    ref.backward()
+    dlp = lp.to(cuda_device).requires_grad_(True)
+    got = approx_kl_loss(dlp, to(base), to(mask), estimator)
+    (got * 1.0).backward()
+    assert got.dim() == 0 and got.item() == pytest.approx(ref.item(), rel=1e-5, abs=1e-7)
+    torch.testing.assert_close(dlp.grad.cpu().double(), ref_lp.grad, rtol=2e-5, atol=1e-9)
+
+
+def test_masked_mean_matches_oracle(cuda_device):
+    from skyrl_amd.policy_loss import masked_mean
+
+    gen = torch.Generator().manual_seed(17)
+    B, S = 9, 1031
+    v = torch.randn(B, S, generator=gen)
+    mask = (torch.rand(B, S, generator=gen) > 0.5).float()
+    mask[3] = 0
+    mask[4, :] = 0
+    mask[4, 5] = 0.25
+    for m in (None, mask):
+        for dim in (None, -1):
+            ref_v = v.double().requires_grad_(True)
+            ref = O.masked_mean(ref_v, None if m is None else m.double(), dim)
+            w = torch.randn(ref.shape, generator=gen).double()
+            (ref * w).sum().backward()
+            dv = v.to(cuda_device).requires_grad_(True)
+            got = masked_mean(dv, None if m is None else m.to(cuda_device), dim)
+            (got * w.float().to(cuda_device)).sum().backward()
+            assert got.shape == ref.shape
+            torch.testing.assert_close(got.detach().cpu().double(), ref.detach(), rtol=1e-5, atol=1e-6)
+            torch.testing.assert_close(dv.grad.cpu().double(), ref_v.grad, rtol=1e-5, atol=1e-9)
+    with pytest.raises(NotImplementedError):
+        masked_mean(v.to(cuda_device), None, 0)
+
+
+def test_loss_argument_errors(cuda_device):
+    lib = _lib.load()
+    x = torch.zeros(16, dtype=torch.float32, device=cuda_device)
+    p = x.data_ptr()
+    assert lib.skyrl_ppo_policy_loss(p, None, None, None, None, 16, 0.2, 0.2, 3.0, 2, p, None, None) == 0   # cross entropy
+    assert lib.skyrl_ppo_policy_loss(p, None, None, None, None, 16, 0.2, 0.2, 3.0, 3, p, None, None) == -1
+    assert lib.skyrl_ppo_policy_loss(p, p, p, None, None, 16, 0.2, 0.2, 3.0, 4, p, None, None) == -5
+    assert lib.skyrl_approx_kl(p, p, None, 4, 4, 3, None, None, p, 0, None, None) == -1
+    assert lib.skyrl_approx_kl(p, p, None, 4, 4, 4, None, p, p, 0, None, None) == -5
+    assert lib.skyrl_approx_kl(p, p, None, 4, 4, 3, None, p, p, 2, None, None) == -1
+    assert lib.skyrl_approx_kl(p, p, None, 0, 4, 3, None, p, p, 0, None, None) == -2
+    assert lib.skyrl_masked_mean(p, None, 4, 4, None, None, None) == -1
+    assert lib.skyrl_masked_mean(p, None, 4, 0, p, None, None) == -2
+    torch.cuda.synchronize()
+
+
 def test_mfma_probe_sums_exactly(cuda_device):
     """The measurement kernel runs the mainloop's MFMA sequence on caller-given operands: with small integers the sum of
     every wavefront's accumulators has a closed form, sum_k (sum_m A[m,k]) (sum_n B[n,k]) per pair of fragments."""
