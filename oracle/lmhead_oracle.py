@@ -30,6 +30,8 @@ What pins each function (all in ``tests/test_oracle.py``; none of them re-types 
     under x ~ p the expectation of k1 and of k3 is KL(p || q) exactly, summed by brute force over a small alphabet and
     compared with ``torch.nn.functional.kl_div`` -- and k3 ~ k2 for small differences; the trainer's reduction against a
     per-row Python loop.
+  * the FSDP forward tail: ``torch.distributions.Categorical`` for entropy and log-probability, and a Python loop that
+    scores action token j of row b against position S - num_actions + j - 1, with and without padding removed.
 No function is left "parity unpinned".
 """
 
@@ -493,3 +495,46 @@ def compute_approx_kl(
 def approx_kl_loss(log_probs, log_probs_base, loss_mask=None, kl_estimator_type: str = "k3") -> torch.Tensor:
     """The KL loss term as the trainer reduces it (skyrl/backends/skyrl_train/workers/worker.py:1071-1077)."""
     return masked_mean(compute_approx_kl(log_probs, log_probs_base, loss_mask, kl_estimator_type), loss_mask, dim=-1).mean()
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# The FSDP worker's forward tail on materialised logits
+# ----------------------------------------------------------------------------------------------------------------------
+def chunked_entropy_from_logits(logits: torch.Tensor, attention_mask: Optional[torch.Tensor] = None, chunk_size: int = 1024):
+    """skyrl/backends/skyrl_train/utils/torch_utils.py:58-111: per sequence chunk ``log_softmax``, ``-sum p log p``, times the
+    attention mask; result in the logits' dtype."""
+    out = torch.zeros(logits.shape[:2], dtype=logits.dtype)
+    for start in range(0, logits.shape[1], chunk_size):
+        chunk = torch.log_softmax(logits[:, start:start + chunk_size], dim=-1)
+        ent = -(chunk.exp() * chunk).sum(-1)
+        if attention_mask is not None:
+            ent = ent * attention_mask[:, start:start + chunk_size]
+        out[:, start:start + chunk_size] = ent
+    return out
+
+
+def hf_wrapper_tail(
+    logits: torch.Tensor,
+    sequences: torch.Tensor,
+    num_actions: int,
+    attention_mask: Optional[torch.Tensor],
+    temperature: float,
+    nnz_indices: Optional[torch.Tensor] = None,
+):
+    """skyrl/backends/skyrl_train/workers/model_wrapper.py:291, 333-393 on given logits ([B,S,V], or [1,nnz,V] with
+    ``nnz_indices`` = flat positions of the real tokens): logits / temperature, log-prob of the stream rolled left by one
+    (torch_utils.py:169-176: log_softmax + gather), entropy (masked by the attention mask only without packing), padding
+    put back as zeros, action slice ``[:, -num_actions-1:-1]``.  Returns ``(action_log_probs, entropy [B,S])``."""
+    batch, seqlen = sequences.shape
+    tokens = sequences if nnz_indices is None else sequences.reshape(-1)[nnz_indices][None]
+    rolled = torch.roll(tokens, shifts=-1, dims=1)
+    z = logits / temperature
+    log_probs = torch.log_softmax(z, dim=-1).gather(-1, rolled.unsqueeze(-1)).squeeze(-1)
+    entropy = chunked_entropy_from_logits(z, None if nnz_indices is not None else attention_mask)
+    if nnz_indices is not None:
+        def pad(v):
+            out = torch.zeros(batch * seqlen, dtype=v.dtype)
+            out[nnz_indices] = v.reshape(-1)
+            return out.view(batch, seqlen)
+        log_probs, entropy = pad(log_probs), pad(entropy)
+    return log_probs[:, -num_actions - 1:-1], entropy

@@ -1,0 +1,93 @@
+"""The tail of the FSDP worker's model forward on the fused LM head: hidden states in, action log-probabilities out.
+
+The reference's ``HFModelWrapper.forward`` (skyrl/backends/skyrl_train/workers/model_wrapper.py:241-398) runs the HF model to
+``logits_BSV`` -- a ``[B, S, V]`` tensor, 9-19 GiB in fp32 at the benchmark shapes -- and then divides by the temperature
+(:334), takes the log-probability of the next token (:337-341), optionally the per-token entropy (:358-386), and slices the
+action tokens (:393).  ``action_log_probs_from_hidden`` is that tail starting one step earlier, from the decoder's
+``last_hidden_state`` and ``lm_head.weight``, so the logits are never materialised; the entropy comes from the same pass
+and can carry its own gradient (``use_entropy_loss``, workers/worker.py:1058-1065).
+
+Integration: in ``HFModelWrapper.forward`` call the decoder without its head (``self.model.model(...)`` for HF causal
+LMs) and replace lines 333-393 by one call of this function with ``self.model.lm_head.weight``.
+"""
+
+from __future__ import annotations
+
+from typing import List, Optional, Tuple, Union
+
+import torch
+
+from .fused_linear_logprob_hip import linear_cross_entropy
+from .model_utils import _fused_lm_head_logprob_apply
+
+__all__ = ["action_log_probs_from_hidden"]
+
+
+def _pad_back(values: torch.Tensor, nnz_indices: torch.Tensor, batch: int, seqlen: int) -> torch.Tensor:
+    """``pad_input`` of the reference (:350-356): packed ``[nnz]`` values to ``[batch, seqlen]``, zeros at padding."""
+    out = torch.zeros(batch * seqlen, dtype=values.dtype, device=values.device)
+    return out.index_copy(0, nnz_indices.to(torch.long), values).view(batch, seqlen)
+
+
+def action_log_probs_from_hidden(
+    last_hidden_state: torch.Tensor,
+    lm_head_weight: torch.Tensor,
+    sequences: torch.Tensor,
+    num_actions: Union[int, List[int]],
+    attention_mask: Optional[torch.Tensor] = None,
+    temperature: float = 1.0,
+    return_output: bool = False,
+    compute_entropy: bool = False,
+    entropy_requires_grad: bool = True,
+    nnz_indices: Optional[torch.Tensor] = None,
+) -> Union[torch.Tensor, Tuple[torch.Tensor, dict]]:
+    """Action log-probabilities ``[B, num_actions]`` (and ``{"entropy": [B, S]}`` with ``return_output``).
+
+    ``last_hidden_state`` is ``[B, S, H]``, or ``[1, nnz, H]`` when the worker removed the micro-batch padding, in which
+    case ``nnz_indices`` are the flat positions of the real tokens (what ``unpad_input`` returned, :281-283) and
+    ``sequences`` / ``attention_mask`` keep their ``[B, S]`` shape.  ``sequences`` are the token ids the model saw;
+    targets are those ids rolled left by one over the stream the model ran on (:291), so with packing the last token of a
+    sequence is scored against the first token of the next one, exactly as in the reference.
+
+    Differences from the reference: the entropy is fp32 (the reference returns it in the logits' dtype, torch_utils.py:92),
+    and both outputs come from one pass over the vocabulary.
+    """
+    if isinstance(num_actions, list):
+        if len(num_actions) != 1:
+            raise NotImplementedError("per-row num_actions is not supported (the reference slices with a numpy array here, "
+                                      "which torch rejects as well)")
+        num_actions = num_actions[0]
+    batch, seqlen = sequences.shape
+    packed = nnz_indices is not None
+    if packed:
+        tokens = sequences.reshape(-1)[nnz_indices.to(torch.long)].unsqueeze(0)
+    else:
+        tokens = sequences
+    if last_hidden_state.shape[:2] != tokens.shape:
+        raise ValueError(f"last_hidden_state {tuple(last_hidden_state.shape)} does not match the token stream "
+                         f"{tuple(tokens.shape)}")
+    rolled = torch.roll(tokens, shifts=-1, dims=1)
+    V = lm_head_weight.shape[0]
+
+    output = {}
+    if compute_entropy:
+        hidden = last_hidden_state.to(lm_head_weight.dtype)
+        log_probs, entropy = linear_cross_entropy(hidden, lm_head_weight.contiguous(), rolled.contiguous(), float(temperature),
+                                                  "none", None)
+        log_probs, entropy = log_probs.reshape(tokens.shape), entropy.reshape(tokens.shape)
+        if not entropy_requires_grad:
+            entropy = entropy.detach()
+        if packed:
+            entropy = _pad_back(entropy.reshape(-1), nnz_indices, batch, seqlen)
+        elif attention_mask is not None:
+            if attention_mask.shape != entropy.shape:
+                raise ValueError(f"attention_mask shape {tuple(attention_mask.shape)} does not match {tuple(entropy.shape)}")
+            entropy = entropy * attention_mask
+        output["entropy"] = entropy
+    else:
+        log_probs = _fused_lm_head_logprob_apply("hip", last_hidden_state, lm_head_weight, rolled, 0, V, tokens.shape[1], None,
+                                                 not torch.is_grad_enabled(), float(temperature))
+    if packed:
+        log_probs = _pad_back(log_probs.reshape(-1), nnz_indices, batch, seqlen)
+    action_log_probs = log_probs[:, -num_actions - 1 : -1]
+    return (action_log_probs, output) if return_output else action_log_probs

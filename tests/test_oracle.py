@@ -545,3 +545,42 @@ def test_approx_kl_loss_reduction_brute_force():
     assert got == pytest.approx(sum(rows) / 3)
     got = O.approx_kl_loss(lp, base, None, "abs").item()
     assert got == pytest.approx(float((lp - base).abs().mean()))
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# the FSDP worker's forward tail
+# ----------------------------------------------------------------------------------------------------------------------
+def test_hf_wrapper_tail_brute_force():
+    gen = torch.Generator().manual_seed(21)
+    B, S, V, A, t = 3, 9, 13, 4, 0.7
+    logits = torch.randn(B, S, V, dtype=torch.float64, generator=gen)
+    seqs = torch.randint(0, V, (B, S), generator=gen)
+    am = torch.ones(B, S, dtype=torch.long)
+    am[0, :3] = 0                                          # left padding
+    am[2, :1] = 0
+    alp, ent = O.hf_wrapper_tail(logits, seqs, A, am, t)
+    dist = torch.distributions.Categorical(logits=logits / t)
+    assert alp.shape == (B, A) and ent.shape == (B, S)
+    for b in range(B):
+        for j in range(A):
+            pos = S - A + j                                 # the j-th action token; predicted from position pos - 1
+            one = torch.distributions.Categorical(logits=logits[b, pos - 1] / t)
+            assert alp[b, j].item() == pytest.approx(one.log_prob(seqs[b, pos]).item(), rel=1e-12)
+    torch.testing.assert_close(ent, dist.entropy() * am, rtol=1e-12, atol=1e-12)
+
+    # padding removed: the model ran on the real tokens only, as one stream
+    nnz = am.flatten().nonzero().flatten()
+    packed_logits = logits.reshape(B * S, V)[nnz][None]
+    alp_p, ent_p = O.hf_wrapper_tail(packed_logits, seqs, A, am, t, nnz_indices=nnz)
+    assert alp_p.shape == (B, A) and ent_p.shape == (B, S)
+    # inside a row the successor in the stream is the successor in the row, so all but each row's last action agree
+    torch.testing.assert_close(alp_p[:, :], alp[:, :], rtol=1e-12, atol=0)
+    torch.testing.assert_close(ent_p, dist.entropy() * am, rtol=1e-12, atol=1e-12)   # zeros come from the padding here
+    # the stream's roll wraps a row's last token onto the next row's first real token (the slice drops that position)
+    tokens = seqs.flatten()[nnz]
+    full, _ = O.hf_wrapper_tail(packed_logits, seqs, S - 1, am, t, nnz_indices=nnz)
+    row0_last = int(am[0].sum()) - 1                                      # stream position of row 0's last token
+    want = torch.log_softmax(packed_logits[0, row0_last] / t, -1)[tokens[row0_last + 1]]
+    lp_all = torch.log_softmax(packed_logits[0] / t, -1).gather(-1, torch.roll(tokens, -1)[:, None])[:, 0]
+    assert lp_all[row0_last].item() == pytest.approx(want.item(), rel=1e-12)
+    assert full.shape == (B, S - 1)

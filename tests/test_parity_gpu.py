@@ -799,6 +799,52 @@ def test_packed_argument_errors(cuda_device):
     torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("compute_entropy,entropy_grad", [(False, False), (True, False), (True, True)])
+def test_fsdp_forward_tail_from_hidden(cuda_device, packed, compute_entropy, entropy_grad):
+    """action_log_probs_from_hidden against the reference tail evaluated on materialised fp64 logits: values, shapes, the
+    zero padding, and the gradients into hidden and weight (log-probability loss, plus an entropy term when it has a grad)."""
+    from skyrl_amd.model_wrapper import action_log_probs_from_hidden
+    dev = cuda_device
+    gen = torch.Generator().manual_seed(61)
+    B, S, H, V, A, t = 3, 24, 128, 700, 7, 0.8
+    seqs = torch.randint(0, V, (B, S), generator=gen)
+    am = torch.ones(B, S, dtype=torch.long)
+    am[0, :5] = 0
+    am[1, :2] = 0
+    weight = (torch.randn(V, H, generator=gen) * 3 / H ** 0.5).to(torch.bfloat16)
+    nnz = am.flatten().nonzero().flatten() if packed else None
+    n_tok = int(am.sum()) if packed else B * S
+    hidden = torch.randn(1 if packed else B, n_tok if packed else S, H, generator=gen).to(torch.bfloat16)
+
+    h64, w64 = hidden.double().requires_grad_(True), weight.double().requires_grad_(True)
+    want_alp, want_ent = O.hf_wrapper_tail(h64 @ w64.t(), seqs, A, am.double(), t, nnz_indices=nnz)
+    G = torch.randn(B, A, generator=gen).double()
+    Q = torch.randn(B, S, generator=gen).double() * 0.1
+    loss = (want_alp * G).sum() + ((want_ent * Q).sum() if entropy_grad else 0.0)
+    loss.backward()
+
+    hd, wd = hidden.to(dev).requires_grad_(True), weight.to(dev).requires_grad_(True)
+    got = action_log_probs_from_hidden(hd, wd, seqs.to(dev), A, am.to(dev), t, return_output=True,
+                                       compute_entropy=compute_entropy, entropy_requires_grad=entropy_grad,
+                                       nnz_indices=None if nnz is None else nnz.to(dev))
+    alp, out = got
+    assert alp.shape == (B, A) and alp.dtype == torch.float32
+    torch.testing.assert_close(alp.detach().cpu().double(), want_alp.detach(), atol=LOGPROB_ATOL, rtol=0)
+    loss = (alp * G.float().to(dev)).sum()
+    if compute_entropy:
+        ent = out["entropy"]
+        assert ent.shape == (B, S) and ent.requires_grad == entropy_grad
+        torch.testing.assert_close(ent.detach().cpu().double(), want_ent.detach(), rtol=ENTROPY_RTOL, atol=1e-6)
+        assert bool((ent.detach().cpu()[am == 0] == 0).all())
+        if entropy_grad:
+            loss = loss + (ent * Q.float().to(dev)).sum()
+    else:
+        assert out == {}
+    loss.backward()
+    assert cos(hd.grad, h64.grad) >= GRAD_COS and cos(wd.grad, w64.grad) >= GRAD_COS
+
+
 def test_opcheck_registration(cuda_device):
     T, H, V = 64, 64, 300
     hidden, weight, labels, _, _ = _rand(T, H, V, seed=2)
