@@ -58,7 +58,7 @@ size_t skyrl_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V);
 
 /* Scratch needed by skyrl_lmhead_bwd for a given vocab chunk width (0 = library default):
  * weight^T bf16 [H, V'+64], hidden^T bf16 [H, T'+64], fp32 dHidden partial sums (T' x H' values, kept in the
- * kernel's accumulator order between chunks) and two bf16 dz panels [T', chunk+64] / [chunk, T'+64]
+ * kernel's accumulator order between chunks) and one bf16 dz panel [T', chunk+64]
  * (T', V', H' = T, V, H rounded up to 256; the 64 extra elements keep row pitches off powers of two).
  * Nothing in it scales with T * V.
  * (Stands in for the `d_logits [T, 9504]` scratch of the reference's default backward,

@@ -21,6 +21,8 @@
 //
 // Data path: 16-byte global_load_lds (global -> LDS without a VGPR round trip) into a ring of five 32 KiB operand
 // slots (2.5 k-tiles, all of the CU's 160 KiB); ds_read_b128 fragments one 32-k step ahead; MFMA, fp32 accumulation.
+// The B operand may also be given K-major (see Operand); its fragments then come through ds_read_b64_tr_b16, the
+// transposing LDS read, so that a producer's output can be contracted along either of its axes without a second copy.
 //
 // LDS operand slot: 256 rows x 64 k bf16 = 256 x 128 B.  The 16-byte chunk (row, kc) lives at byte
 // row*128 + ((kc ^ swz(row)) << 4), see swz() below.
@@ -42,6 +44,7 @@ namespace lmhead {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) short i16x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
@@ -72,12 +75,29 @@ __device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
 
 typedef f32x4 acc_t[TM][TN];
 
+// The n-th (n = 0, 1, ...) MFMA gap of a 64-MFMA step at or behind x that is odd (the even ones carry fragment reads)
+// and is not a copy gap (x % 8 == 5).
+constexpr int free_gap(int x, int n) {
+  for (int g = x | 1;; g += 2)
+    if (g % 8 != 5 && n-- == 0) return g;
+}
+
 struct Operand {
   const uint16_t* ptr;  // bf16 bits, row-major, K contiguous
   int ld;               // elements between rows (multiple of 8)
   int row0;             // first row of this tile
   int rows;             // total valid rows; rows past the end are clamped (their results are masked later)
 };
+// A B operand may instead be "K-major": the same matrix stored transposed, ptr[k * ld + n], so that a 16-byte chunk
+// holds eight consecutive n of one k (what a producer writes when n is its contiguous axis).  Then row0 is the first
+// column n of the tile; the caller guarantees that columns row0 .. row0+255 and every k row of the loop exist.
+//
+// K-major slot layout: 64 k-rows x 256 n = 32 blocks of 1 KiB, block b = rows 2b and 2b+1 (what one wave-wide copy
+// fills).  A block is 16 windows of 64 bytes, a window = 32 bytes (16 n) of the even row, then of the odd row.  The 16 n
+// of pair q sit in window q ^ sigma(b), sigma(b) = (b & 1) + 2 * ((b >> 2) & 1): the transposing fragment read below
+// takes, per 16 lanes, four consecutive rows at one pair, and with this key the eight row pieces of lanes 0-31 (and of
+// lanes 32-63) fall into the eight different 32-byte bank groups.
+__device__ __forceinline__ int kmajor_sigma(int block) { return (block & 1) + 2 * ((block >> 2) & 1); }
 
 // Wait until at most N of this lane's global->LDS copies are still in flight and all of its LDS reads have returned,
 // then meet the rest of the workgroup.  The "memory" clobber keeps the compiler from moving LDS accesses across it.
@@ -125,6 +145,7 @@ struct CopyPlan {
   uint32_t a_src[COPIES_PER_OPERAND], b_src[COPIES_PER_OPERAND];
 };
 
+template <bool BKM>
 __device__ __forceinline__ void make_plan(CopyPlan& p, const Operand& a, const Operand& b, int k_begin) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -133,14 +154,28 @@ __device__ __forceinline__ void make_plan(CopyPlan& p, const Operand& a, const O
     const int c = (j * NWAVES + wave) * 64 + lane;  // chunk index inside the slot
     const int row = c >> 3;
     const int kc = (c & 7) ^ swz(row);
-    int ga = a.row0 + row, gb = b.row0 + row;
+    int ga = a.row0 + row;
     ga = ga < a.rows ? ga : a.rows - 1;
-    gb = gb < b.rows ? gb : b.rows - 1;
     p.a_src[j] = (uint32_t)ga * (uint32_t)a.ld * 2u + (uint32_t)(kc * 16);
-    p.b_src[j] = (uint32_t)gb * (uint32_t)b.ld * 2u + (uint32_t)(kc * 16);
+    if (BKM) {
+      const int block = j * NWAVES + wave;             // rows 2 * block, 2 * block + 1 of the k-tile
+      const int q = (lane >> 2) ^ kmajor_sigma(block);  // the pair whose home is this lane's window
+      const int krow = 2 * block + ((lane >> 1) & 1);
+      p.b_src[j] = (uint32_t)krow * (uint32_t)b.ld * 2u + (uint32_t)((b.row0 + q * 16 + (lane & 1) * 8) * 2);
+    } else {
+      int gb = b.row0 + row;
+      gb = gb < b.rows ? gb : b.rows - 1;
+      p.b_src[j] = (uint32_t)gb * (uint32_t)b.ld * 2u + (uint32_t)(kc * 16);
+    }
   }
   p.a_bytes = (const char*)a.ptr + (size_t)k_begin * 2;
-  p.b_bytes = (const char*)b.ptr + (size_t)k_begin * 2;
+  p.b_bytes = (const char*)b.ptr + (BKM ? (size_t)k_begin * (size_t)b.ld * 2 : (size_t)k_begin * 2);
+}
+
+// Bytes between consecutive k-tiles of the B operand.
+template <bool BKM>
+__device__ __forceinline__ uint32_t b_tile_stride(const Operand& b) {
+  return BKM ? (uint32_t)BK * (uint32_t)b.ld * 2u : (uint32_t)(BK * 2);
 }
 
 // Copies j0 .. j0+n-1 (of COPIES_PER_OPERAND) of one k-tile of one operand into a ring slot.  `g` is the wave-uniform
@@ -170,15 +205,16 @@ __device__ __forceinline__ uint32_t wave_copy_base(char* lds) {
 // Put the first k-tiles of an output tile in flight: A(0) B(0) A(1) B(1) into slots 0..3.  All five slots must be free
 // (true at kernel start and after mainloop() returns).  Called before the epilogue of the previous output tile so that
 // the copy path keeps working while the VALU does the epilogue.
+template <bool BKM = false>
 __device__ __forceinline__ void prefetch_first_tiles(const Operand& a, const Operand& b, int k_begin, int nk, char* lds) {
   CopyPlan p;  // rebuilt by mainloop(): keeping it in registers across an epilogue costs more than recomputing it
-  make_plan(p, a, b, k_begin);
+  make_plan<BKM>(p, a, b, k_begin);
   const uint32_t w0 = wave_copy_base(lds);
   copy_part(p.a_bytes, p.a_src, w0 + 0 * OPERAND_BYTES, 0, COPIES_PER_OPERAND);
   copy_part(p.b_bytes, p.b_src, w0 + 1 * OPERAND_BYTES, 0, COPIES_PER_OPERAND);
   if (nk > 1) {
     copy_part(p.a_bytes + BK * 2, p.a_src, w0 + 2 * OPERAND_BYTES, 0, COPIES_PER_OPERAND);
-    copy_part(p.b_bytes + BK * 2, p.b_src, w0 + 3 * OPERAND_BYTES, 0, COPIES_PER_OPERAND);
+    copy_part(p.b_bytes + b_tile_stride<BKM>(b), p.b_src, w0 + 3 * OPERAND_BYTES, 0, COPIES_PER_OPERAND);
   }
 }
 
@@ -197,9 +233,11 @@ __device__ __forceinline__ void prefetch_first_tiles(const Operand& a, const Ope
 //                register sets), one copy behind every eighth MFMA, in a gap without a read; sched_barrier pins that order.
 // MFMA order inside a step is a serpentine over the 8 x 8 accumulators (the B fragment is kept where the A fragment
 // changes): fewer operand toggles, measurably less power.
+template <bool BKM = false>
 __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int k_begin, int nk, char* lds, acc_t& acc) {
   CopyPlan p;
-  make_plan(p, a, b, k_begin);
+  make_plan<BKM>(p, a, b, k_begin);
+  const uint32_t b_stride = b_tile_stride<BKM>(b);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
@@ -213,24 +251,77 @@ __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int
   const int a_off0 = (wm * WM + lrow) * ROW_BYTES + xsw + rel, a_off1 = (wm * WM + lrow) * ROW_BYTES + (xsw ^ 64) + rel;
   const int b_off0 = (wn * WN + lrow) * ROW_BYTES + xsw + rel, b_off1 = (wn * WN + lrow) * ROW_BYTES + (xsw ^ 64) + rel;
   typedef const __attribute__((address_space(3))) bf16x8* frag_ptr;
+  typedef __attribute__((address_space(3))) i16x4* half_ptr;
 
-  bf16x8 af[2][TM], bfr[2][TN];
-  // Fragment x of a 32-k step: x < TM is the A fragment of MFMA row x, otherwise the B fragment of MFMA column x - TM.
-  auto read_one = [&](uint32_t pa, uint32_t pb, int set, int x) {  // pa, pb: LDS addresses of fragment 0
-    if (x < TM) af[set][x] = *(frag_ptr)(uintptr_t)(pa + x * MT * ROW_BYTES);
-    else bfr[set][x - TM] = *(frag_ptr)(uintptr_t)(pb + (x - TM) * MT * ROW_BYTES);
+  // K-major B: a fragment (16 n x 32 k -> per lane one n, eight k) is two ds_read_b64_tr_b16, each of which takes four
+  // consecutive k-rows at one pair of 16 n from sixteen lanes and hands lane l column l of each.  Lane l = (kq, s)
+  // supplies the address of row kq*8 + half*4 + (s >> 2), n quarter s & 3.  The window key of those rows,
+  // sigma = ((s >> 3) & 1) + 2 * (kq & 1), is a per-lane constant, so pair j of the wave is found at one of four
+  // per-lane offsets (j & 3) ^ sigma plus immediates for j >> 2, the half and the k-step.
+  constexpr int NB = BKM ? 4 : 1;  // B fragment address registers per k-step
+  int kb_off[4];
+  {
+    const int kq = lane >> 4, s = lane & 15, r = s >> 2;
+    const int sigma = ((r >> 1) & 1) + 2 * (kq & 1);
+    const int base = (kq * 4 + (r >> 1)) * 1024 + wn * (WN / 16) * 64 + (r & 1) * 32 + (s & 3) * 8 + rel;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) kb_off[e] = base + ((e ^ sigma) * 64);
+  }
+  constexpr int kKStepBytes = 16 * 1024;  // 32 k-rows of a K-major slot
+  constexpr int kHalfBytes = 2 * 1024;    // 4 k-rows
+
+  // Fragment registers.  A K-major B fragment arrives as two 64-bit halves (k 0-3 and k 4-7 of the lane's eight).
+  bf16x8 af[2][TM], bfr[2][BKM ? 1 : TN];
+  i16x4 bh[2][BKM ? TN : 1][2];
+  auto b_frag = [&](int set, int j) -> bf16x8 {
+    if constexpr (BKM) {
+      typedef __attribute__((ext_vector_type(8))) short i16x8;
+      const i16x8 v = __builtin_shufflevector(bh[set][j][0], bh[set][j][1], 0, 1, 2, 3, 4, 5, 6, 7);
+      return __builtin_bit_cast(bf16x8, v);
+    } else {
+      return bfr[set][j];
+    }
   };
+  // Read instruction y of a 32-k step: y < TM is the A fragment of MFMA row y; then the B fragments, one instruction each
+  // (K-contiguous B) or two (K-major B).  pa: LDS address of A fragment 0; pb: NB LDS addresses for B.
+  constexpr int READS_PER_STEP = TM + (BKM ? 2 * TN : TN);
+  auto read_one = [&](uint32_t pa, const uint32_t (&pb)[NB], int set, int y) {
+    if (y < TM) {
+      af[set][y] = *(frag_ptr)(uintptr_t)(pa + y * MT * ROW_BYTES);
+    } else if constexpr (BKM) {
+      const int j = (y - TM) >> 1, half = (y - TM) & 1;
+      const uint32_t addr = pb[j & 3] + (j >> 2) * 256 + half * kHalfBytes + (set == 1 ? kKStepBytes : 0);
+      bh[set][j][half] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((half_ptr)(uintptr_t)addr);
+    } else {
+      bfr[set][y - TM] = *(frag_ptr)(uintptr_t)(pb[0] + (y - TM) * MT * ROW_BYTES);
+    }
+  };
+  // Lane offsets of the B fragment addresses for k-step 0 / k-step 1 of a slot (the k-step of a K-major slot is an
+  // immediate in read_one, so both are the same four offsets there).
+  int boff0[NB], boff1[NB];
+#pragma unroll
+  for (int e = 0; e < NB; ++e) {
+    boff0[e] = BKM ? kb_off[e] : b_off0;
+    boff1[e] = BKM ? kb_off[e] : b_off1;
+  }
 
   if (nk > 1) wait_copies_and_barrier<2 * COPIES_PER_OPERAND>(); else wait_copies_and_barrier<0>();  // tile 0 has landed
+  {
+    uint32_t pb[NB];
 #pragma unroll
-  for (int x = 0; x < TM + TN; ++x) read_one(w0 + a_off0, w0 + OPERAND_BYTES + b_off0, 0, x);
+    for (int e = 0; e < NB; ++e) pb[e] = w0 + OPERAND_BYTES + boff0[e];
+#pragma unroll
+    for (int y = 0; y < READS_PER_STEP; ++y) read_one(w0 + a_off0, pb, 0, y);
+  }
 
   // Ring state, as byte offsets of the slots in the order A(kt), B(kt), A(kt+1), B(kt+1), free.  Advancing one k-tile
   // rotates the five values by two places, so no arithmetic is needed; the fragment addresses of the next k-tile are
   // formed in the shadow of MFMAs in the middle of a step, not at the top of the loop where nothing would hide them.
   uint32_t o0 = w0, o1 = w0 + OPERAND_BYTES, o2 = w0 + 2 * OPERAND_BYTES, o3 = w0 + 3 * OPERAND_BYTES, o4 = w0 + 4 * OPERAND_BYTES;
-  uint32_t ra1 = o0 + a_off1, rb1 = o1 + b_off1;  // step-0 reads: k-step 1 of this k-tile (LDS addresses)
-  uint32_t ra0 = o2 + a_off0, rb0 = o3 + b_off0;  // step-1 reads: k-step 0 of the next k-tile
+  uint32_t ra1 = o0 + a_off1, ra0 = o2 + a_off0;  // step-0 reads: k-step 1 of this k-tile; step-1 reads: k-step 0 of the next
+  uint32_t rb1[NB], rb0[NB];
+#pragma unroll
+  for (int e = 0; e < NB; ++e) rb1[e] = o1 + boff1[e], rb0[e] = o3 + boff0[e];
   // An add the compiler cannot move: it would otherwise collect these at the top of the loop body.
   auto pinned_add = [](uint32_t slot_off, int lane_off) {
     uint32_t r;
@@ -241,11 +332,16 @@ __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int
   // right behind the last copy that uses them -- the empty asm keeps the compiler from gathering the increments at the
   // end of the loop body, where every instruction is a bubble.
   const char* ga = p.a_bytes + 2 * (BK * 2);
-  const char* gb = p.b_bytes + 2 * (BK * 2);
+  const char* gb = p.b_bytes + 2 * (size_t)b_stride;
   // Three copies of the tile step (steady state, second-to-last, last) instead of conditions inside one loop body: a
   // branch that joins a path with outstanding LDS reads makes the compiler wait for all of them.
   auto tile_step = [&](auto has_next, auto load2) {
-    uint32_t nra1 = ra1, nrb1 = rb1, nra0 = ra0, nrb0 = rb0;
+    // The fragment addresses of the next k-tile are formed in place, one add per MFMA shadow, in gaps behind the last
+    // read of the step (which still uses the old value) that carry neither a read nor a copy.
+    constexpr int kAddX0 = BKM ? 2 * READS_PER_STEP - 1 : 41;
+    constexpr int kGapA = free_gap(kAddX0, 0);
+    constexpr int kGapB[4] = {free_gap(kAddX0, 1), free_gap(kAddX0, 2), free_gap(kAddX0, 3), free_gap(kAddX0, 4)};
+    static_assert(kGapB[3] < TM * TN, "address adds must fit the step");
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       if (ks == 1 && has_next) {
@@ -255,9 +351,9 @@ __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int
 #pragma unroll
       for (int x = 0; x < TM * TN; ++x) {
         const int i = x / TN, j = (i & 1) ? TN - 1 - x % TN : x % TN;
-        mfma_16x16x32(acc[i][j], af[ks][i], bfr[ks][j]);
+        mfma_16x16x32(acc[i][j], af[ks][i], b_frag(ks, j));
         __builtin_amdgcn_sched_barrier(0);
-        if (x % 2 == 0 && x < 2 * (TM + TN)) {
+        if (x % 2 == 0 && x < 2 * READS_PER_STEP) {
           if (ks == 0) read_one(ra1, rb1, 1, x / 2);
           else if (has_next) read_one(ra0, rb0, 0, x / 2);
         }
@@ -270,20 +366,22 @@ __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int
             ga += BK * 2;
             asm volatile("" : "+s"(ga));
           } else {
-            gb += BK * 2;
+            gb += b_stride;
             asm volatile("" : "+s"(gb));
           }
         }
         if (has_next) {  // next k-tile's fragment addresses, one per MFMA shadow, after this step's reads are issued
-          if (ks == 0 && x == 41) nra1 = pinned_add(o2, a_off1);
-          if (ks == 0 && x == 43) nrb1 = pinned_add(o3, b_off1);
-          if (ks == 1 && x == 41) nra0 = pinned_add(o4, a_off0);
-          if (ks == 1 && x == 43) nrb0 = pinned_add(o0, b_off0);
+          if (ks == 0 && x == kGapA) ra1 = pinned_add(o2, a_off1);
+          if (ks == 1 && x == kGapA) ra0 = pinned_add(o4, a_off0);
+#pragma unroll
+          for (int e = 0; e < NB; ++e) {
+            if (ks == 0 && x == kGapB[e]) rb1[e] = pinned_add(o3, boff1[e]);
+            if (ks == 1 && x == kGapB[e]) rb0[e] = pinned_add(o0, boff0[e]);
+          }
         }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    ra1 = nra1, rb1 = nrb1, ra0 = nra0, rb0 = nrb0;
     const uint32_t t0 = o0, t1 = o1;
     o0 = o2, o1 = o3, o2 = o4, o3 = t0, o4 = t1;
   };

@@ -240,15 +240,13 @@ struct DzArgs {
   int vc0, tiles_m, tiles_n;  // first vocab row of the chunk; tiles of the chunk panel along vocab and tokens
   uint16_t* D;                // [tiles_n * 256, ldd]  dz, token-major
   int ldd;
-  uint16_t* DT;               // [tiles_m * 256, lddt] dz, vocab-major
-  int lddt;
 };
 
 template <bool ENTGRAD>
 __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
   const uint16_t* __restrict__ W = z.W;
   const uint16_t* __restrict__ Hd = z.Hd;
-  const int ldw = z.ldw, ldh = z.ldh, T = z.T, H = z.H, V = z.V, vc0 = z.vc0, ldd = z.ldd, lddt = z.lddt;
+  const int ldw = z.ldw, ldh = z.ldh, T = z.T, H = z.H, V = z.V, vc0 = z.vc0, ldd = z.ldd;
   const float rcp_temp = z.rcp_temp;
   const int64_t* __restrict__ labels = z.labels;
   const float* __restrict__ row_lse = z.row_lse;
@@ -256,7 +254,6 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
   const float* __restrict__ dlogprobs = z.dlogprobs;
   const float* __restrict__ dentropy = z.dentropy;
   uint16_t* __restrict__ D = z.D;
-  uint16_t* __restrict__ DT = z.DT;
   int tm, tn;
   tile_coords(id, z.tiles_m, z.tiles_n, kGroupM, tm, tn);
 
@@ -295,82 +292,57 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
   prefetch_first_tiles(a, b, 0, H / BK, lds);
   mainloop(a, b, 0, H / BK, lds, acc);
 
-  // The wave's 128 x 128 dz block leaves through LDS so that both panels are written with 16-byte stores.  A lane holds
-  // four consecutive vocab rows of one token, which is an 8-byte piece of a D row; for D^T the four lanes of a quad
-  // (four consecutive tokens) first transpose their 4 x 4 block in registers (DPP + byte permute).  The block goes in
-  // two halves of 64 tokens; mainloop() left LDS free and every wave uses a private region, so no barrier is needed
-  // (LDS operations of one wave execute in order).
-  constexpr int kTokRow = WM * 2 + 16;            // D staging: 64 token rows x (128 vocab x 2 B + pad)
-  constexpr int kVocRow = 64 * 2 + 16;            // D^T staging: 128 vocab rows x (64 tokens x 2 B + pad)
-  constexpr int kStageD = 64 * kTokRow, kStageDT = WM * kVocRow;
-  static_assert(NWAVES * (kStageD + kStageDT) <= LDS_BYTES, "dz staging does not fit LDS");
-  char* stage_d = lds + wave * (kStageD + kStageDT);
-  char* stage_dt = stage_d + kStageD;
-  const int q4 = lane & 3;
-  const uint32_t sel1 = (q4 & 1) ? 0x03020706u : 0x05040100u;
-  const bool upper = (q4 & 2) != 0;
-  constexpr int JH = TN / 2;  // column tiles per half
+  // The wave's 128 x 128 dz block leaves through LDS so that the panel is written with 16-byte stores: a lane holds four
+  // consecutive vocab rows of one token, an 8-byte piece of a D row.  mainloop() left LDS free and every wave uses a
+  // private region, so no barrier is needed (LDS operations of one wave execute in order).  The stores are marked
+  // non-temporal: the panel is a gigabyte that is read back only by the next launch, and letting it displace the operand
+  // panels from L2 costs the mainloops of the neighbouring tiles more than the stores themselves.
+  constexpr int kTokRow = WM * 2 + 16;  // staging: 128 token rows x (128 vocab x 2 B + pad)
+  constexpr int kStage = WN * kTokRow;
+  static_assert(NWAVES * kStage <= LDS_BYTES, "dz staging does not fit LDS");
+  char* stage = lds + wave * kStage;
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 #pragma unroll
-  for (int half = 0; half < 2; ++half) {
+  for (int j = 0; j < TN; ++j) {
+    const float gs = gs_[j], c0 = c0_[j], c1 = c1_[j], lse2 = lse2_[j];
+    const int yrel = yrel_[j];
+    const bool any_label = __any(yrel >= 0);  // some token of this column tile has its label inside the wave's rows
 #pragma unroll
-    for (int jj = 0; jj < JH; ++jj) {
-      const int j = half * JH + jj;
-      const float gs = gs_[j], c0 = c0_[j], c1 = c1_[j], lse2 = lse2_[j];
-      const int yrel = yrel_[j];
-      const bool any_label = __any(yrel >= 0);  // some token of this column tile has its label inside the wave's rows
+    for (int i = 0; i < TM; ++i) {
+      float d[4];
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        float d[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float x = acc[i][j][r];
-          const float p = __builtin_amdgcn_exp2f(fmaf(x, scale2, -lse2));
-          d[r] = ENTGRAD ? p * fmaf(c1, x, c0) : p * c0;
-        }
-        const int vl = i * MT + kq * 4;  // vocab row inside the wave block; this lane holds vl .. vl+3
-        if (any_label) {
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (yrel == vl + r) d[r] += gs;
-        }
-        if (!full) {
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (vbase + vl + r >= V) d[r] = 0.f;
-        }
-        f32x4 v4 = {d[0], d[1], d[2], d[3]};
-        const bf16x4 b4 = __builtin_convertvector(v4, bf16x4);
-        uint32_t w0 = ((const uint32_t*)&b4)[0], w1 = ((const uint32_t*)&b4)[1];
-        *(uint2*)(stage_d + (jj * MT + lrow) * kTokRow + vl * 2) = make_uint2(w0, w1);
-        // 4 x 4 transpose inside the quad: afterwards lane q4 holds vocab row vl + q4 for the quad's four tokens
-        const uint32_t p0 = (uint32_t)__builtin_amdgcn_mov_dpp((int)w0, 0xB1, 0xF, 0xF, true);  // lane ^ 1
-        const uint32_t p1 = (uint32_t)__builtin_amdgcn_mov_dpp((int)w1, 0xB1, 0xF, 0xF, true);
-        w0 = __builtin_amdgcn_perm(p0, w0, sel1);
-        w1 = __builtin_amdgcn_perm(p1, w1, sel1);
-        const uint32_t send = upper ? w0 : w1;
-        const uint32_t recv = (uint32_t)__builtin_amdgcn_mov_dpp((int)send, 0x4E, 0xF, 0xF, true);  // lane ^ 2
-        const uint32_t t0 = upper ? recv : w0, t1 = upper ? w1 : recv;
-        *(uint2*)(stage_dt + (vl + q4) * kVocRow + (jj * MT + (lrow & ~3)) * 2) = make_uint2(t0, t1);
+      for (int r = 0; r < 4; ++r) {
+        const float x = acc[i][j][r];
+        const float p = __builtin_amdgcn_exp2f(fmaf(x, scale2, -lse2));
+        d[r] = ENTGRAD ? p * fmaf(c1, x, c0) : p * c0;
       }
-    }
-    // 64 tokens x 128 vocab staged both ways: 1024 16-byte pieces each, 16 per lane.
+      const int vl = i * MT + kq * 4;  // vocab row inside the wave block; this lane holds vl .. vl+3
+      if (any_label) {
 #pragma unroll
-    for (int it = 0; it < 16; ++it) {
-      const int idx = it * 64 + lane;
-      {
-        const int n = idx >> 4, c = idx & 15;  // token row, 8-vocab piece
-        const uint4 v = *(const uint4*)(stage_d + n * kTokRow + c * 16);
-        *(uint4*)(D + (size_t)(tbase + half * 64 + n) * (size_t)ldd + vloc_base + c * 8) = v;
+        for (int r = 0; r < 4; ++r)
+          if (yrel == vl + r) d[r] += gs;
       }
-      {
-        const int vr = idx >> 3, c = idx & 7;  // vocab row, 8-token piece
-        const uint4 v = *(const uint4*)(stage_dt + vr * kVocRow + c * 16);
-        *(uint4*)(DT + (size_t)(vloc_base + vr) * (size_t)lddt + tbase + half * 64 + c * 8) = v;
+      if (!full) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (vbase + vl + r >= V) d[r] = 0.f;
       }
+      f32x4 v4 = {d[0], d[1], d[2], d[3]};
+      const bf16x4 b4 = __builtin_convertvector(v4, bf16x4);
+      *(uint2*)(stage + (j * MT + lrow) * kTokRow + vl * 2) = *(const uint2*)&b4;
     }
   }
+  // 128 tokens x 128 vocab staged: 2048 16-byte pieces, 32 per lane; 16 lanes cover one token row (256 bytes).
+#pragma unroll
+  for (int it = 0; it < 32; ++it) {
+    const int idx = it * 64 + lane;
+    const int n = idx >> 4, c = idx & 15;  // token row, 8-vocab piece
+    const u32x4 v = *(const u32x4*)(stage + n * kTokRow + c * 16);
+    __builtin_nontemporal_store(v, (u32x4*)(D + (size_t)(tbase + n) * (size_t)ldd + vloc_base + c * 8));
+  }
 }
+
 
 // ------------------------------------------------------------------------------------------------------------
 // Plain NT GEMM with an fp32 / bf16 store epilogue:  C[N,M] (+)= B[N,K] . A[M,K]^T, i.e. C[n][m] = sum_k A[m][k] B[n][k]:
@@ -399,10 +371,10 @@ struct GemmArgs {
   float* Pout;
 };
 
-__device__ __forceinline__ void gemm_tile(const GemmArgs& p0, const GemmArgs& p1, int tiles0, int id, char* lds) {
-  const bool second = id >= tiles0;
-  const GemmArgs& p = second ? p1 : p0;
-  const int bid = second ? id - tiles0 : id;
+// BKM: the B operand is K-major.  The two variants are separate instantiations of the whole tile (mainloop and
+// epilogue) so that their accumulators never meet at a join, where the register allocator would shuffle all 256 of them.
+template <bool BKM>
+__device__ __forceinline__ void gemm_tile(const GemmArgs& p, int bid, char* lds) {
   const int M = p.M, N = p.N;
   const int tiles_m = (M + BM - 1) / BM;
   const int tiles_n = (N + BN - 1) / BN;
@@ -412,8 +384,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p0, const GemmArgs& p1
   Operand b{p.B, p.ldb, tn * BN, p.b_rows};
   acc_t acc;
   zero_acc(acc);
-  prefetch_first_tiles(a, b, 0, p.nk, lds);
-  mainloop(a, b, 0, p.nk, lds, acc);
+  prefetch_first_tiles<BKM>(a, b, 0, p.nk, lds);
+  mainloop<BKM>(a, b, 0, p.nk, lds, acc);
 
   const float* __restrict__ Cin = p.Cin;
   float* __restrict__ Cf = p.Cf;
@@ -464,7 +436,8 @@ __global__ __launch_bounds__(NTHREADS) void lmhead_bwd_chunk(const DzArgs z, con
                                                              int gemm_tiles) {
   __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
   const int id = blockIdx.x;
-  if (id < gemm_tiles) gemm_tile(p0, p1, tiles0, id, lds);
+  if (id < tiles0) gemm_tile<false>(p0, id, lds);               // dHidden: B = dz panel rows, K (vocab) contiguous
+  else if (id < gemm_tiles) gemm_tile<true>(p1, id - tiles0, lds);  // dW: B = the same panel read K-major (K = tokens)
   else dz_tile<ENTGRAD>(z, id - gemm_tiles, lds);
 }
 
@@ -618,7 +591,7 @@ int64_t default_vocab_chunk(int64_t T, int64_t V) {
 }
 
 struct BwdWorkspace {
-  uint16_t *Wt, *Ht, *D, *DT;
+  uint16_t *Wt, *Ht, *D;
   float* dHacc;
   size_t bytes;
 };
@@ -631,7 +604,6 @@ BwdWorkspace carve_bwd(void* ws, int64_t T, int64_t H, int64_t V, int64_t vc) {
   w.Ht = c.take<uint16_t>((size_t)H * (Tpad + kLdPad));
   w.dHacc = c.take<float>((size_t)Tpad * round_up(H, 256));  // accumulator order, whole tiles
   w.D = c.take<uint16_t>((size_t)Tpad * (vc + kLdPad));
-  w.DT = c.take<uint16_t>((size_t)vc * (Tpad + kLdPad));
   w.bytes = (size_t)round_up((int64_t)c.off, 256);
   return w;
 }
@@ -752,9 +724,9 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
   const int64_t Tpad = round_up(T, 256), Vpad = round_up(V, 256);
   int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(T, V);
   if (vc > Vpad) vc = Vpad;
-  // 32-bit byte offsets inside the scratch matrices as well (weight^T, hidden^T, the two dz panels)
+  // 32-bit byte offsets inside the scratch matrices as well (weight^T, hidden^T, the dz panel)
   if (H * (Vpad + kLdPad) * 2 >= ((int64_t)1 << 32) || H * (Tpad + kLdPad) * 2 >= ((int64_t)1 << 32) ||
-      Tpad * (vc + kLdPad) * 2 >= ((int64_t)1 << 32) || vc * (Tpad + kLdPad) * 2 >= ((int64_t)1 << 32))
+      Tpad * (vc + kLdPad) * 2 >= ((int64_t)1 << 32))
     return SKYRL_LMHEAD_ERR_SHAPE;
   if (!workspace || workspace_bytes < skyrl_lmhead_bwd_workspace_bytes(T, H, V, vc)) return SKYRL_LMHEAD_ERR_WORKSPACE;
   if ((uintptr_t)workspace & 255u) return SKYRL_LMHEAD_ERR_ALIGN;
@@ -784,26 +756,25 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
   auto dz_args = [&](int64_t ci) {
     const int64_t vc0 = ci * vc, vcw = chunk_width(ci);
     return DzArgs{Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)T, (int)H, (int)V, rcp_temperature, labels, row_lse, row_pz,
-                  dlogprobs, dentropy, (int)vc0, (int)(vcw / 256), tiles_t, w.D, (int)(vcw + kLdPad), w.DT,
-                  (int)(Tpad + kLdPad)};
+                  dlogprobs, dentropy, (int)vc0, (int)(vcw / 256), tiles_t, w.D, (int)(vcw + kLdPad)};
   };
   const GemmArgs none{};
   for (int64_t ci = 0; ci < nchunks; ++ci) {
-    // dz panels of this chunk, then the two gradient GEMMs that consume them (one launch, they are independent).
+    // dz panel of this chunk, then the two gradient GEMMs that consume it (one launch, they are independent).
     // Carrying the next chunk's dz tiles in the GEMM launch (to fill its tail) was measured: no gain at the default chunk
-    // width, and it needs a second pair of panels.
+    // width, and it needs a second panel.
     e = launch_bwd_chunk(s, dentropy != nullptr, dz_args(ci), (unsigned)(chunk_width(ci) / 256 * tiles_t), false, none, none);
     if (e != hipSuccess) return (int)e;
     const int64_t vc0 = ci * vc, vcw = chunk_width(ci);
     // dHidden[t, h] (+)= sum_v D[t, v] . weight^T[h, vc0 + v]        (A = weight^T rows at k offset vc0, B = D rows)
-    // dW[vc0 + v, h]  (+)= sum_t D^T[v, t] . hidden^T[h, t]           (A = hidden^T rows, B = D^T rows)
+    // dW[vc0 + v, h]  (+)= sum_t D[t, v] . hidden^T[h, t]             (A = hidden^T rows, B = D read K-major)
     const bool first = ci == 0, last = ci == nchunks - 1;
     const int64_t rows = (V - vc0) < vcw ? (V - vc0) : vcw;
     float* dWc = d_weight + (size_t)vc0 * (size_t)H;
     const GemmArgs gh = make_gemm(w.Wt + vc0, Vpad + kLdPad, H, w.D, vcw + kLdPad, Tpad, vcw / BK, H, T, nullptr, nullptr,
                                   last ? (uint16_t*)d_hidden : (uint16_t*)nullptr, H,
                                   first ? (const float*)nullptr : (const float*)w.dHacc, last ? (float*)nullptr : w.dHacc);
-    const GemmArgs gw = make_gemm(w.Ht, Tpad + kLdPad, H, w.DT, Tpad + kLdPad, vcw, Tpad / BK, H, rows,
+    const GemmArgs gw = make_gemm(w.Ht, Tpad + kLdPad, H, w.D, vcw + kLdPad, vcw, Tpad / BK, H, rows,
                                   accumulate_dw ? (const float*)dWc : (const float*)nullptr, dWc, (uint16_t*)nullptr, H);
     e = launch_bwd_chunk(s, dentropy != nullptr, DzArgs{}, 0, true, gh, gw);
     if (e != hipSuccess) return (int)e;

@@ -50,8 +50,8 @@ def test_workspace_queries():
     fwd = lib.skyrl_lmhead_fwd_workspace_bytes(T, H, V)
     assert 3 * 4 * T * 2 * 594 <= fwd <= 3 * 4 * T * 2 * 594 + 4096
     bwd = lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, 4096)
-    # weight^T + hidden^T + fp32 dHidden + two dz panels; nothing of size T*V
-    expect = 2 * H * V + 2 * H * T + 4 * T * H + 2 * 2 * T * 4096
+    # weight^T + hidden^T + fp32 dHidden + one dz panel; nothing of size T*V
+    expect = 2 * H * V + 2 * H * T + 4 * T * H + 2 * T * 4096
     assert expect <= bwd <= expect + (8 << 20)  # + 128 B of row padding per scratch row
     assert bwd < 2 * T * V
     assert lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, 100) == 0  # not a multiple of 256
