@@ -235,3 +235,36 @@ def test_packed_index_helpers_match_brute_force():
         model_utils._packed_subseq_row_indices_offsets_and_lens(torch.tensor([0, 4, 8]), [[3], [4], [1]], torch.device("cpu"))
     with pytest.raises(ValueError):
         model_utils._packed_subseq_row_indices_offsets_and_lens(torch.tensor([0, 4, 8, 9]), [[3], [4]], torch.device("cpu"))
+
+
+def test_merge_shard_statistics_equals_full_vocabulary_softmax():
+    """The host-side merge of per-slice statistics (what a vocabulary-parallel group's all-reduces compute) against a plain
+    log-softmax over the whole vocabulary, fp64, with a token whose target no slice owns."""
+    from skyrl_amd.vocab_shards import merge_shard_statistics
+
+    gen = torch.Generator().manual_seed(12)
+    T, V = 9, 40
+    z = torch.randn(T, V, dtype=torch.float64, generator=gen) * 3
+    y = torch.randint(0, V, (T,), generator=gen)
+    y[0] = V + 5
+    bounds = [0, 7, 8, 29, 40]
+    lps, lses, pzs, owners = [], [], [], []
+    for lo, hi in zip(bounds[:-1], bounds[1:]):
+        zs = z[:, lo:hi]
+        lse = torch.logsumexp(zs, -1)
+        own = (y >= lo) & (y < hi)
+        idx = (y - lo).clamp(0, hi - lo - 1)
+        lps.append(torch.where(own, zs.gather(-1, idx[:, None])[:, 0] - lse, torch.zeros(T, dtype=torch.float64)))
+        lses.append(lse)
+        pzs.append((torch.softmax(zs, -1) * zs).sum(-1))
+        owners.append(own)
+    lp, ent, lse, pz = merge_shard_statistics(torch.stack(lps), torch.stack(lses), torch.stack(pzs), torch.stack(owners))
+    full = torch.log_softmax(z, -1)
+    want_lp = full.gather(-1, y.clamp(max=V - 1)[:, None])[:, 0]
+    want_lp[0] = 0.0
+    torch.testing.assert_close(lp, want_lp, rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(ent, -(full.exp() * full).sum(-1), rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(lse, torch.logsumexp(z, -1), rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(pz, (full.exp() * z).sum(-1), rtol=1e-12, atol=1e-12)
+    with pytest.raises(ValueError):
+        merge_shard_statistics(lp, lse, pz, torch.stack(owners))

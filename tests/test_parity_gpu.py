@@ -845,6 +845,43 @@ def test_fsdp_forward_tail_from_hidden(cuda_device, packed, compute_entropy, ent
     assert cos(hd.grad, h64.grad) >= GRAD_COS and cos(wd.grad, w64.grad) >= GRAD_COS
 
 
+def test_vocab_shards_reproduce_the_full_vocabulary(cuda_device):
+    """How the path shards over a vocabulary-parallel group, on one GPU: forward per weight slice, the four [T] vectors
+    merged (what the group's all-reduces would do), backward per slice with the global statistics.  The slices' d_weight
+    rows concatenate to the full d_weight and their d_hidden shares add up to the full d_hidden."""
+    from skyrl_amd.vocab_shards import merge_shard_statistics
+    dev = cuda_device
+    T, H, V, t = 300, 128, 1000, 0.7
+    hidden, weight, labels, g, q = _rand(T, H, V, seed=31)
+    labels[:7] = SENTINEL                                  # targets no shard owns
+    h, w, y = hidden.to(dev), weight.to(dev), labels.to(dev)
+    gd, qd = g.to(dev), q.to(dev)
+    full_lp, full_ent, full_lse, full_pz = ops.lmhead_fwd(h, w, y, 1.0 / t, True)
+    full_dh, full_dw = ops.lmhead_bwd(h, w, y, full_lse, full_pz, gd, qd, 1.0 / t, 0)
+
+    bounds = [0, 256, 333, 1000]                           # uneven slices, one narrower than a tile
+    outs, owners, local_labels = [], [], []
+    for lo, hi in zip(bounds[:-1], bounds[1:]):
+        own = (y >= lo) & (y < hi)
+        yl = torch.where(own, y - lo, torch.full_like(y, SENTINEL))
+        outs.append(ops.lmhead_fwd(h, w[lo:hi].contiguous(), yl, 1.0 / t, True))
+        owners.append(own)
+        local_labels.append(yl)
+    lp, ent, lse, pz = merge_shard_statistics(torch.stack([o[0] for o in outs]), torch.stack([o[2] for o in outs]),
+                                              torch.stack([o[3] for o in outs]), torch.stack(owners))
+    torch.testing.assert_close(lp, full_lp, atol=2e-5, rtol=0)
+    torch.testing.assert_close(ent, full_ent, atol=2e-5, rtol=1e-5)
+    torch.testing.assert_close(lse, full_lse, atol=2e-5, rtol=0)
+    assert bool((lp[:7] == 0).all())
+
+    dh_sum = torch.zeros(T, H, dtype=torch.float32, device=dev)
+    for (lo, hi), yl in zip(zip(bounds[:-1], bounds[1:]), local_labels):
+        dh, dw = ops.lmhead_bwd(h, w[lo:hi].contiguous(), yl, lse, pz, gd, qd, 1.0 / t, 0)
+        torch.testing.assert_close(dw, full_dw[lo:hi], atol=2e-4, rtol=2e-3)   # same dz values up to the merged lse's rounding
+        dh_sum += dh.float()
+    assert cos(dh_sum, full_dh) >= 0.9999 and rel_l2(dh_sum, full_dh.float()) < 1e-2   # three bf16 roundings instead of one
+
+
 def test_opcheck_registration(cuda_device):
     T, H, V = 64, 64, 300
     hidden, weight, labels, _, _ = _rand(T, H, V, seed=2)
