@@ -459,7 +459,7 @@ __global__ __launch_bounds__(NTHREADS) void mfma_probe(const bf16x8* __restrict_
     for (int ks = 0; ks < KSTEPS; ++ks)
 #pragma unroll
       for (int x = 0; x < TM * TN; ++x) {
-        const int i = x / TN, j = (i & 1) ? TN - 1 - x % TN : x % TN;
+        const int i = mfma_row(x), j = mfma_col(x);
         mfma_16x16x32(acc[i][j], af[ks][i], bfr[ks][j]);
       }
   }
