@@ -83,7 +83,8 @@ int skyrl_lmhead_fwd(const void* hidden, int64_t ld_hidden, const void* weight, 
  * d_hidden: bf16 [T, H] contiguous, overwritten.  d_weight: fp32 [V, H] contiguous, overwritten, or added to
  * when accumulate_dw != 0 (gradient accumulation across micro-batches).  Both gradients are with respect to
  * the unscaled weight / hidden: the 1/temperature factor is already applied.
- * vocab_chunk: width of the dz panel in vocab columns (multiple of 256; 0 = library default).
+ * vocab_chunk: width of the dz panel in vocab columns (multiple of 256; 0 = library default: the width, with a panel of
+ * at most 1.5 GiB, whose launches divide most evenly over the device's compute units).
  */
 int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight,
                      const int64_t* labels, const float* row_lse, const float* row_pz,

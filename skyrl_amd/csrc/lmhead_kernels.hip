@@ -15,6 +15,7 @@
 #include <math.h>
 #include <stdint.h>
 
+#include <algorithm>
 #include <vector>
 
 #include "../../include/skyrl_lmhead.h"
@@ -582,12 +583,73 @@ int check_common(const void* hidden, int64_t ldh, const void* weight, int64_t ld
   return SKYRL_LMHEAD_OK;
 }
 
-int64_t default_vocab_chunk(int64_t T, int64_t V) {
-  const int64_t Tpad = round_up(T, 256), Vpad = round_up(V, 256);
-  int64_t vc = ((int64_t)1 << 28) / Tpad / 256 * 256;  // ~512 MiB of bf16 per dz panel
-  if (vc < 2048) vc = 2048;
-  if (vc > Vpad) vc = Vpad;
-  return vc;
+// Compute units of the current device (256 on an MI355X); 256 when no device answers, so that the workspace query gives
+// the same figure on a machine without a GPU.
+int compute_units() {
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+      n < 1) {
+    (void)hipGetLastError();
+    return 256;
+  }
+  return n;
+}
+
+// Estimated duration, in k-tiles of mainloop per CU, of `count_a` tiles of length `len_a` followed by `count_b` tiles of
+// length `len_b` handed to `ncu` CUs in order, each CU taking the next tile when it is free (what the dispatcher does with
+// one workgroup per CU).  Closed form: the first kind fills whole rounds plus one partial round; the second kind then
+// runs back to back on CUs that became free at one of two times, so the end is the smallest time by which those CUs can
+// have completed count_b tiles.
+int64_t list_schedule(int64_t count_a, int64_t len_a, int64_t count_b, int64_t len_b, int64_t ncu) {
+  const int64_t rounds = count_a / ncu, late = count_a % ncu, early = ncu - late;
+  const int64_t t_early = rounds * len_a, t_late = late ? (rounds + 1) * len_a : t_early;
+  if (count_b == 0) return t_late;
+  auto done_by = [&](int64_t t) {
+    return early * (t > t_early ? (t - t_early) / len_b : 0) + late * (t > t_late ? (t - t_late) / len_b : 0);
+  };
+  // the end is t_early + m * len_b or t_late + m * len_b for some m >= 1: take the smallest that suffices
+  int64_t best = -1;
+  for (const int64_t t0 : {t_early, t_late}) {
+    int64_t lo = 1, hi = count_b;  // m = count_b always suffices (one CU alone)
+    while (lo < hi) {
+      const int64_t mid = (lo + hi) / 2;
+      if (done_by(t0 + mid * len_b) >= count_b) hi = mid; else lo = mid + 1;
+    }
+    const int64_t t = t0 + lo * len_b;
+    if (best < 0 || t < best) best = t;
+  }
+  return best > t_late ? best : t_late;
+}
+
+// Width of the dz panel in vocab columns when the caller does not choose one.  Wider chunks mean fewer launches (every
+// launch ends with CUs idling for part of a tile), fewer read-modify-write passes over the dHidden partial sums and a
+// larger panel; what matters most is whether the tiles of a launch divide evenly over the CUs.  The candidates
+// (multiples of 2048 columns whose panel holds at most 1.5 GiB of dz values) are rated with a small model of the two launches per
+// chunk -- dz tiles of H/64 k-tiles plus an epilogue, then dHidden tiles of chunk/64 and dW tiles of T'/64 k-tiles,
+// list-scheduled over the CUs, plus a fixed cost per launch -- and the cheapest wins.  At the 7B shape (T = 16384, H = 3584)
+// that is 49152 columns: 4096 x 3 dz tiles and 896 + 2688 GEMM tiles per launch, both multiples of 256 CUs.
+int64_t default_vocab_chunk(int64_t T, int64_t H, int64_t V) {
+  const int64_t Tpad = round_up(T, 256), Vpad = round_up(V, 256), Hpad = round_up(H, 256);
+  const int ncu = compute_units();
+  const int64_t tiles_t = Tpad / 256, tiles_h = Hpad / 256;
+  const int64_t kDzEpilogue = 8, kGemmEpilogue = 6, kLaunch = 24;  // in k-tiles (about 1.3 us each)
+  const int64_t kMaxPanelBytes = (int64_t)3 << 29;  // of dz values, before the row padding
+  int64_t best_vc = 0, best_cost = 0;
+  for (int64_t vc = 2048;; vc += 2048) {
+    if (vc > Vpad) vc = Vpad;
+    const bool fits = Tpad * vc * 2 <= kMaxPanelBytes;
+    if (fits || best_vc == 0) {
+      int64_t cost = 0;
+      for (int64_t v0 = 0; v0 < Vpad; v0 += vc) {
+        const int64_t w = Vpad - v0 < vc ? Vpad - v0 : vc;
+        cost += list_schedule(w / 256 * tiles_t, H / BK + kDzEpilogue, 0, 0, ncu) + kLaunch;
+        cost += list_schedule(tiles_h * tiles_t, w / BK + kGemmEpilogue, tiles_h * (w / 256), Tpad / BK + kGemmEpilogue, ncu) + kLaunch;
+      }
+      if (best_vc == 0 || cost < best_cost) best_vc = vc, best_cost = cost;
+    }
+    if (vc >= Vpad || !fits) break;
+  }
+  return best_vc;
 }
 
 struct BwdWorkspace {
@@ -667,7 +729,7 @@ size_t skyrl_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
 
 size_t skyrl_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t vocab_chunk) {
   if (T < 1 || V < 1 || H < 1 || vocab_chunk < 0 || vocab_chunk % 256 != 0) return 0;
-  int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(T, V);
+  int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(T, H, V);
   if (vc > round_up(V, 256)) vc = round_up(V, 256);
   return carve_bwd(nullptr, T, H, V, vc).bytes;
 }
@@ -722,7 +784,7 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
   if (!aligned16(d_hidden) || !aligned16(d_weight)) return SKYRL_LMHEAD_ERR_ALIGN;
   if (vocab_chunk < 0 || vocab_chunk % 256 != 0) return SKYRL_LMHEAD_ERR_ARG;
   const int64_t Tpad = round_up(T, 256), Vpad = round_up(V, 256);
-  int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(T, V);
+  int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(T, H, V);
   if (vc > Vpad) vc = Vpad;
   // 32-bit byte offsets inside the scratch matrices as well (weight^T, hidden^T, the dz panel)
   if (H * (Vpad + kLdPad) * 2 >= ((int64_t)1 << 32) || H * (Tpad + kLdPad) * 2 >= ((int64_t)1 << 32) ||
