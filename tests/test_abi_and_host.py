@@ -268,3 +268,21 @@ def test_merge_shard_statistics_equals_full_vocabulary_softmax():
     torch.testing.assert_close(pz, (full.exp() * z).sum(-1), rtol=1e-12, atol=1e-12)
     with pytest.raises(ValueError):
         merge_shard_statistics(lp, lse, pz, torch.stack(owners))
+
+
+def test_default_vocab_chunk_respects_the_panel_cap():
+    """With vocab_chunk = 0 the library picks the dz panel width itself: whatever the shape, the panel holds at most 1.5 GiB
+    of dz values (plus row padding), the choice is a multiple of 256 columns no wider than the padded vocabulary, and the
+    same query gives the same answer twice."""
+    lib = _lib.load()
+    for T, H, V in [(16384, 3584, 152064), (32768, 4096, 128256), (8192, 1536, 151936), (300, 128, 1001), (1, 64, 8),
+                    (100000, 1024, 50257), (2048, 8192, 262144)]:
+        Tp, Vp, Hp = -(-T // 256) * 256, -(-V // 256) * 256, -(-H // 256) * 256
+        total = lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, 0)
+        assert total == lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, 0)
+        fixed = 2 * H * (Vp + 64) + 2 * H * (Tp + 64) + 4 * Tp * Hp
+        panel = total - fixed
+        assert 0 < panel <= (3 << 29) + 2 * Tp * 64 + 4096 or panel <= 2 * Tp * (2048 + 64) + 4096, (T, H, V, panel)
+        vc = (panel - 1024) // (2 * Tp) - 64          # the alignment slack is below one row
+        vc = -(-vc // 256) * 256
+        assert 256 <= vc <= Vp and lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, vc) == total, (T, H, V, vc)
