@@ -165,6 +165,26 @@ def test_edge_shapes(T, H, V, temperature, oov, vc, cuda_device):
     assert (out["entropy"] >= -1e-4).all() and (out["entropy"] <= math.log(V) + 1e-4).all()
 
 
+def test_random_shapes_against_the_oracle(cuda_device):
+    """Seeded sweep over ragged shapes: token counts and vocabulary sizes that are not multiples of any tile edge, every
+    hidden size class, chunk widths that split the vocabulary unevenly, temperatures, with and without an entropy gradient."""
+    gen = torch.Generator().manual_seed(2024)
+    ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=gen))  # noqa: E731
+    for case in range(24):
+        T, H, V = ri(1, 700), 64 * ri(1, 8), ri(2, 3500)
+        temperature = [1.0, 0.6, 1.7][ri(0, 2)]
+        oov = [None, "some", "all"][ri(0, 2)] if case % 3 == 0 else None
+        vc = [0, 256, 512, 1024][ri(0, 3)]
+        use_q = case % 2 == 0
+        hidden, weight, labels, g, q = _rand(T, H, V, seed=1000 + case, oov=oov)
+        tag = f"case {case}: T={T} H={H} V={V} t={temperature} oov={oov} vc={vc} q={use_q}"
+        print(tag, flush=True)
+        out = run_hip(cuda_device, hidden, weight, labels, temperature, g, q if use_q else None, True, vc)
+        ex = O.exact_fwd_bwd(hidden, weight, labels, temperature, g, q if use_q else None)
+        check_against(out, ex, True, True, tag)
+        assert torch.isfinite(out["d_hidden"].float()).all() and torch.isfinite(out["d_weight"]).all(), tag
+
+
 def test_zero_weight_known_answer(cuda_device):
     T, H, V = 70, 64, 1000
     hidden = torch.randn(T, H).to(torch.bfloat16)
