@@ -2,7 +2,6 @@
 before touching a device, and the Python host layer mirrors the reference's interface and error behaviour.  No kernel is
 launched here."""
 
-import ctypes
 import inspect
 import os
 import re

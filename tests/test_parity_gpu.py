@@ -5,8 +5,6 @@ gradient cosine similarity >= 0.999, all against an fp32 (here fp64) statement o
 Where a comparison is tighter than that, the tighter bound documents what the kernel actually achieves.
 """
 
-import ctypes
-import dataclasses
 import glob
 import math
 import os
