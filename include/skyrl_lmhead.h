@@ -141,6 +141,25 @@ int skyrl_approx_kl(const float* logprobs, const float* base_logprobs, const flo
                     int estimator, float* kld, float* row_mean, float* mean, int grad_mode, float* dlogprobs, void* stream);
 
 /*
+ * The whole actor loss of a micro-batch and both upstream gradients of the LM-head backward in two launches -- what the
+ * worker assembles from the policy loss, the KL term and the entropy term (skyrl/backends/skyrl_train/workers/worker.py:989-1089,
+ * workers/megatron/megatron_model_wrapper.py:902-941):
+ *     out6[0] = policy_scale * out6[1] + term_scale * (kl_coef * out6[4] - entropy_coef * out6[5])
+ *     out6[1] = policy loss, out6[2] its statistic, out6[3] = sum mask          (as skyrl_ppo_policy_loss's out3)
+ *     out6[4] = KL term: mean over rows of the masked row means of the estimate   (as skyrl_approx_kl's mean; 0 without base_logprobs)
+ *     out6[5] = entropy term: sum entropy * mask / max(sum mask, 1)               (masked_mean over everything; 0 without entropy)
+ *     dlogprobs = d out6[0] / d logprobs        dentropy = d out6[0] / d entropy
+ * All arrays fp32 [rows, cols]; loss_mask, loss_weight, base_logprobs, entropy, dlogprobs, dentropy may be NULL (dentropy needs
+ * entropy).  policy_scale is the factor the worker applies to the pre-scaled policy loss (its data-parallel size), term_scale
+ * the micro-batch weight of the two mean-reduced terms.  row_sums: fp32 scratch [rows, 6].
+ */
+int skyrl_actor_loss(const float* logprobs, const float* old_logprobs, const float* advantages, const float* loss_mask,
+                     const float* loss_weight, const float* base_logprobs, const float* entropy, int64_t rows, int64_t cols,
+                     int loss_type, float eps_clip_low, float eps_clip_high, float clip_ratio_c, int kl_estimator,
+                     float policy_scale, float term_scale, float kl_coef, float entropy_coef, float* row_sums, float* out6,
+                     float* dlogprobs, float* dentropy, void* stream);
+
+/*
  * masked_mean (torch_utils.py:180-184) per row of values fp32 [rows, cols]:
  *     means[b] = sum_s values * mask / max(sum_s mask, 1)          (mask NULL: the plain mean)
  * and, when dvalues is not NULL, dvalues[b,s] = d means[b] / d values[b,s] = mask / max(sum_s mask, 1).

@@ -30,6 +30,7 @@ What pins each function (all in ``tests/test_oracle.py``; none of them re-types 
     under x ~ p the expectation of k1 and of k3 is KL(p || q) exactly, summed by brute force over a small alphabet and
     compared with ``torch.nn.functional.kl_div`` -- and k3 ~ k2 for small differences; the trainer's reduction against a
     per-row Python loop.
+  * the assembled actor loss: a hand-computed two-row case (every term worked out on paper) on top of the pinned parts.
   * the FSDP forward tail: ``torch.distributions.Categorical`` for entropy and log-probability, and a Python loop that
     scores action token j of row b against position S - num_actions + j - 1, with and without padding removed.
 No function is left "parity unpinned".
@@ -538,3 +539,28 @@ def hf_wrapper_tail(
             return out.view(batch, seqlen)
         log_probs, entropy = pad(log_probs), pad(entropy)
     return log_probs[:, -num_actions - 1:-1], entropy
+
+
+def actor_loss(
+    log_probs: torch.Tensor,
+    old_log_probs: torch.Tensor,
+    advantages: torch.Tensor,
+    loss_mask: Optional[torch.Tensor],
+    eps_clip_low: float,
+    eps_clip_high: float,
+    policy_scale: float = 1.0,
+    term_scale: float = 1.0,
+    base_log_probs: Optional[torch.Tensor] = None,
+    kl_estimator_type: str = "k3",
+    kl_coef: float = 0.0,
+    entropy: Optional[torch.Tensor] = None,
+    entropy_coef: float = 0.0,
+):
+    """The per-micro-batch loss the policy worker back-propagates (skyrl/backends/skyrl_train/workers/worker.py:989-1089):
+    ``policy_loss * grad_sum_correction_factor + (kl_loss * kl_loss_coef - entropy * entropy_loss_coef) * microbatch_weight``
+    with ``kl_loss = masked_mean(compute_approx_kl(...), loss_mask, dim=-1).mean()`` and ``entropy = masked_mean(entropy_BS,
+    loss_mask)``.  Policy loss type "regular".  Returns ``(loss, policy_loss, kl, entropy_mean)``."""
+    policy, _ = ppo_policy_loss(log_probs, old_log_probs, advantages, eps_clip_low, eps_clip_high, loss_mask=loss_mask)
+    kl = approx_kl_loss(log_probs, base_log_probs, loss_mask, kl_estimator_type) if base_log_probs is not None else torch.zeros(())
+    ent = masked_mean(entropy, loss_mask) if entropy is not None else torch.zeros(())
+    return policy * policy_scale + (kl * kl_coef - ent * entropy_coef) * term_scale, policy, kl, ent

@@ -11,7 +11,7 @@ import os
 import threading
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libskyrl_lmhead.so")
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _c_i64 = ctypes.c_int64
 _c_p = ctypes.c_void_p
@@ -37,6 +37,10 @@ SIGNATURES = {
         [_c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_int, _c_p, _c_p, _c_p],
     ),
     "skyrl_approx_kl": (ctypes.c_int, [_c_p, _c_p, _c_p, _c_i64, _c_i64, ctypes.c_int, _c_p, _c_p, _c_p, ctypes.c_int, _c_p, _c_p]),
+    "skyrl_actor_loss": (
+        ctypes.c_int,
+        [_c_p] * 7 + [_c_i64, _c_i64, ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_int,
+                      ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float, _c_p, _c_p, _c_p, _c_p, _c_p]),
     "skyrl_masked_mean": (ctypes.c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_p, _c_p, _c_p]),
     "skyrl_packed_next_token_labels": (ctypes.c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_p, _c_p]),
     "skyrl_packed_scatter_logprobs": (

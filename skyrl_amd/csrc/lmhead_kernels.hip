@@ -696,7 +696,7 @@ hipError_t launch_bwd_chunk(hipStream_t s, bool entgrad, const DzArgs& z, unsign
 
 extern "C" {
 
-int skyrl_lmhead_version(void) { return 4; }
+int skyrl_lmhead_version(void) { return 5; }
 
 const char* skyrl_lmhead_strerror(int status) {
   switch (status) {

@@ -33,6 +33,45 @@ namespace {
 // `weight` carries whatever multiplies the loss without depending on lp (the off-policy importance ratio).
 // One workgroup: the data is a few hundred KiB, and a fixed reduction order keeps the sums bit-reproducible.
 // ------------------------------------------------------------------------------------------------------------
+// One token of the policy loss: value, derivative with respect to lp, and the statistic summed for the metric.
+__device__ __forceinline__ void policy_term(int type, float lp, float old, float A, float lo, float hi, float clip_c, float& loss,
+                                            float& dloss, float& stat) {
+  if (type == SKYRL_POLICY_LOSS_CROSS_ENTROPY) {
+    loss = -lp;
+    dloss = -1.f;
+    stat = 0.f;
+    return;
+  }
+  if (type == SKYRL_POLICY_LOSS_IMPORTANCE_SAMPLING) {
+    const float ratio = expf(lp - old);
+    loss = -(ratio * A);
+    dloss = loss;
+    stat = ratio;
+    return;
+  }
+  const float delta = lp - old;
+  const float dc = fminf(fmaxf(delta, -20.f), 20.f);
+  const float ratio = expf(dc);
+  const float d_ratio = (delta >= -20.f && delta <= 20.f) ? ratio : 0.f;  // d ratio / d lp
+  const float surr1 = ratio * A;
+  const float rc = fminf(fmaxf(ratio, lo), hi);
+  const float surr2 = rc * A;
+  const float d1 = d_ratio * A;
+  const float d2 = (ratio >= lo && ratio <= hi) ? d_ratio * A : 0.f;
+  loss = -fminf(surr1, surr2);
+  dloss = surr1 < surr2 ? -d1 : (surr1 > surr2 ? -d2 : -0.5f * (d1 + d2));
+  stat = surr2 < surr1 ? 1.f : 0.f;
+  if (type == SKYRL_POLICY_LOSS_DUAL_CLIP && A < 0.f) {
+    const float pg3 = -A * clip_c;
+    if (pg3 < loss) {
+      loss = pg3;
+      dloss = 0.f;
+    } else if (pg3 == loss) {
+      dloss *= 0.5f;
+    }
+  }
+}
+
 __global__ __launch_bounds__(1024) void policy_loss_kernel(const float* __restrict__ lp, const float* __restrict__ old,
                                                            const float* __restrict__ adv, const float* __restrict__ mask,
                                                            const float* __restrict__ weight, int64_t T, float eps_low,
@@ -43,39 +82,8 @@ __global__ __launch_bounds__(1024) void policy_loss_kernel(const float* __restri
   const float lo = 1.f - eps_low, hi = 1.f + eps_high;
   for (int64_t t = threadIdx.x; t < T; t += blockDim.x) {
     float loss, dloss, stat;
-    if (type == SKYRL_POLICY_LOSS_CROSS_ENTROPY) {
-      loss = -lp[t];
-      dloss = -1.f;
-      stat = 0.f;
-    } else if (type == SKYRL_POLICY_LOSS_IMPORTANCE_SAMPLING) {
-      const float ratio = expf(lp[t] - old[t]);
-      loss = -(ratio * adv[t]);
-      dloss = loss;
-      stat = ratio;
-    } else {
-      const float delta = lp[t] - old[t];
-      const float dc = fminf(fmaxf(delta, -20.f), 20.f);
-      const float ratio = expf(dc);
-      const float A = adv[t];
-      const float d_ratio = (delta >= -20.f && delta <= 20.f) ? ratio : 0.f;  // d ratio / d lp
-      const float surr1 = ratio * A;
-      const float rc = fminf(fmaxf(ratio, lo), hi);
-      const float surr2 = rc * A;
-      const float d1 = d_ratio * A;
-      const float d2 = (ratio >= lo && ratio <= hi) ? d_ratio * A : 0.f;
-      loss = -fminf(surr1, surr2);
-      dloss = surr1 < surr2 ? -d1 : (surr1 > surr2 ? -d2 : -0.5f * (d1 + d2));
-      stat = surr2 < surr1 ? 1.f : 0.f;
-      if (type == SKYRL_POLICY_LOSS_DUAL_CLIP && A < 0.f) {
-        const float pg3 = -A * clip_c;
-        if (pg3 < loss) {
-          loss = pg3;
-          dloss = 0.f;
-        } else if (pg3 == loss) {
-          dloss *= 0.5f;
-        }
-      }
-    }
+    const bool ce = type == SKYRL_POLICY_LOSS_CROSS_ENTROPY;  // reads neither old nor adv
+    policy_term(type, lp[t], ce ? 0.f : old[t], ce ? 0.f : adv[t], lo, hi, clip_c, loss, dloss, stat);
     const float m = mask ? mask[t] : 1.f;
     const float w = weight ? m * weight[t] : m;
     s_loss += loss * w;
@@ -124,6 +132,30 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 // One workgroup per row: mask sum, then values, row sum and gradient in a second sweep.  GRAD: 0 none, 1 the elementwise
 // derivative d kld_masked / d lp, 2 the derivative of mean_b row_mean_b.
 // ------------------------------------------------------------------------------------------------------------
+// One token of the KL estimate: value and derivative with respect to lp (clamp passes the gradient on its closed interval,
+// |.| has derivative 0 at 0, as torch differentiates them).
+__device__ __forceinline__ void kl_term(int estimator, float lp, float base, float& kld, float& dk) {
+  const float d = lp - base;
+  if (estimator == SKYRL_KL_K1) {
+    kld = d;
+    dk = 1.f;
+  } else if (estimator == SKYRL_KL_ABS) {
+    kld = fabsf(d);
+    dk = d > 0.f ? 1.f : (d < 0.f ? -1.f : 0.f);
+  } else if (estimator == SKYRL_KL_K2) {
+    kld = 0.5f * d * d;
+    dk = d;
+  } else {
+    const float kraw = base - lp;
+    const float k = fminf(fmaxf(kraw, -20.f), 20.f);
+    const float ratio = expf(k);
+    const float v = ratio - k - 1.f;
+    kld = fminf(fmaxf(v, -10.f), 10.f);
+    const bool open = kraw >= -20.f && kraw <= 20.f && v >= -10.f && v <= 10.f;
+    dk = open ? 1.f - ratio : 0.f;  // d/d lp of exp(k) - k - 1 with k = base - lp
+  }
+}
+
 __global__ __launch_bounds__(kRowThreads) void approx_kl_rows_kernel(const float* __restrict__ lp, const float* __restrict__ base,
                                                                      const float* __restrict__ mask, int64_t rows, int64_t cols,
                                                                      int estimator, int grad_mode, float* __restrict__ kld_out,
@@ -139,26 +171,8 @@ __global__ __launch_bounds__(kRowThreads) void approx_kl_rows_kernel(const float
   const float gscale = 1.f / (denom * (float)rows);
   float acc = 0.f;
   for (int64_t c = threadIdx.x; c < cols; c += kRowThreads) {
-    const float d = lp[row0 + c] - base[row0 + c];
     float kld, dk;
-    if (estimator == SKYRL_KL_K1) {
-      kld = d;
-      dk = 1.f;
-    } else if (estimator == SKYRL_KL_ABS) {
-      kld = fabsf(d);
-      dk = d > 0.f ? 1.f : (d < 0.f ? -1.f : 0.f);
-    } else if (estimator == SKYRL_KL_K2) {
-      kld = 0.5f * d * d;
-      dk = d;
-    } else {
-      const float kraw = base[row0 + c] - lp[row0 + c];
-      const float k = fminf(fmaxf(kraw, -20.f), 20.f);
-      const float ratio = expf(k);
-      const float v = ratio - k - 1.f;
-      kld = fminf(fmaxf(v, -10.f), 10.f);
-      const bool open = kraw >= -20.f && kraw <= 20.f && v >= -10.f && v <= 10.f;
-      dk = open ? 1.f - ratio : 0.f;  // d/d lp of exp(k) - k - 1 with k = base - lp
-    }
+    kl_term(estimator, lp[row0 + c], base[row0 + c], kld, dk);
     float m = 1.f;
     if (mask) {
       m = mask[row0 + c];
@@ -213,6 +227,90 @@ __global__ __launch_bounds__(kRowThreads) void masked_mean_rows_kernel(const flo
   }
 }
 
+// ------------------------------------------------------------------------------------------------------------
+// The whole per-micro-batch actor loss in two launches (workers/worker.py:989-1089, megatron_model_wrapper.py:902-941):
+//     loss = policy_scale * policy_loss  +  term_scale * ( kl_coef * kl  -  entropy_coef * entropy_mean )
+//     policy_loss  = sum loss_token * mask * weight                                   (policy_term above, reduce_loss)
+//     kl           = mean_b [ sum_s kld * mask / max(sum_s mask, 1) ]                  (kl_term above, masked_mean(dim=-1).mean())
+//     entropy_mean = sum entropy * mask / max(sum mask, 1)                            (masked_mean over everything)
+// and both upstream gradients of the LM-head backward:
+//     dlogprobs = policy_scale * d policy_loss / d lp  +  term_scale * kl_coef * d kl / d lp
+//     dentropy  = -term_scale * entropy_coef * mask / max(sum mask, 1)
+// First launch, one workgroup per row: the row's sums and dlogprobs (the KL gradient needs only the row's own mask count).
+// Second launch, one workgroup: the sums over rows in a fixed order, the six results, and dentropy, which needs the
+// global mask count.
+// ------------------------------------------------------------------------------------------------------------
+struct ActorLossArgs {
+  const float *lp, *old, *adv, *mask, *weight, *base, *entropy;
+  int64_t rows, cols;
+  int loss_type, kl_estimator;
+  float lo, hi, clip_c, policy_scale, term_scale, kl_coef, entropy_coef;
+  float* row_sums;  // [rows, 6]: policy loss, statistic, mask, kl row mean, entropy * mask, (unused)
+  float* out;       // [6]: loss, policy_loss, statistic, mask count, kl, entropy_mean
+  float *dlp, *dent;
+};
+
+__global__ __launch_bounds__(kRowThreads) void actor_loss_rows_kernel(const ActorLossArgs a) {
+  __shared__ float red[kRowThreads / 64];
+  const int64_t row0 = (int64_t)blockIdx.x * a.cols;
+  float msum = 0.f;
+  if (a.mask)
+    for (int64_t c = threadIdx.x; c < a.cols; c += kRowThreads) msum += a.mask[row0 + c];
+  const float row_mask = a.mask ? block_sum(msum, red) : (float)a.cols;
+  const float kl_denom = fmaxf(row_mask, 1.f);
+  const float kl_gscale = a.term_scale * a.kl_coef / (kl_denom * (float)a.rows);
+  const bool ce = a.loss_type == SKYRL_POLICY_LOSS_CROSS_ENTROPY;
+  float s_loss = 0.f, s_stat = 0.f, s_kl = 0.f, s_ent = 0.f;
+  for (int64_t c = threadIdx.x; c < a.cols; c += kRowThreads) {
+    const int64_t i = row0 + c;
+    const float lp = a.lp[i];
+    const float m = a.mask ? a.mask[i] : 1.f;
+    float loss, dloss, stat;
+    policy_term(a.loss_type, lp, ce ? 0.f : a.old[i], ce ? 0.f : a.adv[i], a.lo, a.hi, a.clip_c, loss, dloss, stat);
+    const float w = a.weight ? m * a.weight[i] : m;
+    s_loss += loss * w;
+    s_stat += stat * m;
+    float g = a.policy_scale * dloss * w;
+    if (a.base) {
+      float kld, dk;
+      kl_term(a.kl_estimator, lp, a.base[i], kld, dk);
+      // compute_approx_kl zeroes masked positions with where(); masked_mean multiplies by the mask once more
+      const float km = a.mask ? (m != 0.f ? m * m : 0.f) : 1.f;
+      s_kl += kld * km;
+      g += dk * km * kl_gscale;
+    }
+    if (a.entropy) s_ent += a.entropy[i] * m;
+    if (a.dlp) a.dlp[i] = g;
+  }
+  const float t_loss = block_sum(s_loss, red), t_stat = block_sum(s_stat, red);
+  const float t_kl = a.base ? block_sum(s_kl, red) : 0.f;
+  const float t_ent = a.entropy ? block_sum(s_ent, red) : 0.f;
+  if (threadIdx.x == 0) {
+    float* r = a.row_sums + (int64_t)blockIdx.x * 6;
+    r[0] = t_loss, r[1] = t_stat, r[2] = row_mask, r[3] = t_kl / kl_denom, r[4] = t_ent, r[5] = 0.f;
+  }
+}
+
+__global__ __launch_bounds__(kRowThreads) void actor_loss_finish_kernel(const ActorLossArgs a) {
+  __shared__ float red[kRowThreads / 64];
+  float v[5] = {0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int64_t r = threadIdx.x; r < a.rows; r += kRowThreads)
+    for (int k = 0; k < 5; ++k) v[k] += a.row_sums[r * 6 + k];
+  float t[5];
+  for (int k = 0; k < 5; ++k) t[k] = block_sum(v[k], red);
+  const float mask_denom = fmaxf(t[2], 1.f);
+  const float kl = t[3] / (float)a.rows, ent = t[4] / mask_denom;
+  if (threadIdx.x == 0) {
+    a.out[0] = a.policy_scale * t[0] + a.term_scale * (a.kl_coef * kl - a.entropy_coef * ent);
+    a.out[1] = t[0], a.out[2] = t[1], a.out[3] = t[2], a.out[4] = kl, a.out[5] = ent;
+  }
+  if (a.dent) {
+    const float c = -a.term_scale * a.entropy_coef / mask_denom;
+    const int64_t n = a.rows * a.cols;
+    for (int64_t i = threadIdx.x; i < n; i += kRowThreads) a.dent[i] = a.mask ? c * a.mask[i] : c;
+  }
+}
+
 bool finite(float x) { return std::isfinite(x); }
 
 }  // namespace
@@ -244,6 +342,31 @@ int skyrl_approx_kl(const float* logprobs, const float* base_logprobs, const flo
   hipLaunchKernelGGL(approx_kl_rows_kernel, dim3((unsigned)rows), dim3(kRowThreads), 0, s, logprobs, base_logprobs, loss_mask,
                      rows, cols, estimator, grad_mode, kld, row_mean, dlogprobs);
   hipLaunchKernelGGL(scaled_sum_kernel, dim3(1), dim3(kRowThreads), 0, s, row_mean, rows, 1.f / (float)rows, mean);
+  return (int)hipGetLastError();
+}
+
+int skyrl_actor_loss(const float* logprobs, const float* old_logprobs, const float* advantages, const float* loss_mask,
+                     const float* loss_weight, const float* base_logprobs, const float* entropy, int64_t rows, int64_t cols,
+                     int loss_type, float eps_clip_low, float eps_clip_high, float clip_ratio_c, int kl_estimator,
+                     float policy_scale, float term_scale, float kl_coef, float entropy_coef, float* row_sums, float* out6,
+                     float* dlogprobs, float* dentropy, void* stream) {
+  if (loss_type < SKYRL_POLICY_LOSS_REGULAR || loss_type > SKYRL_POLICY_LOSS_IMPORTANCE_SAMPLING) return SKYRL_LMHEAD_ERR_ARG;
+  if (base_logprobs && (kl_estimator < SKYRL_KL_K1 || kl_estimator > SKYRL_KL_K3)) return SKYRL_LMHEAD_ERR_ARG;
+  const bool needs_old = loss_type != SKYRL_POLICY_LOSS_CROSS_ENTROPY;
+  if (!logprobs || !row_sums || !out6 || (needs_old && (!old_logprobs || !advantages))) return SKYRL_LMHEAD_ERR_NULL;
+  if (dentropy && !entropy) return SKYRL_LMHEAD_ERR_NULL;
+  if (rows < 1 || cols < 1 || rows >= (int64_t(1) << 31)) return SKYRL_LMHEAD_ERR_SHAPE;
+  const bool clips = loss_type == SKYRL_POLICY_LOSS_REGULAR || loss_type == SKYRL_POLICY_LOSS_DUAL_CLIP;
+  if (clips && (!finite(eps_clip_low) || !finite(eps_clip_high))) return SKYRL_LMHEAD_ERR_ARG;
+  if (loss_type == SKYRL_POLICY_LOSS_DUAL_CLIP && !finite(clip_ratio_c)) return SKYRL_LMHEAD_ERR_ARG;
+  if (!finite(policy_scale) || !finite(term_scale) || !finite(kl_coef) || !finite(entropy_coef)) return SKYRL_LMHEAD_ERR_ARG;
+  const ActorLossArgs a{logprobs,   old_logprobs,       advantages,         loss_mask,    loss_weight,  base_logprobs, entropy,
+                        rows,       cols,               loss_type,          kl_estimator, 1.f - eps_clip_low,
+                        1.f + eps_clip_high, clip_ratio_c, policy_scale,    term_scale,   kl_coef,      entropy_coef,
+                        row_sums,   out6,               dlogprobs,          dentropy};
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(actor_loss_rows_kernel, dim3((unsigned)rows), dim3(kRowThreads), 0, s, a);
+  hipLaunchKernelGGL(actor_loss_finish_kernel, dim3(1), dim3(kRowThreads), 0, s, a);
   return (int)hipGetLastError();
 }
 

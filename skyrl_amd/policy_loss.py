@@ -9,7 +9,9 @@ and results:
 * ``compute_approx_kl``         :88-126    -> per-token KL estimate ``[B, S]``
 * ``masked_mean``               torch_utils.py:180-184
 
-plus ``approx_kl_loss``, the reduction the trainer applies to the KL estimate (``masked_mean(kl, mask, dim=-1).mean()``,
+plus ``actor_loss``, the whole per-micro-batch loss of the policy worker (policy loss + KL term - entropy term,
+workers/worker.py:989-1089) with both upstream gradients of the LM head from two launches, and ``approx_kl_loss``, the
+reduction the trainer applies to the KL estimate (``masked_mean(kl, mask, dim=-1).mean()``,
 workers/worker.py:1071-1077) fused with the estimate and its gradient.  The losses are reduced as ``reduce_loss`` does
 (masked sum, :1145-1149; the reference folds the kind of mean into the advantages beforehand, :1152-1181).  The reference
 computes each with a chain of elementwise torch kernels and lets autograd derive the gradient; here one kernel produces
@@ -31,7 +33,7 @@ from . import _lib
 from .ops import _require_device
 
 __all__ = ["ppo_policy_loss", "cross_entropy_loss", "importance_sampling_loss", "compute_approx_kl", "approx_kl_loss",
-           "masked_mean", "ppo_policy_loss_terms"]
+           "masked_mean", "actor_loss", "ppo_policy_loss_terms"]
 
 LOSS_REGULAR, LOSS_DUAL_CLIP, LOSS_CROSS_ENTROPY, LOSS_IMPORTANCE_SAMPLING = 0, 1, 2, 3
 KL_ESTIMATORS = {"k1": 0, "abs": 1, "k2": 2, "k3": 3}
@@ -319,3 +321,130 @@ def masked_mean(tensor: torch.Tensor, mask: Optional[torch.Tensor], dim: Optiona
         raise NotImplementedError("masked_mean reduces everything (dim=None) or the last dimension")
     rows, cols = _rows_cols(tensor)
     return _MaskedMean.apply(tensor, mask, rows, cols, tensor.shape[:-1])
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# the assembled actor loss
+# ----------------------------------------------------------------------------------------------------------------------
+_POLICY_LOSS_TYPES = {"regular": LOSS_REGULAR, "dual_clip": LOSS_DUAL_CLIP, "cross_entropy": LOSS_CROSS_ENTROPY,
+                      "importance_sampling": LOSS_IMPORTANCE_SAMPLING}
+
+
+@torch.library.custom_op("skyrl_amd::actor_loss", mutates_args=())
+def _actor_loss(log_probs: torch.Tensor, old_log_probs: Optional[torch.Tensor], advantages: Optional[torch.Tensor],
+                loss_mask: Optional[torch.Tensor], loss_weight: Optional[torch.Tensor], base_log_probs: Optional[torch.Tensor],
+                entropy: Optional[torch.Tensor], loss_type: int, eps_clip_low: float, eps_clip_high: float, clip_ratio_c: float,
+                kl_estimator: int, policy_scale: float, term_scale: float, kl_coef: float, entropy_coef: float,
+                ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``(out6, dlogprobs, dentropy)`` for contiguous fp32 ``[rows, cols]`` inputs; ``dentropy`` is empty without ``entropy``."""
+    dev = _require_device(log_probs)
+    rows, cols = log_probs.shape
+    for name, t in (("old_log_probs", old_log_probs), ("advantages", advantages), ("loss_mask", loss_mask),
+                    ("loss_weight", loss_weight), ("base_log_probs", base_log_probs), ("entropy", entropy)):
+        if t is not None and (t.dtype != torch.float32 or t.shape != log_probs.shape or not t.is_contiguous()):
+            raise ValueError(f"{name} must be a contiguous fp32 tensor of shape {tuple(log_probs.shape)}")
+    out6 = torch.empty(6, dtype=torch.float32, device=dev)
+    row_sums = torch.empty((rows, 6), dtype=torch.float32, device=dev)
+    dlp = torch.empty_like(log_probs)
+    dent = torch.empty_like(log_probs) if entropy is not None else torch.empty(0, dtype=torch.float32, device=dev)
+    ptr = lambda t: None if t is None else t.data_ptr()  # noqa: E731
+    with torch.cuda.device(dev):
+        st = _lib.load().skyrl_actor_loss(
+            log_probs.data_ptr(), ptr(old_log_probs), ptr(advantages), ptr(loss_mask), ptr(loss_weight), ptr(base_log_probs),
+            ptr(entropy), rows, cols, int(loss_type), float(eps_clip_low), float(eps_clip_high), float(clip_ratio_c),
+            int(kl_estimator), float(policy_scale), float(term_scale), float(kl_coef), float(entropy_coef), row_sums.data_ptr(),
+            out6.data_ptr(), dlp.data_ptr(), dent.data_ptr() if entropy is not None else None,
+            torch.cuda.current_stream(dev).cuda_stream)
+    _lib.check(st, "skyrl_actor_loss")
+    return out6, dlp, dent
+
+
+@_actor_loss.register_fake
+def _(log_probs, old_log_probs, advantages, loss_mask, loss_weight, base_log_probs, entropy, loss_type, eps_clip_low,
+      eps_clip_high, clip_ratio_c, kl_estimator, policy_scale, term_scale, kl_coef, entropy_coef):
+    return (log_probs.new_empty(6), torch.empty_like(log_probs),
+            torch.empty_like(log_probs) if entropy is not None else log_probs.new_empty(0))
+
+
+class _ActorLoss(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, log_probs, entropy, consts, scalars):
+        old, adv, mask, weight, base = consts
+        rows, cols = _rows_cols(log_probs)
+        flat = lambda t: None if t is None else t.detach().to(torch.float32).contiguous().reshape(rows, cols)  # noqa: E731
+        for name, t in (("old_log_probs", old), ("advantages", adv), ("loss_mask", mask), ("loss_weight", weight),
+                        ("base_log_probs", base), ("entropy", entropy)):
+            if t is not None and t.shape != log_probs.shape:
+                raise ValueError(f"{name} has shape {tuple(t.shape)}, expected {tuple(log_probs.shape)}")
+        out6, dlp, dent = _actor_loss(flat(log_probs), flat(old), flat(adv), flat(mask), flat(weight), flat(base), flat(entropy),
+                                      *scalars)
+        ctx.save_for_backward(dlp, dent)
+        ctx.lp_meta = (log_probs.shape, log_probs.dtype)
+        ctx.ent_meta = None if entropy is None else (entropy.shape, entropy.dtype)
+        ctx.mark_non_differentiable(out6)
+        return out6[0].clone(), out6
+
+    @staticmethod
+    def backward(ctx, grad_loss, _grad_out6):
+        dlp, dent = ctx.saved_tensors
+        shape, dtype = ctx.lp_meta
+        g_lp = (dlp * grad_loss).reshape(shape).to(dtype)
+        g_ent = None
+        if ctx.ent_meta is not None:
+            g_ent = (dent * grad_loss).reshape(ctx.ent_meta[0]).to(ctx.ent_meta[1])
+        return g_lp, g_ent, None, None
+
+
+def actor_loss(
+    log_probs: torch.Tensor,
+    old_log_probs: Optional[torch.Tensor],
+    advantages: Optional[torch.Tensor],
+    config: Any,
+    loss_mask: Optional[torch.Tensor] = None,
+    *,
+    base_log_probs: Optional[torch.Tensor] = None,
+    entropy: Optional[torch.Tensor] = None,
+    loss_weight: Optional[torch.Tensor] = None,
+    policy_scale: float = 1.0,
+    term_scale: float = 1.0,
+) -> Tuple[torch.Tensor, Dict[str, torch.Tensor]]:
+    """The loss the policy worker back-propagates for one micro-batch, assembled in two kernel launches together with
+    both upstream gradients of the fused LM head (reference: workers/worker.py:989-1089):
+
+        ``policy_loss * policy_scale + (kl_loss * config.kl_loss_coef - entropy * config.entropy_loss_coef) * term_scale``
+
+    ``config`` is the algorithm config: ``policy_loss_type`` (regular, dual_clip, cross_entropy, importance_sampling),
+    ``eps_clip_low`` / ``eps_clip_high`` / ``clip_ratio_c``, ``use_kl_loss`` + ``kl_loss_coef`` + ``kl_estimator_type``,
+    ``use_entropy_loss`` + ``entropy_loss_coef``.  The KL term needs ``base_log_probs``; the entropy term needs ``entropy``
+    (``[B, S]``, e.g. from ``action_log_probs_from_hidden(..., compute_entropy=True)``) and sends a gradient into it.
+    ``policy_scale`` is the worker's ``grad_sum_correction_factor``, ``term_scale`` its ``microbatch_weight``.
+
+    Returns the loss and a dict of 0-dim tensors (no host synchronisation): ``policy_loss``, ``policy_kl``, ``policy_entropy``
+    and ``clip_ratio`` (``importance_ratio`` for the importance-sampling loss).
+    """
+    name = getattr(config, "policy_loss_type", "regular")
+    if name not in _POLICY_LOSS_TYPES:
+        raise NotImplementedError(f"policy_loss_type {name!r} is not part of the fused actor loss; fused types: "
+                                  f"{sorted(_POLICY_LOSS_TYPES)}")
+    loss_type = _POLICY_LOSS_TYPES[name]
+    use_kl = bool(getattr(config, "use_kl_loss", False))
+    if use_kl and base_log_probs is None:
+        raise ValueError("use_kl_loss needs base_log_probs")
+    use_ent = bool(getattr(config, "use_entropy_loss", False))
+    if use_ent and entropy is None:
+        raise ValueError("use_entropy_loss needs the per-token entropy")
+    estimator = getattr(config, "kl_estimator_type", "k3")
+    if use_kl and estimator not in KL_ESTIMATORS:
+        raise ValueError(f"Invalid KL estimator type: {estimator}")
+    clips = loss_type in (LOSS_REGULAR, LOSS_DUAL_CLIP)
+    scalars = (loss_type, float(config.eps_clip_low) if clips else 0.0, float(config.eps_clip_high) if clips else 0.0,
+               float(getattr(config, "clip_ratio_c", 0.0)) if loss_type == LOSS_DUAL_CLIP else 0.0,
+               KL_ESTIMATORS.get(estimator, 3), float(policy_scale), float(term_scale),
+               float(config.kl_loss_coef) if use_kl else 0.0, float(config.entropy_loss_coef) if use_ent else 0.0)
+    consts = (old_log_probs, advantages, loss_mask, loss_weight, base_log_probs if use_kl else None)
+    # The entropy is reduced for the metric even when it is not part of the loss, as the worker does.
+    loss, out6 = _ActorLoss.apply(log_probs, entropy, consts, scalars)
+    stat = out6[2] / (out6[3] if loss_type == LOSS_IMPORTANCE_SAMPLING else out6[3].clamp(min=1.0))
+    metrics = {"policy_loss": out6[1], "policy_kl": out6[4], "policy_entropy": out6[5],
+               ("importance_ratio" if loss_type == LOSS_IMPORTANCE_SAMPLING else "clip_ratio"): stat}
+    return loss, metrics

@@ -547,6 +547,23 @@ def test_approx_kl_loss_reduction_brute_force():
     assert got == pytest.approx(float((lp - base).abs().mean()))
 
 
+def test_actor_loss_combination_by_hand():
+    # two rows of two tokens; ratios 1 (unclipped), so the policy loss is -sum A * mask
+    lp = torch.tensor([[-1.0, -2.0], [-0.5, -3.0]], dtype=torch.float64)
+    adv = torch.tensor([[1.0, -2.0], [0.5, 4.0]], dtype=torch.float64)
+    mask = torch.tensor([[1.0, 1.0], [1.0, 0.0]], dtype=torch.float64)
+    base = lp - torch.tensor([[0.2, -0.4], [0.6, 9.0]], dtype=torch.float64)        # k1 = lp - base
+    ent = torch.tensor([[2.0, 4.0], [6.0, 100.0]], dtype=torch.float64)
+    loss, policy, kl, e = O.actor_loss(lp, lp.clone(), adv, mask, 0.2, 0.2, policy_scale=8.0, term_scale=0.25,
+                                       base_log_probs=base, kl_estimator_type="k1", kl_coef=0.1, entropy=ent, entropy_coef=0.01)
+    assert policy.item() == pytest.approx(-(1.0 - 2.0 + 0.5))
+    assert kl.item() == pytest.approx(((0.2 - 0.4) / 2 + 0.6 / 1) / 2)            # row means over masked tokens, then over rows
+    assert e.item() == pytest.approx((2.0 + 4.0 + 6.0) / 3)
+    assert loss.item() == pytest.approx(8.0 * 0.5 + 0.25 * (0.1 * 0.25 - 0.01 * 4.0))
+    bare, _, kl0, e0 = O.actor_loss(lp, lp.clone(), adv, mask, 0.2, 0.2)
+    assert bare.item() == pytest.approx(0.5) and kl0.item() == 0.0 and e0.item() == 0.0
+
+
 # ----------------------------------------------------------------------------------------------------------------------
 # the FSDP worker's forward tail
 # ----------------------------------------------------------------------------------------------------------------------

@@ -535,7 +535,62 @@ def test_loss_argument_errors(cuda_device):
     assert lib.skyrl_approx_kl(p, p, None, 0, 4, 3, None, p, p, 0, None, None) == -2
     assert lib.skyrl_masked_mean(p, None, 4, 4, None, None, None) == -1
     assert lib.skyrl_masked_mean(p, None, 4, 0, p, None, None) == -2
+    args = lambda **kw: [kw.get("lp", p), p, p, None, None, None, kw.get("ent"), 4, 4, kw.get("type", 0), 0.2, 0.2, 3.0,  # noqa: E731
+                         3, 1.0, 1.0, 0.0, 0.0, kw.get("rows", p), p, None, kw.get("dent"), None]
+    assert lib.skyrl_actor_loss(*args()) == 0
+    assert lib.skyrl_actor_loss(*args(rows=None)) == -1
+    assert lib.skyrl_actor_loss(*args(dent=p)) == -1          # an entropy gradient without the entropy
+    assert lib.skyrl_actor_loss(*args(type=9)) == -5
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("use_kl,use_ent,masked", [(False, False, True), (True, False, False), (True, True, True)])
+def test_actor_loss_matches_oracle(use_kl, use_ent, masked, cuda_device):
+    """The assembled loss (policy + KL - entropy) and both upstream gradients from the two-launch kernel pair."""
+    from types import SimpleNamespace
+
+    from skyrl_amd.policy_loss import actor_loss
+
+    gen = torch.Generator().manual_seed(23)
+    B, S = 6, 700
+    lp = torch.randn(B, S, generator=gen) * 0.5 - 2.0
+    old = lp + torch.randn(B, S, generator=gen) * 0.3
+    base = lp + torch.randn(B, S, generator=gen) * 0.4
+    adv = torch.randn(B, S, generator=gen)
+    ent = torch.rand(B, S, generator=gen) * 3
+    mask = None
+    if masked:
+        mask = (torch.rand(B, S, generator=gen) > 0.4).float()
+        mask[2] = 0
+    cfg = SimpleNamespace(policy_loss_type="regular", eps_clip_low=0.2, eps_clip_high=0.28, use_kl_loss=use_kl, kl_loss_coef=0.05,
+                          kl_estimator_type="k3", use_entropy_loss=use_ent, entropy_loss_coef=0.01)
+    m64 = None if mask is None else mask.double()
+    r_lp, r_ent = lp.double().requires_grad_(True), ent.double().requires_grad_(True)
+    ref, ref_pol, ref_kl, ref_e = O.actor_loss(r_lp, old.double(), adv.double(), m64, 0.2, 0.28, policy_scale=4.0, term_scale=0.125,
+                                               base_log_probs=base.double() if use_kl else None, kl_estimator_type="k3",
+                                               kl_coef=0.05 if use_kl else 0.0, entropy=r_ent, entropy_coef=0.01 if use_ent else 0.0)
+    ref.backward()
+    to = lambda t: None if t is None else t.to(cuda_device)  # noqa: E731
+    d_lp, d_ent = lp.to(cuda_device).requires_grad_(True), ent.to(cuda_device).requires_grad_(True)
+    loss, metrics = actor_loss(d_lp, to(old), to(adv), cfg, to(mask), base_log_probs=to(base), entropy=d_ent, policy_scale=4.0,
+                               term_scale=0.125)
+    loss.backward()
+    assert loss.item() == pytest.approx(ref.item(), rel=2e-5, abs=1e-4)
+    assert metrics["policy_loss"].item() == pytest.approx(ref_pol.item(), rel=2e-5, abs=1e-4)
+    assert metrics["policy_kl"].item() == pytest.approx(ref_kl.item() if use_kl else 0.0, rel=2e-5, abs=1e-7)
+    assert metrics["policy_entropy"].item() == pytest.approx(ref_e.item(), rel=2e-5)
+    torch.testing.assert_close(d_lp.grad.cpu().double(), r_lp.grad, rtol=2e-5, atol=1e-7)
+    want_dent = r_ent.grad if r_ent.grad is not None else torch.zeros(B, S, dtype=torch.float64)
+    torch.testing.assert_close(d_ent.grad.cpu().double(), want_dent, rtol=2e-5, atol=1e-12)
+    # the same loss from the separate kernels
+    from skyrl_amd.policy_loss import approx_kl_loss, masked_mean, ppo_policy_loss
+    pol, _ = ppo_policy_loss(to(lp), to(old), to(adv), cfg, to(mask))
+    parts = pol * 4.0
+    if use_kl:
+        parts = parts + 0.125 * 0.05 * approx_kl_loss(to(lp), to(base), to(mask), "k3")
+    if use_ent:
+        parts = parts - 0.125 * 0.01 * masked_mean(to(ent), to(mask))
+    assert loss.item() == pytest.approx(parts.item(), rel=1e-5, abs=1e-4)
 
 
 def test_mfma_probe_sums_exactly(cuda_device):
