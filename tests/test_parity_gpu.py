@@ -593,6 +593,50 @@ def test_actor_loss_matches_oracle(use_kl, use_ent, masked, cuda_device):
     assert loss.item() == pytest.approx(parts.item(), rel=1e-5, abs=1e-4)
 
 
+def test_whole_path_hidden_to_actor_loss_gradients(cuda_device):
+    """Decoder output -> fused LM head (log-probabilities and grad-carrying entropy, padding removed) -> assembled actor loss
+    -> gradients in hidden and weight, against the same chain on materialised fp64 logits."""
+    from types import SimpleNamespace
+
+    from skyrl_amd.model_wrapper import action_log_probs_from_hidden
+    from skyrl_amd.policy_loss import actor_loss
+
+    dev = cuda_device
+    gen = torch.Generator().manual_seed(77)
+    B, S, H, V, A, t = 4, 48, 128, 900, 20, 0.9
+    seqs = torch.randint(0, V, (B, S), generator=gen)
+    am = torch.ones(B, S, dtype=torch.long)
+    am[0, :9] = 0
+    am[3, :17] = 0
+    nnz = am.flatten().nonzero().flatten()
+    hidden = torch.randn(1, len(nnz), H, generator=gen).to(torch.bfloat16)
+    weight = (torch.randn(V, H, generator=gen) * 3 / H ** 0.5).to(torch.bfloat16)
+    adv = torch.randn(B, A, generator=gen)
+    loss_mask = (torch.rand(B, A, generator=gen) > 0.3).float()
+    cfg = SimpleNamespace(policy_loss_type="regular", eps_clip_low=0.2, eps_clip_high=0.2, use_kl_loss=True, kl_loss_coef=0.02,
+                          kl_estimator_type="k2", use_entropy_loss=True, entropy_loss_coef=0.005)
+
+    h64, w64 = hidden.double().requires_grad_(True), weight.double().requires_grad_(True)
+    alp, ent = O.hf_wrapper_tail(h64 @ w64.t(), seqs, A, am.double(), t, nnz_indices=nnz)
+    old = (alp.detach() + 0.2 * torch.randn(B, A, generator=gen).double()).float()
+    base = (alp.detach() + 0.3 * torch.randn(B, A, generator=gen).double()).float()
+    ent_act = ent[:, -A - 1:-1]
+    ref, _, _, _ = O.actor_loss(alp, old.double(), adv.double(), loss_mask.double(), 0.2, 0.2, policy_scale=2.0, term_scale=0.5,
+                                base_log_probs=base.double(), kl_estimator_type="k2", kl_coef=0.02, entropy=ent_act,
+                                entropy_coef=0.005)
+    ref.backward()
+
+    hd, wd = hidden.to(dev).requires_grad_(True), weight.to(dev).requires_grad_(True)
+    got_alp, out = action_log_probs_from_hidden(hd, wd, seqs.to(dev), A, am.to(dev), t, return_output=True,
+                                                compute_entropy=True, entropy_requires_grad=True, nnz_indices=nnz.to(dev))
+    loss, metrics = actor_loss(got_alp, old.to(dev), adv.to(dev), cfg, loss_mask.to(dev), base_log_probs=base.to(dev),
+                               entropy=out["entropy"][:, -A - 1:-1], policy_scale=2.0, term_scale=0.5)
+    loss.backward()
+    assert loss.item() == pytest.approx(ref.item(), rel=1e-3, abs=1e-3)
+    assert all(v.dim() == 0 and v.is_cuda for v in metrics.values())
+    assert cos(hd.grad, h64.grad) >= GRAD_COS and cos(wd.grad, w64.grad) >= GRAD_COS
+
+
 def test_mfma_probe_sums_exactly(cuda_device):
     """The measurement kernel runs the mainloop's MFMA sequence on caller-given operands: with small integers the sum of
     every wavefront's accumulators has a closed form, sum_k (sum_m A[m,k]) (sum_n B[n,k]) per pair of fragments."""
