@@ -57,8 +57,9 @@ const char* skyrl_lmhead_strerror(int status);
 size_t skyrl_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V);
 
 /* Scratch needed by skyrl_lmhead_bwd for a given vocab chunk width (0 = library default):
- * weight^T bf16 [H, V'+64], hidden^T bf16 [H, T'+64], fp32 dHidden partial sums (T' x H' values, kept in the
- * kernel's accumulator order between chunks) and one bf16 dz panel [T', chunk+64]
+ * hidden^T bf16 [H, T'+64], fp32 dHidden partial sums (T' x H' values, kept in the kernel's accumulator order between
+ * chunks), one bf16 dz panel [T', chunk+64] and, only when V is not a multiple of 64, weight^T bf16 [H, V'+64] (otherwise
+ * the weight is read where it is)
  * (T', V', H' = T, V, H rounded up to 256; the 64 extra elements keep row pitches off powers of two).
  * Nothing in it scales with T * V.
  * (Stands in for the `d_logits [T, 9504]` scratch of the reference's default backward,

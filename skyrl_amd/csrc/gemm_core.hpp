@@ -99,7 +99,9 @@ struct Operand {
 };
 // A B operand may instead be "K-major": the same matrix stored transposed, ptr[k * ld + n], so that a 16-byte chunk
 // holds eight consecutive n of one k (what a producer writes when n is its contiguous axis).  Then row0 is the first
-// column n of the tile; the caller guarantees that columns row0 .. row0+255 and every k row of the loop exist.
+// column n of the tile and `rows` the number of valid columns (a multiple of 8): a tile may overhang them, the overhanging
+// lanes re-read the last valid chunk (their results belong to output columns that the epilogue drops).  The caller
+// guarantees that every k row of the loop exists.
 //
 // K-major slot layout: 64 k-rows x 256 n = 32 blocks of 1 KiB, block b = rows 2b and 2b+1 (what one wave-wide copy
 // fills).  A block is 16 windows of 64 bytes, a window = 32 bytes (16 n) of the even row, then of the odd row.  The 16 n
@@ -170,7 +172,9 @@ __device__ __forceinline__ void make_plan(CopyPlan& p, const Operand& a, const O
       const int block = j * NWAVES + wave;             // rows 2 * block, 2 * block + 1 of the k-tile
       const int q = (lane >> 2) ^ kmajor_sigma(block);  // the pair whose home is this lane's window
       const int krow = 2 * block + ((lane >> 1) & 1);
-      p.b_src[j] = (uint32_t)krow * (uint32_t)b.ld * 2u + (uint32_t)((b.row0 + q * 16 + (lane & 1) * 8) * 2);
+      int n = b.row0 + q * 16 + (lane & 1) * 8;
+      n = n < b.rows - 8 ? n : b.rows - 8;
+      p.b_src[j] = (uint32_t)krow * (uint32_t)b.ld * 2u + (uint32_t)(n * 2);
     } else {
       int gb = b.row0 + row;
       gb = gb < b.rows ? gb : b.rows - 1;

@@ -359,7 +359,9 @@ struct GemmArgs {
   const uint16_t* A;
   int lda, a_rows;
   const uint16_t* B;
-  int ldb, b_rows;
+  int ldb, b_rows;  // K-major B: b_rows is the number of valid columns (n) of the stored matrix
+  int b_kmajor;     // B is stored K-major, B[k * ldb + n]
+  int c_rows_m;     // the bf16 output is C[m * ldc + n] (n contiguous) instead of C[n * ldc + m]
   int nk, M, N;
   const float* Cin;
   float* Cf;
@@ -409,6 +411,26 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, int bid, char* lds)
   }
   if (!Cf && !Cb) return;
 
+  if (BKM && p.c_rows_m) {
+    // Output rows run along M: a lane's four values belong to four different rows; sixteen lanes (n = lrow) cover 32
+    // contiguous bytes of each.  Only the last vocab chunk's dHidden tiles come through here.
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = tn * BN + wn * WN + j * MT + lrow;
+      if (n >= N) continue;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int m = tm * BM + wm * WM + i * MT + kq * 4;
+        const bf16x4 b4 = __builtin_convertvector(acc[i][j], bf16x4);
+        const uint16_t* h4 = (const uint16_t*)&b4;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (m + r < M) Cb[(size_t)(m + r) * (size_t)ldc + n] = h4[r];
+      }
+    }
+    return;
+  }
+
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int n = tn * BN + wn * WN + j * MT + lrow;
@@ -437,9 +459,15 @@ __global__ __launch_bounds__(NTHREADS) void lmhead_bwd_chunk(const DzArgs z, con
                                                              int gemm_tiles) {
   __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
   const int id = blockIdx.x;
-  if (id < tiles0) gemm_tile<false>(p0, id, lds);               // dHidden: B = dz panel rows, K (vocab) contiguous
-  else if (id < gemm_tiles) gemm_tile<true>(p1, id - tiles0, lds);  // dW: B = the same panel read K-major (K = tokens)
-  else dz_tile<ENTGRAD>(z, id - gemm_tiles, lds);
+  // dW always reads the dz panel K-major (K = tokens); dHidden either reads the weight itself K-major (K = vocab) or,
+  // when the vocabulary is not a multiple of the k-tile, a transposed, zero-padded copy of it with K contiguous.
+  const bool second = id >= tiles0;
+  if (id < gemm_tiles) {
+    if (second || p0.b_kmajor) gemm_tile<true>(second ? p1 : p0, second ? id - tiles0 : id, lds);
+    else gemm_tile<false>(p0, id, lds);
+  } else {
+    dz_tile<ENTGRAD>(z, id - gemm_tiles, lds);
+  }
 }
 
 // Measurement aid: the mainloop's MFMA sequence (two 32-k steps of 64 MFMAs, same order, accumulators in AGPRs) with
@@ -658,11 +686,16 @@ struct BwdWorkspace {
   size_t bytes;
 };
 
+// The dHidden GEMM contracts over the vocabulary.  When V is a multiple of the k-tile it reads the weight rows where they
+// are (K-major B operand); otherwise the last k-tile would reach past the weight's last row, and a transposed copy,
+// zero-padded to whole tiles, is made in the workspace instead.
+inline bool reads_weight_in_place(int64_t V) { return V % BK == 0; }
+
 BwdWorkspace carve_bwd(void* ws, int64_t T, int64_t H, int64_t V, int64_t vc) {
   const int64_t Tpad = round_up(T, 256), Vpad = round_up(V, 256);
   Carver c(ws);
   BwdWorkspace w;
-  w.Wt = c.take<uint16_t>((size_t)H * (Vpad + kLdPad));
+  w.Wt = reads_weight_in_place(V) ? nullptr : c.take<uint16_t>((size_t)H * (Vpad + kLdPad));
   w.Ht = c.take<uint16_t>((size_t)H * (Tpad + kLdPad));
   w.dHacc = c.take<float>((size_t)Tpad * round_up(H, 256));  // accumulator order, whole tiles
   w.D = c.take<uint16_t>((size_t)Tpad * (vc + kLdPad));
@@ -670,10 +703,11 @@ BwdWorkspace carve_bwd(void* ws, int64_t T, int64_t H, int64_t V, int64_t vc) {
   return w;
 }
 
-GemmArgs make_gemm(const uint16_t* A, int64_t lda, int64_t a_rows, const uint16_t* B, int64_t ldb, int64_t b_rows, int64_t nk,
-                   int64_t M, int64_t N, const float* Cin, float* Cf, uint16_t* Cb, int64_t ldc, const float* Pin = nullptr,
-                   float* Pout = nullptr) {
-  return GemmArgs{A, (int)lda, (int)a_rows, B, (int)ldb, (int)b_rows, (int)nk, (int)M, (int)N, Cin, Cf, Cb, (int)ldc, Pin, Pout};
+GemmArgs make_gemm(const uint16_t* A, int64_t lda, int64_t a_rows, const uint16_t* B, int64_t ldb, int64_t b_rows, bool b_kmajor,
+                   bool c_rows_m, int64_t nk, int64_t M, int64_t N, const float* Cin, float* Cf, uint16_t* Cb, int64_t ldc,
+                   const float* Pin = nullptr, float* Pout = nullptr) {
+  return GemmArgs{A,       (int)lda, (int)a_rows, B,  (int)ldb, (int)b_rows, b_kmajor ? 1 : 0, c_rows_m ? 1 : 0, (int)nk,
+                  (int)M,  (int)N,   Cin,         Cf, Cb,       (int)ldc,    Pin,              Pout};
 }
 
 unsigned gemm_tiles(const GemmArgs& g) { return (unsigned)(((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN)); }
@@ -799,8 +833,9 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
   const uint16_t* Hp = (const uint16_t*)hidden;
   hipError_t e;
 
-  // weight^T [H, Vpad] and hidden^T [H, Tpad], zero in the padding columns.
-  {
+  // hidden^T [H, Tpad] and, unless the weight can be read in place, weight^T [H, Vpad]; zero in the padding columns.
+  const bool w_in_place = reads_weight_in_place(V);
+  if (!w_in_place) {
     Timed timed(kTranspose, s);
     hipLaunchKernelGGL(transpose_bf16, dim3((unsigned)(Vpad / 64), (unsigned)(H / 64)), dim3(256), 0, s, Wp, (int)ld_weight,
                        (int)V, (int)H, w.Wt, (int)(Vpad + kLdPad), (int)Vpad);
@@ -833,10 +868,18 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
     const bool first = ci == 0, last = ci == nchunks - 1;
     const int64_t rows = (V - vc0) < vcw ? (V - vc0) : vcw;
     float* dWc = d_weight + (size_t)vc0 * (size_t)H;
-    const GemmArgs gh = make_gemm(w.Wt + vc0, Vpad + kLdPad, H, w.D, vcw + kLdPad, Tpad, vcw / BK, H, T, nullptr, nullptr,
-                                  last ? (uint16_t*)d_hidden : (uint16_t*)nullptr, H,
-                                  first ? (const float*)nullptr : (const float*)w.dHacc, last ? (float*)nullptr : w.dHacc);
-    const GemmArgs gw = make_gemm(w.Ht, Tpad + kLdPad, H, w.D, vcw + kLdPad, vcw, Tpad / BK, H, rows,
+    const uint16_t* dh_out = last ? (uint16_t*)d_hidden : (uint16_t*)nullptr;
+    const float* dh_in = first ? (const float*)nullptr : (const float*)w.dHacc;
+    float* dh_keep = last ? (float*)nullptr : w.dHacc;
+    // In place: C[t, h] with A = D rows (K = vocab, contiguous), B = weight rows vc0.. read K-major; the k extent stops at V.
+    // Otherwise: C[h, t] with A = weight^T rows, B = D rows.  The partial sums are in accumulator order either way.
+    const int64_t kext = (V - vc0) < vcw ? (V - vc0) : vcw;
+    const GemmArgs gh =
+        w_in_place ? make_gemm(w.D, vcw + kLdPad, Tpad, Wp + (size_t)vc0 * (size_t)ld_weight, ld_weight, H, true, true, kext / BK, T,
+                               H, nullptr, nullptr, (uint16_t*)dh_out, H, dh_in, dh_keep)
+                   : make_gemm(w.Wt + vc0, Vpad + kLdPad, H, w.D, vcw + kLdPad, Tpad, false, false, vcw / BK, H, T, nullptr,
+                               nullptr, (uint16_t*)dh_out, H, dh_in, dh_keep);
+    const GemmArgs gw = make_gemm(w.Ht, Tpad + kLdPad, H, w.D, vcw + kLdPad, vcw, true, false, Tpad / BK, H, rows,
                                   accumulate_dw ? (const float*)dWc : (const float*)nullptr, dWc, (uint16_t*)nullptr, H);
     e = launch_bwd_chunk(s, dentropy != nullptr, DzArgs{}, 0, true, gh, gw);
     if (e != hipSuccess) return (int)e;

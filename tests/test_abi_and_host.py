@@ -49,9 +49,12 @@ def test_workspace_queries():
     fwd = lib.skyrl_lmhead_fwd_workspace_bytes(T, H, V)
     assert 3 * 4 * T * 2 * 594 <= fwd <= 3 * 4 * T * 2 * 594 + 4096
     bwd = lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, 4096)
-    # weight^T + hidden^T + fp32 dHidden + one dz panel; nothing of size T*V
-    expect = 2 * H * V + 2 * H * T + 4 * T * H + 2 * T * 4096
+    # hidden^T + fp32 dHidden + one dz panel; nothing of size T*V, and no copy of the weight (V is a multiple of 64)
+    expect = 2 * H * T + 4 * T * H + 2 * T * 4096
     assert expect <= bwd <= expect + (8 << 20)  # + 128 B of row padding per scratch row
+    # a vocabulary that is not a multiple of the k-tile needs the transposed, zero-padded weight as well
+    odd = lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V - 8, 4096)
+    assert expect + 2 * H * (V - 8) <= odd <= expect + 2 * H * V + (8 << 20)
     assert bwd < 2 * T * V
     assert lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, 100) == 0  # not a multiple of 256
     assert lib.skyrl_lmhead_fwd_workspace_bytes(0, H, V) == 0
@@ -279,7 +282,7 @@ def test_default_vocab_chunk_respects_the_panel_cap():
         Tp, Vp, Hp = -(-T // 256) * 256, -(-V // 256) * 256, -(-H // 256) * 256
         total = lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, 0)
         assert total == lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, 0)
-        fixed = 2 * H * (Vp + 64) + 2 * H * (Tp + 64) + 4 * Tp * Hp
+        fixed = (0 if V % 64 == 0 else 2 * H * (Vp + 64)) + 2 * H * (Tp + 64) + 4 * Tp * Hp
         panel = total - fixed
         assert 0 < panel <= (3 << 29) + 2 * Tp * 64 + 4096 or panel <= 2 * Tp * (2048 + 64) + 4096, (T, H, V, panel)
         vc = (panel - 1024) // (2 * Tp) - 64          # the alignment slack is below one row

@@ -149,6 +149,12 @@ def _rand(T, H, V, seed, oov=None):
         (300, 128, 1001, 0.6, None, 256),
         (513, 256, 3000, 1.0, "some", 1024),
         (64, 64, 5000, 2.0, "all", 2048),
+        # vocabularies that are multiples of 64: the dHidden GEMM reads the weight in place (K-major), also with a hidden size
+        # that is not a multiple of the tile (overhanging columns) and ragged token counts
+        (300, 192, 1024, 0.8, None, 0),
+        (257, 128, 64, 1.0, "some", 0),
+        (100, 320, 4096, 1.0, None, 1024),
+        (513, 448, 1984, 0.6, "some", 512),
     ],
 )
 def test_edge_shapes(T, H, V, temperature, oov, vc, cuda_device):
