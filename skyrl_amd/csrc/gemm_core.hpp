@@ -13,8 +13,9 @@
 //   * a CU takes at most ~32 B/clk from L2, through global_load_lds as well as through ordinary loads; a 64 KiB k-tile
 //     (256 + 256 rows x 64 k) therefore needs >= 2048 clk, exactly the MFMA time of a 256 x 256 x 64 tile: the copy
 //     path, not the matrix pipe, is the resource that must never idle;
-//   * every LDS read cycle steals about half a cycle from the direct-to-LDS copies, so LDS is read as little as
-//     possible: 128 x 128 wave tiles need 16 fragment reads per 32-k step (128 x 64 tiles need 24);
+//   * LDS reads and direct-to-LDS copies share the LDS port, so LDS is read as little as possible: 128 x 128 wave
+//     tiles need 16 fragment reads per 32-k step (128 x 64 tiles need 24); the 8 extra reads of a K-major B operand
+//     (two 64-bit transposing reads per fragment) measured free;
 //   * the copy unit takes one 1 KiB copy about every 34 clk for the whole CU and a wave that issues into a full queue
 //     stalls -- with one wave per SIMD that stalls the matrix pipe -- so a lane's 16 copies per k-tile are spread
 //     evenly over its 128 MFMAs.

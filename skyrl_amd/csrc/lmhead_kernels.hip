@@ -7,10 +7,12 @@
 //   lmhead_fwd_merge   per token: merges the partials (online log-sum-exp), gathers the label logit with an
 //                      fp32 dot product hidden[t] . weight[label], writes logprob / entropy / lse / pz.
 // Backward (6*T*V*H flop), looped over vocab chunks of `vocab_chunk` columns:
-//   transpose_bf16     weight^T and hidden^T once per call, so that every contraction is K-contiguous.
-//   lmhead_bwd_chunk   dz tiles: recompute a logits tile and form dz in registers; write it (bf16) row-major and
-//                      transposed into two chunk-sized panels.  GEMM tiles: dHidden (+)= dz . weight and
-//                      dW[chunk] = dz^T . hidden, fp32 accumulation.
+//   transpose_bf16     hidden^T once per call (and weight^T only when V is not a multiple of 64).
+//   lmhead_bwd_chunk   dz tiles: recompute a logits tile, form dz in registers and write it (bf16) into one token-major
+//                      panel of the chunk.  GEMM tiles: dHidden (+)= dz . weight and dW[chunk] = dz^T . hidden with fp32
+//                      accumulation, both from that panel -- dW reads it K-major, dHidden reads the weight K-major in
+//                      place -- through the transposing LDS read (gemm_core.hpp).
+// The per-token loss kernels and the packed-sequence index kernels live in loss_kernels.hip and packed_kernels.hip.
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdint.h>
