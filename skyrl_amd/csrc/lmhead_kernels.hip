@@ -402,14 +402,22 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, int bid, char* lds)
 
   if (p.Pin || p.Pout) {
     const size_t base = ((size_t)(tm * tiles_n + tn) * NWAVES + wave) * (TM * TN * 64 * 4) + (size_t)lane * 4;
+    if (p.Pin) {  // sixteen loads in flight at a time: one at a time costs a round trip to HBM each (36 us per tile)
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+      for (int i = 0; i < TM; i += 2) {
+        f32x4 t[2 * TN];
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const size_t off = base + (size_t)(i * TN + j) * (64 * 4);
-        if (p.Pin) acc[i][j] += *(const f32x4*)(p.Pin + off);
-        if (p.Pout) *(f32x4*)(p.Pout + off) = acc[i][j];
+        for (int x = 0; x < 2 * TN; ++x) t[x] = *(const f32x4*)(p.Pin + base + (size_t)(i * TN + x) * (64 * 4));
+#pragma unroll
+        for (int x = 0; x < 2 * TN; ++x) acc[i + x / TN][x % TN] += t[x];
       }
+    }
+    if (p.Pout) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) *(f32x4*)(p.Pout + base + (size_t)(i * TN + j) * (64 * 4)) = acc[i][j];
+    }
   }
   if (!Cf && !Cb) return;
 
