@@ -117,6 +117,27 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
 #define SKYRL_POLICY_LOSS_DUAL_CLIP 1
 #define SKYRL_POLICY_LOSS_CROSS_ENTROPY 2
 #define SKYRL_POLICY_LOSS_IMPORTANCE_SAMPLING 3
+/* Further types of the reference's registry (ppo_utils.py), same outputs; r = exp(clamp(logprobs - old_logprobs, -20, 20)):
+ *   GSPO (gspo_policy_loss, :663-729; skyrl_actor_loss only, it needs rows): the clipped surrogate of REGULAR with every
+ *     token's ratio replaced by its sequence's, exp(min(masked row mean of logprobs - old_logprobs, 10)), whose gradient
+ *     reaches each token's own logprob with weight 1.
+ *   SAPO (sapo_policy_loss, :590-660): loss = -sigmoid(tau (r - 1)) (4 / tau) A, tau = A > 0 ? eps_clip_low : eps_clip_high
+ *     (the two arguments carry tau_pos and tau_neg); out3[1] = 0.
+ *   CISPO (compute_policy_loss_cispo, :732-821, anchor "old"; pass the rollout log-probabilities as old_logprobs for the
+ *     "rollout" anchor): loss = -A stopgrad(clamp(r, 1 - eps_clip_low, 1 + eps_clip_high)) logprobs; out3[1] counts r outside.
+ *   ROLLOUT_IS (rollout_is_policy_loss, :824-863; old_logprobs = rollout log-probabilities):
+ *     loss = -stopgrad(r inside the open interval (1 - eps_clip_low, 1 + eps_clip_high) ? r : 0) A logprobs; out3[1] counts outside.
+ *   DPPO_TV, DPPO_KL (dppo_policy_loss, :866-935; old_logprobs = rollout log-probabilities when there are any):
+ *     loss = -r A keep, keep = 0 where the probability moved too far in the advantage's direction -- TV: p - p_old >
+ *     eps_clip_high (A > 0) or p_old - p > eps_clip_low (A < 0); KL: the binary KL of p_old to p exceeds the same thresholds
+ *     (the two arguments carry delta_low and delta_high); out3[1] counts keep == 0.
+ * Not covered: clip_cov and kl_cov (a random subset / a top-k over the whole batch). */
+#define SKYRL_POLICY_LOSS_GSPO 4
+#define SKYRL_POLICY_LOSS_SAPO 5
+#define SKYRL_POLICY_LOSS_CISPO 6
+#define SKYRL_POLICY_LOSS_ROLLOUT_IS 7
+#define SKYRL_POLICY_LOSS_DPPO_TV 8
+#define SKYRL_POLICY_LOSS_DPPO_KL 9
 int skyrl_ppo_policy_loss(const float* logprobs, const float* old_logprobs, const float* advantages,
                           const float* loss_mask, const float* loss_weight, int64_t T,
                           float eps_clip_low, float eps_clip_high, float clip_ratio_c, int loss_type,

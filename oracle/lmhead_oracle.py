@@ -26,6 +26,11 @@ What pins each function (all in ``tests/test_oracle.py``; none of them re-types 
     the advantage, dual-clip active / inactive, the +-20 clamp of the log-ratio), fp64 central finite differences of the
     loss for the gradient autograd derives from it, and the masked-mean definition of clip_ratio counted by hand.
   * cross-entropy and importance-sampling losses, masked_mean: values worked out by hand on small inputs.
+  * SAPO, GSPO, CISPO, rollout-IS and DPPO losses: per-token values worked out with ``math`` on either side of every branch
+    (sign of the advantage, inside / on / outside the interval, both trust-region tests, the clamps at 20 and 10), the
+    limits that tie them to pinned functions (GSPO on rows of one token is the clipped surrogate; DPPO with nothing masked
+    and SAPO's gate near r = 1 are the importance-sampling surrogate; CISPO and rollout-IS agree inside the interval), and
+    fp64 central finite differences of the surrogate with the stop-gradient factors held fixed.
   * approximate KL: hand values at d = 0, ln 2, -1 and in both clamps; the identities the estimators are built on --
     under x ~ p the expectation of k1 and of k3 is KL(p || q) exactly, summed by brute force over a small alphabet and
     compared with ``torch.nn.functional.kl_div`` -- and k3 ~ k2 for small differences; the trainer's reduction against a
@@ -444,6 +449,80 @@ def ppo_policy_loss(
         loss = loss * loss_weight
     loss = (loss * loss_mask).sum() if loss_mask is not None else loss.sum()            # reduce_loss
     return loss, clip_ratio.detach()
+
+
+def _reduce(loss: torch.Tensor, loss_mask: Optional[torch.Tensor]) -> torch.Tensor:
+    """reduce_loss, ppo_utils.py:1145-1149: the masked sum."""
+    return (loss * loss_mask).sum() if loss_mask is not None else loss.sum()
+
+
+def _safe_ratio(log_probs: torch.Tensor, behaviour: torch.Tensor) -> torch.Tensor:
+    """safe_exp_delta with clip = 20, torch_utils.py:187-192."""
+    return torch.clamp(log_probs - behaviour, -20.0, 20.0).exp()
+
+
+def sapo_policy_loss(log_probs, old_log_probs, advantages, tau_pos: float, tau_neg: float, loss_mask=None):
+    """ppo_utils.py:590-660: the sigmoid gate ``sigmoid(tau (r - 1)) 4 / tau`` in place of the clipped ratio, tau chosen by
+    the sign of the advantage (:639-643: tau_pos where A > 0, tau_neg elsewhere).  Returns ``(loss, clip_ratio = 0)``."""
+    ratio = _safe_ratio(log_probs, old_log_probs)
+    taus = torch.where(advantages > 0, torch.as_tensor(tau_pos, dtype=advantages.dtype),
+                       torch.as_tensor(tau_neg, dtype=advantages.dtype))
+    gates = torch.sigmoid(taus * (ratio - 1.0)) * (4.0 / taus)
+    return _reduce(-gates * advantages, loss_mask), torch.zeros(())
+
+
+def gspo_policy_loss(log_probs, old_log_probs, advantages, eps_clip_low: float, eps_clip_high: float, loss_mask=None):
+    """ppo_utils.py:663-729: every token of a sequence carries the sequence's importance weight, the masked row mean of the
+    log-ratio (:701), re-attached to the token's own log-probability so that the gradient reaches it (:707), clamped from
+    above at 10 (:709), then the clipped surrogate.  Returns ``(loss, clip_ratio)``."""
+    row = masked_mean(log_probs - old_log_probs, loss_mask, dim=-1).unsqueeze(-1)
+    log_w = torch.clamp(log_probs - log_probs.detach() + row.detach(), max=10)
+    ratio = log_w.exp()
+    surr1 = ratio * advantages
+    surr2 = ratio.clamp(1 - eps_clip_low, 1 + eps_clip_high) * advantages
+    clip_ratio = masked_mean((-surr2 > -surr1).to(log_probs.dtype), loss_mask)
+    return _reduce(-torch.min(surr1, surr2), loss_mask), clip_ratio.detach()
+
+
+def cispo_policy_loss(log_probs, behaviour_log_probs, advantages, eps_clip_low: float, eps_clip_high: float, loss_mask=None):
+    """ppo_utils.py:732-821: ``-A stopgrad(clamp(r, 1 - lo, 1 + hi)) log_probs``; ``behaviour_log_probs`` is the anchor the
+    config selects (:769-780).  Returns ``(loss, clip_ratio)``, the fraction of tokens whose ratio lies outside (:786-787)."""
+    ratio = _safe_ratio(log_probs, behaviour_log_probs)
+    clamped = torch.clamp(ratio, 1 - eps_clip_low, 1 + eps_clip_high)
+    clipped = ((ratio < 1 - eps_clip_low) | (ratio > 1 + eps_clip_high)).to(log_probs.dtype)
+    return _reduce(-advantages * clamped.detach() * log_probs, loss_mask), masked_mean(clipped, loss_mask).detach()
+
+
+def rollout_is_policy_loss(log_probs, rollout_logprobs, advantages, eps_clip_low: float, eps_clip_high: float, loss_mask=None):
+    """ppo_utils.py:824-863: as CISPO on the rollout log-probabilities, with the weight set to zero outside the open interval
+    (1 - lo, 1 + hi) (:850-851).  Returns ``(loss, clip_ratio)``."""
+    ratio = _safe_ratio(log_probs, rollout_logprobs)
+    in_range = (ratio > 1 - eps_clip_low) & (ratio < 1 + eps_clip_high)
+    weight = torch.where(in_range, ratio, torch.zeros_like(ratio))
+    loss = -(weight.detach() * advantages * log_probs)
+    return _reduce(loss, loss_mask), masked_mean((~in_range).to(log_probs.dtype), loss_mask).detach()
+
+
+def dppo_policy_loss(log_probs, mu_log_probs, advantages, dppo_type: str, delta_low: float, delta_high: float, loss_mask=None):
+    """ppo_utils.py:866-935: the unclipped surrogate times a 0/1 trust-region mask computed without gradient from the token's
+    probability under the two policies -- "binary_tv" (:902-906) on the probability difference, "binary_kl" (:908-917) on the
+    Bernoulli KL of the behaviour policy to the current one.  Returns ``(loss, clip_ratio)``, the fraction masked out."""
+    ratio = _safe_ratio(log_probs, mu_log_probs)
+    with torch.no_grad():
+        p, mu = log_probs.exp(), mu_log_probs.exp()
+        diff = p - mu
+        keep = torch.ones_like(advantages)
+        if dppo_type == "binary_tv":
+            keep[(advantages > 0) & (diff > delta_high)] = 0.0
+            keep[(advantages < 0) & (-diff > delta_low)] = 0.0
+        elif dppo_type == "binary_kl":
+            eps = 1e-8
+            bkl = mu * (mu_log_probs - log_probs) + (1 - mu) * torch.log((1 - mu + eps) / (1 - p + eps))
+            keep[(advantages > 0) & (diff > 0) & (bkl > delta_high)] = 0.0
+            keep[(advantages < 0) & (diff < 0) & (bkl > delta_low)] = 0.0
+        else:
+            raise ValueError(f"Unknown DPPO type: {dppo_type}. Must be 'binary_tv' or 'binary_kl'.")
+    return _reduce(-(ratio * advantages * keep), loss_mask), masked_mean((keep == 0).to(log_probs.dtype), loss_mask).detach()
 
 
 def cross_entropy_loss(log_probs: torch.Tensor, loss_mask: Optional[torch.Tensor] = None) -> torch.Tensor:

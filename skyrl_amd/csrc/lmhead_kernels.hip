@@ -740,7 +740,7 @@ hipError_t launch_bwd_chunk(hipStream_t s, bool entgrad, const DzArgs& z, unsign
 
 extern "C" {
 
-int skyrl_lmhead_version(void) { return 5; }
+int skyrl_lmhead_version(void) { return 6; }
 
 const char* skyrl_lmhead_strerror(int status) {
   switch (status) {

@@ -34,8 +34,10 @@ namespace {
 // One workgroup: the data is a few hundred KiB, and a fixed reduction order keeps the sums bit-reproducible.
 // ------------------------------------------------------------------------------------------------------------
 // One token of the policy loss: value, derivative with respect to lp, and the statistic summed for the metric.
-__device__ __forceinline__ void policy_term(int type, float lp, float old, float A, float lo, float hi, float clip_c, float& loss,
-                                            float& dloss, float& stat) {
+// (lo, hi, c) are the type's three parameters as the header lists them; row_lr is the masked row mean of lp - old, used by
+// the sequence-level type only.
+__device__ __forceinline__ void policy_term(int type, float lp, float old, float A, float lo, float hi, float c, float row_lr,
+                                            float& loss, float& dloss, float& stat) {
   if (type == SKYRL_POLICY_LOSS_CROSS_ENTROPY) {
     loss = -lp;
     dloss = -1.f;
@@ -49,10 +51,53 @@ __device__ __forceinline__ void policy_term(int type, float lp, float old, float
     stat = ratio;
     return;
   }
+  // safe_exp_delta: the log-ratio clamped to +-20; the clamp passes the gradient on its closed interval
   const float delta = lp - old;
-  const float dc = fminf(fmaxf(delta, -20.f), 20.f);
-  const float ratio = expf(dc);
-  const float d_ratio = (delta >= -20.f && delta <= 20.f) ? ratio : 0.f;  // d ratio / d lp
+  float ratio = expf(fminf(fmaxf(delta, -20.f), 20.f));
+  float d_ratio = (delta >= -20.f && delta <= 20.f) ? ratio : 0.f;  // d ratio / d lp
+  if (type == SKYRL_POLICY_LOSS_GSPO) {  // the sequence's ratio for every token, clamp(max = 10) on the log
+    ratio = expf(fminf(row_lr, 10.f));
+    d_ratio = row_lr <= 10.f ? ratio : 0.f;
+  }
+  if (type == SKYRL_POLICY_LOSS_SAPO) {  // lo = tau_pos, hi = tau_neg
+    const float tau = A > 0.f ? lo : hi;
+    const float sg = 1.f / (1.f + expf(-tau * (ratio - 1.f)));
+    loss = -(sg * (4.f / tau)) * A;
+    dloss = -4.f * A * sg * (1.f - sg) * d_ratio;
+    stat = 0.f;
+    return;
+  }
+  if (type == SKYRL_POLICY_LOSS_CISPO) {  // lo, hi: bounds of the stop-gradient weight; the gradient flows through lp only
+    const float w = fminf(fmaxf(ratio, lo), hi);
+    loss = -A * w * lp;
+    dloss = -A * w;
+    stat = (ratio < lo || ratio > hi) ? 1.f : 0.f;
+    return;
+  }
+  if (type == SKYRL_POLICY_LOSS_ROLLOUT_IS) {  // old = rollout log-probabilities; weight zeroed outside the open interval
+    const bool in_range = ratio > lo && ratio < hi;
+    const float w = in_range ? ratio : 0.f;
+    loss = -(w * A * lp);
+    dloss = -(w * A);
+    stat = in_range ? 0.f : 1.f;
+    return;
+  }
+  if (type == SKYRL_POLICY_LOSS_DPPO_TV || type == SKYRL_POLICY_LOSS_DPPO_KL) {  // lo = delta_low, hi = delta_high
+    const float p = expf(lp), pm = expf(old), diff = p - pm;
+    bool keep = true;
+    if (type == SKYRL_POLICY_LOSS_DPPO_TV) {
+      if ((A > 0.f && diff > hi) || (A < 0.f && -diff > lo)) keep = false;
+    } else {
+      const float eps = 1e-8f;
+      const float bkl = pm * (old - lp) + (1.f - pm) * logf((1.f - pm + eps) / (1.f - p + eps));
+      if ((A > 0.f && diff > 0.f && bkl > hi) || (A < 0.f && diff < 0.f && bkl > lo)) keep = false;
+    }
+    loss = keep ? -(ratio * A) : 0.f;
+    dloss = keep ? -(d_ratio * A) : 0.f;
+    stat = keep ? 0.f : 1.f;
+    return;
+  }
+  // REGULAR, DUAL_CLIP, GSPO: the clipped surrogate
   const float surr1 = ratio * A;
   const float rc = fminf(fmaxf(ratio, lo), hi);
   const float surr2 = rc * A;
@@ -62,7 +107,7 @@ __device__ __forceinline__ void policy_term(int type, float lp, float old, float
   dloss = surr1 < surr2 ? -d1 : (surr1 > surr2 ? -d2 : -0.5f * (d1 + d2));
   stat = surr2 < surr1 ? 1.f : 0.f;
   if (type == SKYRL_POLICY_LOSS_DUAL_CLIP && A < 0.f) {
-    const float pg3 = -A * clip_c;
+    const float pg3 = -A * c;
     if (pg3 < loss) {
       loss = pg3;
       dloss = 0.f;
@@ -72,6 +117,12 @@ __device__ __forceinline__ void policy_term(int type, float lp, float old, float
   }
 }
 
+// The interval parameters of a type: clip types take (1 - eps_low, 1 + eps_high), the others their two values as given.
+__device__ __forceinline__ bool is_interval_type(int type) {
+  return type == SKYRL_POLICY_LOSS_REGULAR || type == SKYRL_POLICY_LOSS_DUAL_CLIP || type == SKYRL_POLICY_LOSS_GSPO ||
+         type == SKYRL_POLICY_LOSS_CISPO || type == SKYRL_POLICY_LOSS_ROLLOUT_IS;
+}
+
 __global__ __launch_bounds__(1024) void policy_loss_kernel(const float* __restrict__ lp, const float* __restrict__ old,
                                                            const float* __restrict__ adv, const float* __restrict__ mask,
                                                            const float* __restrict__ weight, int64_t T, float eps_low,
@@ -79,11 +130,11 @@ __global__ __launch_bounds__(1024) void policy_loss_kernel(const float* __restri
                                                            float* __restrict__ g) {
   __shared__ float red[3][16];
   float s_loss = 0.f, s_clip = 0.f, s_mask = 0.f;
-  const float lo = 1.f - eps_low, hi = 1.f + eps_high;
+  const float lo = is_interval_type(type) ? 1.f - eps_low : eps_low, hi = is_interval_type(type) ? 1.f + eps_high : eps_high;
   for (int64_t t = threadIdx.x; t < T; t += blockDim.x) {
     float loss, dloss, stat;
     const bool ce = type == SKYRL_POLICY_LOSS_CROSS_ENTROPY;  // reads neither old nor adv
-    policy_term(type, lp[t], ce ? 0.f : old[t], ce ? 0.f : adv[t], lo, hi, clip_c, loss, dloss, stat);
+    policy_term(type, lp[t], ce ? 0.f : old[t], ce ? 0.f : adv[t], lo, hi, clip_c, 0.f, loss, dloss, stat);
     const float m = mask ? mask[t] : 1.f;
     const float w = weight ? m * weight[t] : m;
     s_loss += loss * w;
@@ -257,6 +308,13 @@ __global__ __launch_bounds__(kRowThreads) void actor_loss_rows_kernel(const Acto
   if (a.mask)
     for (int64_t c = threadIdx.x; c < a.cols; c += kRowThreads) msum += a.mask[row0 + c];
   const float row_mask = a.mask ? block_sum(msum, red) : (float)a.cols;
+  float row_lr = 0.f;  // masked mean of lp - old over the row: the sequence-level log-ratio
+  if (a.loss_type == SKYRL_POLICY_LOSS_GSPO) {
+    float lr = 0.f;
+    for (int64_t c = threadIdx.x; c < a.cols; c += kRowThreads)
+      lr += (a.lp[row0 + c] - a.old[row0 + c]) * (a.mask ? a.mask[row0 + c] : 1.f);
+    row_lr = block_sum(lr, red) / (a.mask ? fmaxf(row_mask, 1.f) : (float)a.cols);
+  }
   const float kl_denom = fmaxf(row_mask, 1.f);
   const float kl_gscale = a.term_scale * a.kl_coef / (kl_denom * (float)a.rows);
   const bool ce = a.loss_type == SKYRL_POLICY_LOSS_CROSS_ENTROPY;
@@ -266,7 +324,7 @@ __global__ __launch_bounds__(kRowThreads) void actor_loss_rows_kernel(const Acto
     const float lp = a.lp[i];
     const float m = a.mask ? a.mask[i] : 1.f;
     float loss, dloss, stat;
-    policy_term(a.loss_type, lp, ce ? 0.f : a.old[i], ce ? 0.f : a.adv[i], a.lo, a.hi, a.clip_c, loss, dloss, stat);
+    policy_term(a.loss_type, lp, ce ? 0.f : a.old[i], ce ? 0.f : a.adv[i], a.lo, a.hi, a.clip_c, row_lr, loss, dloss, stat);
     const float w = a.weight ? m * a.weight[i] : m;
     s_loss += loss * w;
     s_stat += stat * m;
@@ -312,6 +370,18 @@ __global__ __launch_bounds__(kRowThreads) void actor_loss_finish_kernel(const Ac
 }
 
 bool finite(float x) { return std::isfinite(x); }
+bool valid_loss_type(int t) { return t >= SKYRL_POLICY_LOSS_REGULAR && t <= SKYRL_POLICY_LOSS_DPPO_KL; }
+bool interval_type(int t) {
+  return t == SKYRL_POLICY_LOSS_REGULAR || t == SKYRL_POLICY_LOSS_DUAL_CLIP || t == SKYRL_POLICY_LOSS_GSPO ||
+         t == SKYRL_POLICY_LOSS_CISPO || t == SKYRL_POLICY_LOSS_ROLLOUT_IS;
+}
+// Types that read their two parameters need them finite (SAPO's temperatures also non-zero); the dual clip its third.
+bool valid_loss_params(int t, float a, float b, float c) {
+  if (t == SKYRL_POLICY_LOSS_CROSS_ENTROPY || t == SKYRL_POLICY_LOSS_IMPORTANCE_SAMPLING) return true;
+  if (!finite(a) || !finite(b)) return false;
+  if (t == SKYRL_POLICY_LOSS_SAPO && (a == 0.f || b == 0.f)) return false;
+  return t != SKYRL_POLICY_LOSS_DUAL_CLIP || finite(c);
+}
 
 }  // namespace
 
@@ -320,13 +390,12 @@ extern "C" {
 int skyrl_ppo_policy_loss(const float* logprobs, const float* old_logprobs, const float* advantages, const float* loss_mask,
                           const float* loss_weight, int64_t T, float eps_clip_low, float eps_clip_high, float clip_ratio_c,
                           int loss_type, float* out3, float* dlogprobs, void* stream) {
-  if (loss_type < SKYRL_POLICY_LOSS_REGULAR || loss_type > SKYRL_POLICY_LOSS_IMPORTANCE_SAMPLING) return SKYRL_LMHEAD_ERR_ARG;
+  // the sequence-level type needs rows: it is part of skyrl_actor_loss only
+  if (!valid_loss_type(loss_type) || loss_type == SKYRL_POLICY_LOSS_GSPO) return SKYRL_LMHEAD_ERR_ARG;
   const bool needs_old = loss_type != SKYRL_POLICY_LOSS_CROSS_ENTROPY;
   if (!logprobs || !out3 || (needs_old && (!old_logprobs || !advantages))) return SKYRL_LMHEAD_ERR_NULL;
   if (T < 1) return SKYRL_LMHEAD_ERR_SHAPE;
-  const bool clips = loss_type == SKYRL_POLICY_LOSS_REGULAR || loss_type == SKYRL_POLICY_LOSS_DUAL_CLIP;
-  if (clips && (!finite(eps_clip_low) || !finite(eps_clip_high))) return SKYRL_LMHEAD_ERR_ARG;
-  if (loss_type == SKYRL_POLICY_LOSS_DUAL_CLIP && !finite(clip_ratio_c)) return SKYRL_LMHEAD_ERR_ARG;
+  if (!valid_loss_params(loss_type, eps_clip_low, eps_clip_high, clip_ratio_c)) return SKYRL_LMHEAD_ERR_ARG;
   hipLaunchKernelGGL(policy_loss_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, logprobs, old_logprobs, advantages,
                      loss_mask, loss_weight, T, eps_clip_low, eps_clip_high, clip_ratio_c, loss_type, out3, dlogprobs);
   return (int)hipGetLastError();
@@ -350,19 +419,18 @@ int skyrl_actor_loss(const float* logprobs, const float* old_logprobs, const flo
                      int loss_type, float eps_clip_low, float eps_clip_high, float clip_ratio_c, int kl_estimator,
                      float policy_scale, float term_scale, float kl_coef, float entropy_coef, float* row_sums, float* out6,
                      float* dlogprobs, float* dentropy, void* stream) {
-  if (loss_type < SKYRL_POLICY_LOSS_REGULAR || loss_type > SKYRL_POLICY_LOSS_IMPORTANCE_SAMPLING) return SKYRL_LMHEAD_ERR_ARG;
+  if (!valid_loss_type(loss_type)) return SKYRL_LMHEAD_ERR_ARG;
   if (base_logprobs && (kl_estimator < SKYRL_KL_K1 || kl_estimator > SKYRL_KL_K3)) return SKYRL_LMHEAD_ERR_ARG;
   const bool needs_old = loss_type != SKYRL_POLICY_LOSS_CROSS_ENTROPY;
   if (!logprobs || !row_sums || !out6 || (needs_old && (!old_logprobs || !advantages))) return SKYRL_LMHEAD_ERR_NULL;
   if (dentropy && !entropy) return SKYRL_LMHEAD_ERR_NULL;
   if (rows < 1 || cols < 1 || rows >= (int64_t(1) << 31)) return SKYRL_LMHEAD_ERR_SHAPE;
-  const bool clips = loss_type == SKYRL_POLICY_LOSS_REGULAR || loss_type == SKYRL_POLICY_LOSS_DUAL_CLIP;
-  if (clips && (!finite(eps_clip_low) || !finite(eps_clip_high))) return SKYRL_LMHEAD_ERR_ARG;
-  if (loss_type == SKYRL_POLICY_LOSS_DUAL_CLIP && !finite(clip_ratio_c)) return SKYRL_LMHEAD_ERR_ARG;
+  if (!valid_loss_params(loss_type, eps_clip_low, eps_clip_high, clip_ratio_c)) return SKYRL_LMHEAD_ERR_ARG;
   if (!finite(policy_scale) || !finite(term_scale) || !finite(kl_coef) || !finite(entropy_coef)) return SKYRL_LMHEAD_ERR_ARG;
   const ActorLossArgs a{logprobs,   old_logprobs,       advantages,         loss_mask,    loss_weight,  base_logprobs, entropy,
-                        rows,       cols,               loss_type,          kl_estimator, 1.f - eps_clip_low,
-                        1.f + eps_clip_high, clip_ratio_c, policy_scale,    term_scale,   kl_coef,      entropy_coef,
+                        rows,       cols,               loss_type,          kl_estimator,
+                        interval_type(loss_type) ? 1.f - eps_clip_low : eps_clip_low,
+                        interval_type(loss_type) ? 1.f + eps_clip_high : eps_clip_high, clip_ratio_c, policy_scale,    term_scale,   kl_coef,      entropy_coef,
                         row_sums,   out6,               dlogprobs,          dentropy};
   hipStream_t s = (hipStream_t)stream;
   hipLaunchKernelGGL(actor_loss_rows_kernel, dim3((unsigned)rows), dim3(kRowThreads), 0, s, a);

@@ -6,6 +6,8 @@ and results:
 * ``ppo_policy_loss``           :555-588  (policy loss types "regular" and "dual_clip") -> ``(loss, {"clip_ratio": ...})``
 * ``cross_entropy_loss``        :1056-1092 -> ``(loss, {"clip_ratio": 0.0})``
 * ``importance_sampling_loss``  :1095-1142 -> ``(loss, {"importance_ratio": ...})``
+* ``sapo_policy_loss``          :590-660, ``gspo_policy_loss`` :663-729, ``compute_policy_loss_cispo`` :732-821,
+  ``rollout_is_policy_loss`` :824-863, ``dppo_policy_loss`` :866-935 -> ``(loss, {"clip_ratio": ...})``
 * ``compute_approx_kl``         :88-126    -> per-token KL estimate ``[B, S]``
 * ``masked_mean``               torch_utils.py:180-184
 
@@ -19,8 +21,11 @@ value, statistics and gradient, so the upstream gradient of ``skyrl_lmhead_bwd``
 ``[B, S]`` tensors and, with ``sync_metrics=False``, without a host synchronisation.
 
 Off-policy correction (``apply_off_policy_correction``, off_policy_correction_utils.py:351-385) multiplies the per-token
-loss by an importance ratio that does not depend on the policy's log-probabilities: pass that ratio as ``loss_weight``.
-Computing it from ``rollout_logprobs`` is outside this module, so ``ppo_policy_loss`` needs ``rollout_logprobs=None``.
+loss by an importance ratio that does not depend on the policy's log-probabilities and may thin the loss mask: compute both
+with the trainer's own helper and pass the ratio as ``loss_weight`` and the thinned mask as ``loss_mask``.  Computing them
+from ``rollout_logprobs`` is outside this module: the losses raise when the config switches a correction on, and otherwise
+use ``rollout_logprobs`` only where the loss itself is anchored on them (rollout-IS, DPPO, CISPO with the rollout anchor).
+The two covariance-based types (clip_cov, kl_cov) pick a random subset / a top-k over the whole batch and are not here.
 """
 
 from __future__ import annotations
@@ -32,10 +37,37 @@ import torch
 from . import _lib
 from .ops import _require_device
 
-__all__ = ["ppo_policy_loss", "cross_entropy_loss", "importance_sampling_loss", "compute_approx_kl", "approx_kl_loss",
+__all__ = ["ppo_policy_loss", "cross_entropy_loss", "importance_sampling_loss", "sapo_policy_loss", "gspo_policy_loss",
+           "compute_policy_loss_cispo", "rollout_is_policy_loss", "dppo_policy_loss", "compute_approx_kl", "approx_kl_loss",
            "masked_mean", "actor_loss", "ppo_policy_loss_terms"]
 
 LOSS_REGULAR, LOSS_DUAL_CLIP, LOSS_CROSS_ENTROPY, LOSS_IMPORTANCE_SAMPLING = 0, 1, 2, 3
+LOSS_GSPO, LOSS_SAPO, LOSS_CISPO, LOSS_ROLLOUT_IS, LOSS_DPPO_TV, LOSS_DPPO_KL = 4, 5, 6, 7, 8, 9
+
+
+def _get(obj: Any, name: str, default: Any = None) -> Any:
+    """Field of a config given as an object or as a mapping."""
+    if obj is None:
+        return default
+    if isinstance(obj, dict):
+        return obj.get(name, default)
+    return getattr(obj, name, default)
+
+
+def _reject_off_policy_correction(config: Any, rollout_logprobs: Optional[torch.Tensor]) -> None:
+    """The reference corrects only when rollout log-probabilities are given and one of the config's switches is on
+    (off_policy_correction_utils.py:285-305, 388-391)."""
+    opc = _get(config, "off_policy_correction")
+    if rollout_logprobs is None or opc is None:
+        return
+    on = (_get(opc, "tis_ratio_type") is not None or _get(opc, "sequence_mask_metric") is not None
+          or _get(opc, "outlier_token_is_threshold_low") is not None
+          or _get(opc, "outlier_token_is_threshold_high") is not None
+          or (_get(opc, "token_mask_is_threshold_low") is not None and _get(opc, "token_mask_is_threshold_high") is not None))
+    if on:
+        raise NotImplementedError(
+            "off-policy correction from rollout_logprobs is not part of the fused loss; compute the importance ratio and the "
+            "thinned mask with the trainer's own helper and pass them as loss_weight and loss_mask")
 KL_ESTIMATORS = {"k1": 0, "abs": 1, "k2": 2, "k3": 3}
 
 
@@ -130,10 +162,7 @@ def ppo_policy_loss(
     """
     loss_type = getattr(config, "policy_loss_type", "regular")
     assert loss_type in ["regular", "dual_clip"], "loss_type must be either 'regular' or 'dual_clip'"
-    if rollout_logprobs is not None:
-        raise NotImplementedError(
-            "off-policy correction from rollout_logprobs is not part of the fused loss; compute the importance ratio with "
-            "the trainer's own helper and pass it as loss_weight")
+    _reject_off_policy_correction(config, rollout_logprobs)
     dual = loss_type == "dual_clip"
     loss, sums = _PolicyLoss.apply(log_probs, old_log_probs, advantages, loss_mask, loss_weight, float(config.eps_clip_low),
                                    float(config.eps_clip_high), float(getattr(config, "clip_ratio_c", 0.0)) if dual else 0.0,
@@ -172,6 +201,110 @@ def importance_sampling_loss(
                                    LOSS_IMPORTANCE_SAMPLING)
     ratio = sums[1] / sums[2]
     return loss, {"importance_ratio": ratio.item() if sync_metrics else ratio}
+
+
+def _type_parameters(config: Any, name: str, rollout_logprobs: Optional[torch.Tensor], old_log_probs):
+    """``(loss_type, a, b, c, behaviour log-probabilities)`` of a policy-loss type as the kernels take them: the two bounds
+    (or temperatures, or thresholds), the dual-clip constant, and the log-probabilities its ratio is anchored on."""
+    if name in ("regular", "dual_clip", "gspo"):
+        dual = name == "dual_clip"
+        return ({"regular": LOSS_REGULAR, "dual_clip": LOSS_DUAL_CLIP, "gspo": LOSS_GSPO}[name], float(config.eps_clip_low),
+                float(config.eps_clip_high), float(getattr(config, "clip_ratio_c", 0.0)) if dual else 0.0, old_log_probs)
+    if name in ("cross_entropy", "importance_sampling"):
+        return (LOSS_CROSS_ENTROPY if name == "cross_entropy" else LOSS_IMPORTANCE_SAMPLING), 0.0, 0.0, 0.0, old_log_probs
+    if name == "sapo":
+        sapo = _get(config, "sapo")
+        return LOSS_SAPO, float(_get(sapo, "tau_pos", 1.0)), float(_get(sapo, "tau_neg", 1.05)), 0.0, old_log_probs
+    if name == "cispo":
+        cispo = _get(config, "cispo")
+        behaviour = old_log_probs
+        if _get(cispo, "cispo_anchor", "old") == "rollout":
+            assert rollout_logprobs is not None, "rollout_logprobs are required for cispo with cispo_anchor='rollout'"
+            tis = _get(_get(config, "off_policy_correction"), "tis_ratio_type")
+            if tis is not None:
+                raise ValueError("cispo_anchor='rollout' is already rollout-anchored and performs the off-policy correction; "
+                                 f"TIS (tis_ratio_type={tis!r}) would double-count it. Set "
+                                 "off_policy_correction.tis_ratio_type=None.")
+            behaviour = rollout_logprobs
+        return (LOSS_CISPO, float(_get(cispo, "cispo_eps_clip_low", 1.0)), float(_get(cispo, "cispo_eps_clip_high", 4.0)), 0.0,
+                behaviour)
+    if name == "rollout_is":
+        assert rollout_logprobs is not None, "rollout_logprobs are required for rollout_is"
+        return LOSS_ROLLOUT_IS, float(config.eps_clip_low), float(config.eps_clip_high), 0.0, rollout_logprobs
+    if name == "dppo":
+        dppo = _get(config, "dppo")
+        kind = _get(dppo, "dppo_type", "binary_tv")
+        if kind not in ("binary_tv", "binary_kl"):
+            raise ValueError(f"Unknown DPPO type: {kind}. Must be 'binary_tv' or 'binary_kl'.")
+        return (LOSS_DPPO_TV if kind == "binary_tv" else LOSS_DPPO_KL, float(_get(dppo, "delta_low", 0.2)),
+                float(_get(dppo, "delta_high", 0.2)), 0.0, rollout_logprobs if rollout_logprobs is not None else old_log_probs)
+    raise NotImplementedError(f"policy_loss_type {name!r} is not part of the fused losses; fused types: "
+                              f"{sorted(_POLICY_LOSS_NAMES)}")
+
+
+_POLICY_LOSS_NAMES = ("regular", "dual_clip", "cross_entropy", "importance_sampling", "gspo", "sapo", "cispo", "rollout_is",
+                      "dppo")
+
+
+def _elementwise_loss(name: str, log_probs, old_log_probs, advantages, config, loss_mask, rollout_logprobs, loss_weight,
+                      sync_metrics: bool):
+    _reject_off_policy_correction(config, rollout_logprobs)
+    loss_type, a, b, c, behaviour = _type_parameters(config, name, rollout_logprobs, old_log_probs)
+    loss, sums = _PolicyLoss.apply(log_probs, behaviour, advantages, loss_mask, loss_weight, a, b, c, loss_type)
+    clip_ratio = sums[1] / sums[2].clamp(min=1.0)
+    return loss, {"clip_ratio": clip_ratio.item() if sync_metrics else clip_ratio}
+
+
+def sapo_policy_loss(log_probs, old_log_probs, advantages, config, loss_mask=None, rollout_logprobs=None, *,
+                     loss_weight=None) -> Tuple[torch.Tensor, Dict[str, Any]]:
+    """Soft adaptive policy optimisation (reference ``sapo_policy_loss``, ppo_utils.py:590-660): the gate
+    ``sigmoid(tau (r - 1)) 4 / tau`` replaces the clipped ratio, ``tau = config.sapo.tau_pos`` where the advantage is
+    positive, ``tau_neg`` elsewhere.  ``clip_ratio`` is 0.0 as in the reference."""
+    loss, _ = _elementwise_loss("sapo", log_probs, old_log_probs, advantages, config, loss_mask, rollout_logprobs, loss_weight,
+                                False)
+    return loss, {"clip_ratio": 0.0}
+
+
+def compute_policy_loss_cispo(log_probs, old_log_probs, advantages, config, loss_mask=None, rollout_logprobs=None, *,
+                              loss_weight=None, sync_metrics: bool = True) -> Tuple[torch.Tensor, Dict[str, Any]]:
+    """Clipped importance-weight policy optimisation (reference ``compute_policy_loss_cispo``, ppo_utils.py:732-821):
+    ``-A stopgrad(clamp(r, 1 - cispo_eps_clip_low, 1 + cispo_eps_clip_high)) log_probs`` with the ratio anchored as
+    ``config.cispo.cispo_anchor`` says.  Returns ``clip_ratio``; the reference's four ``cispo/ratio_*`` diagnostics are not
+    computed."""
+    return _elementwise_loss("cispo", log_probs, old_log_probs, advantages, config, loss_mask, rollout_logprobs, loss_weight,
+                             sync_metrics)
+
+
+def rollout_is_policy_loss(log_probs, old_log_probs, advantages, config, loss_mask=None, rollout_logprobs=None, *,
+                           loss_weight=None, sync_metrics: bool = True) -> Tuple[torch.Tensor, Dict[str, Any]]:
+    """Calibrated importance-weighted policy gradient on the rollout log-probabilities (reference
+    ``rollout_is_policy_loss``, ppo_utils.py:824-863): the weight is the ratio inside the open interval
+    ``(1 - eps_clip_low, 1 + eps_clip_high)`` and zero outside; ``old_log_probs`` is not read."""
+    return _elementwise_loss("rollout_is", log_probs, old_log_probs, advantages, config, loss_mask, rollout_logprobs,
+                             loss_weight, sync_metrics)
+
+
+def dppo_policy_loss(log_probs, old_log_probs, advantages, config, loss_mask=None, rollout_logprobs=None, *,
+                     loss_weight=None, sync_metrics: bool = True) -> Tuple[torch.Tensor, Dict[str, Any]]:
+    """Divergence proximal policy optimisation (reference ``dppo_policy_loss``, ppo_utils.py:866-935): the unclipped
+    surrogate times a binary trust-region mask (``config.dppo.dppo_type`` "binary_tv" or "binary_kl", thresholds
+    ``delta_low`` / ``delta_high``); the rollout log-probabilities are the behaviour policy when given."""
+    return _elementwise_loss("dppo", log_probs, old_log_probs, advantages, config, loss_mask, rollout_logprobs, loss_weight,
+                             sync_metrics)
+
+
+def gspo_policy_loss(log_probs, old_log_probs, advantages, config, loss_mask=None, rollout_logprobs=None, *,
+                     loss_weight=None, sync_metrics: bool = True) -> Tuple[torch.Tensor, Dict[str, Any]]:
+    """Group sequence policy optimisation, token-level variant (reference ``gspo_policy_loss``, ppo_utils.py:663-729): the
+    clipped surrogate with every token's ratio replaced by its sequence's, ``exp(min(masked row mean of the log-ratio,
+    10))``.  ``log_probs`` is ``[B, S]``; the rows are the sequences."""
+    _reject_off_policy_correction(config, rollout_logprobs)
+    if log_probs.dim() < 2:
+        raise ValueError("gspo_policy_loss needs [B, S] inputs: the importance weight is a row mean")
+    scalars = (LOSS_GSPO, float(config.eps_clip_low), float(config.eps_clip_high), 0.0, 3, 1.0, 1.0, 0.0, 0.0)
+    loss, out6 = _ActorLoss.apply(log_probs, None, (old_log_probs, advantages, loss_mask, loss_weight, None), scalars)
+    clip_ratio = out6[2] / out6[3].clamp(min=1.0)
+    return loss, {"clip_ratio": clip_ratio.item() if sync_metrics else clip_ratio}
 
 
 # ----------------------------------------------------------------------------------------------------------------------
@@ -326,10 +459,6 @@ def masked_mean(tensor: torch.Tensor, mask: Optional[torch.Tensor], dim: Optiona
 # ----------------------------------------------------------------------------------------------------------------------
 # the assembled actor loss
 # ----------------------------------------------------------------------------------------------------------------------
-_POLICY_LOSS_TYPES = {"regular": LOSS_REGULAR, "dual_clip": LOSS_DUAL_CLIP, "cross_entropy": LOSS_CROSS_ENTROPY,
-                      "importance_sampling": LOSS_IMPORTANCE_SAMPLING}
-
-
 @torch.library.custom_op("skyrl_amd::actor_loss", mutates_args=())
 def _actor_loss(log_probs: torch.Tensor, old_log_probs: Optional[torch.Tensor], advantages: Optional[torch.Tensor],
                 loss_mask: Optional[torch.Tensor], loss_weight: Optional[torch.Tensor], base_log_probs: Optional[torch.Tensor],
@@ -405,6 +534,7 @@ def actor_loss(
     base_log_probs: Optional[torch.Tensor] = None,
     entropy: Optional[torch.Tensor] = None,
     loss_weight: Optional[torch.Tensor] = None,
+    rollout_logprobs: Optional[torch.Tensor] = None,
     policy_scale: float = 1.0,
     term_scale: float = 1.0,
 ) -> Tuple[torch.Tensor, Dict[str, torch.Tensor]]:
@@ -413,9 +543,10 @@ def actor_loss(
 
         ``policy_loss * policy_scale + (kl_loss * config.kl_loss_coef - entropy * config.entropy_loss_coef) * term_scale``
 
-    ``config`` is the algorithm config: ``policy_loss_type`` (regular, dual_clip, cross_entropy, importance_sampling),
-    ``eps_clip_low`` / ``eps_clip_high`` / ``clip_ratio_c``, ``use_kl_loss`` + ``kl_loss_coef`` + ``kl_estimator_type``,
-    ``use_entropy_loss`` + ``entropy_loss_coef``.  The KL term needs ``base_log_probs``; the entropy term needs ``entropy``
+    ``config`` is the algorithm config: ``policy_loss_type`` (regular, dual_clip, cross_entropy, importance_sampling, gspo,
+    sapo, cispo, rollout_is, dppo) with that type's parameters (``eps_clip_low`` / ``eps_clip_high`` / ``clip_ratio_c``,
+    ``sapo``, ``cispo``, ``dppo``), ``use_kl_loss`` + ``kl_loss_coef`` + ``kl_estimator_type``, ``use_entropy_loss`` +
+    ``entropy_loss_coef``.  ``rollout_logprobs`` are read by the types anchored on them.  The KL term needs ``base_log_probs``; the entropy term needs ``entropy``
     (``[B, S]``, e.g. from ``action_log_probs_from_hidden(..., compute_entropy=True)``) and sends a gradient into it.
     ``policy_scale`` is the worker's ``grad_sum_correction_factor``, ``term_scale`` its ``microbatch_weight``.
 
@@ -423,10 +554,8 @@ def actor_loss(
     and ``clip_ratio`` (``importance_ratio`` for the importance-sampling loss).
     """
     name = getattr(config, "policy_loss_type", "regular")
-    if name not in _POLICY_LOSS_TYPES:
-        raise NotImplementedError(f"policy_loss_type {name!r} is not part of the fused actor loss; fused types: "
-                                  f"{sorted(_POLICY_LOSS_TYPES)}")
-    loss_type = _POLICY_LOSS_TYPES[name]
+    _reject_off_policy_correction(config, rollout_logprobs)
+    loss_type, a, b, c, behaviour = _type_parameters(config, name, rollout_logprobs, old_log_probs)
     use_kl = bool(getattr(config, "use_kl_loss", False))
     if use_kl and base_log_probs is None:
         raise ValueError("use_kl_loss needs base_log_probs")
@@ -436,12 +565,9 @@ def actor_loss(
     estimator = getattr(config, "kl_estimator_type", "k3")
     if use_kl and estimator not in KL_ESTIMATORS:
         raise ValueError(f"Invalid KL estimator type: {estimator}")
-    clips = loss_type in (LOSS_REGULAR, LOSS_DUAL_CLIP)
-    scalars = (loss_type, float(config.eps_clip_low) if clips else 0.0, float(config.eps_clip_high) if clips else 0.0,
-               float(getattr(config, "clip_ratio_c", 0.0)) if loss_type == LOSS_DUAL_CLIP else 0.0,
-               KL_ESTIMATORS.get(estimator, 3), float(policy_scale), float(term_scale),
+    scalars = (loss_type, a, b, c, KL_ESTIMATORS.get(estimator, 3), float(policy_scale), float(term_scale),
                float(config.kl_loss_coef) if use_kl else 0.0, float(config.entropy_loss_coef) if use_ent else 0.0)
-    consts = (old_log_probs, advantages, loss_mask, loss_weight, base_log_probs if use_kl else None)
+    consts = (behaviour, advantages, loss_mask, loss_weight, base_log_probs if use_kl else None)
     # The entropy is reduced for the metric even when it is not part of the loss, as the worker does.
     loss, out6 = _ActorLoss.apply(log_probs, entropy, consts, scalars)
     stat = out6[2] / (out6[3] if loss_type == LOSS_IMPORTANCE_SAMPLING else out6[3].clamp(min=1.0))

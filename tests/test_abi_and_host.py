@@ -135,7 +135,13 @@ def test_ppo_policy_loss_mirror_contract():
     cfg = SimpleNamespace(policy_loss_type="regular", eps_clip_low=0.2, eps_clip_high=0.2, clip_ratio_c=3.0)
     with pytest.raises(AssertionError):
         ppo_policy_loss(x, x, x, SimpleNamespace(policy_loss_type="gspo", eps_clip_low=0.2, eps_clip_high=0.2))
+    # rollout log-probabilities are used for off-policy correction only: refused when the config switches one on,
+    # ignored (as in the reference) when it does not
+    cfg.off_policy_correction = SimpleNamespace(tis_ratio_type="token")
     with pytest.raises(NotImplementedError):
+        ppo_policy_loss(x, x, x, cfg, rollout_logprobs=x)
+    cfg.off_policy_correction = {"tis_ratio_type": None, "sequence_mask_metric": None}
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
         ppo_policy_loss(x, x, x, cfg, rollout_logprobs=x)
     with pytest.raises(RuntimeError, match="no CPU implementation"):
         ppo_policy_loss(x, x, x, cfg)

@@ -479,6 +479,174 @@ def test_cross_entropy_and_importance_sampling_by_hand():
     assert big.item() == pytest.approx(-math.exp(30.0), rel=1e-6)
 
 
+def _grad(fn, lp):
+    x = torch.tensor(lp, dtype=torch.float64, requires_grad=True)
+    loss, stat = fn(x)
+    loss.backward()
+    return loss.item(), stat.item(), x.grad.tolist()
+
+
+def _t(v):
+    return torch.tensor(v, dtype=torch.float64)
+
+
+def test_sapo_by_hand():
+    sig = lambda u: 1.0 / (1.0 + math.exp(-u))  # noqa: E731
+    # ratio 1: the gate is sigmoid(0) * 4 / tau = 2 / tau, whatever the sign of A picks
+    loss, stat, g = _grad(lambda x: O.sapo_policy_loss(x, _t([0.3, 0.3]), _t([1.5, -1.5]), 1.0, 1.25), [0.3, 0.3])
+    assert loss == pytest.approx(-(2.0 / 1.0) * 1.5 + (2.0 / 1.25) * 1.5) and stat == 0.0
+    # d gate / d lp at ratio 1 = 4 s (1 - s) ratio = 1 for every tau: there SAPO moves like the plain surrogate -ratio*A
+    assert g == pytest.approx([-1.5, 1.5])
+    # ratio 2, A = 3 > 0 -> tau_pos = 0.5; ratio 1/2, A = -2 (A <= 0 -> tau_neg = 2); A = 0 takes tau_neg and gives 0
+    loss, _, g = _grad(lambda x: O.sapo_policy_loss(x, _t([0.0, 0.0, 0.0]), _t([3.0, -2.0, 0.0]), 0.5, 2.0),
+                       [math.log(2.0), math.log(0.5), 0.7])
+    s1, s2 = sig(0.5 * 1.0), sig(2.0 * -0.5)
+    assert loss == pytest.approx(-s1 * 8.0 * 3.0 + s2 * 2.0 * 2.0)
+    assert g == pytest.approx([-4 * 3.0 * s1 * (1 - s1) * 2.0, 4 * 2.0 * s2 * (1 - s2) * 0.5, 0.0])
+    # the log-ratio is clamped at 20 and passes no gradient beyond
+    loss, _, g = _grad(lambda x: O.sapo_policy_loss(x, _t([0.0]), _t([1.0]), 1.0, 1.0), [25.0])
+    assert loss == pytest.approx(-4.0) and g == pytest.approx([0.0])
+    # mask: the masked sum
+    loss, _, _ = _grad(lambda x: O.sapo_policy_loss(x, _t([0.0, 0.0]), _t([1.0, 1.0]), 1.0, 1.0, _t([0.0, 1.0])), [0.0, 0.0])
+    assert loss == pytest.approx(-2.0)
+
+
+def test_gspo_by_hand_and_single_token_rows_are_ppo():
+    ln2 = math.log(2.0)
+    # one row, log-ratios (ln 2, 0, 3 ln 2) -> mean = 4/3 ln 2, masked (1, 1, 0) -> mean = ln 2 / 2: ratio sqrt 2 for all
+    lp, old, adv = [[ln2, 0.0, 3 * ln2]], _t([[0.0, 0.0, 0.0]]), _t([[1.0, -1.0, 5.0]])
+    mask = _t([[1.0, 1.0, 0.0]])
+    r = math.sqrt(2.0)
+    loss, clip, g = _grad(lambda x: O.gspo_policy_loss(x, old, adv, 0.2, 0.5, mask), lp)
+    # token 0: A > 0, ratio 1.414 inside [0.8, 1.5] -> -r, gradient -r (to the token's own log-prob, weight 1);
+    # token 1: A < 0 -> +r, gradient +r; token 2 masked
+    assert loss == pytest.approx(-r + r) and clip == 0.0 and g[0] == pytest.approx([-r, r, 0.0])
+    # tighter interval [0.8, 1.2]: token 0 clipped (-1.2, no gradient), token 1 takes the unclipped branch
+    loss, clip, g = _grad(lambda x: O.gspo_policy_loss(x, old, adv, 0.2, 0.2, mask), lp)
+    assert loss == pytest.approx(-1.2 + r) and clip == pytest.approx(0.5) and g[0] == pytest.approx([0.0, r, 0.0])
+    # without a mask the row mean is the plain mean: ratio 2^(4/3)
+    loss, _, _ = _grad(lambda x: O.gspo_policy_loss(x, old, adv, 0.2, 9.0), lp)
+    assert loss == pytest.approx(-(2 ** (4 / 3)) * (1.0 - 1.0 + 5.0))
+    # the clamp of the log weight at 10: ratio e^10, no gradient
+    loss, _, g = _grad(lambda x: O.gspo_policy_loss(x, _t([[0.0]]), _t([[-1.0]]), 0.2, 0.2), [[12.0]])
+    assert loss == pytest.approx(math.exp(10.0)) and g[0] == pytest.approx([0.0])
+    # rows of one token: the sequence ratio is the token ratio, so GSPO is the clipped surrogate pinned above
+    gen = torch.Generator().manual_seed(5)
+    lp1 = torch.randn(40, 1, generator=gen, dtype=torch.float64) * 0.4
+    old1 = torch.randn(40, 1, generator=gen, dtype=torch.float64) * 0.4
+    adv1 = torch.randn(40, 1, generator=gen, dtype=torch.float64)
+    x, y = lp1.clone().requires_grad_(True), lp1.clone().requires_grad_(True)
+    a, ca = O.gspo_policy_loss(x, old1, adv1, 0.2, 0.28)
+    b, cb = O.ppo_policy_loss(y, old1, adv1, 0.2, 0.28)
+    a.backward(), b.backward()
+    assert a.item() == pytest.approx(b.item()) and ca.item() == cb.item()
+    assert torch.allclose(x.grad, y.grad, atol=1e-12)
+
+
+def test_cispo_and_rollout_is_by_hand():
+    ln2, ln3, lnh = math.log(2.0), math.log(3.0), math.log(0.5)
+    lp = [ln2 - 1.0, ln3 - 1.0, lnh - 1.0, -1.0]                   # ratios 2, 3, 1/2, 1 against old = -1
+    old, adv = _t([-1.0] * 4), _t([1.0, 2.0, -1.0, -3.0])
+    # CISPO with [0.75, 2.5]: weights 2, 2.5 (capped), 0.75 (capped), 1
+    loss, clip, g = _grad(lambda x: O.cispo_policy_loss(x, old, adv, 0.25, 1.5), lp)
+    w = [2.0, 2.5, 0.75, 1.0]
+    assert loss == pytest.approx(-sum(a * wi * l for a, wi, l in zip(adv.tolist(), w, lp)))
+    assert clip == pytest.approx(0.5) and g == pytest.approx([-2.0, -5.0, 0.75, 3.0])
+    # every token keeps a gradient; with a mask the clip fraction counts unmasked tokens only
+    _, clip, g = _grad(lambda x: O.cispo_policy_loss(x, old, adv, 0.25, 1.5, _t([1.0, 0.0, 1.0, 1.0])), lp)
+    assert clip == pytest.approx(1 / 3) and g == pytest.approx([-2.0, 0.0, 0.75, 3.0])
+    # rollout-IS with the same interval: the two outside tokens drop to weight 0
+    loss, clip, g = _grad(lambda x: O.rollout_is_policy_loss(x, old, adv, 0.25, 1.5), lp)
+    assert loss == pytest.approx(-(1.0 * 2.0 * lp[0] + -3.0 * 1.0 * lp[3]))
+    assert clip == pytest.approx(0.5) and g == pytest.approx([-2.0, 0.0, 0.0, 3.0])
+    # the interval is open: a ratio exactly on the bound is out for rollout-IS, not clipped for CISPO
+    loss, clip, g = _grad(lambda x: O.rollout_is_policy_loss(x, _t([0.0]), _t([1.0]), 0.5, 1.0), [ln2])
+    assert loss == 0.0 and clip == 1.0 and g == [0.0]
+    loss, clip, g = _grad(lambda x: O.cispo_policy_loss(x, _t([0.0]), _t([1.0]), 0.5, 1.0), [ln2])
+    assert loss == pytest.approx(-2.0 * ln2) and clip == 0.0 and g == pytest.approx([-2.0])
+    # inside the interval the two are the same function
+    a = _grad(lambda x: O.cispo_policy_loss(x, old, adv, 0.9, 9.0), lp)
+    b = _grad(lambda x: O.rollout_is_policy_loss(x, old, adv, 0.9, 9.0), lp)
+    assert a[0] == pytest.approx(b[0]) and a[2] == pytest.approx(b[2]) and a[1] == b[1] == 0.0
+
+
+def test_dppo_by_hand():
+    ln = math.log
+    # probabilities now / behaviour: (0.5, 0.2), (0.2, 0.5), (0.5, 0.2), (0.2, 0.5), (0.3, 0.2)
+    lp = [ln(0.5), ln(0.2), ln(0.5), ln(0.2), ln(0.3)]
+    mu = _t([ln(0.2), ln(0.5), ln(0.2), ln(0.5), ln(0.2)])
+    adv = _t([1.0, 1.0, -1.0, -1.0, 2.0])
+    # TV, delta_low 0.25, delta_high 0.2: token 0 (A > 0, rose by 0.3 > 0.2) out; token 3 (A < 0, fell by 0.3 > 0.25) out;
+    # tokens 1 and 2 moved against their advantage's direction and stay; token 4 rose by 0.1 only
+    loss, clip, g = _grad(lambda x: O.dppo_policy_loss(x, mu, adv, "binary_tv", 0.25, 0.2), lp)
+    assert loss == pytest.approx(-(0.4 * 1.0) + 2.5 * 1.0 - 1.5 * 2.0) and clip == pytest.approx(0.4)
+    assert g == pytest.approx([0.0, -0.4, 2.5, 0.0, -3.0])
+    # the thresholds are per direction: delta_low 0.35 lets token 3 back in
+    loss, clip, _ = _grad(lambda x: O.dppo_policy_loss(x, mu, adv, "binary_tv", 0.35, 0.2), lp)
+    assert loss == pytest.approx(-0.4 + 2.5 + 0.4 - 3.0) and clip == pytest.approx(0.2)
+    # KL: Bernoulli KL(mu || p) = mu ln(mu/p) + (1-mu) ln((1-mu)/(1-p))
+    bkl = lambda m, p: m * ln(m / p) + (1 - m) * ln((1 - m) / (1 - p))  # noqa: E731
+    k0, k3, k4 = bkl(0.2, 0.5), bkl(0.5, 0.2), bkl(0.2, 0.3)
+    assert k4 < 0.05 < k0 < 0.21 < k3                                  # 0.0257, 0.1927, 0.2231
+    loss, clip, g = _grad(lambda x: O.dppo_policy_loss(x, mu, adv, "binary_kl", 0.21, 0.05), lp)
+    assert clip == pytest.approx(0.4) and g == pytest.approx([0.0, -0.4, 2.5, 0.0, -3.0])
+    loss, clip, g = _grad(lambda x: O.dppo_policy_loss(x, mu, adv, "binary_kl", 0.23, 0.2), lp)
+    assert clip == 0.0 and g == pytest.approx([-2.5, -0.4, 2.5, 0.4, -3.0])
+    # nothing masked: the importance-sampling surrogate pinned above
+    ref, _ = O.importance_sampling_loss(_t(lp), mu, adv)
+    assert loss == pytest.approx(ref.item())
+    with pytest.raises(ValueError):
+        O.dppo_policy_loss(_t(lp), mu, adv, "topk_tv", 0.2, 0.2)
+
+
+@pytest.mark.parametrize("kind", ["sapo", "gspo", "cispo", "rollout_is", "dppo_tv", "dppo_kl"])
+def test_further_losses_gradient_matches_finite_differences(kind):
+    """Autograd of the restatement against fp64 central differences of the same surrogate with its stop-gradient factors
+    (the CISPO / rollout-IS weight, the DPPO mask, GSPO's sequence weight) evaluated once at the base point."""
+    gen = torch.Generator().manual_seed(23)
+    rows, cols = 6, 9
+    old = -torch.rand(rows, cols, generator=gen, dtype=torch.float64) * 2 - 0.1
+    lp = (old + torch.randn(rows, cols, generator=gen, dtype=torch.float64) * 0.3).clamp(max=-0.01)
+    adv = torch.randn(rows, cols, generator=gen, dtype=torch.float64)
+    mask = (torch.rand(rows, cols, generator=gen) > 0.3).double()
+    ratio0 = (lp - old).exp()
+    if kind == "sapo":
+        f = lambda x: O.sapo_policy_loss(x, old, adv, 1.0, 1.05, mask)[0]  # noqa: E731
+        frozen = f
+    elif kind == "gspo":
+        f = lambda x: O.gspo_policy_loss(x, old, adv, 0.1, 0.15, mask)[0]  # noqa: E731
+        row0 = O.masked_mean(lp - old, mask, dim=-1).unsqueeze(-1)
+
+        def frozen(x):  # s_i fixed at the base point, times pi(x) / pi(base)
+            r = (x - lp + row0).exp()
+            return -(torch.min(r * adv, r.clamp(0.9, 1.15) * adv) * mask).sum()
+    elif kind == "cispo":
+        f = lambda x: O.cispo_policy_loss(x, old, adv, 0.2, 0.3, mask)[0]  # noqa: E731
+        frozen = lambda x: -(adv * ratio0.clamp(0.8, 1.3) * x * mask).sum()  # noqa: E731
+    elif kind == "rollout_is":
+        f = lambda x: O.rollout_is_policy_loss(x, old, adv, 0.2, 0.3, mask)[0]  # noqa: E731
+        w0 = torch.where((ratio0 > 0.8) & (ratio0 < 1.3), ratio0, torch.zeros_like(ratio0))
+        frozen = lambda x: -(adv * w0 * x * mask).sum()  # noqa: E731
+    else:
+        name = "binary_tv" if kind == "dppo_tv" else "binary_kl"
+        lo, hi = (0.05, 0.04) if kind == "dppo_tv" else (0.02, 0.015)
+        f = lambda x: O.dppo_policy_loss(x, old, adv, name, lo, hi, mask)[0]  # noqa: E731
+        x0 = lp.clone().requires_grad_(True)
+        keep0 = (torch.autograd.grad(f(x0), x0)[0] != 0) | (mask == 0) | (adv == 0)
+        assert 0 < (~keep0).sum() < keep0.numel() / 2                   # the mask does cut some tokens, not most
+        frozen = lambda x: -((x - old).exp() * adv * keep0 * mask).sum()  # noqa: E731
+    x = lp.clone().requires_grad_(True)
+    f(x).backward()
+    assert frozen(lp).item() == pytest.approx(f(lp).item(), rel=1e-12)
+    eps = 1e-6
+    for i in range(rows):
+        for j in range(cols):
+            d = torch.zeros(rows, cols, dtype=torch.float64)
+            d[i, j] = eps
+            fd = (frozen(lp + d) - frozen(lp - d)).item() / (2 * eps)
+            assert x.grad[i, j].item() == pytest.approx(fd, abs=1e-6), f"token {i},{j}"
+
+
 def test_masked_mean_by_hand():
     t = torch.tensor([[1.0, 2.0, 3.0], [4.0, 5.0, 6.0]])
     m = torch.tensor([[1.0, 0.0, 1.0], [0.0, 0.0, 0.0]])

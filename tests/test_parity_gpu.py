@@ -456,6 +456,148 @@ def test_cross_entropy_and_importance_sampling_losses_match_oracle(masked, cuda_
     assert bool((err <= 1e-5 * ref_lp.grad.abs().clamp(min=1.0)).all())
 
 
+def _further_loss_case(kind, masked):
+    """Inputs for one of the further loss types, its config, and the oracle's loss / clip ratio / gradient in fp64.  Tokens
+    whose branch decision sits within 1e-4 of a threshold in fp64 are moved to ratio 1 so that fp32 takes the same branch."""
+    from types import SimpleNamespace
+
+    gen = torch.Generator().manual_seed(31)
+    B, S = 7, 411
+    lp = (torch.randn(B, S, generator=gen) * 0.7 - 1.5).clamp(max=-0.02)
+    old = lp + torch.randn(B, S, generator=gen) * 0.35
+    adv = torch.randn(B, S, generator=gen)
+    adv[3, :5] = 0.0                                            # A = 0: tau_neg side of SAPO, neither DPPO direction
+    mask = None
+    if masked:
+        mask = (torch.rand(B, S, generator=gen) > 0.4).float()
+        mask[2] = 0                                             # a row without loss tokens
+        mask[4, :7] = 0.5                                       # fractional weights
+    weight = (torch.rand(B, S, generator=gen) + 0.5) if masked else None
+    lo, hi = {"sapo": (1.0, 1.05), "gspo": (0.02, 0.03), "cispo": (0.3, 0.5), "rollout_is": (0.3, 0.5),
+              "dppo_tv": (0.06, 0.05), "dppo_kl": (0.02, 0.015)}[kind]
+    ratio = (lp.double() - old.double()).exp()
+    fragile = torch.zeros(B, S, dtype=torch.bool)
+    if kind in ("cispo", "rollout_is"):
+        fragile = ((ratio - (1 - lo)).abs() < 1e-4) | ((ratio - (1 + hi)).abs() < 1e-4)
+    elif kind == "dppo_tv":
+        diff = lp.double().exp() - old.double().exp()
+        fragile = ((diff - hi).abs() < 1e-4) | ((-diff - lo).abs() < 1e-4)
+    elif kind == "dppo_kl":
+        p, mu = lp.double().exp(), old.double().exp()
+        bkl = mu * (old.double() - lp.double()) + (1 - mu) * torch.log((1 - mu) / (1 - p))
+        fragile = ((bkl - hi).abs() < 1e-4) | ((bkl - lo).abs() < 1e-4) | ((p - mu).abs() < 1e-6)
+    old = torch.where(fragile, lp, old)
+    old[1, 0], old[1, 1] = lp[1, 0] - 30.0, lp[1, 1] + 30.0     # beyond the +-20 clamp of the log-ratio
+    if kind == "gspo":
+        old[5] = lp[5] - 11.0                                   # a row beyond the clamp of the sequence weight at 10
+        row = O.masked_mean(lp.double() - old.double(), None if mask is None else mask.double(), dim=-1).exp()
+        assert bool((((row - (1 - lo)).abs() > 1e-3) & ((row - (1 + hi)).abs() > 1e-3)).all())
+        assert bool((row < 1 - lo).any()) and bool((row > 1 + hi).any())
+
+    cfg = SimpleNamespace(policy_loss_type={"dppo_tv": "dppo", "dppo_kl": "dppo"}.get(kind, kind), eps_clip_low=lo,
+                          eps_clip_high=hi, loss_reduction="sequence_mean",
+                          sapo=SimpleNamespace(tau_pos=lo, tau_neg=hi),
+                          cispo=SimpleNamespace(cispo_eps_clip_low=lo, cispo_eps_clip_high=hi, cispo_anchor="old"),
+                          dppo=SimpleNamespace(dppo_type="binary_kl" if kind == "dppo_kl" else "binary_tv", delta_low=lo,
+                                               delta_high=hi),
+                          off_policy_correction=SimpleNamespace(tis_ratio_type=None, sequence_mask_metric=None))
+    m64 = None if mask is None else mask.double()
+    x = lp.double().requires_grad_(True)
+    if kind == "dppo_tv" or kind == "dppo_kl":
+        per_token = lambda msk: O.dppo_policy_loss(x, old.double(), adv.double(), cfg.dppo.dppo_type, lo, hi, msk)  # noqa: E731
+    else:
+        fn = {"sapo": O.sapo_policy_loss, "gspo": O.gspo_policy_loss, "cispo": O.cispo_policy_loss,
+              "rollout_is": O.rollout_is_policy_loss}[kind]
+        per_token = lambda msk: fn(x, old.double(), adv.double(), lo, hi, msk)  # noqa: E731
+    # the importance weight of off-policy correction multiplies the per-token loss before the masked sum: fold it into the mask
+    # for the loss, keep the plain mask for the statistic (and, for GSPO, for the row mean)
+    if weight is None:
+        ref_loss, ref_clip = per_token(m64)
+    elif kind == "gspo":
+        row = O.masked_mean(x - old.double(), m64, dim=-1).unsqueeze(-1)
+        r = torch.clamp(x - x.detach() + row.detach(), max=10).exp()
+        a64 = adv.double()
+        ref_loss = (-torch.min(r * a64, r.clamp(1 - lo, 1 + hi) * a64) * weight.double() * m64).sum()
+        ref_clip = per_token(m64)[1]
+    else:
+        ref_loss, ref_clip = per_token(m64 * weight.double())[0], per_token(m64)[1]
+    ref_loss.backward()
+    return lp, old, adv, mask, weight, cfg, ref_loss.item(), ref_clip.item(), x.grad
+
+
+@pytest.mark.parametrize("kind", ["sapo", "gspo", "cispo", "rollout_is", "dppo_tv", "dppo_kl"])
+@pytest.mark.parametrize("masked", [False, True])
+def test_further_policy_losses_match_oracle(kind, masked, cuda_device):
+    from skyrl_amd import policy_loss as PL
+
+    lp, old, adv, mask, weight, cfg, ref_loss, ref_clip, ref_grad = _further_loss_case(kind, masked)
+    fn = {"sapo": PL.sapo_policy_loss, "gspo": PL.gspo_policy_loss, "cispo": PL.compute_policy_loss_cispo,
+          "rollout_is": PL.rollout_is_policy_loss, "dppo_tv": PL.dppo_policy_loss, "dppo_kl": PL.dppo_policy_loss}[kind]
+    to = lambda t: None if t is None else t.to(cuda_device)  # noqa: E731
+    dlp = lp.to(cuda_device).requires_grad_(True)
+    if kind == "rollout_is":     # anchored on the rollout log-probabilities; the old ones are not read
+        loss, metrics = fn(dlp, to(old) + 5.0, to(adv), cfg, to(mask), to(old), loss_weight=to(weight))
+    else:
+        loss, metrics = fn(dlp, to(old), to(adv), cfg, to(mask), loss_weight=to(weight))
+    loss.backward()
+    scale = max(abs(ref_loss), float(ref_grad.abs().max()), 1e3)
+    assert abs(loss.item() - ref_loss) <= 5e-6 * scale, (loss.item(), ref_loss)
+    assert metrics["clip_ratio"] == pytest.approx(ref_clip, abs=1e-6)
+    if kind not in ("sapo",):
+        assert 0.0 < ref_clip < 1.0                             # both sides of the branch are exercised
+    err = (dlp.grad.double().cpu() - ref_grad).abs().max().item()
+    assert err <= 1e-5 * max(1.0, ref_grad.abs().max().item()), f"gradient max abs err {err}"
+    if mask is not None:
+        assert bool((dlp.grad.cpu()[mask == 0] == 0).all())
+
+    # the same type inside the assembled actor loss, with a KL term on top
+    cfg.use_kl_loss, cfg.kl_loss_coef, cfg.kl_estimator_type, cfg.use_entropy_loss = True, 0.05, "k2", False
+    base = lp + 0.25
+    d2 = lp.to(cuda_device).requires_grad_(True)
+    rollout = to(old) if kind == "rollout_is" else None
+    loss2, m2 = PL.actor_loss(d2, to(old), to(adv), cfg, to(mask), base_log_probs=to(base), loss_weight=to(weight),
+                              rollout_logprobs=rollout, policy_scale=2.0, term_scale=0.5)
+    loss2.backward()
+    kl_ref_lp = lp.double().requires_grad_(True)
+    kl_ref = O.approx_kl_loss(kl_ref_lp, base.double(), None if mask is None else mask.double(), "k2")
+    kl_ref.backward()
+    want = 2.0 * ref_loss + 0.5 * 0.05 * kl_ref.item()
+    assert abs(loss2.item() - want) <= 5e-6 * scale
+    assert m2["clip_ratio"].item() == pytest.approx(ref_clip, abs=1e-6)
+    want_grad = 2.0 * ref_grad + 0.5 * 0.05 * kl_ref_lp.grad
+    err = (d2.grad.double().cpu() - want_grad).abs().max().item()
+    assert err <= 2e-5 * max(1.0, want_grad.abs().max().item()), f"actor-loss gradient max abs err {err}"
+
+
+def test_further_policy_losses_argument_handling(cuda_device):
+    from types import SimpleNamespace
+
+    from skyrl_amd import policy_loss as PL
+
+    x = torch.full((2, 8), -1.0, device=cuda_device)
+    cfg = SimpleNamespace(policy_loss_type="cispo", eps_clip_low=0.2, eps_clip_high=0.2,
+                          cispo=SimpleNamespace(cispo_eps_clip_low=1.0, cispo_eps_clip_high=4.0, cispo_anchor="rollout"),
+                          dppo=SimpleNamespace(dppo_type="topk", delta_low=0.2, delta_high=0.2),
+                          off_policy_correction=SimpleNamespace(tis_ratio_type="token", sequence_mask_metric=None))
+    with pytest.raises(AssertionError):                          # the rollout anchor needs rollout log-probabilities
+        PL.compute_policy_loss_cispo(x, x, x, cfg)
+    with pytest.raises(NotImplementedError):                     # a correction switched on is not silently skipped
+        PL.ppo_policy_loss(x, x, x, SimpleNamespace(policy_loss_type="regular", eps_clip_low=0.2, eps_clip_high=0.2,
+                                                    off_policy_correction=cfg.off_policy_correction), None, x)
+    cfg.off_policy_correction.tis_ratio_type = None
+    loss, m = PL.compute_policy_loss_cispo(x, x + 9.0, x, cfg, None, x)   # ratio 1 against the rollout anchor
+    assert loss.item() == pytest.approx(-16.0) and m["clip_ratio"] == 0.0
+    with pytest.raises(AssertionError):
+        PL.rollout_is_policy_loss(x, x, x, cfg)
+    with pytest.raises(ValueError):
+        PL.dppo_policy_loss(x, x, x, cfg)
+    with pytest.raises(ValueError):
+        PL.gspo_policy_loss(x[0], x[0], x[0], cfg)
+    cfg.policy_loss_type = "clip_cov"
+    with pytest.raises(NotImplementedError):
+        PL.actor_loss(x, x, x, cfg)
+
+
 @pytest.mark.parametrize("estimator", ["k1", "abs", "k2", "k3"])
 @pytest.mark.parametrize("masked", [False, True])
 def test_approx_kl_matches_oracle(estimator, masked, cuda_device):
@@ -546,7 +688,10 @@ def test_loss_argument_errors(cuda_device):
     assert lib.skyrl_actor_loss(*args()) == 0
     assert lib.skyrl_actor_loss(*args(rows=None)) == -1
     assert lib.skyrl_actor_loss(*args(dent=p)) == -1          # an entropy gradient without the entropy
-    assert lib.skyrl_actor_loss(*args(type=9)) == -5
+    assert lib.skyrl_actor_loss(*args(type=4)) == 0           # the sequence-level type is part of this entry point only
+    assert lib.skyrl_actor_loss(*args(type=10)) == -5
+    # SAPO's temperatures divide: zero is refused
+    assert lib.skyrl_ppo_policy_loss(p, p, p, None, None, 16, 0.0, 1.0, 0.0, 5, p, None, None) == -5
     torch.cuda.synchronize()
 
 
