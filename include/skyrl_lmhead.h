@@ -224,6 +224,39 @@ int skyrl_packed_gather_grad(const float* d_out, const int64_t* cu_seqlens, int6
                              const uint8_t* attention_mask, int64_t rows, int64_t cols, float* d_packed, void* stream);
 
 /*
+ * Soft cross-entropy of a draft head against the policy's own next-token distribution, from hidden states.
+ * Replaces, for the full-vocabulary branch on one vocabulary shard, draft_soft_ce / _VocabParallelSoftCrossEntropy
+ * (skyrl/backends/skyrl_train/mtp/soft_ce.py:123-154, 200-240) together with the two output-layer products that feed it
+ * (project_mtp_hidden_to_logits, mtp/adapter.py:37-64, and the policy's own logits) and the teacher roll
+ * (build_teacher_logits, soft_ce.py:22-34):
+ *
+ *     z_s[t] = student_hidden[t] . weight^T / temperature        z_t[t] = teacher_hidden[roll(t)] . weight^T / temperature
+ *     loss[t] = -sum_v softmax(z_t[t])_v * log_softmax(z_s[t])_v
+ *
+ * roll(t) for t = b * seq_len + s is b * seq_len + (s + shift) mod seq_len (shift = MTP depth + 1; seq_len = T for one packed
+ * row); the caller's loss mask removes the wrapped positions, as in the reference.  Neither [T, V] logits tensor exists:
+ * both hidden rows of a token go through one tile of the MFMA kernel side by side.  student_hidden / teacher_hidden are
+ * bf16 [T, H] with leading dimensions ld_student / ld_teacher; weight is bf16 [V, H]; T must be a multiple of seq_len.
+ *
+ * skyrl_softce_fwd writes loss [T] and the two row log-sum-exps [T] (fp32) that skyrl_softce_bwd takes back.
+ * skyrl_softce_bwd writes d_student_hidden [T, H] bf16 = sum_v dloss[t] * (softmax(z_s) - softmax(z_t))_v / temperature *
+ * weight[v] (soft_ce.py:146-151 followed by the output layer's input gradient).  The teacher and the weight get no gradient:
+ * the reference detaches both (soft_ce.py:16-19, mtp/adapter.py:51-56).  Workspaces: 256-byte aligned device memory of at
+ * least the queried size (0 = bad arguments); vocab_chunk as in skyrl_lmhead_bwd.  Not covered: the top-k variant
+ * (draft_soft_ce_topk, soft_ce.py:243-341) and more than one vocabulary shard.
+ */
+size_t skyrl_softce_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V);
+size_t skyrl_softce_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t vocab_chunk);
+int skyrl_softce_fwd(const void* student_hidden, int64_t ld_student, const void* teacher_hidden, int64_t ld_teacher,
+                     const void* weight, int64_t ld_weight, int64_t T, int64_t seq_len, int64_t shift, int64_t H, int64_t V,
+                     float rcp_temperature, float* loss, float* lse_student, float* lse_teacher, void* workspace,
+                     size_t workspace_bytes, void* stream);
+int skyrl_softce_bwd(const void* student_hidden, int64_t ld_student, const void* teacher_hidden, int64_t ld_teacher,
+                     const void* weight, int64_t ld_weight, const float* lse_student, const float* lse_teacher,
+                     const float* dloss, int64_t T, int64_t seq_len, int64_t shift, int64_t H, int64_t V, float rcp_temperature,
+                     void* d_student_hidden, int64_t vocab_chunk, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Measurement aid for benchmarks (no counterpart in the reference): what the matrix pipe sustains on a given kind of
  * data.  Launches `workgroups` workgroups of 4 wavefronts; each wavefront loads 32 operand fragments once from
  * `operands` (bf16, 32 fragments x 256 lanes x 8 values = 128 KiB) and then issues iters x 128 v_mfma_f32_16x16x32_bf16

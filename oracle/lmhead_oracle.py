@@ -38,6 +38,11 @@ What pins each function (all in ``tests/test_oracle.py``; none of them re-types 
   * the assembled actor loss: a hand-computed two-row case (every term worked out on paper) on top of the pinned parts.
   * the FSDP forward tail: ``torch.distributions.Categorical`` for entropy and log-probability, and a Python loop that
     scores action token j of row b against position S - num_actions + j - 1, with and without padding removed.
+  * MTP soft cross-entropy: the reference's own golden masks for ``shift_mask_for_mtp`` (tests/backends/skyrl_train/mtp/
+    test_soft_ce.py:224-245) plus a per-position Python loop for the packed form; the decomposition soft CE = H(p) + KL(p || q)
+    against ``torch.distributions`` / ``torch.nn.functional.kl_div``, the limits "teacher = student -> entropy" (the
+    reference's known answer, test_soft_ce.py:248-284) and "one-hot teacher -> -log q(label)" (the pinned log-probability),
+    and the gradient softmax(student) - softmax(teacher) (test_soft_ce.py:171-181) by fp64 finite differences.
 No function is left "parity unpinned".
 """
 
@@ -643,3 +648,62 @@ def actor_loss(
     kl = approx_kl_loss(log_probs, base_log_probs, loss_mask, kl_estimator_type) if base_log_probs is not None else torch.zeros(())
     ent = masked_mean(entropy, loss_mask) if entropy is not None else torch.zeros(())
     return policy * policy_scale + (kl * kl_coef - ent * entropy_coef) * term_scale, policy, kl, ent
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# Multi-token-prediction draft loss: soft cross-entropy against the policy's own next-token distribution
+# ----------------------------------------------------------------------------------------------------------------------
+MTP = "skyrl/backends/skyrl_train/mtp/soft_ce.py"
+
+
+def build_teacher_logits(main_logits: torch.Tensor, mtp_layer_number: int = 0) -> torch.Tensor:
+    """mtp/soft_ce.py:22-34: the policy's logits rolled left by depth + 1 along the sequence, detached."""
+    return torch.roll(main_logits.detach(), shifts=-(mtp_layer_number + 1), dims=1)
+
+
+def shift_mask_for_mtp(mask: torch.Tensor, mtp_layer_number: int = 0, cu_seqlens=None) -> torch.Tensor:
+    """mtp/soft_ce.py:37-79: the mask rolled like the teacher with the wrapped tail zeroed, AND-ed with the source mask;
+    with ``cu_seqlens`` the roll is done segment by segment and each segment's tail is zeroed."""
+    shift = mtp_layer_number + 1
+    if cu_seqlens is None:
+        rolled = torch.roll(mask, shifts=-shift, dims=1)
+        rolled[:, -shift:] = 0
+        return mask * rolled
+    bounds = [int(b) for b in (cu_seqlens.tolist() if torch.is_tensor(cu_seqlens) else cu_seqlens)]
+    rolled = torch.zeros_like(mask)
+    for start, end in zip(bounds[:-1], bounds[1:]):
+        if end - start <= 0:
+            continue
+        seg = torch.roll(mask[:, start:end], shifts=-shift, dims=1)
+        if shift < end - start:
+            seg[:, -shift:] = 0
+        else:
+            seg.zero_()
+        rolled[:, start:end] = seg
+    return mask * rolled
+
+
+def soft_ce_per_token(student_logits: torch.Tensor, teacher_logits: torch.Tensor) -> torch.Tensor:
+    """mtp/soft_ce.py:230-233 (and :137-143 for the vocabulary-parallel form on one shard):
+    ``-sum_v softmax(teacher)_v log_softmax(student)_v`` in fp32 or wider."""
+    up = torch.float64 if student_logits.dtype == torch.float64 else torch.float32
+    return -(torch.softmax(teacher_logits.to(up), dim=-1) * torch.log_softmax(student_logits.to(up), dim=-1)).sum(dim=-1)
+
+
+def draft_soft_ce(student_logits, teacher_logits, mask, global_normalization_factor=None) -> torch.Tensor:
+    """mtp/soft_ce.py:200-240 with the reduction of :154-159: masked mean over the local mask count, or the masked sum over
+    ``clamp(global_normalization_factor, min=1)``.  Sequence chunking (:162-197) does not change the value."""
+    assert not teacher_logits.requires_grad, "MTP draft loss: teacher_logits must be detached"
+    per_token = soft_ce_per_token(student_logits, teacher_logits)
+    if global_normalization_factor is not None:
+        return (per_token * mask).sum() / global_normalization_factor.clamp(min=1.0)
+    return masked_mean(per_token, mask)
+
+
+def draft_soft_ce_from_hidden(student_hidden, teacher_hidden, weight, mask, mtp_layer_number=0, global_normalization_factor=None):
+    """The call chain around it: both hidden states through the shared, detached output layer (mtp/adapter.py:51-64), the
+    teacher rolled to the draft depth, then ``draft_soft_ce`` (megatron_model_wrapper.py:766-775)."""
+    w = weight.detach()
+    student_logits = student_hidden @ w.t()
+    teacher_logits = build_teacher_logits(teacher_hidden.detach() @ w.t(), mtp_layer_number)
+    return draft_soft_ce(student_logits, teacher_logits, mask, global_normalization_factor)

@@ -11,7 +11,7 @@ import os
 import threading
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libskyrl_lmhead.so")
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 _c_i64 = ctypes.c_int64
 _c_p = ctypes.c_void_p
@@ -47,6 +47,18 @@ SIGNATURES = {
         ctypes.c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_p, _c_p]),
     "skyrl_packed_gather_grad": (
         ctypes.c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_p, _c_p]),
+    "skyrl_softce_fwd_workspace_bytes": (ctypes.c_size_t, [_c_i64, _c_i64, _c_i64]),
+    "skyrl_softce_bwd_workspace_bytes": (ctypes.c_size_t, [_c_i64, _c_i64, _c_i64, _c_i64]),
+    "skyrl_softce_fwd": (
+        ctypes.c_int,
+        [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, ctypes.c_float, _c_p, _c_p, _c_p,
+         _c_p, ctypes.c_size_t, _c_p],
+    ),
+    "skyrl_softce_bwd": (
+        ctypes.c_int,
+        [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, ctypes.c_float,
+         _c_p, _c_i64, _c_p, ctypes.c_size_t, _c_p],
+    ),
     "skyrl_lmhead_mfma_probe": (ctypes.c_int, [_c_p, ctypes.c_int, ctypes.c_int, _c_p, _c_p]),
     "skyrl_lmhead_num_kernel_kinds": (ctypes.c_int, []),
     "skyrl_lmhead_kernel_name": (ctypes.c_char_p, [ctypes.c_int]),

@@ -45,9 +45,12 @@ __host__ __device__ inline int64_t round_up(int64_t x, int64_t m) { return (x + 
 // (fused_linear_logprob_triton.py:296-385): scale, running max, sum exp, sum z*exp; vocab rows past V take no part.
 // The label-logit gather of that kernel (:364-385) is done in lmhead_fwd_merge instead.
 // ------------------------------------------------------------------------------------------------------------
-template <bool ENTROPY, bool MASKED>
+// PAIRED (the soft cross-entropy, below): token blocks j >= TN / 2 hold teacher rows, and their third statistic weighs the
+// *student's* logit -- the same lane's accumulator TN / 2 blocks earlier -- with the teacher's exp: sum z_student e^(z_teacher - m).
+template <bool ENTROPY, bool MASKED, bool PAIRED>
 __device__ __forceinline__ void fwd_tile_stats(const acc_t& acc, int j, int vbase, int V, float scale2, int kq, float& m_out,
                                                float& s_out, float& e_out) {
+  const int jy = (PAIRED && j >= TN / 2) ? j - TN / 2 : j;  // j is a constant of the caller's unrolled loop
   // Two read-only passes over the accumulators (they live in AGPRs; writing scaled values back would cost a move each
   // way).  scale2 > 0, so the maximum commutes with the scaling, and sum z*p = scale2 * sum x*p.
   float mx = -INFINITY;
@@ -76,7 +79,7 @@ __device__ __forceinline__ void fwd_tile_stats(const acc_t& acc, int j, int vbas
         if (v >= V) p = 0.f;
       }
       s += p;
-      if (ENTROPY) e = fmaf(x, p, e);
+      if (ENTROPY) e = fmaf(PAIRED ? acc[i][jy][r] : x, p, e);
     }
   s = col_sum(s);
   if (ENTROPY) e = col_sum(e);
@@ -85,12 +88,10 @@ __device__ __forceinline__ void fwd_tile_stats(const acc_t& acc, int j, int vbas
   e_out = e * scale2 * kLn2;
 }
 
-template <bool ENTROPY>
-__global__ __launch_bounds__(NTHREADS) void lmhead_fwd_tiles(const uint16_t* __restrict__ W, int ldw,
-                                                             const uint16_t* __restrict__ Hd, int ldh, int T, int H, int V,
-                                                             float rcp_temp, float* __restrict__ part_max,
-                                                             float* __restrict__ part_sum, float* __restrict__ part_pz) {
-  __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
+template <bool ENTROPY, bool PAIRED>
+__device__ __forceinline__ void fwd_tile(const uint16_t* __restrict__ W, int ldw, const uint16_t* __restrict__ Hd, int ldh, int T,
+                                         int H, int V, float rcp_temp, float* __restrict__ part_max,
+                                         float* __restrict__ part_sum, float* __restrict__ part_pz, char* lds) {
   const int tiles_m = (V + BM - 1) / BM;
   const int tiles_n = (T + BN - 1) / BN;
   int tm, tn;
@@ -114,9 +115,9 @@ __global__ __launch_bounds__(NTHREADS) void lmhead_fwd_tiles(const uint16_t* __r
     const int t = tn * BN + wn * WN + j * MT + lrow;
     float m = -INFINITY, s = 0.f, e = 0.f;
     if (vbase + WM <= V) {
-      fwd_tile_stats<ENTROPY, false>(acc, j, vbase, V, scale2, kq, m, s, e);
+      fwd_tile_stats<ENTROPY, false, PAIRED>(acc, j, vbase, V, scale2, kq, m, s, e);
     } else if (vbase < V) {
-      fwd_tile_stats<ENTROPY, true>(acc, j, vbase, V, scale2, kq, m, s, e);
+      fwd_tile_stats<ENTROPY, true, PAIRED>(acc, j, vbase, V, scale2, kq, m, s, e);
     }
     if (kq == 0 && t < T) {
       part_max[part + t] = m;
@@ -124,6 +125,15 @@ __global__ __launch_bounds__(NTHREADS) void lmhead_fwd_tiles(const uint16_t* __r
       if (ENTROPY) part_pz[part + t] = e;
     }
   }
+}
+
+template <bool ENTROPY>
+__global__ __launch_bounds__(NTHREADS) void lmhead_fwd_tiles(const uint16_t* __restrict__ W, int ldw,
+                                                             const uint16_t* __restrict__ Hd, int ldh, int T, int H, int V,
+                                                             float rcp_temp, float* __restrict__ part_max,
+                                                             float* __restrict__ part_sum, float* __restrict__ part_pz) {
+  __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
+  fwd_tile<ENTROPY, false>(W, ldw, Hd, ldh, T, H, V, rcp_temp, part_max, part_sum, part_pz, lds);
 }
 
 // ------------------------------------------------------------------------------------------------------------
@@ -190,7 +200,7 @@ __global__ __launch_bounds__(256) void lmhead_fwd_merge(const float* __restrict_
   const int t = blockIdx.x * kMergeTokens + tl;
   float dot = 0.f;
   bool has_label = false;
-  if (t < T) {
+  if (t < T && labels) {
     const int64_t y = labels[t];
     has_label = (y >= 0 && y < (int64_t)V);
     if (has_label) {
@@ -213,7 +223,7 @@ __global__ __launch_bounds__(256) void lmhead_fwd_merge(const float* __restrict_
   for (int o = 1; o < kMergeGroups; o <<= 1) dot += __shfl_xor(dot, o, 64);
   if (sub == 0 && t < T) {
     const float lse = sm_lse[tl], pz = sm_pz[tl];
-    logprobs[t] = has_label ? dot * rcp_temp - lse : 0.f;
+    if (logprobs) logprobs[t] = has_label ? dot * rcp_temp - lse : 0.f;
     if (entropy) entropy[t] = lse - pz;
     if (row_lse) row_lse[t] = lse;
     if (row_pz) row_pz[t] = pz;
@@ -346,6 +356,156 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
   }
 }
 
+
+// ------------------------------------------------------------------------------------------------------------
+// Soft cross-entropy from hidden states (the draft-head loss of multi-token prediction, skyrl/backends/skyrl_train/mtp/
+// soft_ce.py:200-240):  loss[t] = -sum_v softmax(z_teacher[t])_v * log_softmax(z_student[t])_v = lse_student - E_teacher[z_student],
+// both logits rows being products with the same (detached) output weight.  The reference materialises both [T, V] logits
+// tensors and their fp32 softmaxes; here the two hidden rows of a token sit in one "stacked" operand so that one lane
+// holds z_student and z_teacher of the same (token, vocab) pair, TN / 2 accumulator blocks apart:
+//   stacked row of token t:   student  (t / 64) * 128 + t % 64,   teacher  (t / 64) * 128 + 64 + t % 64
+// i.e. each wave's 128 token rows are 64 student rows followed by the 64 teacher rows of the same tokens.  The forward
+// is the ordinary tile kernel on the stacked rows with the paired third statistic; the backward recomputes a tile and
+// writes  d loss / d z_student = g * (softmax(z_student) - softmax(z_teacher))  (soft_ce.py:146-151) for the student rows
+// into the token-major dz panel, from which the ordinary dHidden GEMM runs.  The weight gets no gradient (it is detached
+// in the reference, mtp/adapter.py:51-56), neither does the teacher.
+// ------------------------------------------------------------------------------------------------------------
+constexpr int kPairRows = WN / 2;  // 64 tokens per wave
+
+__host__ __device__ inline int64_t stacked_row(int64_t t, bool teacher) {
+  return (t / kPairRows) * WN + (teacher ? kPairRows : 0) + t % kPairRows;
+}
+
+// One workgroup per stacked row: copies the student's or the teacher's hidden row, zeros for the padding tokens.
+// Teacher row of token t = b * seq_len + s is the teacher's hidden row b * seq_len + (s + shift) mod seq_len: the roll of
+// build_teacher_logits (soft_ce.py:22-34) applied to the hidden states instead of the logits.
+__global__ __launch_bounds__(256) void softce_pack_rows(const uint16_t* __restrict__ student, int lds_,
+                                                        const uint16_t* __restrict__ teacher, int ldt, int T, int seq_len,
+                                                        int shift, int H, uint16_t* __restrict__ stacked) {
+  const int r = blockIdx.x;
+  const bool is_teacher = (r / kPairRows) & 1;
+  const int t = (r / WN) * kPairRows + r % kPairRows;
+  const uint16_t* src = nullptr;
+  if (t < T) {
+    if (is_teacher) {
+      const int b = t / seq_len, sft = (t % seq_len + shift) % seq_len;
+      src = teacher + (size_t)(b * seq_len + sft) * (size_t)ldt;
+    } else {
+      src = student + (size_t)t * (size_t)lds_;
+    }
+  }
+  uint16_t* dst = stacked + (size_t)r * (size_t)H;
+  for (int c = threadIdx.x * 8; c < H; c += 256 * 8)
+    *(uint4*)(dst + c) = src ? *(const uint4*)(src + c) : make_uint4(0, 0, 0, 0);
+}
+
+template <bool ENTROPY>
+__global__ __launch_bounds__(NTHREADS) void softce_fwd_tiles(const uint16_t* __restrict__ W, int ldw,
+                                                             const uint16_t* __restrict__ Hd, int ldh, int T, int H, int V,
+                                                             float rcp_temp, float* __restrict__ part_max,
+                                                             float* __restrict__ part_sum, float* __restrict__ part_pz) {
+  __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
+  fwd_tile<ENTROPY, true>(W, ldw, Hd, ldh, T, H, V, rcp_temp, part_max, part_sum, part_pz, lds);
+}
+
+// Per token: the merged statistics of its two stacked rows -> loss and the two log-sum-exps the backward needs.
+__global__ __launch_bounds__(256) void softce_finish(const float* __restrict__ row_lse, const float* __restrict__ row_pz, int T,
+                                                     float* __restrict__ loss, float* __restrict__ lse_student,
+                                                     float* __restrict__ lse_teacher) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= T) return;
+  const int64_t rs = stacked_row(t, false), rt = stacked_row(t, true);
+  const float ls = row_lse[rs];
+  loss[t] = ls - row_pz[rt];  // row_pz of a teacher row is E_teacher[z_student]
+  lse_student[t] = ls;
+  lse_teacher[t] = row_lse[rt];
+}
+
+struct SoftCeDzArgs {
+  const uint16_t* W;
+  int ldw;
+  const uint16_t* S;  // stacked hidden rows [2 * Tp, H], Tp = T rounded up to whole 128-token tiles
+  int T, Tp, H, V;
+  float rcp_temp;
+  const float* lse_student;
+  const float* lse_teacher;
+  const float* dloss;
+  int vc0, tiles_m, tiles_n;  // first vocab row of the chunk; tiles along the chunk's vocab rows and the stacked rows
+  uint16_t* D;                // [Tp, ldd]  dz of the student rows, token-major
+  int ldd;
+};
+
+__global__ __launch_bounds__(NTHREADS) void softce_dz_tiles(const SoftCeDzArgs z) {
+  __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
+  const uint16_t* __restrict__ W = z.W;
+  const uint16_t* __restrict__ S = z.S;
+  const int T = z.T, H = z.H, V = z.V, vc0 = z.vc0, ldd = z.ldd;
+  uint16_t* __restrict__ D = z.D;
+  int tm, tn;
+  tile_coords(blockIdx.x, z.tiles_m, z.tiles_n, kGroupM, tm, tn);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int lrow = lane & 15, kq = lane >> 4;
+  const int vloc_base = tm * BM + wm * WM;
+  const int vbase = vc0 + vloc_base;
+  const int tokbase = (tn * WAVES_N + wn) * kPairRows;  // first token of this wave
+  const bool full = vbase + WM <= V;
+  const float scale2 = z.rcp_temp * kLog2e;
+
+  float gs_[TN / 2], ls2_[TN / 2], lt2_[TN / 2];
+#pragma unroll
+  for (int j = 0; j < TN / 2; ++j) {
+    const int t = tokbase + j * MT + lrow;
+    const bool valid = t < T;
+    gs_[j] = valid ? z.dloss[t] * z.rcp_temp : 0.f;
+    ls2_[j] = valid ? z.lse_student[t] * kLog2e : INFINITY;
+    lt2_[j] = valid ? z.lse_teacher[t] * kLog2e : INFINITY;
+  }
+
+  Operand a{W, z.ldw, vc0 + tm * BM, V};
+  Operand b{S, H, tn * BN, 2 * z.Tp};
+  acc_t acc;
+  zero_acc(acc);
+  prefetch_first_tiles(a, b, 0, H / BK, lds);
+  mainloop(a, b, 0, H / BK, lds, acc);
+
+  // Staging as in dz_tile: a private region per wave, 64 token rows of 128 vocab columns, then 16-byte non-temporal stores.
+  constexpr int kTokRow = WM * 2 + 16;
+  constexpr int kStage = WN * kTokRow;
+  char* stage = lds + wave * kStage;
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+  for (int j = 0; j < TN / 2; ++j) {
+    const float gs = gs_[j], ls2 = ls2_[j], lt2 = lt2_[j];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      float d[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float q = __builtin_amdgcn_exp2f(fmaf(acc[i][j][r], scale2, -ls2));
+        const float p = __builtin_amdgcn_exp2f(fmaf(acc[i][j + TN / 2][r], scale2, -lt2));
+        d[r] = gs * (q - p);
+      }
+      const int vl = i * MT + kq * 4;
+      if (!full) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (vbase + vl + r >= V) d[r] = 0.f;
+      }
+      f32x4 v4 = {d[0], d[1], d[2], d[3]};
+      const bf16x4 b4 = __builtin_convertvector(v4, bf16x4);
+      *(uint2*)(stage + (j * MT + lrow) * kTokRow + vl * 2) = *(const uint2*)&b4;
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < 16; ++it) {
+    const int idx = it * 64 + lane;
+    const int n = idx >> 4, c = idx & 15;
+    const u32x4 v = *(const u32x4*)(stage + n * kTokRow + c * 16);
+    __builtin_nontemporal_store(v, (u32x4*)(D + (size_t)(tokbase + n) * (size_t)ldd + vloc_base + c * 8));
+  }
+}
 
 // ------------------------------------------------------------------------------------------------------------
 // Plain NT GEMM with an fp32 / bf16 store epilogue:  C[N,M] (+)= B[N,K] . A[M,K]^T, i.e. C[n][m] = sum_k A[m][k] B[n][k]:
@@ -563,9 +723,13 @@ __global__ __launch_bounds__(256) void transpose_bf16(const uint16_t* __restrict
 // ------------------------------------------------------------------------------------------------------------
 // Optional per-kernel timing: while a profile is open on the calling thread every launch below is bracketed by a pair of
 // HIP events on the launch stream.  Closed profiles cost one thread-local load per launch.
-enum KernelKind { kFwdTiles = 0, kFwdMerge, kTranspose, kBwdChunkDz, kBwdChunkGemm, kNumKernelKinds };
+enum KernelKind {
+  kFwdTiles = 0, kFwdMerge, kTranspose, kBwdChunkDz, kBwdChunkGemm, kSoftCePack, kSoftCeFwdTiles, kSoftCeFinish, kSoftCeDz,
+  kNumKernelKinds
+};
 const char* const kKernelNames[kNumKernelKinds] = {"lmhead_fwd_tiles", "lmhead_fwd_merge", "transpose_bf16",
-                                                   "lmhead_bwd_chunk[dz]", "lmhead_bwd_chunk[gemm]"};
+                                                   "lmhead_bwd_chunk[dz]", "lmhead_bwd_chunk[gemm]", "softce_pack_rows",
+                                                   "softce_fwd_tiles", "softce_finish", "softce_dz_tiles"};
 struct Profile {
   struct Rec {
     int kind;
@@ -736,11 +900,74 @@ hipError_t launch_bwd_chunk(hipStream_t s, bool entgrad, const DzArgs& z, unsign
   return hipGetLastError();
 }
 
+// Workspaces of the soft cross-entropy: the stacked hidden rows first in both.
+constexpr int64_t kPairTile = BN / 2;  // tokens per workgroup tile of stacked rows
+
+struct SoftCeFwdWorkspace {
+  uint16_t* S;
+  float *pmax, *psum, *ppz, *row_lse, *row_pz;
+  size_t nparts, bytes;
+};
+
+SoftCeFwdWorkspace carve_softce_fwd(void* ws, int64_t T, int64_t H, int64_t V) {
+  const int64_t Tp = round_up(T, kPairTile);
+  Carver c(ws);
+  SoftCeFwdWorkspace w;
+  w.nparts = (size_t)((V + BM - 1) / BM) * WAVES_M;
+  w.S = c.take<uint16_t>((size_t)(2 * Tp) * (size_t)H);
+  w.pmax = c.take<float>(w.nparts * (size_t)(2 * Tp));
+  w.psum = c.take<float>(w.nparts * (size_t)(2 * Tp));
+  w.ppz = c.take<float>(w.nparts * (size_t)(2 * Tp));
+  w.row_lse = c.take<float>((size_t)(2 * Tp));
+  w.row_pz = c.take<float>((size_t)(2 * Tp));
+  w.bytes = (size_t)round_up((int64_t)c.off, 256);
+  return w;
+}
+
+struct SoftCeBwdWorkspace {
+  uint16_t *S, *Wt, *D;
+  float* dHacc;
+  size_t bytes;
+};
+
+SoftCeBwdWorkspace carve_softce_bwd(void* ws, int64_t T, int64_t H, int64_t V, int64_t vc) {
+  const int64_t Tp = round_up(T, kPairTile), Vpad = round_up(V, 256);
+  Carver c(ws);
+  SoftCeBwdWorkspace w;
+  w.S = c.take<uint16_t>((size_t)(2 * Tp) * (size_t)H);
+  w.Wt = reads_weight_in_place(V) ? nullptr : c.take<uint16_t>((size_t)H * (Vpad + kLdPad));
+  w.dHacc = c.take<float>((size_t)round_up(T, 256) * round_up(H, 256));
+  w.D = c.take<uint16_t>((size_t)Tp * (vc + kLdPad));
+  w.bytes = (size_t)round_up((int64_t)c.off, 256);
+  return w;
+}
+
+int check_softce(const void* student, int64_t lds_, const void* teacher, int64_t ldt, const void* weight, int64_t ldw, int64_t T,
+                 int64_t seq_len, int64_t shift, int64_t H, int64_t V, float rcp_temperature) {
+  static const int64_t no_labels = 0;  // check_common wants a labels pointer; this path has none
+  int st = check_common(student, lds_, weight, ldw, &no_labels, T, H, V, rcp_temperature);
+  if (st) return st;
+  if (!teacher) return SKYRL_LMHEAD_ERR_NULL;
+  if (ldt < H || ldt > (int64_t)1 << 30 || T * ldt * 2 >= ((int64_t)1 << 32)) return SKYRL_LMHEAD_ERR_SHAPE;
+  if (seq_len < 1 || T % seq_len != 0 || shift < 0) return SKYRL_LMHEAD_ERR_SHAPE;
+  if (2 * round_up(T, kPairTile) * H * 2 >= ((int64_t)1 << 32)) return SKYRL_LMHEAD_ERR_SHAPE;  // the stacked rows
+  if (!aligned16(teacher) || ldt % 8 != 0) return SKYRL_LMHEAD_ERR_ALIGN;
+  return SKYRL_LMHEAD_OK;
+}
+
+hipError_t launch_softce_pack(hipStream_t s, const void* student, int64_t lds_, const void* teacher, int64_t ldt, int64_t T,
+                              int64_t seq_len, int64_t shift, int64_t H, uint16_t* S) {
+  Timed timed(kSoftCePack, s);
+  hipLaunchKernelGGL(softce_pack_rows, dim3((unsigned)(2 * round_up(T, kPairTile))), dim3(256), 0, s, (const uint16_t*)student,
+                     (int)lds_, (const uint16_t*)teacher, (int)ldt, (int)T, (int)seq_len, (int)(shift % seq_len), (int)H, S);
+  return hipGetLastError();
+}
+
 }  // namespace
 
 extern "C" {
 
-int skyrl_lmhead_version(void) { return 6; }
+int skyrl_lmhead_version(void) { return 7; }
 
 const char* skyrl_lmhead_strerror(int status) {
   switch (status) {
@@ -892,6 +1119,115 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
     const GemmArgs gw = make_gemm(w.Ht, Tpad + kLdPad, H, w.D, vcw + kLdPad, vcw, true, false, Tpad / BK, H, rows,
                                   accumulate_dw ? (const float*)dWc : (const float*)nullptr, dWc, (uint16_t*)nullptr, H);
     e = launch_bwd_chunk(s, dentropy != nullptr, DzArgs{}, 0, true, gh, gw);
+    if (e != hipSuccess) return (int)e;
+  }
+  return SKYRL_LMHEAD_OK;
+}
+
+size_t skyrl_softce_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
+  if (T < 1 || V < 1 || H < 1) return 0;
+  return carve_softce_fwd(nullptr, T, H, V).bytes;
+}
+
+size_t skyrl_softce_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t vocab_chunk) {
+  if (T < 1 || V < 1 || H < 1 || vocab_chunk < 0 || vocab_chunk % 256 != 0) return 0;
+  int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(T, H, V);
+  if (vc > round_up(V, 256)) vc = round_up(V, 256);
+  return carve_softce_bwd(nullptr, T, H, V, vc).bytes;
+}
+
+int skyrl_softce_fwd(const void* student_hidden, int64_t ld_student, const void* teacher_hidden, int64_t ld_teacher,
+                     const void* weight, int64_t ld_weight, int64_t T, int64_t seq_len, int64_t shift, int64_t H, int64_t V,
+                     float rcp_temperature, float* loss, float* lse_student, float* lse_teacher, void* workspace,
+                     size_t workspace_bytes, void* stream) {
+  int st = check_softce(student_hidden, ld_student, teacher_hidden, ld_teacher, weight, ld_weight, T, seq_len, shift, H, V,
+                        rcp_temperature);
+  if (st) return st;
+  if (!loss || !lse_student || !lse_teacher) return SKYRL_LMHEAD_ERR_NULL;
+  if (!workspace || workspace_bytes < skyrl_softce_fwd_workspace_bytes(T, H, V)) return SKYRL_LMHEAD_ERR_WORKSPACE;
+  if ((uintptr_t)workspace & 255u) return SKYRL_LMHEAD_ERR_ALIGN;
+
+  hipStream_t s = (hipStream_t)stream;
+  const SoftCeFwdWorkspace w = carve_softce_fwd(workspace, T, H, V);
+  const int64_t rows = 2 * round_up(T, kPairTile);
+  const uint16_t* Wp = (const uint16_t*)weight;
+  hipError_t e = launch_softce_pack(s, student_hidden, ld_student, teacher_hidden, ld_teacher, T, seq_len, shift, H, w.S);
+  if (e != hipSuccess) return (int)e;
+  const int tiles_m = (int)((V + BM - 1) / BM), tiles_n = (int)(rows / BN);
+  {
+    Timed timed(kSoftCeFwdTiles, s);
+    hipLaunchKernelGGL(softce_fwd_tiles<true>, dim3((unsigned)(tiles_m * tiles_n)), dim3(NTHREADS), 0, s, Wp, (int)ld_weight, w.S,
+                       (int)H, (int)rows, (int)H, (int)V, rcp_temperature, w.pmax, w.psum, w.ppz);
+  }
+  if ((e = hipGetLastError()) != hipSuccess) return (int)e;
+  {
+    Timed timed(kFwdMerge, s);
+    hipLaunchKernelGGL(lmhead_fwd_merge, dim3((unsigned)((rows + kMergeTokens - 1) / kMergeTokens)), dim3(256), 0, s, w.pmax,
+                       w.psum, w.ppz, (int)w.nparts, (int)rows, w.S, (int)H, Wp, (int)ld_weight, (const int64_t*)nullptr, (int)H,
+                       (int)V, rcp_temperature, (float*)nullptr, (float*)nullptr, w.row_lse, w.row_pz);
+  }
+  if ((e = hipGetLastError()) != hipSuccess) return (int)e;
+  Timed timed(kSoftCeFinish, s);
+  hipLaunchKernelGGL(softce_finish, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, s, w.row_lse, w.row_pz, (int)T, loss,
+                     lse_student, lse_teacher);
+  e = hipGetLastError();
+  return e == hipSuccess ? SKYRL_LMHEAD_OK : (int)e;
+}
+
+int skyrl_softce_bwd(const void* student_hidden, int64_t ld_student, const void* teacher_hidden, int64_t ld_teacher,
+                     const void* weight, int64_t ld_weight, const float* lse_student, const float* lse_teacher,
+                     const float* dloss, int64_t T, int64_t seq_len, int64_t shift, int64_t H, int64_t V, float rcp_temperature,
+                     void* d_student_hidden, int64_t vocab_chunk, void* workspace, size_t workspace_bytes, void* stream) {
+  int st = check_softce(student_hidden, ld_student, teacher_hidden, ld_teacher, weight, ld_weight, T, seq_len, shift, H, V,
+                        rcp_temperature);
+  if (st) return st;
+  if (!lse_student || !lse_teacher || !dloss || !d_student_hidden) return SKYRL_LMHEAD_ERR_NULL;
+  if (!aligned16(d_student_hidden)) return SKYRL_LMHEAD_ERR_ALIGN;
+  if (vocab_chunk < 0 || vocab_chunk % 256 != 0) return SKYRL_LMHEAD_ERR_ARG;
+  const int64_t Tp = round_up(T, kPairTile), Vpad = round_up(V, 256);
+  int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(T, H, V);
+  if (vc > Vpad) vc = Vpad;
+  if (H * (Vpad + kLdPad) * 2 >= ((int64_t)1 << 32) || Tp * (vc + kLdPad) * 2 >= ((int64_t)1 << 32))
+    return SKYRL_LMHEAD_ERR_SHAPE;
+  if (!workspace || workspace_bytes < skyrl_softce_bwd_workspace_bytes(T, H, V, vc)) return SKYRL_LMHEAD_ERR_WORKSPACE;
+  if ((uintptr_t)workspace & 255u) return SKYRL_LMHEAD_ERR_ALIGN;
+
+  hipStream_t s = (hipStream_t)stream;
+  const SoftCeBwdWorkspace w = carve_softce_bwd(workspace, T, H, V, vc);
+  const uint16_t* Wp = (const uint16_t*)weight;
+  hipError_t e = launch_softce_pack(s, student_hidden, ld_student, teacher_hidden, ld_teacher, T, seq_len, shift, H, w.S);
+  if (e != hipSuccess) return (int)e;
+  const bool w_in_place = reads_weight_in_place(V);
+  if (!w_in_place) {
+    Timed timed(kTranspose, s);
+    hipLaunchKernelGGL(transpose_bf16, dim3((unsigned)(Vpad / 64), (unsigned)(H / 64)), dim3(256), 0, s, Wp, (int)ld_weight,
+                       (int)V, (int)H, w.Wt, (int)(Vpad + kLdPad), (int)Vpad);
+    if ((e = hipGetLastError()) != hipSuccess) return (int)e;
+  }
+  const int64_t nchunks = (Vpad + vc - 1) / vc;
+  const GemmArgs none{};
+  for (int64_t ci = 0; ci < nchunks; ++ci) {
+    const int64_t vc0 = ci * vc, vcw = (Vpad - vc0) < vc ? (Vpad - vc0) : vc;
+    const SoftCeDzArgs z{Wp, (int)ld_weight, w.S, (int)T, (int)Tp, (int)H, (int)V, rcp_temperature, lse_student, lse_teacher,
+                         dloss, (int)vc0, (int)(vcw / 256), (int)(2 * Tp / BN), w.D, (int)(vcw + kLdPad)};
+    {
+      Timed timed(kSoftCeDz, s);
+      hipLaunchKernelGGL(softce_dz_tiles, dim3((unsigned)(z.tiles_m * z.tiles_n)), dim3(NTHREADS), 0, s, z);
+    }
+    if ((e = hipGetLastError()) != hipSuccess) return (int)e;
+    // d student hidden [t, h] (+)= sum_v D[t, v] . weight[vc0 + v, h]: the dHidden GEMM of the log-probability backward,
+    // partial sums carried from chunk to chunk in accumulator order, bf16 rows written by the last chunk.
+    const bool first = ci == 0, last = ci == nchunks - 1;
+    uint16_t* dh_out = last ? (uint16_t*)d_student_hidden : (uint16_t*)nullptr;
+    const float* dh_in = first ? (const float*)nullptr : (const float*)w.dHacc;
+    float* dh_keep = last ? (float*)nullptr : w.dHacc;
+    const int64_t kext = (V - vc0) < vcw ? (V - vc0) : vcw;
+    const GemmArgs gh =
+        w_in_place ? make_gemm(w.D, vcw + kLdPad, Tp, Wp + (size_t)vc0 * (size_t)ld_weight, ld_weight, H, true, true, kext / BK, T,
+                               H, nullptr, nullptr, dh_out, H, dh_in, dh_keep)
+                   : make_gemm(w.Wt + vc0, Vpad + kLdPad, H, w.D, vcw + kLdPad, Tp, false, false, vcw / BK, H, T, nullptr,
+                               nullptr, dh_out, H, dh_in, dh_keep);
+    e = launch_bwd_chunk(s, false, DzArgs{}, 0, true, gh, none);
     if (e != hipSuccess) return (int)e;
   }
   return SKYRL_LMHEAD_OK;

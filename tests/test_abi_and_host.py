@@ -19,7 +19,7 @@ HEADER = os.path.join(ROOT, "include", "skyrl_lmhead.h")
 def _declared_functions():
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(skyrl_(?:lmhead|ppo|packed|approx|masked|actor)_\w+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(skyrl_(?:lmhead|ppo|packed|approx|masked|actor|softce)_\w+)\s*\(", text)))
 
 
 def test_library_exports_every_declared_symbol():

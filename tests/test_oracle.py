@@ -769,3 +769,121 @@ def test_hf_wrapper_tail_brute_force():
     lp_all = torch.log_softmax(packed_logits[0] / t, -1).gather(-1, torch.roll(tokens, -1)[:, None])[:, 0]
     assert lp_all[row0_last].item() == pytest.approx(want.item(), rel=1e-12)
     assert full.shape == (B, S - 1)
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# MTP draft loss: soft cross-entropy
+# ----------------------------------------------------------------------------------------------------------------------
+def test_shift_mask_for_mtp_reference_golden_masks():
+    """The masks the reference's tests spell out (tests/backends/skyrl_train/mtp/test_soft_ce.py:224-245)."""
+    m = torch.ones(1, 4)
+    assert O.shift_mask_for_mtp(m, 0).tolist() == [[1.0, 1.0, 1.0, 0.0]]
+    assert O.shift_mask_for_mtp(m, 1).tolist() == [[1.0, 1.0, 0.0, 0.0]]
+    left = torch.tensor([[0.0, 0.0, 1.0, 1.0, 1.0]])
+    assert O.shift_mask_for_mtp(left, 0).tolist() == [[0.0, 0.0, 1.0, 1.0, 0.0]]
+    assert O.shift_mask_for_mtp(left, 1).tolist() == [[0.0, 0.0, 1.0, 0.0, 0.0]]
+    right = torch.tensor([[1.0, 1.0, 1.0, 0.0, 0.0]])
+    assert O.shift_mask_for_mtp(right, 0).tolist() == [[1.0, 1.0, 0.0, 0.0, 0.0]]
+
+
+def _shift_mask_loop(mask, shift, bounds):
+    out = torch.zeros_like(mask)
+    for b in range(mask.shape[0]):
+        for start, end in zip(bounds[:-1], bounds[1:]):
+            for t in range(start, end):
+                if t + shift < end and mask[b, t] != 0 and mask[b, t + shift] != 0:
+                    out[b, t] = mask[b, t] * mask[b, t + shift]
+    return out
+
+
+def test_shift_mask_for_mtp_packed_brute_force_and_product_mirror():
+    from skyrl_amd.mtp_soft_ce import shift_mask_for_mtp as product
+
+    gen = torch.Generator().manual_seed(3)
+    for bounds in ([0, 5, 5, 6, 14, 20], [0, 1, 3, 20], [0, 20], [0, 7, 12]):   # empty / one-token segments, a tail outside
+        mask = (torch.rand(2, 20, generator=gen) > 0.25).float()
+        for depth in (0, 1, 2, 6):
+            want = _shift_mask_loop(mask, depth + 1, bounds)
+            assert torch.equal(O.shift_mask_for_mtp(mask.clone(), depth, torch.tensor(bounds)), want), (bounds, depth)
+            assert torch.equal(product(mask.clone(), depth, torch.tensor(bounds)), want), (bounds, depth)
+            assert torch.equal(product(mask.clone(), depth, bounds), want)
+    mask = (torch.rand(3, 9, generator=gen) > 0.3).float()
+    for depth in (0, 1, 3, 8, 11):
+        want = _shift_mask_loop(mask, depth + 1, [0, 9])
+        assert torch.equal(O.shift_mask_for_mtp(mask.clone(), depth), want)
+        assert torch.equal(product(mask.clone(), depth), want)
+
+
+def test_soft_ce_is_entropy_plus_kl_and_its_limits():
+    gen = torch.Generator().manual_seed(12)
+    student = torch.randn(3, 5, 11, generator=gen, dtype=torch.float64) * 2
+    teacher = torch.randn(3, 5, 11, generator=gen, dtype=torch.float64) * 2
+    got = O.soft_ce_per_token(student, teacher)
+    p = torch.distributions.Categorical(logits=teacher)
+    kl = torch.nn.functional.kl_div(torch.log_softmax(student, -1), torch.softmax(teacher, -1), reduction="none").sum(-1)
+    torch.testing.assert_close(got, p.entropy() + kl, rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(got, p.entropy() + torch.distributions.kl_divergence(p, torch.distributions.Categorical(logits=student)))
+    # teacher = student: the entropy; a shift of either logits row changes nothing
+    torch.testing.assert_close(O.soft_ce_per_token(teacher + 3.0, teacher - 1.0), p.entropy())
+    # a one-hot teacher: minus the student's log-probability of that token, i.e. the pinned forward with these labels
+    labels = torch.randint(0, 11, (3, 5), generator=gen)
+    hot = torch.full((3, 5, 11), -1e4, dtype=torch.float64).scatter_(-1, labels[..., None], 0.0)
+    want = -O.distributed_log_softmax(student).gather(-1, labels[..., None])[..., 0]
+    torch.testing.assert_close(O.soft_ce_per_token(student, hot), want)
+    # uniform teacher over V: ln V + mean of (lse - z)
+    uni = torch.zeros(3, 5, 11, dtype=torch.float64)
+    torch.testing.assert_close(O.soft_ce_per_token(student, uni), torch.logsumexp(student, -1) - student.mean(-1))
+
+
+def test_draft_soft_ce_reduction_gradient_and_teacher_checks():
+    gen = torch.Generator().manual_seed(13)
+    student = torch.randn(2, 4, 6, generator=gen, dtype=torch.float64)
+    teacher = torch.randn(2, 4, 6, generator=gen, dtype=torch.float64)
+    mask = torch.tensor([[1.0, 1.0, 0.0, 1.0], [0.0, 1.0, 1.0, 0.0]], dtype=torch.float64)
+    per = O.soft_ce_per_token(student, teacher)
+    by_hand = sum(per[b, t].item() for b in range(2) for t in range(4) if mask[b, t]) / 5
+    assert O.draft_soft_ce(student, teacher, mask).item() == pytest.approx(by_hand)
+    assert O.draft_soft_ce(student, teacher, mask, torch.tensor(20.0)).item() == pytest.approx(by_hand * 5 / 20)
+    assert O.draft_soft_ce(student, teacher, mask, torch.tensor(0.25)).item() == pytest.approx(by_hand * 5)   # clamp(min=1)
+    # masked-out positions do not enter (test_soft_ce.py:184-194)
+    other = teacher.clone()
+    other[0, 2] = torch.randn(6, generator=gen, dtype=torch.float64)
+    assert O.draft_soft_ce(student, other, mask).item() == pytest.approx(by_hand)
+    # gradient: (softmax(student) - softmax(teacher)) * mask / n (test_soft_ce.py:171-181), against central differences
+    x = student.clone().requires_grad_(True)
+    O.draft_soft_ce(x, teacher, mask).backward()
+    want = (torch.softmax(student, -1) - torch.softmax(teacher, -1)) * mask[..., None] / 5
+    torch.testing.assert_close(x.grad, want, rtol=1e-10, atol=1e-12)
+    eps = 1e-6
+    for idx in [(0, 0, 1), (0, 2, 3), (1, 1, 5), (1, 2, 0)]:
+        d = torch.zeros_like(student)
+        d[idx] = eps
+        fd = (O.draft_soft_ce(student + d, teacher, mask) - O.draft_soft_ce(student - d, teacher, mask)).item() / (2 * eps)
+        assert x.grad[idx].item() == pytest.approx(fd, abs=1e-8)
+    assert x.grad.sum(-1).abs().max().item() < 1e-14                  # rows of the gradient sum to zero
+    with pytest.raises(AssertionError, match="must be detached"):
+        O.draft_soft_ce(student, teacher.clone().requires_grad_(True), mask)
+
+
+def test_build_teacher_logits_and_hidden_chain():
+    ml = torch.arange(2 * 4 * 3, dtype=torch.float64, requires_grad=True).reshape(2, 4, 3)
+    assert torch.equal(O.build_teacher_logits(ml, 0), torch.roll(ml.detach(), -1, dims=1))
+    assert torch.equal(O.build_teacher_logits(ml, 1), torch.roll(ml.detach(), -2, dims=1))
+    assert not O.build_teacher_logits(ml, 0).requires_grad
+    # the hidden-state chain: position t of the student against position t + depth + 1 of the policy, by a per-position loop
+    gen = torch.Generator().manual_seed(14)
+    B, S, H, V, depth = 2, 6, 8, 13, 1
+    hs = torch.randn(B, S, H, generator=gen, dtype=torch.float64, requires_grad=True)
+    ht = torch.randn(B, S, H, generator=gen, dtype=torch.float64)
+    w = torch.randn(V, H, generator=gen, dtype=torch.float64, requires_grad=True)
+    mask = O.shift_mask_for_mtp(torch.ones(B, S, dtype=torch.float64), depth)
+    got = O.draft_soft_ce_from_hidden(hs, ht, w, mask, depth)
+    total, n = 0.0, 0
+    for b in range(B):
+        for t in range(S - depth - 1):
+            p = torch.softmax(w.detach() @ ht[b, t + depth + 1], -1)
+            total += -(p * torch.log_softmax(w.detach() @ hs[b, t].detach(), -1)).sum().item()
+            n += 1
+    assert got.item() == pytest.approx(total / n)
+    got.backward()
+    assert w.grad is None and hs.grad is not None                      # the output weight is detached

@@ -1244,3 +1244,119 @@ def test_full_size_forward_qwen05b(cuda_device):
 
 def test_full_size_forward_backward_qwen7b(cuda_device):
     _full_size_check(CONFIGS["qwen2.5-7b-fwdbwd"], cuda_device)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# MTP draft loss: soft cross-entropy from hidden states
+# ---------------------------------------------------------------------------------------------------------------------
+SOFTCE_ATOL = 5e-3   # per-token loss, absolute (values are of the order of ln V)
+
+
+def _softce_case(B, S, H, V, seed, spread=3.0):
+    gen = torch.Generator().manual_seed(seed)
+    hs = torch.randn(B, S, H, generator=gen).bfloat16()
+    ht = torch.randn(B, S, H, generator=gen).bfloat16()
+    w = (torch.randn(V, H, generator=gen) * spread / H ** 0.5).bfloat16()
+    return hs, ht, w
+
+
+@pytest.mark.parametrize("B,S,H,V,depth,temperature,vocab_chunk", [
+    (3, 50, 128, 1000, 0, 1.0, 0),        # ragged tokens and vocabulary, transposed-weight fallback (V % 64 != 0)
+    (2, 200, 192, 1088, 1, 0.7, 0),       # weight read in place, depth 1, a temperature
+    (1, 333, 128, 1000, 2, 1.0, 256),     # one packed row, four vocabulary chunks
+    (4, 128, 256, 8192, 0, 1.0, 2048),    # whole tiles, four chunks in place
+])
+def test_soft_ce_from_hidden_matches_oracle(B, S, H, V, depth, temperature, vocab_chunk, cuda_device):
+    from skyrl_amd.mtp_soft_ce import soft_ce_from_hidden
+
+    hs, ht, w = _softce_case(B, S, H, V, 40 + depth)
+    gen = torch.Generator().manual_seed(77)
+    g = torch.randn(B, S, generator=gen) * (torch.rand(B, S, generator=gen) > 0.3)
+
+    hs64 = hs.double().requires_grad_(True)
+    student_logits = hs64 @ w.double().t() / temperature
+    teacher_logits = O.build_teacher_logits(ht.double() @ w.double().t() / temperature, depth)
+    ref = O.soft_ce_per_token(student_logits, teacher_logits)
+    (ref * g.double()).sum().backward()
+
+    d_hs = hs.to(cuda_device).requires_grad_(True)
+    got = soft_ce_from_hidden(d_hs, ht.to(cuda_device), w.to(cuda_device), shift=depth + 1, temperature=temperature,
+                              vocab_chunk=vocab_chunk)
+    assert got.shape == (B, S) and got.dtype == torch.float32
+    (got * g.to(cuda_device)).sum().backward()
+    err = (got.detach().cpu().double() - ref.detach()).abs().max().item()
+    assert err <= SOFTCE_ATOL, f"per-token loss max abs err {err}"
+    assert d_hs.grad.dtype == torch.bfloat16 and d_hs.grad.shape == hs.shape
+    assert cos(d_hs.grad.float(), hs64.grad) >= GRAD_COS
+    rel = (d_hs.grad.cpu().double() - hs64.grad).norm() / hs64.grad.norm()
+    assert rel.item() <= 2e-2, f"gradient relative error {rel.item()}"
+    assert bool((d_hs.grad.cpu()[g == 0] == 0).all())           # tokens without an upstream gradient get exact zeros
+
+
+def test_soft_ce_limits_against_the_logprob_kernels(cuda_device):
+    """Teacher = student, no roll: the loss is the entropy the log-probability forward reports, and the gradient is exactly
+    zero (both softmaxes come from the same accumulator values)."""
+    from skyrl_amd.mtp_soft_ce import soft_ce_from_hidden
+
+    hs, _, w = _softce_case(2, 300, 128, 2000, 51)
+    d_hs = hs.to(cuda_device).requires_grad_(True)
+    dw = w.to(cuda_device)
+    loss = soft_ce_from_hidden(d_hs, d_hs.detach(), dw, shift=0)
+    loss.sum().backward()
+    labels = torch.zeros(600, dtype=torch.int64, device=cuda_device)
+    _, entropy, _, _ = ops.lmhead_fwd(d_hs.detach().reshape(600, 128), dw, labels, 1.0, True)
+    torch.testing.assert_close(loss.detach().reshape(-1), entropy, rtol=1e-5, atol=1e-5)
+    assert bool((d_hs.grad == 0).all())
+
+
+def test_draft_soft_ce_from_hidden_matches_oracle(cuda_device):
+    from skyrl_amd.mtp_soft_ce import draft_soft_ce_from_hidden, shift_mask_for_mtp
+
+    B, S, H, V, depth = 3, 70, 128, 1500, 1
+    hs, ht, w = _softce_case(B, S, H, V, 60)
+    gen = torch.Generator().manual_seed(61)
+    attn = (torch.rand(B, S, generator=gen) > 0.2).float()
+    attn[1, :9] = 0                                              # left padding
+    mask = O.shift_mask_for_mtp(attn.clone(), depth)
+    for factor in (None, torch.tensor(57.0), torch.tensor(0.5)):
+        hs64 = hs.double().requires_grad_(True)
+        ref = O.draft_soft_ce_from_hidden(hs64, ht.double(), w.double(), mask.double(), depth, factor)
+        ref.backward()
+        d_hs = hs.to(cuda_device).requires_grad_(True)
+        d_mask = shift_mask_for_mtp(attn.to(cuda_device), depth)
+        assert torch.equal(d_mask.cpu(), mask)
+        got = draft_soft_ce_from_hidden(d_hs, ht.to(cuda_device), w.to(cuda_device), d_mask, depth,
+                                        None if factor is None else factor.to(cuda_device))
+        got.backward()
+        assert got.dim() == 0 and got.item() == pytest.approx(ref.item(), abs=SOFTCE_ATOL * max(1.0, ref.item() / 10))
+        assert cos(d_hs.grad.float(), hs64.grad) >= GRAD_COS
+    with pytest.raises(AssertionError, match="must be detached"):
+        draft_soft_ce_from_hidden(d_hs, ht.to(cuda_device).requires_grad_(True), w.to(cuda_device), d_mask, depth)
+
+
+def test_soft_ce_argument_errors(cuda_device):
+    lib = _lib.load()
+    x = torch.zeros(256, 128, dtype=torch.bfloat16, device=cuda_device)
+    f = torch.zeros(256, dtype=torch.float32, device=cuda_device)
+    ws = torch.zeros(lib.skyrl_softce_fwd_workspace_bytes(256, 128, 256), dtype=torch.uint8, device=cuda_device)
+    p, fp = x.data_ptr(), f.data_ptr()
+
+    def fwd(**kw):
+        a = dict(s=p, lds=128, t=p, ldt=128, w=p, ldw=128, T=256, seq=64, shift=1, H=128, V=256, rt=1.0, loss=fp, ls=fp, lt=fp,
+                 ws=ws.data_ptr(), wsb=ws.numel())
+        a.update(kw)
+        return lib.skyrl_softce_fwd(a["s"], a["lds"], a["t"], a["ldt"], a["w"], a["ldw"], a["T"], a["seq"], a["shift"], a["H"],
+                                    a["V"], a["rt"], a["loss"], a["ls"], a["lt"], a["ws"], a["wsb"], None)
+
+    assert fwd() == 0
+    assert fwd(t=None) == -1 and fwd(loss=None) == -1
+    assert fwd(seq=100) == -2 and fwd(seq=0) == -2 and fwd(shift=-1) == -2 and fwd(ldt=64) == -2
+    assert fwd(t=p + 8) == -3
+    assert fwd(wsb=1024) == -4 and fwd(ws=None) == -4
+    assert fwd(rt=0.0) == -5
+    assert lib.skyrl_softce_bwd_workspace_bytes(256, 128, 256, 100) == 0
+    assert lib.skyrl_softce_bwd(p, 128, p, 128, p, 128, fp, fp, None, 256, 64, 1, 128, 256, 1.0, p, 0, ws.data_ptr(), ws.numel(),
+                                None) == -1
+    assert lib.skyrl_softce_bwd(p, 128, p, 128, p, 128, fp, fp, fp, 256, 64, 1, 128, 256, 1.0, p, 0, ws.data_ptr(), 1024,
+                                None) == -4
+    torch.cuda.synchronize()
