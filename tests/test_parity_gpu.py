@@ -1360,3 +1360,34 @@ def test_soft_ce_argument_errors(cuda_device):
     assert lib.skyrl_softce_bwd(p, 128, p, 128, p, 128, fp, fp, fp, 256, 64, 1, 128, 256, 1.0, p, 0, ws.data_ptr(), 1024,
                                 None) == -4
     torch.cuda.synchronize()
+
+
+def test_soft_ce_full_size_properties(cuda_device):
+    """The benchmark shape (T=16384, H=3584, V=152064), through size-independent properties: teacher = student gives the
+    entropy of the log-probability forward and an exactly zero gradient; the per-token loss is at least the teacher's
+    entropy (Gibbs); the gradient is linear in the upstream gradient for power-of-two factors, bit for bit."""
+    from skyrl_amd.mtp_soft_ce import softce_bwd, softce_fwd
+
+    T, H, V = 16384, 3584, 152064
+    gen = torch.Generator(device=cuda_device).manual_seed(9)
+    hs = torch.randn(T, H, generator=gen, device=cuda_device).bfloat16()
+    ht = torch.randn(T, H, generator=gen, device=cuda_device).bfloat16()
+    w = (torch.randn(V, H, generator=gen, device=cuda_device) * 3 / H ** 0.5).bfloat16()
+    g = torch.randn(T, generator=gen, device=cuda_device)
+    labels = torch.zeros(T, dtype=torch.int64, device=cuda_device)
+
+    loss_self, lse_s, lse_t = softce_fwd(ht, ht, w, T, 0, 1.0)
+    _, entropy, lse, _ = ops.lmhead_fwd(ht, w, labels, 1.0, True)
+    torch.testing.assert_close(loss_self, entropy, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(lse_t, lse, rtol=1e-6, atol=1e-6)
+    assert bool((softce_bwd(ht, ht, w, lse_s, lse_t, g, T, 0, 1.0, 0) == 0).all())
+
+    loss, lse_s, lse_t = softce_fwd(hs, ht, w, T, 1, 1.0)
+    rolled_entropy = torch.roll(entropy, -1)                      # the teacher of token t is row t + 1
+    assert bool((loss >= rolled_entropy - 1e-3).all()) and bool(torch.isfinite(loss).all())
+    d1 = softce_bwd(hs, ht, w, lse_s, lse_t, g, T, 1, 1.0, 0)
+    d4 = softce_bwd(hs, ht, w, lse_s, lse_t, g * 4.0, T, 1, 1.0, 0)
+    assert torch.equal(d4.float(), d1.float() * 4.0) and bool(torch.isfinite(d1.float()).all())
+    # a different vocabulary chunking changes the order of the fp32 partial sums only
+    d_chunked = softce_bwd(hs, ht, w, lse_s, lse_t, g, T, 1, 1.0, 16384)
+    assert cos(d_chunked.float(), d1.float()) >= 0.99999
