@@ -22,6 +22,8 @@ What pins each function (all in ``tests/test_oracle.py``; none of them re-types 
   * packed-sequence roll and scatter-back (plain, sub-sequence and attention-mask layouts): per-sequence Python loops that
     place each token by hand, over ragged cases with length-1 and empty sequences, padded segments, left- and
     interior-padded masks and outputs narrower than a row's content.
+  * packed action-token entropy: a per-row Python loop that walks each row's real tokens (or listed sub-sequences) and
+    adds up entropy times weight by hand, with loss masks, left padding and a row without action weight.
   * PPO policy loss: hand-computed cases on both sides of every branch (unclipped, clipped high / low for either sign of
     the advantage, dual-clip active / inactive, the +-20 clamp of the log-ratio), fp64 central finite differences of the
     loss for the gradient autograd derives from it, and the masked-mean definition of clip_ratio counted by hand.
@@ -370,6 +372,43 @@ def packed_scatter_back(
 # ----------------------------------------------------------------------------------------------------------------------
 # Convenience used by the parity tests and the CPU baseline: one call = forward + backward of the whole path
 # ----------------------------------------------------------------------------------------------------------------------
+def packed_action_entropy(
+    entropy_tokens: torch.Tensor,
+    cu_seqlens: torch.Tensor,
+    unpacked_seqlen: int,
+    num_actions: int,
+    attention_mask: torch.Tensor,
+    loss_mask: Optional[torch.Tensor],
+    sub_seq_lengths: Optional[Sequence[Sequence[int]]] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """MU:1124-1208 at CP = 1, after the per-token entropy: the action weights (ones, or the loss mask, in the last
+    ``num_actions`` columns of [B, unpacked_seqlen - 1], MU:1153-1157) are carried to the packed stream by the inverse of the
+    scatter-back mapping (sub-sequences MU:1160-1172, attention mask MU:1173-1179) and the entropy is their weighted mean
+    with the weight sum clamped at 1 (MU:1196-1207).  Returns ``(entropy, entropy_for_loss)``, equal at CP = 1."""
+    batch = int(attention_mask.shape[0])
+    weights = torch.zeros((batch, unpacked_seqlen - 1), dtype=entropy_tokens.dtype)
+    weights[:, -num_actions:] = 1.0 if loss_mask is None else loss_mask.to(entropy_tokens.dtype)
+    packed = torch.zeros(int(cu_seqlens[-1]), dtype=entropy_tokens.dtype)
+    if sub_seq_lengths is not None:
+        seq_idx, seq_off, _ = packed_sequence_indices(cu_seqlens, int(packed.shape[0]))
+        rows, offs, lens = packed_subseq_rows_offsets_lens(cu_seqlens, sub_seq_lengths)
+        take = seq_off < torch.clamp(lens - 1, min=0)[seq_idx]
+        cols = offs[seq_idx[take]] + seq_off[take]
+        rws = rows[seq_idx[take]]
+        inb = cols < weights.shape[1]
+        packed[torch.arange(int(packed.shape[0]))[take][inb]] = weights[rws[inb], cols[inb]]
+    else:
+        am = attention_mask.to(torch.bool)
+        real = am.sum(dim=1, dtype=torch.long)
+        ordinal = am.to(torch.long).cumsum(dim=1)
+        out_mask = am[:, :-1] & (ordinal[:, :-1] < real.unsqueeze(1))
+        where = cu_seqlens.to(torch.long)[:-1].unsqueeze(1) + (ordinal - 1)
+        packed[where[:, :-1][out_mask]] = weights[out_mask]
+    total = (entropy_tokens * packed).sum()
+    count = packed.sum().clamp(min=1.0)
+    return total / count, total / count
+
+
 def reference_faithful_fwd_bwd(
     hidden: torch.Tensor,
     weight: torch.Tensor,

@@ -12,6 +12,9 @@
 //                      panel of the chunk.  GEMM tiles: dHidden (+)= dz . weight and dW[chunk] = dz^T . hidden with fp32
 //                      accumulation, both from that panel -- dW reads it K-major, dHidden reads the weight K-major in
 //                      place -- through the transposing LDS read (gemm_core.hpp).
+// Soft cross-entropy of a draft head against the policy (10*T*V*H flop): softce_pack_rows stacks the two hidden rows of every
+//   token, softce_fwd_tiles is the forward tile with a paired third statistic, softce_dz_tiles the matching dz producer; merge
+//   and dHidden GEMM are the kernels above.
 // The per-token loss kernels and the packed-sequence index kernels live in loss_kernels.hip and packed_kernels.hip.
 #include <hip/hip_runtime.h>
 #include <math.h>

@@ -7,6 +7,7 @@ trainer can import these instead:
 * ``from_parallel_hidden_to_logprobs``                   (:713-770)
 * ``from_parallel_hidden_to_logprobs_packed_sequences``  (:773-883)
 * ``_fused_vocab_parallel_entropy_from_hidden``          (:1090-1121)
+* ``from_parallel_hidden_to_entropy_packed_sequences``   (:1124-1208)
 * ``_packed_sequence_indices``, ``_packed_subseq_row_indices_offsets_and_lens``  (:920-928, :886-917)
 
 The packed variant prepares its labels and scatters its result back with one HIP kernel each (``skyrl_amd/packed.py``)
@@ -200,6 +201,52 @@ def _fused_vocab_parallel_entropy_from_hidden(
         _, entropy, _, _ = ops.lmhead_fwd(hidden.reshape(B * S, H).to(lm_head_weight.dtype).contiguous(),
                                           lm_head_weight.contiguous(), labels, 1.0 / float(temperature), True)
     return entropy.reshape(B, S)
+
+
+def from_parallel_hidden_to_entropy_packed_sequences(
+    hidden: torch.Tensor,
+    lm_head_weight: torch.Tensor,
+    cu_seqlens_padded: torch.Tensor,
+    unpacked_seqlen: int,
+    num_actions: int,
+    attention_mask: torch.Tensor,
+    loss_mask: Optional[torch.Tensor],
+    cp_group: Optional[dist.ProcessGroup],
+    tp_group: Optional[dist.ProcessGroup],
+    sub_seq_lengths: Optional[list] = None,
+    chunk_size: Optional[int] = None,
+    temperature: float = 1.0,
+):
+    """Action-token mean of the per-token entropy of a packed ``hidden`` [1, T, H]: ``(entropy, entropy_for_loss)``, both
+    0-dim and without gradient (the metric the Megatron worker logs).
+
+    The reference carries the ``[B, unpacked_seqlen - 1]`` action weights to the packed stream with boolean-mask indexing
+    and one ``.item()`` (:1153-1179); here the per-token entropy goes the other way through the scatter-back kernel, together
+    with a vector of ones that marks the positions a packed token lands on, and the weighted mean is taken in the
+    ``[B, unpacked_seqlen - 1]`` layout -- the same sums, no host synchronisation.
+    """
+    if _group_size(cp_group) > 1:
+        raise NotImplementedError("context parallelism is outside the one-GPU scope of the HIP fused LM-head path")
+    entropy_tokens = _fused_vocab_parallel_entropy_from_hidden(hidden, lm_head_weight, tp_group, chunk_size=chunk_size,
+                                                               temperature=temperature).squeeze(0)
+    device = entropy_tokens.device
+    batch_size = attention_mask.shape[0]
+    cols = unpacked_seqlen - 1
+    with torch.no_grad():
+        action_weights = torch.zeros((batch_size, cols), dtype=entropy_tokens.dtype, device=device)
+        action_weights[:, -num_actions:] = 1.0 if loss_mask is None else loss_mask.to(device=device, dtype=entropy_tokens.dtype)
+        cu = cu_seqlens_padded.to(device=device, dtype=torch.long)
+        if sub_seq_lengths is not None:
+            rows, row_offs, seq_lens = _packed_subseq_row_indices_offsets_and_lens(cu, sub_seq_lengths, device)
+            layout = dict(seg_row=rows, seg_col=row_offs, seg_len=seq_lens)
+        else:
+            layout = dict(attention_mask=attention_mask.to(device=device, dtype=torch.bool))
+        entropy_bs = packed_scatter_logprobs(entropy_tokens.contiguous(), cu, batch_size, cols, **layout)
+        landed = packed_scatter_logprobs(torch.ones_like(entropy_tokens), cu, batch_size, cols, **layout)
+        total = (entropy_bs * action_weights).sum()
+        count = (landed * action_weights).sum().clamp(min=1.0)
+        entropy = total / count
+    return entropy, entropy.clone()
 
 
 def fused_logprobs_and_entropy_from_hidden(

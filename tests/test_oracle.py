@@ -771,6 +771,59 @@ def test_hf_wrapper_tail_brute_force():
     assert full.shape == (B, S - 1)
 
 
+def test_packed_action_entropy_brute_force():
+    gen = torch.Generator().manual_seed(21)
+    # attention-mask layout: rows with left, right and interior padding; row b owns packed tokens cu[b] .. cu[b]+real_b-1
+    L, num_actions = 9, 4
+    am = torch.tensor([[1, 1, 1, 1, 1, 1, 1, 1, 1],
+                       [0, 0, 1, 1, 1, 1, 1, 0, 0],
+                       [1, 1, 0, 1, 1, 0, 1, 1, 1],
+                       [0, 0, 0, 0, 0, 0, 0, 1, 1]])
+    real = am.sum(1).tolist()
+    padded = [r + (-r) % 4 for r in real]                       # segments padded to a multiple of 4
+    cu = torch.tensor([0] + list(np.cumsum(padded)))
+    ent = torch.rand(int(cu[-1]), generator=gen, dtype=torch.float64) * 3
+    for loss_mask in (None, (torch.rand(4, num_actions, generator=gen) > 0.4).double()):
+        total = count = 0.0
+        for b in range(4):
+            j = 0                                               # index of the real token inside row b
+            for c in range(L - 1):
+                if am[b, c]:
+                    if j + 1 < real[b] and c >= L - 1 - num_actions:
+                        wgt = 1.0 if loss_mask is None else loss_mask[b, c - (L - 1 - num_actions)].item()
+                        total += ent[cu[b] + j].item() * wgt
+                        count += wgt
+                    j += 1
+        got, for_loss = O.packed_action_entropy(ent, cu, L, num_actions, am, loss_mask)
+        assert got.item() == pytest.approx(total / max(count, 1.0)) and for_loss.item() == got.item()
+    # no action weight at all: 0 / clamp(0, 1)
+    got, _ = O.packed_action_entropy(ent, cu, L, num_actions, am, torch.zeros(4, num_actions, dtype=torch.float64))
+    assert got.item() == 0.0
+
+    # sub-sequence layout: two output rows, three and two packed segments; true lengths shorter than the padded ones
+    sub = [[3, 1, 4], [5, 2]]
+    pad = [4, 4, 4, 8, 4]
+    cu = torch.tensor([0] + list(np.cumsum(pad)))
+    ent = torch.rand(int(cu[-1]), generator=gen, dtype=torch.float64)
+    L, num_actions = 12, 6
+    loss_mask = (torch.rand(2, num_actions, generator=gen) > 0.3).double()
+    total = count = 0.0
+    k = 0
+    for r, row in enumerate(sub):
+        col0 = 0
+        for n in row:
+            for o in range(max(n - 1, 0)):
+                c = col0 + o
+                if c < L - 1 and c >= L - 1 - num_actions:
+                    wgt = loss_mask[r, c - (L - 1 - num_actions)].item()
+                    total += ent[cu[k] + o].item() * wgt
+                    count += wgt
+            col0 += pad[k]
+            k += 1
+    got, _ = O.packed_action_entropy(ent, cu, L, num_actions, torch.ones(2, L), loss_mask, sub)
+    assert count > 0 and got.item() == pytest.approx(total / count)
+
+
 # ----------------------------------------------------------------------------------------------------------------------
 # MTP draft loss: soft cross-entropy
 # ----------------------------------------------------------------------------------------------------------------------

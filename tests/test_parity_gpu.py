@@ -1391,3 +1391,45 @@ def test_soft_ce_full_size_properties(cuda_device):
     # a different vocabulary chunking changes the order of the fp32 partial sums only
     d_chunked = softce_bwd(hs, ht, w, lse_s, lse_t, g, T, 1, 1.0, 16384)
     assert cos(d_chunked.float(), d1.float()) >= 0.99999
+
+
+@pytest.mark.parametrize("layout", ["attention_mask", "sub_sequences"])
+@pytest.mark.parametrize("with_loss_mask", [False, True])
+def test_packed_action_entropy_matches_oracle(layout, with_loss_mask, cuda_device):
+    """The Megatron worker's entropy metric on a packed micro-batch: per-token entropy from the forward kernel, action-token
+    weighted mean through the scatter kernels, against the oracle's restatement of the reference's packed-weight route."""
+    gen = torch.Generator().manual_seed(33)
+    H, V, temperature = 128, 1500, 0.8
+    if layout == "attention_mask":
+        L, num_actions = 40, 17
+        real = [40, 23, 31, 5, 1]
+        am = torch.zeros(len(real), L, dtype=torch.long)
+        am[0] = 1
+        am[1, L - 23:] = 1                                       # left padding
+        am[2, :31] = 1                                           # right padding
+        am[3, 10:15] = 1
+        am[4, L - 1] = 1                                         # a single real token: nothing to score
+        padded = [r + (-r) % 8 for r in real]
+        sub = None
+    else:
+        L, num_actions = 48, 30
+        sub = [[9, 1, 14], [20, 6], [33]]
+        padded = [16, 8, 16, 24, 8, 40]
+        am = torch.ones(len(sub), L, dtype=torch.long)
+    B = am.shape[0]
+    cu = torch.tensor([0] + list(np.cumsum(padded)))
+    T = int(cu[-1])
+    hidden = torch.randn(1, T, H, generator=gen).bfloat16()
+    weight = (torch.randn(V, H, generator=gen) * 3 / H ** 0.5).bfloat16()
+    loss_mask = (torch.rand(B, num_actions, generator=gen) > 0.35).float() if with_loss_mask else None
+
+    ent64 = O.fused_entropy_from_hidden(hidden.double(), weight.double(), None, temperature).double().squeeze(0)
+    want, want_loss = O.packed_action_entropy(ent64, cu, L, num_actions, am, None if loss_mask is None else loss_mask.double(), sub)
+
+    to = lambda t: None if t is None else t.to(cuda_device)  # noqa: E731
+    got, got_loss = model_utils.from_parallel_hidden_to_entropy_packed_sequences(
+        to(hidden), to(weight), to(cu), L, num_actions, to(am), to(loss_mask), None, None, sub_seq_lengths=sub,
+        temperature=temperature)
+    assert got.dim() == 0 and not got.requires_grad
+    assert want.item() > 0.5                                     # the case does put weight on real tokens
+    assert got.item() == pytest.approx(want.item(), rel=ENTROPY_RTOL) and got_loss.item() == pytest.approx(want_loss.item(), rel=ENTROPY_RTOL)
