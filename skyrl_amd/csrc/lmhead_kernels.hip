@@ -772,9 +772,10 @@ struct Carver {
 
 inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
-int check_common(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
-                 int64_t H, int64_t V, float rcp_temperature) {
-  if (!hidden || !weight || !labels) return SKYRL_LMHEAD_ERR_NULL;
+// The two bf16 operands of every entry point: hidden rows [T, H] and weight rows [V, H].
+int check_operands(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, int64_t T, int64_t H, int64_t V,
+                   float rcp_temperature) {
+  if (!hidden || !weight) return SKYRL_LMHEAD_ERR_NULL;
   if (T < 1 || V < 1 || H < BK || H % BK != 0 || ldh < H || ldw < H) return SKYRL_LMHEAD_ERR_SHAPE;
   if (T > (int64_t)1 << 30 || V > (int64_t)1 << 30 || ldh > (int64_t)1 << 30 || ldw > (int64_t)1 << 30)
     return SKYRL_LMHEAD_ERR_SHAPE;
@@ -782,10 +783,18 @@ int check_common(const void* hidden, int64_t ldh, const void* weight, int64_t ld
   // never larger than these two transposed) must stay below 4 GiB.
   const int64_t kMaxBytes = (int64_t)1 << 32;
   if (T * ldh * 2 >= kMaxBytes || V * ldw * 2 >= kMaxBytes) return SKYRL_LMHEAD_ERR_SHAPE;
-  if (!aligned16(hidden) || !aligned16(weight) || ((uintptr_t)labels & 7u) || ldh % 8 != 0 || ldw % 8 != 0)
-    return SKYRL_LMHEAD_ERR_ALIGN;
+  if (!aligned16(hidden) || !aligned16(weight) || ldh % 8 != 0 || ldw % 8 != 0) return SKYRL_LMHEAD_ERR_ALIGN;
   if (!(rcp_temperature > 0.f) || !isfinite(rcp_temperature)) return SKYRL_LMHEAD_ERR_ARG;
   return SKYRL_LMHEAD_OK;
+}
+
+int check_common(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
+                 int64_t H, int64_t V, float rcp_temperature) {
+  if (!hidden || !weight || !labels) return SKYRL_LMHEAD_ERR_NULL;
+  const int st = check_operands(hidden, ldh, weight, ldw, T, H, V, rcp_temperature);
+  if (st == SKYRL_LMHEAD_ERR_SHAPE) return st;  // shape errors are reported before alignment errors, labels included
+  if ((uintptr_t)labels & 7u) return SKYRL_LMHEAD_ERR_ALIGN;
+  return st;
 }
 
 // Compute units of the current device (256 on an MI355X); 256 when no device answers, so that the workspace query gives
@@ -947,10 +956,9 @@ SoftCeBwdWorkspace carve_softce_bwd(void* ws, int64_t T, int64_t H, int64_t V, i
 
 int check_softce(const void* student, int64_t lds_, const void* teacher, int64_t ldt, const void* weight, int64_t ldw, int64_t T,
                  int64_t seq_len, int64_t shift, int64_t H, int64_t V, float rcp_temperature) {
-  static const int64_t no_labels = 0;  // check_common wants a labels pointer; this path has none
-  int st = check_common(student, lds_, weight, ldw, &no_labels, T, H, V, rcp_temperature);
-  if (st) return st;
   if (!teacher) return SKYRL_LMHEAD_ERR_NULL;
+  int st = check_operands(student, lds_, weight, ldw, T, H, V, rcp_temperature);
+  if (st) return st;
   if (ldt < H || ldt > (int64_t)1 << 30 || T * ldt * 2 >= ((int64_t)1 << 32)) return SKYRL_LMHEAD_ERR_SHAPE;
   if (seq_len < 1 || T % seq_len != 0 || shift < 0) return SKYRL_LMHEAD_ERR_SHAPE;
   if (2 * round_up(T, kPairTile) * H * 2 >= ((int64_t)1 << 32)) return SKYRL_LMHEAD_ERR_SHAPE;  // the stacked rows
