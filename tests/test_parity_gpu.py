@@ -1433,3 +1433,33 @@ def test_packed_action_entropy_matches_oracle(layout, with_loss_mask, cuda_devic
     assert got.dim() == 0 and not got.requires_grad
     assert want.item() > 0.5                                     # the case does put weight on real tokens
     assert got.item() == pytest.approx(want.item(), rel=ENTROPY_RTOL) and got_loss.item() == pytest.approx(want_loss.item(), rel=ENTROPY_RTOL)
+
+
+@pytest.mark.parametrize("B,S,H,V,shift,vocab_chunk", [
+    (1, 1, 64, 5, 1, 0),             # one token, a vocabulary smaller than a tile; the roll of a one-token row is itself
+    (1, 63, 64, 255, 2, 0),          # one token short of the 64-token pairing unit, one row short of a vocabulary tile
+    (3, 43, 320, 257, 1, 256),       # 129 tokens: one more than a 128-token tile; second chunk holds a single vocab row
+    (5, 128, 128, 4104, 3, 1024),    # whole token tiles, V a multiple of 8 but not of 64, five chunks
+    (7, 19, 192, 777, 20, 0),        # a shift larger than the row: wraps modulo the row length
+    (1, 100, 128, 20032, 1, 4096),   # V a multiple of 64 (weight read in place), five chunks with a short last one
+])
+def test_soft_ce_edge_shapes_match_oracle(B, S, H, V, shift, vocab_chunk, cuda_device):
+    from skyrl_amd.mtp_soft_ce import soft_ce_from_hidden
+
+    hs, ht, w = _softce_case(B, S, H, V, 500 + V)
+    gen = torch.Generator().manual_seed(V)
+    g = torch.randn(B, S, generator=gen)
+    hs64 = hs.double().requires_grad_(True)
+    teacher_logits = torch.roll(ht.double() @ w.double().t(), -shift, dims=1)
+    ref = O.soft_ce_per_token(hs64 @ w.double().t(), teacher_logits)
+    (ref * g.double()).sum().backward()
+    d_hs = hs.to(cuda_device).requires_grad_(True)
+    got = soft_ce_from_hidden(d_hs, ht.to(cuda_device), w.to(cuda_device), shift=shift, vocab_chunk=vocab_chunk)
+    (got * g.to(cuda_device)).sum().backward()
+    err = (got.detach().cpu().double() - ref.detach()).abs().max().item()
+    assert err <= SOFTCE_ATOL, f"per-token loss max abs err {err}"
+    assert bool(torch.isfinite(d_hs.grad.float()).all())
+    if hs64.grad.norm() > 0:
+        assert cos(d_hs.grad.float(), hs64.grad) >= GRAD_COS
+        rel = (d_hs.grad.cpu().double() - hs64.grad).norm() / hs64.grad.norm()
+        assert rel.item() <= 2e-2, f"gradient relative error {rel.item()}"
