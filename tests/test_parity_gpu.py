@@ -1382,10 +1382,33 @@ def test_soft_ce_full_size_properties(cuda_device):
     torch.testing.assert_close(lse_t, lse, rtol=1e-6, atol=1e-6)
     assert bool((softce_bwd(ht, ht, w, lse_s, lse_t, g, T, 0, 1.0, 0) == 0).all())
 
+    lib = _lib.load()
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
     loss, lse_s, lse_t = softce_fwd(hs, ht, w, T, 1, 1.0)
+    torch.cuda.synchronize()
+    peak = torch.cuda.max_memory_allocated() - base
+    assert peak < lib.skyrl_softce_fwd_workspace_bytes(T, H, V) + 16 * 4 * T + (64 << 20)
+    assert peak < 2 * T * V / 4                                   # far below one bf16 T x V buffer, let alone two in fp32
+    # sampled tokens against fp64 logits of just those rows
+    rows = torch.randperm(T - 1, generator=torch.Generator().manual_seed(3))[:12].sort().values
+    w64 = w.cpu().double()
+    zs = hs.cpu()[rows].double() @ w64.t()
+    zt = ht.cpu()[rows + 1].double() @ w64.t()
+    want = O.soft_ce_per_token(zs, zt)
+    assert (loss.cpu()[rows].double() - want).abs().max().item() <= SOFTCE_ATOL
     rolled_entropy = torch.roll(entropy, -1)                      # the teacher of token t is row t + 1
     assert bool((loss >= rolled_entropy - 1e-3).all()) and bool(torch.isfinite(loss).all())
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
     d1 = softce_bwd(hs, ht, w, lse_s, lse_t, g, T, 1, 1.0, 0)
+    torch.cuda.synchronize()
+    peak = torch.cuda.max_memory_allocated() - base
+    assert peak < lib.skyrl_softce_bwd_workspace_bytes(T, H, V, 0) + 2 * T * H + (64 << 20)
+    assert lib.skyrl_softce_bwd_workspace_bytes(T, H, V, 0) < 2 * T * V
+    want_rows = ((torch.softmax(zs, -1) - torch.softmax(zt, -1)) * g.cpu()[rows].double()[:, None]) @ w64
+    assert cos(d1.cpu()[rows].float(), want_rows) >= GRAD_COS
     d4 = softce_bwd(hs, ht, w, lse_s, lse_t, g * 4.0, T, 1, 1.0, 0)
     assert torch.equal(d4.float(), d1.float() * 4.0) and bool(torch.isfinite(d1.float()).all())
     # a different vocabulary chunking changes the order of the fp32 partial sums only
