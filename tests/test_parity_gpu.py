@@ -1486,3 +1486,19 @@ def test_soft_ce_edge_shapes_match_oracle(B, S, H, V, shift, vocab_chunk, cuda_d
         assert cos(d_hs.grad.float(), hs64.grad) >= GRAD_COS
         rel = (d_hs.grad.cpu().double() - hs64.grad).norm() / hs64.grad.norm()
         assert rel.item() <= 2e-2, f"gradient relative error {rel.item()}"
+
+
+@pytest.mark.parametrize("B,S,chunk", [(2, 4, 3), (2, 4, 8), (2, 4, 16), (1, 8, 3), (4, 1, 2), (1, 1, 1)])
+def test_identity_lm_head_known_answer(B, S, chunk, cuda_device):
+    """The reference's chunk-boundary cases (tests/tx/utils/test_logits_processor.py:39-58) on its deterministic input: an
+    identity LM head and hidden = arange / n, so the logits are the hidden states themselves and the answer is
+    log_softmax(hidden)[target] whatever the sequence chunk is.  H = V = 64 here (the kernel's k-tile) instead of 16."""
+    V = 64
+    hidden = (torch.arange(B * S * V, dtype=torch.float32).reshape(B, S, V) / (B * S * V)).bfloat16()
+    target = (torch.arange(B * S).reshape(B, S) % V)
+    weight = torch.eye(V).bfloat16()
+    want = torch.log_softmax(hidden.double(), -1).gather(-1, target[..., None])[..., 0]
+    got = FusedLinearLogprobHip.apply(hidden.to(cuda_device), weight.to(cuda_device), target.to(cuda_device), 0, V, chunk, None,
+                                      True)
+    assert got.shape == (B, S)
+    torch.testing.assert_close(got.cpu().double(), want, rtol=1e-5, atol=1e-5)   # the reference's own tolerance
