@@ -1502,3 +1502,49 @@ def test_identity_lm_head_known_answer(B, S, chunk, cuda_device):
                                       True)
     assert got.shape == (B, S)
     torch.testing.assert_close(got.cpu().double(), want, rtol=1e-5, atol=1e-5)   # the reference's own tolerance
+
+
+def test_entry_points_replay_from_a_hip_graph(cuda_device):
+    """The C-ABI entry points neither allocate nor synchronise, so a forward + backward step can be captured into a HIP graph
+    (workspaces and outputs come from the capturing allocator's pool).  Three replays, with eager work and synchronisations
+    of the program's own between them and new values in the static inputs each time, must each reproduce the eager result
+    bit for bit."""
+    gen = torch.Generator().manual_seed(91)
+    T, H, V = 300, 128, 1500
+    weight = (torch.randn(V, H, generator=gen) * 3 / H ** 0.5).bfloat16().to(cuda_device)
+    hidden = torch.zeros(T, H, dtype=torch.bfloat16, device=cuda_device)
+    labels = torch.zeros(T, dtype=torch.int64, device=cuda_device)
+    g = torch.zeros(T, device=cuda_device)
+    q = torch.zeros(T, device=cuda_device)
+
+    def step():
+        lp, ent, lse, pz = ops.lmhead_fwd(hidden, weight, labels, 0.8, True)
+        dh, dw = ops.lmhead_bwd(hidden, weight, labels, lse, pz, g, q, 0.8, 512)
+        return lp, ent, dh, dw
+
+    def refill(seed):
+        gen_ = torch.Generator().manual_seed(seed)
+        hidden.copy_(torch.randn(T, H, generator=gen_).bfloat16())
+        labels.copy_(torch.randint(0, V, (T,), generator=gen_))
+        g.copy_(torch.randn(T, generator=gen_))
+        q.copy_(torch.randn(T, generator=gen_) * 0.01)
+
+    refill(0)
+    side = torch.cuda.Stream(device=cuda_device)
+    side.wait_stream(torch.cuda.current_stream(cuda_device))
+    with torch.cuda.stream(side):
+        step()                                                   # warm-up outside the capture (library load, first launches)
+    torch.cuda.current_stream(cuda_device).wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step()
+    for seed in (1, 2, 3):
+        refill(seed)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in captured]
+        want = step()                                            # eager, on the same inputs
+        torch.cuda.synchronize()
+        for a, b in zip(got, want):
+            assert torch.equal(a, b)
