@@ -13,6 +13,12 @@ kernel's host code (fused_linear_logprob_triton.py:749-801).
 shard per rank the same arithmetic is: ``m = all_reduce(row_lse, MAX)``; ``lse = m + log(all_reduce(exp(row_lse - m), SUM))``;
 ``pz = all_reduce(exp(row_lse - lse) * row_pz, SUM)``; ``z_y = all_reduce(owner ? logprob + row_lse : 0, SUM)``; and the
 ``d_hidden`` shares are summed by the all-reduce (or the sequence-parallel reduce-scatter) that follows the LM head.
+The soft cross-entropy of the draft head shards the same way (``merge_soft_ce_shard_statistics``): per slice ``softce_fwd``
+returns the two log-sum-exps of the slice and ``loss = lse_student - E_teacher[z_student]`` with the teacher normalised over
+the slice; the group exchanges three ``[T]`` vectors (the MAX / SUM all-reduces of ``_vocab_parallel_softmax`` /
+``_vocab_parallel_log_softmax`` and the SUM of the per-token dot product, skyrl/backends/skyrl_train/mtp/soft_ce.py:97-143), and
+``softce_bwd`` with the global log-sum-exps gives every slice its share of the student's gradient.
+
 This module runs no collective: process groups larger than one are refused by the autograd front ends.
 """
 
@@ -22,7 +28,7 @@ from typing import Tuple
 
 import torch
 
-__all__ = ["merge_shard_statistics"]
+__all__ = ["merge_shard_statistics", "merge_soft_ce_shard_statistics"]
 
 
 def merge_shard_statistics(logprobs: torch.Tensor, row_lse: torch.Tensor, row_pz: torch.Tensor,
@@ -39,3 +45,17 @@ def merge_shard_statistics(logprobs: torch.Tensor, row_lse: torch.Tensor, row_pz
     z_target = torch.where(owner, logprobs + row_lse, torch.zeros_like(logprobs)).sum(dim=0)
     merged_logprobs = torch.where(owned, z_target - lse, torch.zeros_like(lse))
     return merged_logprobs, lse - pz, lse, pz
+
+
+def merge_soft_ce_shard_statistics(loss: torch.Tensor, lse_student: torch.Tensor,
+                                   lse_teacher: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Per-shard outputs of ``softce_fwd`` (each ``[shards, T]`` fp32) -> global ``(loss, lse_student, lse_teacher)``.
+
+    A shard's ``lse_student - loss`` is the teacher-weighted mean of the student's logits over that shard; weighting the
+    shards by their share of the teacher's probability mass, ``exp(lse_teacher_shard - lse_teacher)``, gives the global mean."""
+    if not (loss.shape == lse_student.shape == lse_teacher.shape and loss.dim() == 2):
+        raise ValueError("expected three [shards, T] tensors")
+    lse_s = torch.logsumexp(lse_student, dim=0)
+    lse_t = torch.logsumexp(lse_teacher, dim=0)
+    mean_z = (torch.exp(lse_teacher - lse_t) * (lse_student - loss)).sum(dim=0)
+    return lse_s - mean_z, lse_s, lse_t

@@ -245,6 +245,30 @@ def test_packed_index_helpers_match_brute_force():
         model_utils._packed_subseq_row_indices_offsets_and_lens(torch.tensor([0, 4, 8, 9]), [[3], [4]], torch.device("cpu"))
 
 
+def test_merge_soft_ce_shard_statistics_equals_full_vocabulary():
+    """Per-slice soft cross-entropy statistics merged on the host against the full-vocabulary value, fp64."""
+    from skyrl_amd.vocab_shards import merge_soft_ce_shard_statistics
+
+    gen = torch.Generator().manual_seed(13)
+    T, V = 11, 37
+    zs = torch.randn(T, V, dtype=torch.float64, generator=gen) * 3
+    zt = torch.randn(T, V, dtype=torch.float64, generator=gen) * 3
+    bounds = [0, 1, 9, 30, 37]
+    loss, ls, lt = [], [], []
+    for lo, hi in zip(bounds[:-1], bounds[1:]):
+        a, b = zs[:, lo:hi], zt[:, lo:hi]
+        loss.append(-(torch.softmax(b, -1) * torch.log_softmax(a, -1)).sum(-1))
+        ls.append(torch.logsumexp(a, -1))
+        lt.append(torch.logsumexp(b, -1))
+    got, got_ls, got_lt = merge_soft_ce_shard_statistics(torch.stack(loss), torch.stack(ls), torch.stack(lt))
+    want = -(torch.softmax(zt, -1) * torch.log_softmax(zs, -1)).sum(-1)
+    torch.testing.assert_close(got, want, rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(got_ls, torch.logsumexp(zs, -1), rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(got_lt, torch.logsumexp(zt, -1), rtol=1e-12, atol=1e-12)
+    with pytest.raises(ValueError):
+        merge_soft_ce_shard_statistics(got, got_ls, got_lt)
+
+
 def test_merge_shard_statistics_equals_full_vocabulary_softmax():
     """The host-side merge of per-slice statistics (what a vocabulary-parallel group's all-reduces compute) against a plain
     log-softmax over the whole vocabulary, fp64, with a token whose target no slice owns."""

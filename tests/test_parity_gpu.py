@@ -1548,3 +1548,29 @@ def test_entry_points_replay_from_a_hip_graph(cuda_device):
         torch.cuda.synchronize()
         for a, b in zip(got, want):
             assert torch.equal(a, b)
+
+
+def test_soft_ce_vocab_shards_reproduce_the_full_vocabulary(cuda_device):
+    """The soft cross-entropy over a vocabulary-parallel group, on one GPU: forward per weight slice, three [T] vectors
+    merged, backward per slice with the global log-sum-exps; the slices' gradient shares add up to the unsharded gradient."""
+    from skyrl_amd.mtp_soft_ce import softce_bwd, softce_fwd
+    from skyrl_amd.vocab_shards import merge_soft_ce_shard_statistics
+
+    B, S, H, V = 2, 150, 128, 1000
+    hs, ht, w = _softce_case(B, S, H, V, 71)
+    T = B * S
+    hs, ht, w = hs.reshape(T, H).to(cuda_device), ht.reshape(T, H).to(cuda_device), w.to(cuda_device)
+    g = torch.randn(T, generator=torch.Generator().manual_seed(72)).to(cuda_device)
+    full_loss, full_ls, full_lt = softce_fwd(hs, ht, w, S, 1, 1.0)
+    full_d = softce_bwd(hs, ht, w, full_ls, full_lt, g, S, 1, 1.0, 0)
+
+    bounds = [0, 256, 333, 1000]
+    outs = [softce_fwd(hs, ht, w[lo:hi].contiguous(), S, 1, 1.0) for lo, hi in zip(bounds[:-1], bounds[1:])]
+    loss, ls, lt = merge_soft_ce_shard_statistics(*(torch.stack([o[k] for o in outs]) for k in range(3)))
+    torch.testing.assert_close(loss, full_loss, atol=5e-5, rtol=0)
+    torch.testing.assert_close(ls, full_ls, atol=2e-5, rtol=0)
+    torch.testing.assert_close(lt, full_lt, atol=2e-5, rtol=0)
+    d_sum = torch.zeros(T, H, dtype=torch.float32, device=cuda_device)
+    for lo, hi in zip(bounds[:-1], bounds[1:]):
+        d_sum += softce_bwd(hs, ht, w[lo:hi].contiguous(), ls, lt, g, S, 1, 1.0, 0).float()
+    assert cos(d_sum, full_d) >= 0.9999 and rel_l2(d_sum, full_d.float()) < 1e-2
