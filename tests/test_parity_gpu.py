@@ -1574,3 +1574,16 @@ def test_soft_ce_vocab_shards_reproduce_the_full_vocabulary(cuda_device):
     for lo, hi in zip(bounds[:-1], bounds[1:]):
         d_sum += softce_bwd(hs, ht, w[lo:hi].contiguous(), ls, lt, g, S, 1, 1.0, 0).float()
     assert cos(d_sum, full_d) >= 0.9999 and rel_l2(d_sum, full_d.float()) < 1e-2
+
+
+def test_opcheck_registration_of_the_soft_ce_ops(cuda_device):
+    import skyrl_amd.mtp_soft_ce  # noqa: F401  (registers the ops)
+
+    T, H, V = 128, 64, 300
+    hs, ht, w = _softce_case(1, T, H, V, 5)
+    hs, ht, w = hs[0].to(cuda_device), ht[0].to(cuda_device), w.to(cuda_device)
+    checks = ("test_schema", "test_faketensor")
+    torch.library.opcheck(torch.ops.skyrl_amd.softce_fwd.default, (hs, ht, w, T, 1, 1.0), test_utils=checks)
+    _, ls, lt = torch.ops.skyrl_amd.softce_fwd(hs, ht, w, T, 1, 1.0)
+    g = torch.ones(T, device=cuda_device)
+    torch.library.opcheck(torch.ops.skyrl_amd.softce_bwd.default, (hs, ht, w, ls, lt, g, T, 1, 1.0, 0), test_utils=checks)
