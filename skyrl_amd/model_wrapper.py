@@ -40,6 +40,7 @@ def action_log_probs_from_hidden(
     compute_entropy: bool = False,
     entropy_requires_grad: bool = True,
     nnz_indices: Optional[torch.Tensor] = None,
+    action_only: bool = False,
 ) -> Union[torch.Tensor, Tuple[torch.Tensor, dict]]:
     """Action log-probabilities ``[B, num_actions]`` (and ``{"entropy": [B, S]}`` with ``return_output``).
 
@@ -51,6 +52,11 @@ def action_log_probs_from_hidden(
 
     Differences from the reference: the entropy is fp32 (the reference returns it in the logits' dtype, torch_utils.py:92),
     and both outputs come from one pass over the vocabulary.
+
+    ``action_only=True`` (an extension) runs the LM head on the ``B * num_actions`` rows the result is read from -- positions
+    ``S - num_actions - 1 .. S - 2`` of every sequence -- instead of on all tokens: the same action log-probabilities, and
+    the same entropy inside that window, which is the only part the policy worker reads (workers/worker.py:1060-1062);
+    outside it the entropy is 0.  Forward and backward then cost ``num_actions / S`` of the full pass.
     """
     if isinstance(num_actions, list):
         if len(num_actions) != 1:
@@ -68,6 +74,9 @@ def action_log_probs_from_hidden(
                          f"{tuple(tokens.shape)}")
     rolled = torch.roll(tokens, shifts=-1, dims=1)
     V = lm_head_weight.shape[0]
+    if action_only:
+        return _action_rows_only(last_hidden_state, lm_head_weight, rolled, batch, seqlen, int(num_actions), attention_mask,
+                                 float(temperature), return_output, compute_entropy, entropy_requires_grad, nnz_indices)
 
     output = {}
     if compute_entropy:
@@ -90,4 +99,45 @@ def action_log_probs_from_hidden(
     if packed:
         log_probs = _pad_back(log_probs.reshape(-1), nnz_indices, batch, seqlen)
     action_log_probs = log_probs[:, -num_actions - 1 : -1]
+    return (action_log_probs, output) if return_output else action_log_probs
+
+
+def _action_rows_only(last_hidden_state, lm_head_weight, rolled, batch, seqlen, num_actions, attention_mask, temperature,
+                      return_output, compute_entropy, entropy_requires_grad, nnz_indices):
+    """The LM head on the action window only: rows are gathered (differentiably) from the token stream, scored, and put back."""
+    dev = last_hidden_state.device
+    first = seqlen - num_actions - 1
+    if num_actions < 1 or first < 0:
+        raise ValueError(f"num_actions {num_actions} does not fit sequences of length {seqlen}")
+    cols = torch.arange(first, seqlen - 1, device=dev)
+    flat = (torch.arange(batch, device=dev).unsqueeze(1) * seqlen + cols.unsqueeze(0)).reshape(-1)   # positions in [B, S]
+    if nnz_indices is not None:
+        to_stream = torch.full((batch * seqlen,), -1, dtype=torch.long, device=dev)
+        to_stream[nnz_indices.to(torch.long)] = torch.arange(nnz_indices.numel(), device=dev)
+        src = to_stream[flat]
+        present = src >= 0                                       # padding positions hold no token: 0, as pad_input leaves them
+        src = src.clamp(min=0)
+    else:
+        src, present = flat, None
+    H = last_hidden_state.shape[-1]
+    rows = last_hidden_state.reshape(-1, H).index_select(0, src).to(lm_head_weight.dtype).unsqueeze(0)
+    labels = rolled.reshape(-1).index_select(0, src).unsqueeze(0).contiguous()
+    output = {}
+    if compute_entropy:
+        log_probs, entropy = linear_cross_entropy(rows, lm_head_weight.contiguous(), labels, temperature, "none", None)
+        entropy = entropy.reshape(batch, num_actions)
+        if not entropy_requires_grad:
+            entropy = entropy.detach()
+        if present is not None:
+            entropy = entropy * present.reshape(batch, num_actions)
+        elif attention_mask is not None:
+            entropy = entropy * attention_mask[:, first:seqlen - 1]
+        full = torch.zeros((batch, seqlen), dtype=entropy.dtype, device=dev)
+        output["entropy"] = torch.cat([full[:, :first], entropy, full[:, seqlen - 1:]], dim=1)
+    else:
+        log_probs = _fused_lm_head_logprob_apply("hip", rows, lm_head_weight, labels, 0, lm_head_weight.shape[0], rows.shape[1],
+                                                 None, not torch.is_grad_enabled(), temperature)
+    action_log_probs = log_probs.reshape(batch, num_actions)
+    if present is not None:
+        action_log_probs = action_log_probs * present.reshape(batch, num_actions)
     return (action_log_probs, output) if return_output else action_log_probs

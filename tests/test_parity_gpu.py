@@ -1587,3 +1587,48 @@ def test_opcheck_registration_of_the_soft_ce_ops(cuda_device):
     _, ls, lt = torch.ops.skyrl_amd.softce_fwd(hs, ht, w, T, 1, 1.0)
     g = torch.ones(T, device=cuda_device)
     torch.library.opcheck(torch.ops.skyrl_amd.softce_bwd.default, (hs, ht, w, ls, lt, g, T, 1, 1.0, 0), test_utils=checks)
+
+
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("compute_entropy", [False, True])
+def test_fsdp_tail_action_window_only(cuda_device, packed, compute_entropy):
+    """action_only=True scores only the rows the action window reads: the same action log-probabilities and in-window entropy
+    as the full pass (each token's row is computed independently of the others), zeros outside, and the same gradients."""
+    from skyrl_amd.model_wrapper import action_log_probs_from_hidden
+    dev = cuda_device
+    gen = torch.Generator().manual_seed(62)
+    B, S, H, V, A, t = 4, 40, 128, 900, 11, 0.9
+    seqs = torch.randint(0, V, (B, S), generator=gen).to(dev)
+    am = torch.ones(B, S, dtype=torch.long)
+    am[0, :9] = 0                                                # left padding
+    am[2, -4:] = 0                                               # right padding inside the action window
+    am = am.to(dev)
+    weight = (torch.randn(V, H, generator=gen) * 3 / H ** 0.5).to(torch.bfloat16).to(dev)
+    nnz = am.flatten().nonzero().flatten() if packed else None
+    n_tok = int(am.sum()) if packed else B * S
+    hidden = torch.randn(1 if packed else B, n_tok if packed else S, H, generator=gen).to(torch.bfloat16).to(dev)
+    G = torch.randn(B, A, generator=gen).to(dev)
+    Q = (torch.randn(B, S, generator=gen) * 0.1).to(dev)
+
+    results = []
+    for action_only in (False, True):
+        hd, wd = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
+        alp, out = action_log_probs_from_hidden(hd, wd, seqs, A, am, t, return_output=True, compute_entropy=compute_entropy,
+                                                entropy_requires_grad=True, nnz_indices=nnz, action_only=action_only)
+        loss = (alp * G).sum()
+        if compute_entropy:
+            loss = loss + (out["entropy"][:, -A - 1:-1] * Q[:, -A - 1:-1]).sum()
+        loss.backward()
+        results.append((alp.detach(), out.get("entropy"), hd.grad, wd.grad))
+    (alp0, ent0, dh0, dw0), (alp1, ent1, dh1, dw1) = results
+    torch.testing.assert_close(alp1, alp0, rtol=0, atol=1e-6)
+    if packed:
+        assert bool((alp1[2, -3:] == 0).all())                   # window positions that hold padding
+    if compute_entropy:
+        assert ent1.shape == (B, S)
+        torch.testing.assert_close(ent1.detach()[:, -A - 1:-1], ent0.detach()[:, -A - 1:-1], rtol=0, atol=1e-6)
+        outside = torch.ones(S, dtype=torch.bool, device=dev)
+        outside[-A - 1:-1] = False
+        assert bool((ent1.detach()[:, outside] == 0).all())
+    assert cos(dh1, dh0) >= 0.9999 and cos(dw1, dw0) >= 0.9999
+    assert bool((dh1.reshape(-1, H).float().abs().sum(-1) > 0).sum() <= B * A)   # only window rows receive a gradient
