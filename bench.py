@@ -103,7 +103,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--config", default="qwen2.5-7b-fwdbwd")
     ap.add_argument("--vocab-chunk", type=int, default=0)
-    ap.add_argument("--cpu-sample-tokens", type=int, default=4096)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=6144)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-mfma-probe", action="store_true")
     ap.add_argument("--skip-masked-rows", action="store_true",
