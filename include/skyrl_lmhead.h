@@ -112,7 +112,10 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
  * depend on logprobs (the off-policy importance ratio).  out3 = { sum loss*mask*weight, (see above), sum mask }.
  * dlogprobs (may be NULL) receives d out3[0] / d logprobs, i.e. the upstream gradient skyrl_lmhead_bwd takes when the
  * loss is that sum.  The eps / clip_ratio_c arguments are ignored by the loss types that do not clip.
+ * partials: fp32 scratch of 3 * SKYRL_POLICY_LOSS_PARTIALS elements for the partial sums of the workgroups; may be NULL
+ * for T <= 8192 (one workgroup), ERR_WORKSPACE otherwise.  The sums are added in a fixed order: reproducible bit for bit.
  */
+#define SKYRL_POLICY_LOSS_PARTIALS 256
 #define SKYRL_POLICY_LOSS_REGULAR 0
 #define SKYRL_POLICY_LOSS_DUAL_CLIP 1
 #define SKYRL_POLICY_LOSS_CROSS_ENTROPY 2
@@ -141,7 +144,7 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
 int skyrl_ppo_policy_loss(const float* logprobs, const float* old_logprobs, const float* advantages,
                           const float* loss_mask, const float* loss_weight, int64_t T,
                           float eps_clip_low, float eps_clip_high, float clip_ratio_c, int loss_type,
-                          float* out3, float* dlogprobs, void* stream);
+                          float* out3, float* dlogprobs, float* partials, void* stream);
 
 /*
  * Approximate KL divergence to a base policy per token (compute_approx_kl, ppo_utils.py:88-126), reduced as the trainer

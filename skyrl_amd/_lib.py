@@ -11,7 +11,7 @@ import os
 import threading
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libskyrl_lmhead.so")
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _c_i64 = ctypes.c_int64
 _c_p = ctypes.c_void_p
@@ -34,7 +34,8 @@ SIGNATURES = {
     ),
     "skyrl_ppo_policy_loss": (
         ctypes.c_int,
-        [_c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_int, _c_p, _c_p, _c_p],
+        [_c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_int, _c_p, _c_p, _c_p,
+         _c_p],
     ),
     "skyrl_approx_kl": (ctypes.c_int, [_c_p, _c_p, _c_p, _c_i64, _c_i64, ctypes.c_int, _c_p, _c_p, _c_p, ctypes.c_int, _c_p, _c_p]),
     "skyrl_actor_loss": (

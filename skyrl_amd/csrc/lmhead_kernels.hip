@@ -978,7 +978,7 @@ hipError_t launch_softce_pack(hipStream_t s, const void* student, int64_t lds_, 
 
 extern "C" {
 
-int skyrl_lmhead_version(void) { return 7; }
+int skyrl_lmhead_version(void) { return 8; }
 
 const char* skyrl_lmhead_strerror(int status) {
   switch (status) {

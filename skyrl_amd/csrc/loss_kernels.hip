@@ -123,15 +123,18 @@ __device__ __forceinline__ bool is_interval_type(int type) {
          type == SKYRL_POLICY_LOSS_CISPO || type == SKYRL_POLICY_LOSS_ROLLOUT_IS;
 }
 
+// Workgroup b sums tokens [b * slice, (b + 1) * slice) in a fixed order and writes its three sums to out[k * out_stride + b]:
+// with one workgroup that is the result itself, with several the partial sums policy_loss_finish_kernel adds up.
 __global__ __launch_bounds__(1024) void policy_loss_kernel(const float* __restrict__ lp, const float* __restrict__ old,
                                                            const float* __restrict__ adv, const float* __restrict__ mask,
-                                                           const float* __restrict__ weight, int64_t T, float eps_low,
-                                                           float eps_high, float clip_c, int type, float* __restrict__ out,
-                                                           float* __restrict__ g) {
+                                                           const float* __restrict__ weight, int64_t T, int64_t slice,
+                                                           float eps_low, float eps_high, float clip_c, int type,
+                                                           float* __restrict__ out, int out_stride, float* __restrict__ g) {
   __shared__ float red[3][16];
   float s_loss = 0.f, s_clip = 0.f, s_mask = 0.f;
   const float lo = is_interval_type(type) ? 1.f - eps_low : eps_low, hi = is_interval_type(type) ? 1.f + eps_high : eps_high;
-  for (int64_t t = threadIdx.x; t < T; t += blockDim.x) {
+  const int64_t t0 = (int64_t)blockIdx.x * slice, t1 = t0 + slice < T ? t0 + slice : T;
+  for (int64_t t = t0 + threadIdx.x; t < t1; t += blockDim.x) {
     float loss, dloss, stat;
     const bool ce = type == SKYRL_POLICY_LOSS_CROSS_ENTROPY;  // reads neither old nor adv
     policy_term(type, lp[t], ce ? 0.f : old[t], ce ? 0.f : adv[t], lo, hi, clip_c, 0.f, loss, dloss, stat);
@@ -155,11 +158,23 @@ __global__ __launch_bounds__(1024) void policy_loss_kernel(const float* __restri
   if (threadIdx.x < 3) {
     float v = 0.f;
     for (int k = 0; k < (int)(blockDim.x >> 6); ++k) v += red[threadIdx.x][k];
+    out[threadIdx.x * out_stride + blockIdx.x] = v;
+  }
+}
+
+constexpr int kMaxLossSlices = SKYRL_POLICY_LOSS_PARTIALS;
+constexpr int64_t kLossSliceTokens = 8192;  // at least this many tokens per workgroup
+
+__global__ __launch_bounds__(64) void policy_loss_finish_kernel(const float* __restrict__ partials, int slices,
+                                                                float* __restrict__ out) {
+  if (threadIdx.x < 3) {
+    float v = 0.f;
+    for (int b = 0; b < slices; ++b) v += partials[threadIdx.x * kMaxLossSlices + b];
     out[threadIdx.x] = v;
   }
 }
 
-constexpr int kRowThreads = 256;
+constexpr int kRowThreads = 1024;  // one workgroup per row of [B, S]: rows are few and long
 
 // Sum of one value per thread over the workgroup, in a fixed order; every thread receives it.
 __device__ __forceinline__ float block_sum(float v, float* red) {
@@ -362,11 +377,14 @@ __global__ __launch_bounds__(kRowThreads) void actor_loss_finish_kernel(const Ac
     a.out[0] = a.policy_scale * t[0] + a.term_scale * (a.kl_coef * kl - a.entropy_coef * ent);
     a.out[1] = t[0], a.out[2] = t[1], a.out[3] = t[2], a.out[4] = kl, a.out[5] = ent;
   }
-  if (a.dent) {
-    const float c = -a.term_scale * a.entropy_coef / mask_denom;
-    const int64_t n = a.rows * a.cols;
-    for (int64_t i = threadIdx.x; i < n; i += kRowThreads) a.dent[i] = a.mask ? c * a.mask[i] : c;
-  }
+}
+
+// d loss / d entropy = -term_scale * entropy_coef * mask / max(sum mask, 1): elementwise once the finish kernel has the count.
+__global__ __launch_bounds__(256) void actor_loss_dentropy_kernel(const ActorLossArgs a) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= a.rows * a.cols) return;
+  const float c = -a.term_scale * a.entropy_coef / fmaxf(a.out[3], 1.f);
+  a.dent[i] = a.mask ? c * a.mask[i] : c;
 }
 
 bool finite(float x) { return std::isfinite(x); }
@@ -389,15 +407,24 @@ extern "C" {
 
 int skyrl_ppo_policy_loss(const float* logprobs, const float* old_logprobs, const float* advantages, const float* loss_mask,
                           const float* loss_weight, int64_t T, float eps_clip_low, float eps_clip_high, float clip_ratio_c,
-                          int loss_type, float* out3, float* dlogprobs, void* stream) {
+                          int loss_type, float* out3, float* dlogprobs, float* partials, void* stream) {
   // the sequence-level type needs rows: it is part of skyrl_actor_loss only
   if (!valid_loss_type(loss_type) || loss_type == SKYRL_POLICY_LOSS_GSPO) return SKYRL_LMHEAD_ERR_ARG;
   const bool needs_old = loss_type != SKYRL_POLICY_LOSS_CROSS_ENTROPY;
   if (!logprobs || !out3 || (needs_old && (!old_logprobs || !advantages))) return SKYRL_LMHEAD_ERR_NULL;
   if (T < 1) return SKYRL_LMHEAD_ERR_SHAPE;
   if (!valid_loss_params(loss_type, eps_clip_low, eps_clip_high, clip_ratio_c)) return SKYRL_LMHEAD_ERR_ARG;
-  hipLaunchKernelGGL(policy_loss_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, logprobs, old_logprobs, advantages,
-                     loss_mask, loss_weight, T, eps_clip_low, eps_clip_high, clip_ratio_c, loss_type, out3, dlogprobs);
+  // One workgroup up to kLossSliceTokens tokens; beyond that the tokens are cut into equal slices (a fixed number for a given
+  // T, so the result is reproducible) whose partial sums a second launch adds in order.
+  int64_t slices = (T + kLossSliceTokens - 1) / kLossSliceTokens;
+  if (slices > kMaxLossSlices) slices = kMaxLossSlices;
+  if (slices > 1 && !partials) return SKYRL_LMHEAD_ERR_WORKSPACE;
+  const int64_t slice = (T + slices - 1) / slices;
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(policy_loss_kernel, dim3((unsigned)slices), dim3(1024), 0, s, logprobs, old_logprobs, advantages, loss_mask,
+                     loss_weight, T, slice, eps_clip_low, eps_clip_high, clip_ratio_c, loss_type, slices > 1 ? partials : out3,
+                     slices > 1 ? kMaxLossSlices : 1, dlogprobs);
+  if (slices > 1) hipLaunchKernelGGL(policy_loss_finish_kernel, dim3(1), dim3(64), 0, s, partials, (int)slices, out3);
   return (int)hipGetLastError();
 }
 
@@ -435,6 +462,11 @@ int skyrl_actor_loss(const float* logprobs, const float* old_logprobs, const flo
   hipStream_t s = (hipStream_t)stream;
   hipLaunchKernelGGL(actor_loss_rows_kernel, dim3((unsigned)rows), dim3(kRowThreads), 0, s, a);
   hipLaunchKernelGGL(actor_loss_finish_kernel, dim3(1), dim3(kRowThreads), 0, s, a);
+  if (dentropy) {
+    const int64_t n = rows * cols;
+    if (n >= (int64_t(1) << 31) * 256) return SKYRL_LMHEAD_ERR_SHAPE;
+    hipLaunchKernelGGL(actor_loss_dentropy_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, a);
+  }
   return (int)hipGetLastError();
 }
 

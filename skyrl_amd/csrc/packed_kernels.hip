@@ -17,6 +17,7 @@
 namespace {
 
 constexpr int kThreads = 256;
+constexpr int kMaskThreads = 1024;  // workgroup of the attention-mask scatter: one per row, rows are few and long
 constexpr int64_t kNotInVocab = INT64_MAX;
 
 // Sequence that holds packed token t: the smallest s with cu[s+1] > t (what searchsorted(cu[1:], t, right=True) returns,
@@ -93,12 +94,12 @@ __global__ void __launch_bounds__(kThreads) scatter_kernel(float* __restrict__ p
 
 // Attention-mask branch (model_utils.py:873-878): row b of the [rows, cols + 1] mask marks the real tokens of sequence b;
 // its j-th real token (j = 0 ..) takes packed token cu[b] + j, for every real token but the last one.  One workgroup per
-// row walks the row in pieces of 256 columns, numbering the real tokens with wave ballots.
+// row walks the row in pieces of 1024 columns, numbering the real tokens with wave ballots.
 template <bool ADJOINT>
-__global__ void __launch_bounds__(kThreads) scatter_masked_kernel(float* __restrict__ packed, const int64_t* __restrict__ cu,
+__global__ void __launch_bounds__(kMaskThreads) scatter_masked_kernel(float* __restrict__ packed, const int64_t* __restrict__ cu,
                                                                   int64_t T, const uint8_t* __restrict__ mask, int64_t cols,
                                                                   float* __restrict__ out) {
-  __shared__ int wave_count[kThreads / 64];
+  __shared__ int wave_count[kMaskThreads / 64];
   const int64_t b = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const uint8_t* mrow = mask + b * (cols + 1);
@@ -106,23 +107,23 @@ __global__ void __launch_bounds__(kThreads) scatter_masked_kernel(float* __restr
 
   // Number of real tokens in the row.
   int mine = 0;
-  for (int64_t c = threadIdx.x; c <= cols; c += kThreads) mine += mrow[c] != 0;
+  for (int64_t c = threadIdx.x; c <= cols; c += kMaskThreads) mine += mrow[c] != 0;
   for (int o = 32; o > 0; o >>= 1) mine += __shfl_xor(mine, o);
   if (lane == 0) wave_count[wave] = mine;
   __syncthreads();
   int64_t seq_len = 0;
-  for (int w = 0; w < kThreads / 64; ++w) seq_len += wave_count[w];
+  for (int w = 0; w < kMaskThreads / 64; ++w) seq_len += wave_count[w];
   __syncthreads();
 
   int64_t seen = 0;  // real tokens in the columns before this piece
-  for (int64_t c0 = 0; c0 < cols; c0 += kThreads) {
+  for (int64_t c0 = 0; c0 < cols; c0 += kMaskThreads) {
     const int64_t c = c0 + threadIdx.x;
     const bool real = c < cols && mrow[c] != 0;
     const unsigned long long ballot = __ballot(real);
     if (lane == 0) wave_count[wave] = __popcll(ballot);
     __syncthreads();
     int64_t before = seen, piece = 0;
-    for (int w = 0; w < kThreads / 64; ++w) {
+    for (int w = 0; w < kMaskThreads / 64; ++w) {
       if (w < wave) before += wave_count[w];
       piece += wave_count[w];
     }
@@ -178,7 +179,7 @@ int skyrl_packed_scatter_logprobs(const float* packed, const int64_t* cu_seqlens
   if (rows * cols == 0) return SKYRL_LMHEAD_OK;
   hipStream_t s = (hipStream_t)stream;
   if (attention_mask) {
-    hipLaunchKernelGGL(scatter_masked_kernel<false>, dim3((unsigned)rows), dim3(kThreads), 0, s, const_cast<float*>(packed),
+    hipLaunchKernelGGL(scatter_masked_kernel<false>, dim3((unsigned)rows), dim3(kMaskThreads), 0, s, const_cast<float*>(packed),
                        cu_seqlens, T, attention_mask, cols, out);
     return (int)hipGetLastError();
   }
@@ -200,7 +201,7 @@ int skyrl_packed_gather_grad(const float* d_out, const int64_t* cu_seqlens, int6
   if (attention_mask) {
     hipLaunchKernelGGL(fill_f32_kernel, dim3(blocks_for(T)), dim3(kThreads), 0, s, d_packed, T, 0.f);
     if (rows * cols > 0)
-      hipLaunchKernelGGL(scatter_masked_kernel<true>, dim3((unsigned)rows), dim3(kThreads), 0, s, d_packed, cu_seqlens, T,
+      hipLaunchKernelGGL(scatter_masked_kernel<true>, dim3((unsigned)rows), dim3(kMaskThreads), 0, s, d_packed, cu_seqlens, T,
                          attention_mask, cols, src);
     return (int)hipGetLastError();
   }

@@ -69,6 +69,7 @@ def _reject_off_policy_correction(config: Any, rollout_logprobs: Optional[torch.
             "off-policy correction from rollout_logprobs is not part of the fused loss; compute the importance ratio and the "
             "thinned mask with the trainer's own helper and pass them as loss_weight and loss_mask")
 KL_ESTIMATORS = {"k1": 0, "abs": 1, "k2": 2, "k3": 3}
+_LOSS_PARTIALS = 256  # SKYRL_POLICY_LOSS_PARTIALS of the header
 
 
 def _flat_f32(name: str, t: Optional[torch.Tensor], numel: int) -> Optional[torch.Tensor]:
@@ -109,12 +110,13 @@ def ppo_policy_loss_terms(
         return torch.zeros(3, dtype=torch.float32, device=dev), torch.empty(0, dtype=torch.float32, device=dev)
     sums = torch.empty(3, dtype=torch.float32, device=dev)
     grad = torch.empty(n, dtype=torch.float32, device=dev)
+    partials = torch.empty(3 * _LOSS_PARTIALS, dtype=torch.float32, device=dev)   # per-workgroup sums of the kernel
     ptr = lambda t: None if t is None else t.data_ptr()  # noqa: E731
     with torch.cuda.device(dev):
         st = _lib.load().skyrl_ppo_policy_loss(
             log_probs.data_ptr(), ptr(old_log_probs), ptr(advantages), ptr(loss_mask), ptr(loss_weight), n,
             float(eps_clip_low), float(eps_clip_high), float(clip_ratio_c), int(loss_type), sums.data_ptr(),
-            grad.data_ptr(), torch.cuda.current_stream(dev).cuda_stream)
+            grad.data_ptr(), partials.data_ptr(), torch.cuda.current_stream(dev).cuda_stream)
     _lib.check(st, "skyrl_ppo_policy_loss")
     return sums, grad
 

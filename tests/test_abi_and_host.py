@@ -116,14 +116,15 @@ def test_mfma_probe_argument_errors():
 def test_ppo_policy_loss_argument_errors():
     lib = _lib.load()
     call = lambda **kw: lib.skyrl_ppo_policy_loss(*[{**dict(lp=0x1000, old=0x2000, adv=0x3000, mask=None, w=None, T=8, lo=0.2,  # noqa: E731
-                                                        hi=0.2, c=3.0, dual=0, out=0x4000, g=None, stream=None), **kw}[k]
+                                                        hi=0.2, c=3.0, dual=0, out=0x4000, g=None, part=None, stream=None), **kw}[k]
                                                      for k in ("lp", "old", "adv", "mask", "w", "T", "lo", "hi", "c", "dual", "out", "g",
-                                                               "stream")])
+                                                               "part", "stream")])
     assert call(lp=None) == -1
     assert call(out=None) == -1
     assert call(T=0) == -2
     assert call(lo=float("nan")) == -5
     assert call(dual=1, c=float("inf")) == -5
+    assert call(T=8193) == -4 and call(T=8193, part=None, lp=None) == -1   # several workgroups need the partial-sum scratch
 
 
 def test_ppo_policy_loss_mirror_contract():

@@ -355,13 +355,14 @@ def test_c_abi_called_directly(cuda_device):
 # ---------------------------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("loss_type", ["regular", "dual_clip"])
 @pytest.mark.parametrize("masked", [False, True])
-def test_ppo_policy_loss_matches_oracle(loss_type, masked, cuda_device):
+@pytest.mark.parametrize("B", [6, 67])   # 3102 tokens: one workgroup; 34639 tokens: five slices and their partial sums
+def test_ppo_policy_loss_matches_oracle(loss_type, masked, B, cuda_device):
     from types import SimpleNamespace
 
     from skyrl_amd.policy_loss import ppo_policy_loss
 
     gen = torch.Generator().manual_seed(5)
-    B, S = 6, 517
+    S = 517
     lp = (torch.randn(B, S, generator=gen) * 0.5 - 2.0)
     old = lp + torch.randn(B, S, generator=gen) * 0.3
     old[0, :4] = lp[0, :4]                       # exact ties of the two surrogates
@@ -391,6 +392,7 @@ def test_ppo_policy_loss_matches_oracle(loss_type, masked, cuda_device):
     loss2, m2 = ppo_policy_loss(dlp2, to(old), to(adv), cfg, to(mask), loss_weight=to(weight), sync_metrics=False)
     (loss2 * 3.0).backward()
     assert torch.equal(dlp2.grad, dlp.grad * 3.0) and torch.is_tensor(m2["clip_ratio"])
+    assert loss2.item() == loss.item()                           # fixed summation order: reproducible bit for bit
 
 
 def test_policy_loss_feeds_the_fused_backward(cuda_device):
@@ -674,9 +676,9 @@ def test_loss_argument_errors(cuda_device):
     lib = _lib.load()
     x = torch.zeros(16, dtype=torch.float32, device=cuda_device)
     p = x.data_ptr()
-    assert lib.skyrl_ppo_policy_loss(p, None, None, None, None, 16, 0.2, 0.2, 3.0, 2, p, None, None) == 0   # cross entropy
-    assert lib.skyrl_ppo_policy_loss(p, None, None, None, None, 16, 0.2, 0.2, 3.0, 3, p, None, None) == -1
-    assert lib.skyrl_ppo_policy_loss(p, p, p, None, None, 16, 0.2, 0.2, 3.0, 4, p, None, None) == -5
+    assert lib.skyrl_ppo_policy_loss(p, None, None, None, None, 16, 0.2, 0.2, 3.0, 2, p, None, None, None) == 0   # cross entropy
+    assert lib.skyrl_ppo_policy_loss(p, None, None, None, None, 16, 0.2, 0.2, 3.0, 3, p, None, None, None) == -1
+    assert lib.skyrl_ppo_policy_loss(p, p, p, None, None, 16, 0.2, 0.2, 3.0, 4, p, None, None, None) == -5
     assert lib.skyrl_approx_kl(p, p, None, 4, 4, 3, None, None, p, 0, None, None) == -1
     assert lib.skyrl_approx_kl(p, p, None, 4, 4, 4, None, p, p, 0, None, None) == -5
     assert lib.skyrl_approx_kl(p, p, None, 4, 4, 3, None, p, p, 2, None, None) == -1
@@ -691,7 +693,10 @@ def test_loss_argument_errors(cuda_device):
     assert lib.skyrl_actor_loss(*args(type=4)) == 0           # the sequence-level type is part of this entry point only
     assert lib.skyrl_actor_loss(*args(type=10)) == -5
     # SAPO's temperatures divide: zero is refused
-    assert lib.skyrl_ppo_policy_loss(p, p, p, None, None, 16, 0.0, 1.0, 0.0, 5, p, None, None) == -5
+    assert lib.skyrl_ppo_policy_loss(p, p, p, None, None, 16, 0.0, 1.0, 0.0, 5, p, None, None, None) == -5
+    # more than one workgroup's worth of tokens needs the scratch for the partial sums
+    big = torch.zeros(20000, dtype=torch.float32, device=cuda_device)
+    assert lib.skyrl_ppo_policy_loss(big.data_ptr(), None, None, None, None, 20000, 0.2, 0.2, 3.0, 2, p, None, None, None) == -4
     torch.cuda.synchronize()
 
 
