@@ -110,6 +110,8 @@ def main() -> int:
                     help="run the backward pass through skyrl_amd.ops.lmhead_bwd_active_rows, which drops the tokens whose "
                          "upstream gradients are zero (the configurations with a response mask); value stays tokens/s over "
                          "all T tokens, the roofline figures count the flop actually executed")
+    ap.add_argument("--frozen-lm-head", action="store_true",
+                    help="the weight takes no gradient (adapter training): d_weight = NULL, the dW product is skipped")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain 1 GiB device-to-device copy (a kernel of known HBM traffic) so that rocprofv3 "
                          "--pmc FETCH_SIZE / WRITE_SIZE readings of the same run can be scaled to bytes")
@@ -165,11 +167,12 @@ def main() -> int:
         _lib.check(st, "skyrl_lmhead_fwd")
         if skip:
             ops.lmhead_bwd_active_rows(hidden, weight, labels, row_lse, row_pz if q is not None else None, g, q, rcp_t,
-                                       args.vocab_chunk)
+                                       args.vocab_chunk, want_dweight=not args.frozen_lm_head)
         elif cfg.backward:
             st = lib.skyrl_lmhead_bwd(hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0),
                                       labels.data_ptr(), row_lse.data_ptr(), ptr(row_pz) if q is not None else None,
-                                      g.data_ptr(), ptr(q), T, H, V, rcp_t, d_hidden.data_ptr(), d_weight.data_ptr(), 0,
+                                      g.data_ptr(), ptr(q), T, H, V, rcp_t, d_hidden.data_ptr(),
+                                      None if args.frozen_lm_head else d_weight.data_ptr(), 0,
                                       args.vocab_chunk, ws_b.data_ptr(), ws_b.numel(), stream)
             _lib.check(st, "skyrl_lmhead_bwd")
 
@@ -198,7 +201,8 @@ def main() -> int:
     kernels = {k: {"ms_per_step": ms / args.steps, "launches_per_step": n / args.steps, "avg_launch_ms": ms / n}
                for k, (ms, n) in prof.results.items() if n}
     # Executed flop: forward over all T tokens, backward over the tokens that were not dropped.
-    step_flop = cfg.total_flop if not skip else 2.0 * T * V * H + 6.0 * t_active * V * H
+    bwd_gemms = 2.0 if args.frozen_lm_head else 3.0  # logits recompute + dHidden (+ dWeight)
+    step_flop = 2.0 * T * V * H + (2.0 * bwd_gemms * t_active * V * H if cfg.backward else 0.0)
     step_roofline = {"bound": "mfma", "achieved": step_flop / (ms_per_step * 1e-3) / 1e12, "peak": PEAK_BF16_DENSE_FLOPS / 1e12,
                      "unit": "TFLOP/s"}
     step_roofline["frac"] = step_roofline["achieved"] / step_roofline["peak"]
@@ -208,7 +212,7 @@ def main() -> int:
         # lmhead_bwd_chunk: every backward launch (per vocab chunk one with the dz tiles, one with the gradient GEMM tiles);
         # over a step the launches add up to the logits recompute, dHidden and dWeight = 6*T*V*H flop.
         ks = [kernels[n] for n in ("lmhead_bwd_chunk[dz]", "lmhead_bwd_chunk[gemm]")]  # the same kernel, two kinds of launch
-        dom_name, dom_flop = "lmhead_bwd_chunk", 6.0 * t_active * V * H
+        dom_name, dom_flop = "lmhead_bwd_chunk", 2.0 * bwd_gemms * t_active * V * H
         dom_ms, dom_launches = sum(k["ms_per_step"] for k in ks), sum(k["launches_per_step"] for k in ks)
     else:
         k = kernels["lmhead_fwd_tiles"]
@@ -243,7 +247,8 @@ def main() -> int:
         "config": {
             "workload": f"{cfg.name}: LM head T={T} H={H} V={V}, temperature {cfg.temperature}, "
                         f"{'forward+backward' if cfg.backward else 'forward'}"
-                        f"{', entropy with upstream grad' if cfg.entropy_grad else (', entropy' if cfg.entropy else '')}",
+                        f"{', entropy with upstream grad' if cfg.entropy_grad else (', entropy' if cfg.entropy else '')}"
+                        f"{', frozen LM head (no dW)' if args.frozen_lm_head and cfg.backward else ''}",
             "T": T, "H": H, "V": V, "temperature": cfg.temperature,
             "vocab_chunk": args.vocab_chunk or "library default",
             "backward_tokens": t_active,

@@ -82,8 +82,10 @@ int skyrl_lmhead_fwd(const void* hidden, int64_t ld_hidden, const void* weight, 
  * Backward.  Same hidden / weight / labels as the forward call; row_lse, row_pz from it (row_pz may be NULL
  * iff dentropy is NULL); dlogprobs fp32 [T] (required), dentropy fp32 [T] or NULL.
  * d_hidden: bf16 [T, H] contiguous, overwritten.  d_weight: fp32 [V, H] contiguous, overwritten, or added to
- * when accumulate_dw != 0 (gradient accumulation across micro-batches).  Both gradients are with respect to
- * the unscaled weight / hidden: the 1/temperature factor is already applied.
+ * when accumulate_dw != 0 (gradient accumulation across micro-batches); NULL when the weight takes no gradient (a frozen
+ * LM head, e.g. adapter training: autograd would drop grad_weight of model_utils.py:419-428 too) -- the dW product, a third
+ * of the backward's work, is then not computed.  Both gradients are with respect to the unscaled weight / hidden: the
+ * 1/temperature factor is already applied.
  * vocab_chunk: width of the dz panel in vocab columns (multiple of 256; 0 = library default: the width, with a panel of
  * at most 1.5 GiB, whose launches divide most evenly over the device's compute units).
  */

@@ -978,7 +978,7 @@ hipError_t launch_softce_pack(hipStream_t s, const void* student, int64_t lds_, 
 
 extern "C" {
 
-int skyrl_lmhead_version(void) { return 8; }
+int skyrl_lmhead_version(void) { return 9; }
 
 const char* skyrl_lmhead_strerror(int status) {
   switch (status) {
@@ -1061,9 +1061,9 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
                      int64_t vocab_chunk, void* workspace, size_t workspace_bytes, void* stream) {
   int st = check_common(hidden, ld_hidden, weight, ld_weight, labels, T, H, V, rcp_temperature);
   if (st) return st;
-  if (!row_lse || !dlogprobs || !d_hidden || !d_weight) return SKYRL_LMHEAD_ERR_NULL;
+  if (!row_lse || !dlogprobs || !d_hidden) return SKYRL_LMHEAD_ERR_NULL;
   if (dentropy && !row_pz) return SKYRL_LMHEAD_ERR_NULL;
-  if (!aligned16(d_hidden) || !aligned16(d_weight)) return SKYRL_LMHEAD_ERR_ALIGN;
+  if (!aligned16(d_hidden) || !aligned16(d_weight)) return SKYRL_LMHEAD_ERR_ALIGN;  // d_weight NULL: no dW wanted
   if (vocab_chunk < 0 || vocab_chunk % 256 != 0) return SKYRL_LMHEAD_ERR_ARG;
   const int64_t Tpad = round_up(T, 256), Vpad = round_up(V, 256);
   int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(T, H, V);
@@ -1088,7 +1088,7 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
     hipLaunchKernelGGL(transpose_bf16, dim3((unsigned)(Vpad / 64), (unsigned)(H / 64)), dim3(256), 0, s, Wp, (int)ld_weight,
                        (int)V, (int)H, w.Wt, (int)(Vpad + kLdPad), (int)Vpad);
   }
-  {
+  if (d_weight) {  // only the dW product reads hidden^T
     Timed timed(kTranspose, s);
     hipLaunchKernelGGL(transpose_bf16, dim3((unsigned)(Tpad / 64), (unsigned)(H / 64)), dim3(256), 0, s, Hp, (int)ld_hidden,
                        (int)T, (int)H, w.Ht, (int)(Tpad + kLdPad), (int)Tpad);
@@ -1115,7 +1115,7 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
     // dW[vc0 + v, h]  (+)= sum_t D[t, v] . hidden^T[h, t]             (A = hidden^T rows, B = D read K-major)
     const bool first = ci == 0, last = ci == nchunks - 1;
     const int64_t rows = (V - vc0) < vcw ? (V - vc0) : vcw;
-    float* dWc = d_weight + (size_t)vc0 * (size_t)H;
+    float* dWc = d_weight ? d_weight + (size_t)vc0 * (size_t)H : (float*)nullptr;
     const uint16_t* dh_out = last ? (uint16_t*)d_hidden : (uint16_t*)nullptr;
     const float* dh_in = first ? (const float*)nullptr : (const float*)w.dHacc;
     float* dh_keep = last ? (float*)nullptr : w.dHacc;
@@ -1127,8 +1127,10 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
                                H, nullptr, nullptr, (uint16_t*)dh_out, H, dh_in, dh_keep)
                    : make_gemm(w.Wt + vc0, Vpad + kLdPad, H, w.D, vcw + kLdPad, Tpad, false, false, vcw / BK, H, T, nullptr,
                                nullptr, (uint16_t*)dh_out, H, dh_in, dh_keep);
-    const GemmArgs gw = make_gemm(w.Ht, Tpad + kLdPad, H, w.D, vcw + kLdPad, vcw, true, false, Tpad / BK, H, rows,
-                                  accumulate_dw ? (const float*)dWc : (const float*)nullptr, dWc, (uint16_t*)nullptr, H);
+    // A frozen LM head (d_weight == NULL) needs no dW: the launch then carries the dHidden tiles alone.
+    const GemmArgs gw = d_weight ? make_gemm(w.Ht, Tpad + kLdPad, H, w.D, vcw + kLdPad, vcw, true, false, Tpad / BK, H, rows,
+                                             accumulate_dw ? (const float*)dWc : (const float*)nullptr, dWc, (uint16_t*)nullptr, H)
+                                 : none;
     e = launch_bwd_chunk(s, dentropy != nullptr, DzArgs{}, 0, true, gh, gw);
     if (e != hipSuccess) return (int)e;
   }

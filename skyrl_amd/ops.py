@@ -17,7 +17,8 @@ import torch
 
 from . import _lib
 
-__all__ = ["lmhead_fwd", "lmhead_bwd", "lmhead_bwd_active_rows", "fwd_workspace_bytes", "bwd_workspace_bytes"]
+__all__ = ["lmhead_fwd", "lmhead_bwd", "lmhead_bwd_hidden", "lmhead_bwd_active_rows", "fwd_workspace_bytes",
+           "bwd_workspace_bytes"]
 
 
 def _require_device(*tensors: torch.Tensor) -> torch.device:
@@ -131,6 +132,33 @@ def lmhead_bwd(
     return d_hidden, d_weight
 
 
+@torch.library.custom_op("skyrl_amd::lmhead_bwd_hidden", mutates_args=())
+def lmhead_bwd_hidden(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    row_lse: torch.Tensor,
+    row_pz: Optional[torch.Tensor],
+    dlogprobs: torch.Tensor,
+    dentropy: Optional[torch.Tensor],
+    rcp_temperature: float,
+    vocab_chunk: int,
+) -> torch.Tensor:
+    """``d_hidden`` bf16 [T,H] alone, for a weight that takes no gradient (a frozen LM head): the dW product is skipped."""
+    T, H, V = _check_operands(hidden, weight, labels)
+    dev = _require_device(hidden, weight, labels, row_lse, dlogprobs)
+    d_hidden = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    if T > 0:
+        _bwd_into(_lib.load(), hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk,
+                  d_hidden, None, False)
+    return d_hidden
+
+
+@lmhead_bwd_hidden.register_fake
+def _(hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk):
+    return torch.empty_like(hidden, memory_format=torch.contiguous_format)
+
+
 def lmhead_bwd_active_rows(
     hidden: torch.Tensor,
     weight: torch.Tensor,
@@ -142,7 +170,8 @@ def lmhead_bwd_active_rows(
     rcp_temperature: float,
     vocab_chunk: int = 0,
     min_skip_fraction: float = 0.125,
-) -> Tuple[torch.Tensor, torch.Tensor]:
+    want_dweight: bool = True,
+) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """``lmhead_bwd`` that first drops the tokens whose upstream gradients are all zero.
 
     A token with ``dlogprobs == 0`` (and ``dentropy == 0``) has a zero dz row: it adds nothing to dW and its dHidden row is
@@ -150,7 +179,8 @@ def lmhead_bwd_active_rows(
     megatron_model_wrapper.py:607-985; half of the tokens in the Qwen2.5-1.5B benchmark configuration), so the three
     backward GEMMs run on the remaining rows only: rows are gathered, the kernels run on the compact ``[T_active, H]``
     problem, and dHidden rows are scattered back into zeros.  Counting the active rows costs one host synchronisation; when
-    fewer than ``min_skip_fraction`` of the rows would be dropped the dense path is used.
+    fewer than ``min_skip_fraction`` of the rows would be dropped the dense path is used.  With ``want_dweight=False`` (the
+    weight takes no gradient) the dW product is skipped and ``None`` is returned in its place.
     """
     T = hidden.shape[0]
     active = dlogprobs != 0
@@ -158,14 +188,19 @@ def lmhead_bwd_active_rows(
         active |= dentropy != 0
     idx = active.nonzero(as_tuple=True)[0]
     n = int(idx.numel())
+    def run(*args):
+        if want_dweight:
+            return lmhead_bwd(*args)
+        return lmhead_bwd_hidden(*args), None
+
     if n == 0:
-        return torch.zeros_like(hidden, memory_format=torch.contiguous_format), torch.zeros(
-            weight.shape, dtype=torch.float32, device=weight.device)
+        return torch.zeros_like(hidden, memory_format=torch.contiguous_format), (
+            torch.zeros(weight.shape, dtype=torch.float32, device=weight.device) if want_dweight else None)
     if T - n < min_skip_fraction * T:
-        return lmhead_bwd(hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk)
+        return run(hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk)
     take = lambda t: None if t is None else t.index_select(0, idx)  # noqa: E731
-    dh_c, d_weight = lmhead_bwd(take(hidden), weight, take(labels), take(row_lse), take(row_pz) if dentropy is not None else None,
-                                take(dlogprobs), take(dentropy), rcp_temperature, vocab_chunk)
+    dh_c, d_weight = run(take(hidden), weight, take(labels), take(row_lse), take(row_pz) if dentropy is not None else None,
+                         take(dlogprobs), take(dentropy), rcp_temperature, vocab_chunk)
     d_hidden = torch.zeros((T, hidden.shape[1]), dtype=torch.bfloat16, device=hidden.device)
     d_hidden.index_copy_(0, idx, dh_c)
     return d_hidden, d_weight
@@ -194,7 +229,7 @@ def _bwd_into(lib, hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy,
         st = lib.skyrl_lmhead_bwd(
             hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), labels.data_ptr(),
             row_lse.data_ptr(), _ptr(row_pz if dentropy is not None else None), dlogprobs.data_ptr(), _ptr(dentropy),
-            T, H, V, float(rcp_temperature), d_hidden.data_ptr(), d_weight.data_ptr(), int(bool(accumulate_dw)),
+            T, H, V, float(rcp_temperature), d_hidden.data_ptr(), _ptr(d_weight), int(bool(accumulate_dw)),
             int(vocab_chunk), ws.data_ptr(), ws_bytes, stream,
         )
     _lib.check(st, "skyrl_lmhead_bwd")
@@ -238,9 +273,9 @@ def _backward(ctx, d_logprobs, d_entropy, d_row_lse, d_row_pz):
     if ctx.want_entropy and d_entropy is not None:
         dent = d_entropy.to(torch.float32).contiguous()
     d_hidden, d_weight = lmhead_bwd_active_rows(hidden, weight, labels, row_lse, row_pz if dent is not None else None,
-                                                d_logprobs, dent, ctx.rcp_temperature, 0)
+                                                d_logprobs, dent, ctx.rcp_temperature, 0, want_dweight=ctx.needs_input_grad[1])
     # grad_weight is handed back in the weight's dtype, as the reference does (model_utils.py:428).
-    return d_hidden, d_weight.to(weight.dtype), None, None, None
+    return d_hidden, None if d_weight is None else d_weight.to(weight.dtype), None, None, None
 
 
 lmhead_fwd.register_autograd(_backward, setup_context=_setup_context)

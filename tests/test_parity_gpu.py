@@ -1637,3 +1637,41 @@ def test_fsdp_tail_action_window_only(cuda_device, packed, compute_entropy):
         assert bool((ent1.detach()[:, outside] == 0).all())
     assert cos(dh1, dh0) >= 0.9999 and cos(dw1, dw0) >= 0.9999
     assert bool((dh1.reshape(-1, H).float().abs().sum(-1) > 0).sum() <= B * A)   # only window rows receive a gradient
+
+
+def test_frozen_lm_head_skips_the_weight_gradient(cuda_device):
+    """A weight that takes no gradient (adapter training with a frozen LM head): the backward computes dHidden alone -- the
+    same dHidden bit for bit (the dHidden tiles do not depend on what else the launch carries) -- through the C ABI with
+    d_weight = NULL, the functional op and both autograd adapters."""
+    T, H, V, t = 300, 128, 1000, 0.7
+    hidden, weight, labels, g, q = _rand(T, H, V, seed=41)
+    h, w, y, gd, qd = (x.to(cuda_device) for x in (hidden, weight, labels, g, q))
+    lp, ent, lse, pz = ops.lmhead_fwd(h, w, y, 1.0 / t, True)
+    for chunk in (0, 256):
+        dh_full, _ = ops.lmhead_bwd(h, w, y, lse, pz, gd, qd, 1.0 / t, chunk)
+        assert torch.equal(ops.lmhead_bwd_hidden(h, w, y, lse, pz, gd, qd, 1.0 / t, chunk), dh_full)
+    # autograd: the verl-style function and the SkyRL adapter
+    for frozen in (False, True):
+        hd = h.clone().requires_grad_(True)
+        wd = w.clone().requires_grad_(not frozen)
+        out_lp, out_ent = linear_cross_entropy(hd, wd, y, t, "none", None)
+        ((out_lp * gd).sum() + (out_ent * qd).sum()).backward()
+        if frozen:
+            assert wd.grad is None and torch.equal(hd.grad, kept)
+        else:
+            kept = hd.grad.clone()
+            assert wd.grad is not None
+    hd = h.clone().requires_grad_(True)
+    out = FusedLinearLogprobHip.apply(hd[None], w, y[None], 0, V, 1024, None, False)
+    (out[0] * gd).sum().backward()
+    assert hd.grad is not None and w.grad is None
+    # the kernel profile of a frozen-head backward has no hidden transposition and GEMM launches of dHidden tiles only
+    lib = _lib.load()
+    handle = lib.skyrl_lmhead_profile_begin()
+    ops.lmhead_bwd_hidden(h, w, y, lse, pz, gd, qd, 1.0 / t, 0)
+    import ctypes
+    n = lib.skyrl_lmhead_num_kernel_kinds()
+    ms, cnt = (ctypes.c_double * n)(), (ctypes.c_int64 * n)()
+    assert lib.skyrl_lmhead_profile_end(handle, ms, cnt) == 0
+    names = [lib.skyrl_lmhead_kernel_name(k).decode() for k in range(n)]
+    assert cnt[names.index("transpose_bf16")] == 1               # weight^T only (V = 1000 is not a multiple of 64)
