@@ -190,11 +190,15 @@ def main() -> int:
     # Timed region: exactly K steps, bracketed by synchronize on both sides; per-kernel HIP events ride along.
     with _lib.KernelProfile() as prof:
         torch.cuda.synchronize()
+        marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]  # per-step times ride along
         t0 = time.perf_counter()
-        for _ in range(args.steps):
+        marks[0].record()
+        for k in range(args.steps):
             step()
+            marks[k + 1].record()
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - t0
+    per_step = sorted(marks[k].elapsed_time(marks[k + 1]) for k in range(args.steps))
     ms_per_step = elapsed * 1e3 / args.steps
     tokens_per_s = T * args.steps / elapsed
 
@@ -239,6 +243,8 @@ def main() -> int:
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms_per_step,
+        "ms_per_step_median": per_step[len(per_step) // 2],
+        "ms_per_step_min": per_step[0],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
