@@ -235,6 +235,10 @@ def main() -> int:
         "launches_per_step": dom_launches,
     }
 
+    import ctypes
+    cus, khz = ctypes.c_int(0), ctypes.c_int(0)
+    _lib.check(lib.skyrl_lmhead_device_info(ctypes.byref(cus), ctypes.byref(khz)), "skyrl_lmhead_device_info")
+    box_cus, box_khz = cus.value, khz.value
     out = {
         "metric": METRIC,
         "value": tokens_per_s,
@@ -260,6 +264,9 @@ def main() -> int:
             "backward_tokens": t_active,
             "device": torch.cuda.get_device_name(0),
             "compute_units": torch.cuda.get_device_properties(0).multi_processor_count,
+            # the box's own figure for the denominator: CUs x 4096 bf16 flop per clock per CU x the maximum shader clock
+            "max_clock_mhz": box_khz / 1e3,
+            "peak_from_box_tflops": box_cus * 4096 * box_khz * 1e3 / 1e12,
         },
         "tflops": step_roofline["achieved"],
         "pct_of_bf16_mfma_peak": 100.0 * step_roofline["frac"],

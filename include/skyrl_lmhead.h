@@ -271,6 +271,10 @@ int skyrl_softce_bwd(const void* student_hidden, int64_t ld_student, const void*
  */
 int skyrl_lmhead_mfma_probe(const void* operands, int workgroups, int iters, float* sink, void* stream);
 
+/* Measurement aid (no counterpart in the reference): compute units and maximum shader clock (kHz) of the current device, the
+ * two figures the published matrix peak is made of (compute units x 4096 bf16 flop per clock x clock). */
+int skyrl_lmhead_device_info(int* compute_units, int* max_clock_khz);
+
 /*
  * Per-kernel timing for benchmarks (no counterpart in the reference, which times whole calls from Python with
  * torch.cuda.synchronize, skyrl/benchmarks/bench_fused_linear_logprob.py:96-101).

@@ -978,7 +978,7 @@ hipError_t launch_softce_pack(hipStream_t s, const void* student, int64_t lds_, 
 
 extern "C" {
 
-int skyrl_lmhead_version(void) { return 9; }
+int skyrl_lmhead_version(void) { return 10; }
 
 const char* skyrl_lmhead_strerror(int status) {
   switch (status) {
@@ -1253,6 +1253,15 @@ int skyrl_lmhead_mfma_probe(const void* operands, int workgroups, int iters, flo
   hipLaunchKernelGGL(mfma_probe, dim3((unsigned)workgroups), dim3(NTHREADS), 0, (hipStream_t)stream, (const bf16x8*)operands, iters,
                      sink);
   return (int)hipGetLastError();
+}
+
+int skyrl_lmhead_device_info(int* compute_units_out, int* max_clock_khz) {
+  if (!compute_units_out || !max_clock_khz) return SKYRL_LMHEAD_ERR_NULL;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e == hipSuccess) e = hipDeviceGetAttribute(compute_units_out, hipDeviceAttributeMultiprocessorCount, dev);
+  if (e == hipSuccess) e = hipDeviceGetAttribute(max_clock_khz, hipDeviceAttributeClockRate, dev);
+  return e == hipSuccess ? SKYRL_LMHEAD_OK : (int)e;
 }
 
 int skyrl_lmhead_num_kernel_kinds(void) { return kNumKernelKinds; }
