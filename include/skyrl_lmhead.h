@@ -168,7 +168,7 @@ int skyrl_approx_kl(const float* logprobs, const float* base_logprobs, const flo
                     int estimator, float* kld, float* row_mean, float* mean, int grad_mode, float* dlogprobs, void* stream);
 
 /*
- * The whole actor loss of a micro-batch and both upstream gradients of the LM-head backward in two launches -- what the
+ * The whole actor loss of a micro-batch and both upstream gradients of the LM-head backward in two launches (three with dentropy) -- what the
  * worker assembles from the policy loss, the KL term and the entropy term (skyrl/backends/skyrl_train/workers/worker.py:989-1089,
  * workers/megatron/megatron_model_wrapper.py:902-941):
  *     out6[0] = policy_scale * out6[1] + term_scale * (kl_coef * out6[4] - entropy_coef * out6[5])

@@ -12,7 +12,7 @@ and results:
 * ``masked_mean``               torch_utils.py:180-184
 
 plus ``actor_loss``, the whole per-micro-batch loss of the policy worker (policy loss + KL term - entropy term,
-workers/worker.py:989-1089) with both upstream gradients of the LM head from two launches, and ``approx_kl_loss``, the
+workers/worker.py:989-1089) with both upstream gradients of the LM head from two launches (three with an entropy gradient), and ``approx_kl_loss``, the
 reduction the trainer applies to the KL estimate (``masked_mean(kl, mask, dim=-1).mean()``,
 workers/worker.py:1071-1077) fused with the estimate and its gradient.  The losses are reduced as ``reduce_loss`` does
 (masked sum, :1145-1149; the reference folds the kind of mean into the advantages beforehand, :1152-1181).  The reference
@@ -540,7 +540,7 @@ def actor_loss(
     policy_scale: float = 1.0,
     term_scale: float = 1.0,
 ) -> Tuple[torch.Tensor, Dict[str, torch.Tensor]]:
-    """The loss the policy worker back-propagates for one micro-batch, assembled in two kernel launches together with
+    """The loss the policy worker back-propagates for one micro-batch, assembled in two kernel launches (three when the entropy takes a gradient) together with
     both upstream gradients of the fused LM head (reference: workers/worker.py:989-1089):
 
         ``policy_loss * policy_scale + (kl_loss * config.kl_loss_coef - entropy * config.entropy_loss_coef) * term_scale``

@@ -702,7 +702,7 @@ def test_loss_argument_errors(cuda_device):
 
 @pytest.mark.parametrize("use_kl,use_ent,masked", [(False, False, True), (True, False, False), (True, True, True)])
 def test_actor_loss_matches_oracle(use_kl, use_ent, masked, cuda_device):
-    """The assembled loss (policy + KL - entropy) and both upstream gradients from the two-launch kernel pair."""
+    """The assembled loss (policy + KL - entropy) and both upstream gradients from the row / finish / entropy-gradient kernels."""
     from types import SimpleNamespace
 
     from skyrl_amd.policy_loss import actor_loss
