@@ -51,7 +51,7 @@ int skyrl_lmhead_version(void);
 /* Human-readable text for a status code returned by this library (never NULL). */
 const char* skyrl_lmhead_strerror(int status);
 
-/* Scratch needed by skyrl_lmhead_fwd: per-vocab-tile (max, sum-exp, sum z*exp) partials, 24 * T * ceil(V/256) bytes
+/* Scratch needed by skyrl_lmhead_fwd: per-vocab-tile (max, sum-exp, sum z*exp) partials, 24 * T * ceil(V/256) bytes (T rounded up to a multiple of 64)
  * plus alignment slack.  (The reference allocates the same kind of buffers: `_max/_accu/_entropy_b [T, num_splits]`,
  * fused_linear_logprob_triton.py:670-672.) */
 size_t skyrl_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V);

@@ -3,8 +3,9 @@
 // Forward  (2*T*V*H flop):
 //   lmhead_fwd_tiles   one 256(vocab) x 256(token) logits tile per workgroup: bf16 MFMA GEMM, then in registers
 //                      scale by 1/temperature, per-token max / sum-exp / sum z*exp over the tile's vocab rows;
-//                      writes one (max, sum, pz) partial per token per 128-row half tile.  Logits never leave VGPRs.
-//   lmhead_fwd_merge   per token: merges the partials (online log-sum-exp), gathers the label logit with an
+//                      writes one (max, sum, pz) partial per token per 128-row half tile, in blocks of 64 tokens.  Logits
+//                      never leave VGPRs.
+//   lmhead_fwd_merge   per block of 64 tokens: merges the partials (online log-sum-exp), gathers the label logit with an
 //                      fp32 dot product hidden[t] . weight[label], writes logprob / entropy / lse / pz.
 // Backward (6*T*V*H flop), looped over vocab chunks of `vocab_chunk` columns:
 //   transpose_bf16     hidden^T once per call (and weight^T only when V is not a multiple of 64).
@@ -41,6 +42,17 @@ constexpr int kGroupM = LMHEAD_GROUP_M;
 constexpr int kLdPad = 64;
 
 __host__ __device__ inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+
+// Partial statistics live in blocks of 64 tokens: [token block][part][64 tokens].  A wave of the tile kernel writes 64
+// contiguous bytes (16 tokens) of one part; the merge kernel reads a token block's parts as one contiguous stream, 256 bytes
+// per wave instruction.  The arrays hold nparts * round_up(T, 64) floats.
+constexpr int kPartTokens = 64;
+__host__ __device__ inline size_t part_index(int part, int t, int nparts) {
+  return ((size_t)(t / kPartTokens) * (size_t)nparts + (size_t)part) * kPartTokens + (size_t)(t % kPartTokens);
+}
+__host__ __device__ inline size_t part_elems(size_t nparts, int64_t T) {
+  return nparts * (size_t)((T + kPartTokens - 1) / kPartTokens * kPartTokens);
+}
 
 // ------------------------------------------------------------------------------------------------------------
 // Forward tile kernel.  M axis = vocab (A = weight), N axis = tokens (B = hidden).
@@ -111,7 +123,7 @@ __device__ __forceinline__ void fwd_tile(const uint16_t* __restrict__ W, int ldw
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int lrow = lane & 15, kq = lane >> 4;
   const int vbase = tm * BM + wm * WM;
-  const size_t part = (size_t)(tm * WAVES_M + wm) * (size_t)T;
+  const int part = tm * WAVES_M + wm, nparts = tiles_m * WAVES_M;
   const float scale2 = rcp_temp * kLog2e;
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
@@ -123,9 +135,10 @@ __device__ __forceinline__ void fwd_tile(const uint16_t* __restrict__ W, int ldw
       fwd_tile_stats<ENTROPY, true, PAIRED>(acc, j, vbase, V, scale2, kq, m, s, e);
     }
     if (kq == 0 && t < T) {
-      part_max[part + t] = m;
-      part_sum[part + t] = s;
-      if (ENTROPY) part_pz[part + t] = e;
+      const size_t idx = part_index(part, t, nparts);
+      part_max[idx] = m;
+      part_sum[idx] = s;
+      if (ENTROPY) part_pz[idx] = e;
     }
   }
 }
@@ -140,66 +153,82 @@ __global__ __launch_bounds__(NTHREADS) void lmhead_fwd_tiles(const uint16_t* __r
 }
 
 // ------------------------------------------------------------------------------------------------------------
-// Forward merge.  8 tokens per workgroup of 256 threads (32 threads per token).
+// Forward merge.  One workgroup of 16 waves per block of 64 tokens: lane = token, wave w merges parts w, w + 16, ... of that
+// token (every load of a wave is 256 contiguous bytes), the sixteen running triples meet in LDS; then sixteen lanes per
+// token gather the label logit.
 // Merge algebra as in efficient_entropy_triton_kernel_epilogue (fused_linear_logprob_triton.py:417-467) except that
 // the running max starts at -inf (that kernel starts it at 0, which loses rows whose logits are all << 0).
 // Out-of-range labels give logprob 0 (model_utils.py:337; fused_linear_logprob_triton.py:1898-1905).
 // ------------------------------------------------------------------------------------------------------------
-constexpr int kMergeTokens = 8;
-constexpr int kMergeGroups = 256 / kMergeTokens;  // partial groups per token
+constexpr int kMergeTokens = kPartTokens;
+constexpr int kMergeThreads = 1024;
+constexpr int kMergeWaves = kMergeThreads / 64;
+constexpr int kDotLanes = kMergeThreads / kMergeTokens;  // lanes per token in the label-logit phase
 
-__global__ __launch_bounds__(256) void lmhead_fwd_merge(const float* __restrict__ part_max, const float* __restrict__ part_sum,
-                                                        const float* __restrict__ part_pz, int nparts, int T,
-                                                        const uint16_t* __restrict__ Hd, int ldh,
-                                                        const uint16_t* __restrict__ W, int ldw,
-                                                        const int64_t* __restrict__ labels, int H, int V, float rcp_temp,
-                                                        float* __restrict__ logprobs, float* __restrict__ entropy,
-                                                        float* __restrict__ row_lse, float* __restrict__ row_pz) {
-  __shared__ float sm_m[kMergeGroups][kMergeTokens], sm_s[kMergeGroups][kMergeTokens], sm_e[kMergeGroups][kMergeTokens];
+__global__ __launch_bounds__(kMergeThreads) void lmhead_fwd_merge(const float* __restrict__ part_max,
+                                                                  const float* __restrict__ part_sum,
+                                                                  const float* __restrict__ part_pz, int nparts, int T,
+                                                                  const uint16_t* __restrict__ Hd, int ldh,
+                                                                  const uint16_t* __restrict__ W, int ldw,
+                                                                  const int64_t* __restrict__ labels, int H, int V, float rcp_temp,
+                                                                  float* __restrict__ logprobs, float* __restrict__ entropy,
+                                                                  float* __restrict__ row_lse, float* __restrict__ row_pz) {
+  __shared__ float sm_m[kMergeWaves][kMergeTokens], sm_s[kMergeWaves][kMergeTokens], sm_e[kMergeWaves][kMergeTokens];
   __shared__ float sm_lse[kMergeTokens], sm_pz[kMergeTokens];
   const int tid = threadIdx.x;
   {
-    const int tl = tid % kMergeTokens, grp = tid / kMergeTokens;
-    const int t = blockIdx.x * kMergeTokens + tl;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int t = blockIdx.x * kMergeTokens + lane;
+    const size_t base = (size_t)blockIdx.x * (size_t)nparts * kPartTokens + lane;
     float M = -INFINITY, S = 0.f, E = 0.f;
     if (t < T) {
-      for (int p = grp; p < nparts; p += kMergeGroups) {
-        const size_t idx = (size_t)p * (size_t)T + t;
-        const float m = part_max[idx];
-        if (m > -INFINITY) {
-          const float s = part_sum[idx];
-          const float e = part_pz ? part_pz[idx] : 0.f;
-          const float Mn = fmaxf(M, m);
-          const float ca = expf(M - Mn), cb = expf(m - Mn);
-          S = S * ca + s * cb;
-          E = E * ca + e * cb;
-          M = Mn;
+      constexpr int kBatch = 4;  // loads in flight per array before the dependent merge chain
+      for (int p0 = wave; p0 < nparts; p0 += kMergeWaves * kBatch) {
+        float m[kBatch], sv[kBatch], ev[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+          const int p = p0 + u * kMergeWaves;
+          const bool in = p < nparts;
+          const size_t idx = base + (size_t)(in ? p : p0) * kPartTokens;
+          m[u] = in ? part_max[idx] : -INFINITY;
+          sv[u] = part_sum[idx];
+          ev[u] = part_pz ? part_pz[idx] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+          if (m[u] > -INFINITY) {
+            const float Mn = fmaxf(M, m[u]);
+            const float ca = expf(M - Mn), cb = expf(m[u] - Mn);
+            S = S * ca + sv[u] * cb;
+            E = E * ca + ev[u] * cb;
+            M = Mn;
+          }
         }
       }
     }
-    sm_m[grp][tl] = M;
-    sm_s[grp][tl] = S;
-    sm_e[grp][tl] = E;
+    sm_m[wave][lane] = M;
+    sm_s[wave][lane] = S;
+    sm_e[wave][lane] = E;
     __syncthreads();
-    if (grp == 0) {
+    if (wave == 0) {
       float Mg = -INFINITY;
-      for (int g = 0; g < kMergeGroups; ++g) Mg = fmaxf(Mg, sm_m[g][tl]);
+      for (int g = 0; g < kMergeWaves; ++g) Mg = fmaxf(Mg, sm_m[g][lane]);
       float Sg = 0.f, Eg = 0.f;
-      for (int g = 0; g < kMergeGroups; ++g) {
-        const float m = sm_m[g][tl];
+      for (int g = 0; g < kMergeWaves; ++g) {
+        const float m = sm_m[g][lane];
         if (m > -INFINITY) {
           const float c = expf(m - Mg);
-          Sg += sm_s[g][tl] * c;
-          Eg += sm_e[g][tl] * c;
+          Sg += sm_s[g][lane] * c;
+          Eg += sm_e[g][lane] * c;
         }
       }
-      sm_lse[tl] = Mg + logf(Sg);
-      sm_pz[tl] = Eg / Sg;
+      sm_lse[lane] = Mg + logf(Sg);
+      sm_pz[lane] = Eg / Sg;
     }
     __syncthreads();
   }
-  // Label logit: 32 lanes per token, 16-byte loads, fp32 accumulation.
-  const int tl = tid / kMergeGroups, sub = tid % kMergeGroups;
+  // Label logit: 16 lanes per token, 16-byte loads, fp32 accumulation.
+  const int tl = tid / kDotLanes, sub = tid % kDotLanes;
   const int t = blockIdx.x * kMergeTokens + tl;
   float dot = 0.f;
   bool has_label = false;
@@ -209,7 +238,7 @@ __global__ __launch_bounds__(256) void lmhead_fwd_merge(const float* __restrict_
     if (has_label) {
       const uint16_t* hp = Hd + (size_t)t * (size_t)ldh;
       const uint16_t* wp = W + (size_t)y * (size_t)ldw;
-      for (int c = sub * 8; c < H; c += kMergeGroups * 8) {
+      for (int c = sub * 8; c < H; c += kDotLanes * 8) {
         const uint4 hv = *(const uint4*)(hp + c);
         const uint4 wv = *(const uint4*)(wp + c);
         const uint32_t hh[4] = {hv.x, hv.y, hv.z, hv.w};
@@ -223,7 +252,7 @@ __global__ __launch_bounds__(256) void lmhead_fwd_merge(const float* __restrict_
     }
   }
 #pragma unroll
-  for (int o = 1; o < kMergeGroups; o <<= 1) dot += __shfl_xor(dot, o, 64);
+  for (int o = 1; o < kDotLanes; o <<= 1) dot += __shfl_xor(dot, o, 64);
   if (sub == 0 && t < T) {
     const float lse = sm_lse[tl], pz = sm_pz[tl];
     if (logprobs) logprobs[t] = has_label ? dot * rcp_temp - lse : 0.f;
@@ -927,9 +956,9 @@ SoftCeFwdWorkspace carve_softce_fwd(void* ws, int64_t T, int64_t H, int64_t V) {
   SoftCeFwdWorkspace w;
   w.nparts = (size_t)((V + BM - 1) / BM) * WAVES_M;
   w.S = c.take<uint16_t>((size_t)(2 * Tp) * (size_t)H);
-  w.pmax = c.take<float>(w.nparts * (size_t)(2 * Tp));
-  w.psum = c.take<float>(w.nparts * (size_t)(2 * Tp));
-  w.ppz = c.take<float>(w.nparts * (size_t)(2 * Tp));
+  w.pmax = c.take<float>(part_elems(w.nparts, 2 * Tp));
+  w.psum = c.take<float>(part_elems(w.nparts, 2 * Tp));
+  w.ppz = c.take<float>(part_elems(w.nparts, 2 * Tp));
   w.row_lse = c.take<float>((size_t)(2 * Tp));
   w.row_pz = c.take<float>((size_t)(2 * Tp));
   w.bytes = (size_t)round_up((int64_t)c.off, 256);
@@ -978,7 +1007,7 @@ hipError_t launch_softce_pack(hipStream_t s, const void* student, int64_t lds_, 
 
 extern "C" {
 
-int skyrl_lmhead_version(void) { return 10; }
+int skyrl_lmhead_version(void) { return 11; }
 
 const char* skyrl_lmhead_strerror(int status) {
   switch (status) {
@@ -1003,9 +1032,9 @@ size_t skyrl_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
   if (T < 1 || V < 1) return 0;
   const size_t nparts = (size_t)((V + BM - 1) / BM) * WAVES_M;
   Carver c(nullptr);
-  c.take<float>(nparts * (size_t)T);
-  c.take<float>(nparts * (size_t)T);
-  c.take<float>(nparts * (size_t)T);
+  c.take<float>(part_elems(nparts, T));
+  c.take<float>(part_elems(nparts, T));
+  c.take<float>(part_elems(nparts, T));
   return (size_t)round_up((int64_t)c.off, 256);
 }
 
@@ -1029,9 +1058,9 @@ int skyrl_lmhead_fwd(const void* hidden, int64_t ld_hidden, const void* weight, 
   const int tiles_m = (int)((V + BM - 1) / BM), tiles_n = (int)((T + BN - 1) / BN);
   const size_t nparts = (size_t)tiles_m * WAVES_M;
   Carver c(workspace);
-  float* pmax = c.take<float>(nparts * (size_t)T);
-  float* psum = c.take<float>(nparts * (size_t)T);
-  float* ppz = c.take<float>(nparts * (size_t)T);
+  float* pmax = c.take<float>(part_elems(nparts, T));
+  float* psum = c.take<float>(part_elems(nparts, T));
+  float* ppz = c.take<float>(part_elems(nparts, T));
   const bool want_pz = entropy || row_pz;
   const uint16_t* Wp = (const uint16_t*)weight;
   const uint16_t* Hp = (const uint16_t*)hidden;
@@ -1048,7 +1077,7 @@ int skyrl_lmhead_fwd(const void* hidden, int64_t ld_hidden, const void* weight, 
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
   Timed timed(kFwdMerge, s);
-  hipLaunchKernelGGL(lmhead_fwd_merge, dim3((unsigned)((T + kMergeTokens - 1) / kMergeTokens)), dim3(256), 0, s, pmax, psum,
+  hipLaunchKernelGGL(lmhead_fwd_merge, dim3((unsigned)((T + kMergeTokens - 1) / kMergeTokens)), dim3(kMergeThreads), 0, s, pmax, psum,
                      want_pz ? ppz : (float*)nullptr, (int)nparts, (int)T, Hp, (int)ld_hidden, Wp, (int)ld_weight, labels,
                      (int)H, (int)V, rcp_temperature, logprobs, entropy, row_lse, row_pz);
   e = hipGetLastError();
@@ -1175,7 +1204,7 @@ int skyrl_softce_fwd(const void* student_hidden, int64_t ld_student, const void*
   if ((e = hipGetLastError()) != hipSuccess) return (int)e;
   {
     Timed timed(kFwdMerge, s);
-    hipLaunchKernelGGL(lmhead_fwd_merge, dim3((unsigned)((rows + kMergeTokens - 1) / kMergeTokens)), dim3(256), 0, s, w.pmax,
+    hipLaunchKernelGGL(lmhead_fwd_merge, dim3((unsigned)((rows + kMergeTokens - 1) / kMergeTokens)), dim3(kMergeThreads), 0, s, w.pmax,
                        w.psum, w.ppz, (int)w.nparts, (int)rows, w.S, (int)H, Wp, (int)ld_weight, (const int64_t*)nullptr, (int)H,
                        (int)V, rcp_temperature, (float*)nullptr, (float*)nullptr, w.row_lse, w.row_pz);
   }
