@@ -37,7 +37,7 @@ METRIC = "fused LM-head fwd+bwd tokens/sec on 1 MI355X; % bf16 MFMA peak"
 # Bytes beyond L2 per lmhead_bwd_chunk launch from two `rocprofv3 --pmc` passes (FETCH_SIZE, then WRITE_SIZE), each scaled by what
 # the same counter reads for the 1 GiB copy of --copy-probe (x2048 and x1024 bytes per count).  Not measurable live; None for
 # workloads that have not been profiled.  Keyed by config name.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"qwen2.5-7b-fwdbwd": 12842285100}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"qwen2.5-7b-fwdbwd": 12781769720}
 
 
 def cpu_baseline(cfg, sample_tokens: int):
