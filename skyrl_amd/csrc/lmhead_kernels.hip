@@ -801,13 +801,16 @@ struct Carver {
 
 inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
+// Largest T, H, V or leading dimension any entry point accepts (the 4 GiB limit per matrix is far tighter in practice);
+// the workspace queries answer 0 beyond it instead of computing with sizes that no call would accept.
+constexpr int64_t kMaxExtent = (int64_t)1 << 30;
+
 // The two bf16 operands of every entry point: hidden rows [T, H] and weight rows [V, H].
 int check_operands(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, int64_t T, int64_t H, int64_t V,
                    float rcp_temperature) {
   if (!hidden || !weight) return SKYRL_LMHEAD_ERR_NULL;
   if (T < 1 || V < 1 || H < BK || H % BK != 0 || ldh < H || ldw < H) return SKYRL_LMHEAD_ERR_SHAPE;
-  if (T > (int64_t)1 << 30 || V > (int64_t)1 << 30 || ldh > (int64_t)1 << 30 || ldw > (int64_t)1 << 30)
-    return SKYRL_LMHEAD_ERR_SHAPE;
+  if (T > kMaxExtent || V > kMaxExtent || ldh > kMaxExtent || ldw > kMaxExtent) return SKYRL_LMHEAD_ERR_SHAPE;
   // The copy plan addresses an operand with 32-bit byte offsets: each operand (and each backward scratch matrix, which is
   // never larger than these two transposed) must stay below 4 GiB.
   const int64_t kMaxBytes = (int64_t)1 << 32;
@@ -882,12 +885,12 @@ int64_t default_vocab_chunk(int64_t T, int64_t H, int64_t V) {
     if (vc > Vpad) vc = Vpad;
     const bool fits = Tpad * vc * 2 <= kMaxPanelBytes;
     if (fits || best_vc == 0) {
-      int64_t cost = 0;
-      for (int64_t v0 = 0; v0 < Vpad; v0 += vc) {
-        const int64_t w = Vpad - v0 < vc ? Vpad - v0 : vc;
-        cost += list_schedule(w / 256 * tiles_t, H / BK + kDzEpilogue, 0, 0, ncu) + kLaunch;
-        cost += list_schedule(tiles_h * tiles_t, w / BK + kGemmEpilogue, tiles_h * (w / 256), Tpad / BK + kGemmEpilogue, ncu) + kLaunch;
-      }
+      auto chunk_cost = [&](int64_t w) {  // the two launches of a chunk of w columns
+        return list_schedule(w / 256 * tiles_t, H / BK + kDzEpilogue, 0, 0, ncu) + kLaunch +
+               list_schedule(tiles_h * tiles_t, w / BK + kGemmEpilogue, tiles_h * (w / 256), Tpad / BK + kGemmEpilogue, ncu) + kLaunch;
+      };
+      const int64_t full = Vpad / vc, rest = Vpad % vc;  // all chunks but the last have the same width
+      const int64_t cost = full * chunk_cost(vc) + (rest ? chunk_cost(rest) : 0);
       if (best_vc == 0 || cost < best_cost) best_vc = vc, best_cost = cost;
     }
     if (vc >= Vpad || !fits) break;
@@ -1029,7 +1032,7 @@ const char* skyrl_lmhead_strerror(int status) {
 
 size_t skyrl_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
   (void)H;
-  if (T < 1 || V < 1) return 0;
+  if (T < 1 || V < 1 || T > kMaxExtent || V > kMaxExtent) return 0;
   const size_t nparts = (size_t)((V + BM - 1) / BM) * WAVES_M;
   Carver c(nullptr);
   c.take<float>(part_elems(nparts, T));
@@ -1040,6 +1043,7 @@ size_t skyrl_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
 
 size_t skyrl_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t vocab_chunk) {
   if (T < 1 || V < 1 || H < 1 || vocab_chunk < 0 || vocab_chunk % 256 != 0) return 0;
+  if (T > kMaxExtent || V > kMaxExtent || H > kMaxExtent || vocab_chunk > kMaxExtent) return 0;
   int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(T, H, V);
   if (vc > round_up(V, 256)) vc = round_up(V, 256);
   return carve_bwd(nullptr, T, H, V, vc).bytes;
@@ -1167,12 +1171,13 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
 }
 
 size_t skyrl_softce_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
-  if (T < 1 || V < 1 || H < 1) return 0;
+  if (T < 1 || V < 1 || H < 1 || T > kMaxExtent || V > kMaxExtent || H > kMaxExtent) return 0;
   return carve_softce_fwd(nullptr, T, H, V).bytes;
 }
 
 size_t skyrl_softce_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t vocab_chunk) {
   if (T < 1 || V < 1 || H < 1 || vocab_chunk < 0 || vocab_chunk % 256 != 0) return 0;
+  if (T > kMaxExtent || V > kMaxExtent || H > kMaxExtent || vocab_chunk > kMaxExtent) return 0;
   int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(T, H, V);
   if (vc > round_up(V, 256)) vc = round_up(V, 256);
   return carve_softce_bwd(nullptr, T, H, V, vc).bytes;

@@ -433,7 +433,7 @@ int skyrl_approx_kl(const float* logprobs, const float* base_logprobs, const flo
   if (!logprobs || !base_logprobs || !row_mean || !mean) return SKYRL_LMHEAD_ERR_NULL;
   if (grad_mode < 0 || grad_mode > 2 || estimator < SKYRL_KL_K1 || estimator > SKYRL_KL_K3) return SKYRL_LMHEAD_ERR_ARG;
   if (grad_mode != 0 && !dlogprobs) return SKYRL_LMHEAD_ERR_NULL;
-  if (rows < 1 || cols < 1 || rows >= (int64_t(1) << 31)) return SKYRL_LMHEAD_ERR_SHAPE;
+  if (rows < 1 || cols < 1 || rows >= (int64_t(1) << 31) || cols >= (int64_t(1) << 31)) return SKYRL_LMHEAD_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   hipLaunchKernelGGL(approx_kl_rows_kernel, dim3((unsigned)rows), dim3(kRowThreads), 0, s, logprobs, base_logprobs, loss_mask,
                      rows, cols, estimator, grad_mode, kld, row_mean, dlogprobs);
@@ -451,7 +451,7 @@ int skyrl_actor_loss(const float* logprobs, const float* old_logprobs, const flo
   const bool needs_old = loss_type != SKYRL_POLICY_LOSS_CROSS_ENTROPY;
   if (!logprobs || !row_sums || !out6 || (needs_old && (!old_logprobs || !advantages))) return SKYRL_LMHEAD_ERR_NULL;
   if (dentropy && !entropy) return SKYRL_LMHEAD_ERR_NULL;
-  if (rows < 1 || cols < 1 || rows >= (int64_t(1) << 31)) return SKYRL_LMHEAD_ERR_SHAPE;
+  if (rows < 1 || cols < 1 || rows >= (int64_t(1) << 31) || cols >= (int64_t(1) << 31)) return SKYRL_LMHEAD_ERR_SHAPE;
   if (!valid_loss_params(loss_type, eps_clip_low, eps_clip_high, clip_ratio_c)) return SKYRL_LMHEAD_ERR_ARG;
   if (!finite(policy_scale) || !finite(term_scale) || !finite(kl_coef) || !finite(entropy_coef)) return SKYRL_LMHEAD_ERR_ARG;
   const ActorLossArgs a{logprobs,   old_logprobs,       advantages,         loss_mask,    loss_weight,  base_logprobs, entropy,
@@ -473,7 +473,7 @@ int skyrl_actor_loss(const float* logprobs, const float* old_logprobs, const flo
 int skyrl_masked_mean(const float* values, const float* mask, int64_t rows, int64_t cols, float* means, float* dvalues,
                       void* stream) {
   if (!values || !means) return SKYRL_LMHEAD_ERR_NULL;
-  if (rows < 1 || cols < 1 || rows >= (int64_t(1) << 31)) return SKYRL_LMHEAD_ERR_SHAPE;
+  if (rows < 1 || cols < 1 || rows >= (int64_t(1) << 31) || cols >= (int64_t(1) << 31)) return SKYRL_LMHEAD_ERR_SHAPE;
   hipLaunchKernelGGL(masked_mean_rows_kernel, dim3((unsigned)rows), dim3(kRowThreads), 0, (hipStream_t)stream, values, mask, cols,
                      means, dvalues);
   return (int)hipGetLastError();

@@ -152,8 +152,10 @@ int check_scatter(const void* packed, const int64_t* cu, int64_t n, int64_t T, c
   if (given == 3 && mask) return SKYRL_LMHEAD_ERR_ARG;
   if (n < 0 || T < 0 || rows < 0 || cols < 0) return SKYRL_LMHEAD_ERR_SHAPE;
   if (mask && rows != n) return SKYRL_LMHEAD_ERR_SHAPE;
-  if (T >= (int64_t(1) << 31) * kThreads || rows * cols >= (int64_t(1) << 31) * kThreads || rows >= (int64_t(1) << 31))
-    return SKYRL_LMHEAD_ERR_SHAPE;
+  // one thread per token or output element, at most 2^31 workgroups; rows and columns are bounded first so that their
+  // product cannot overflow
+  const int64_t kMaxDim = int64_t(1) << 31, kMaxElems = kMaxDim * kThreads;
+  if (T >= kMaxElems || rows >= kMaxDim || cols >= kMaxDim || rows * cols >= kMaxElems) return SKYRL_LMHEAD_ERR_SHAPE;
   return SKYRL_LMHEAD_OK;
 }
 
