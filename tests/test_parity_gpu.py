@@ -1675,3 +1675,50 @@ def test_frozen_lm_head_skips_the_weight_gradient(cuda_device):
     assert lib.skyrl_lmhead_profile_end(handle, ms, cnt) == 0
     names = [lib.skyrl_lmhead_kernel_name(k).decode() for k in range(n)]
     assert cnt[names.index("transpose_bf16")] == 1               # weight^T only (V = 1000 is not a multiple of 64)
+
+
+def test_entry_points_are_reentrant_across_threads_and_streams(cuda_device):
+    """Two host threads, each with its own stream, inputs and workspaces, run forward + backward steps at the same time; every
+    result equals the one a single thread gets (the library keeps no state between calls apart from the per-thread profile)."""
+    import threading
+
+    T, H, V = 500, 128, 3000
+    cases = []
+    for seed in (101, 102):
+        hidden, weight, labels, g, q = _rand(T, H, V, seed=seed)
+        cases.append([x.to(cuda_device) for x in (hidden, weight, labels, g, q)])
+
+    def run(case):
+        h, w, y, g, q = case
+        lp, ent, lse, pz = ops.lmhead_fwd(h, w, y, 0.9, True)
+        dh, dw = ops.lmhead_bwd(h, w, y, lse, pz, g, q, 0.9, 1024)
+        return lp, ent, dh, dw
+
+    want = [run(c) for c in cases]
+    torch.cuda.synchronize()
+    got = [[], []]
+    errors = []
+
+    def worker(k):
+        try:
+            stream = torch.cuda.Stream(device=cuda_device)
+            with torch.cuda.stream(stream):
+                for _ in range(8):
+                    got[k].append(run(cases[k]))
+            stream.synchronize()
+        except Exception as e:  # surfaced in the main thread below
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(k,)) for k in range(2)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=100)
+    assert not errors, errors
+    assert not any(th.is_alive() for th in threads)
+    torch.cuda.synchronize()
+    for k in range(2):
+        assert len(got[k]) == 8
+        for outs in got[k]:
+            for a, b in zip(outs, want[k]):
+                assert torch.equal(a, b)
