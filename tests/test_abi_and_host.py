@@ -319,3 +319,36 @@ def test_default_vocab_chunk_respects_the_panel_cap():
         vc = (panel - 1024) // (2 * Tp) - 64          # the alignment slack is below one row
         vc = -(-vc // 256) * 256
         assert 256 <= vc <= Vp and lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, vc) == total, (T, H, V, vc)
+
+
+def test_product_never_touches_the_oracle_or_the_working_folder():
+    """The checker stays test infrastructure: no module of the package imports, reads or names ``oracle`` or ``_work``, and
+    of the two scripts at the root only ``smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` import the oracle."""
+    import ast
+
+    def imports(path):
+        tree = ast.parse(open(path).read())
+        found = set()
+        for node in ast.walk(tree):
+            if isinstance(node, ast.Import):
+                found.update(a.name.split(".")[0] for a in node.names)
+            elif isinstance(node, ast.ImportFrom) and node.module and node.level == 0:
+                found.add(node.module.split(".")[0])
+        return found
+
+    pkg = os.path.join(ROOT, "skyrl_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".h")):
+                path = os.path.join(dirpath, f)
+                text = open(path).read()
+                assert "_work" not in text.replace("_workspace", "").replace("_workgroup", ""), path
+                if f.endswith(".py"):
+                    assert "oracle" not in imports(path), path
+    for script, allowed in (("bench.py", "cpu_baseline"), ("__graft_entry__.py", "smoke")):
+        tree = ast.parse(open(os.path.join(ROOT, script)).read())
+        for fn in [n for n in ast.walk(tree) if isinstance(n, ast.FunctionDef)]:
+            uses = any(isinstance(n, ast.ImportFrom) and n.module == "oracle" for n in ast.walk(fn))
+            assert not uses or fn.name == allowed, f"{script}:{fn.name} imports the oracle"
+        top_level = [n for n in tree.body if isinstance(n, (ast.Import, ast.ImportFrom))]
+        assert not any(isinstance(n, ast.ImportFrom) and n.module == "oracle" for n in top_level)
