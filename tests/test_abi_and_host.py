@@ -16,8 +16,13 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "skyrl_lmhead.h")
 
 
+def _read(path):
+    with open(path) as f:
+        return f.read()
+
+
 def _declared_functions():
-    text = open(HEADER).read()
+    text = _read(HEADER)
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(skyrl_(?:lmhead|ppo|packed|approx|masked|actor|softce)_\w+)\s*\(", text)))
 
@@ -33,7 +38,8 @@ def test_library_exports_every_declared_symbol():
 
 def test_library_is_in_tree_and_has_no_torch_dependency():
     assert _lib.lib_path().startswith(ROOT)
-    out = os.popen(f"ldd {_lib.lib_path()}").read()
+    import subprocess
+    out = subprocess.run(["ldd", _lib.lib_path()], capture_output=True, text=True).stdout
     assert "libamdhip64" in out and "torch" not in out and "libc10" not in out
 
 
@@ -327,7 +333,7 @@ def test_product_never_touches_the_oracle_or_the_working_folder():
     import ast
 
     def imports(path):
-        tree = ast.parse(open(path).read())
+        tree = ast.parse(_read(path))
         found = set()
         for node in ast.walk(tree):
             if isinstance(node, ast.Import):
@@ -341,12 +347,12 @@ def test_product_never_touches_the_oracle_or_the_working_folder():
         for f in files:
             if f.endswith((".py", ".hip", ".hpp", ".h")):
                 path = os.path.join(dirpath, f)
-                text = open(path).read()
+                text = _read(path)
                 assert "_work" not in text.replace("_workspace", "").replace("_workgroup", ""), path
                 if f.endswith(".py"):
                     assert "oracle" not in imports(path), path
     for script, allowed in (("bench.py", "cpu_baseline"), ("__graft_entry__.py", "smoke")):
-        tree = ast.parse(open(os.path.join(ROOT, script)).read())
+        tree = ast.parse(_read(os.path.join(ROOT, script)))
         for fn in [n for n in ast.walk(tree) if isinstance(n, ast.FunctionDef)]:
             uses = any(isinstance(n, ast.ImportFrom) and n.module == "oracle" for n in ast.walk(fn))
             assert not uses or fn.name == allowed, f"{script}:{fn.name} imports the oracle"
