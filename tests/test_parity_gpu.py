@@ -1722,3 +1722,23 @@ def test_entry_points_are_reentrant_across_threads_and_streams(cuda_device):
         for outs in got[k]:
             for a, b in zip(outs, want[k]):
                 assert torch.equal(a, b)
+
+
+def test_soft_ce_extreme_logits(cuda_device):
+    """Logits of the order of +-150 (a near one-hot teacher, a confident and often wrong student): losses of tens to hundreds
+    of nats without overflow, against fp64; the tolerance scales with the loss, as the fp32 accumulation error does."""
+    from skyrl_amd.mtp_soft_ce import soft_ce_from_hidden
+
+    B, S, H, V = 2, 130, 128, 1500
+    hs, ht, w = _softce_case(B, S, H, V, 81, spread=45.0)
+    hs64 = hs.double().requires_grad_(True)
+    ref = O.soft_ce_per_token(hs64 @ w.double().t(), torch.roll(ht.double() @ w.double().t(), -1, dims=1))
+    ref.sum().backward()
+    assert ref.max().item() > 100.0
+    d_hs = hs.to(cuda_device).requires_grad_(True)
+    got = soft_ce_from_hidden(d_hs, ht.to(cuda_device), w.to(cuda_device), shift=1)
+    got.sum().backward()
+    assert bool(torch.isfinite(got).all()) and bool(torch.isfinite(d_hs.grad.float()).all())
+    err = (got.detach().cpu().double() - ref.detach()).abs()
+    assert bool((err <= 1e-4 * ref.detach().abs() + 1e-3).all()), err.max().item()
+    assert cos(d_hs.grad.float(), hs64.grad) >= GRAD_COS
