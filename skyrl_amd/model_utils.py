@@ -152,8 +152,16 @@ def from_parallel_hidden_to_logprobs_packed_sequences(
     sub_seq_lengths: Optional[list] = None,
     temperature: float = 1.0,
     fused_backend: str = "hip",
+    *,
+    action_window: Optional[int] = None,
 ) -> torch.Tensor:
-    """Packed variant: ``hidden`` [1, T, H], ``target`` [1, T], ``cu_seqlens_padded`` [n+1] -> [batch, unpacked_seqlen-1]."""
+    """Packed variant: ``hidden`` [1, T, H], ``target`` [1, T], ``cu_seqlens_padded`` [n+1] -> [batch, unpacked_seqlen-1].
+
+    ``action_window = n`` (an extension) returns the last ``n`` columns only, ``[batch, n]`` -- what the Megatron worker
+    slices next (``token_logprobs[:, -num_actions:]``, megatron_model_wrapper.py:707) -- and runs the LM head on just the
+    packed tokens that land there: the scatter kernel, applied to the token numbers, is its own inverse map, so the rows are
+    found without a host synchronisation and the shapes stay static (``batch * n`` rows, absent ones masked).
+    """
     if _group_size(cp_group) > 1:
         raise NotImplementedError("context parallelism is outside the one-GPU scope of the HIP fused LM-head path")
     hidden = hidden.squeeze(0)
@@ -166,6 +174,32 @@ def from_parallel_hidden_to_logprobs_packed_sequences(
     cu = cu_seqlens_padded.to(device=target.device, dtype=torch.long)
     rolled_targets = packed_next_token_labels(target.to(torch.long).contiguous(), cu).unsqueeze(0)
     hidden = hidden.unsqueeze(0)
+    cols = unpacked_seqlen - 1
+    if sub_seq_lengths is not None:
+        rows, row_offs, seq_lens = _packed_subseq_row_indices_offsets_and_lens(cu, sub_seq_lengths, target.device)
+        layout = dict(seg_row=rows, seg_col=row_offs, seg_len=seq_lens)
+    elif attention_mask is not None:
+        layout = dict(attention_mask=attention_mask)
+    else:
+        layout = {}
+
+    if action_window is not None:
+        n_act, T = int(action_window), hidden.shape[1]
+        if not 0 < n_act <= cols:
+            raise ValueError(f"action_window {action_window} does not fit {cols} columns")
+        if T >= 1 << 24:
+            raise ValueError("action_window numbers the packed tokens in fp32: at most 2^24 - 1 tokens")
+        with torch.no_grad():  # token number + 1 where a token lands, 0 elsewhere
+            number = torch.arange(1, T + 1, dtype=torch.float32, device=target.device)
+            landed = packed_scatter_logprobs(number, cu, batch_size, cols, **layout)[:, cols - n_act:]
+            src = landed.reshape(-1).to(torch.long) - 1
+            present = (src >= 0).reshape(batch_size, n_act)
+            src = src.clamp(min=0)
+        rows_h = hidden.reshape(T, -1).index_select(0, src).unsqueeze(0)          # differentiable gather of the rows
+        rows_y = rolled_targets.reshape(-1).index_select(0, src).unsqueeze(0).contiguous()
+        window = _fused_lm_head_logprob_apply(fused_backend, rows_h, lm_head_weight, rows_y, vocab_start_index, vocab_end_index,
+                                              rows_h.shape[1], group, inference_only, temperature)
+        return window.reshape(batch_size, n_act) * present
 
     seq_len_local = hidden.shape[1]
     eff_chunk = chunk_size if (chunk_size is not None and chunk_size < seq_len_local) else seq_len_local
@@ -177,13 +211,7 @@ def from_parallel_hidden_to_logprobs_packed_sequences(
         raise ValueError(f"Expected probs to be 1D after squeezing, but got shape {probs.shape}.")
 
     # Scatter-back to [batch, unpacked_seqlen - 1], one kernel per direction (reference: boolean-mask indexing, :851-883).
-    cols = unpacked_seqlen - 1
-    if sub_seq_lengths is not None:
-        rows, row_offs, seq_lens = _packed_subseq_row_indices_offsets_and_lens(cu, sub_seq_lengths, probs.device)
-        return packed_scatter_logprobs(probs, cu, batch_size, cols, seg_row=rows, seg_col=row_offs, seg_len=seq_lens)
-    if attention_mask is not None:
-        return packed_scatter_logprobs(probs, cu, batch_size, cols, attention_mask=attention_mask)
-    return packed_scatter_logprobs(probs, cu, batch_size, cols)
+    return packed_scatter_logprobs(probs, cu, batch_size, cols, **layout)
 
 
 def _fused_vocab_parallel_entropy_from_hidden(

@@ -203,10 +203,13 @@ def test_signatures_mirror_the_reference():
         "hidden", "lm_head_weight", "target", "vocab_start_index", "vocab_end_index", "tp_group", "inference_only",
         "cp_group", "chunk_size", "temperature", "fused_backend"]
     # model_utils.py:773-789
-    assert list(inspect.signature(model_utils.from_parallel_hidden_to_logprobs_packed_sequences).parameters) == [
+    packed = inspect.signature(model_utils.from_parallel_hidden_to_logprobs_packed_sequences).parameters
+    assert list(packed)[:15] == [
         "hidden", "lm_head_weight", "target", "cu_seqlens_padded", "unpacked_seqlen", "vocab_start_index", "vocab_end_index",
         "group", "inference_only", "cp_group", "chunk_size", "attention_mask", "sub_seq_lengths", "temperature",
         "fused_backend"]
+    # anything beyond the reference's list is keyword-only and optional, so every reference call site binds unchanged
+    assert all(v.kind is inspect.Parameter.KEYWORD_ONLY and v.default is None for v in list(packed.values())[15:])
     # model_utils.py:1090-1096
     assert list(inspect.signature(model_utils._fused_vocab_parallel_entropy_from_hidden).parameters) == [
         "hidden", "lm_head_weight", "tp_group", "chunk_size", "temperature"]

@@ -1057,6 +1057,44 @@ def test_packed_wrapper_all_layouts_with_gradient(cuda_device):
         assert cos(hd.grad[0], ex["d_hidden"]) >= GRAD_COS and cos(wd.grad, ex["d_weight"]) >= GRAD_COS, name
 
 
+def test_packed_wrapper_action_window(cuda_device):
+    """action_window = n: the last n columns of the full result, from an LM head that ran on the landing rows only -- equal
+    values (a token's row is computed independently of the others) and the same gradients as the full pass with an
+    upstream gradient that is zero outside the window."""
+    dev = cuda_device
+    H, V, t = 128, 515, 0.8
+    gen = torch.Generator().manual_seed(53)
+    true_lens = [9, 1, 17, 13, 6]
+    padded = [10, 2, 17, 16, 6]
+    cu = torch.cat([torch.zeros(1, dtype=torch.long), torch.tensor(padded).cumsum(0)]).to(dev)
+    T = int(cu[-1])
+    hidden = torch.randn(1, T, H, generator=gen).to(torch.bfloat16).to(dev)
+    weight = (torch.randn(V, H, generator=gen) * 3 / H**0.5).to(torch.bfloat16).to(dev)
+    tokens = torch.randint(0, V, (1, T), generator=gen).to(dev)
+    L = 20
+    am = torch.zeros(len(true_lens), L, dtype=torch.bool)
+    for b, n in enumerate(true_lens):
+        am[b, L - n:] = True
+    cases = {"plain": (dict(), L), "mask": (dict(attention_mask=am.to(dev)), L), "sub": (dict(sub_seq_lengths=[[9, 1], [17], [13, 6]]), 31)}
+    for name, (kw, seqlen) in cases.items():
+        for window in (4, 11, seqlen - 1):
+            hd, wd = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
+            full = model_utils.from_parallel_hidden_to_logprobs_packed_sequences(hd, wd, tokens, cu, seqlen, 0, V, None,
+                                                                                 temperature=t, **kw)
+            G = torch.randn(full.shape[0], window, generator=gen).to(dev)
+            (full[:, -window:] * G).sum().backward()
+            h2, w2 = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
+            got = model_utils.from_parallel_hidden_to_logprobs_packed_sequences(h2, w2, tokens, cu, seqlen, 0, V, None,
+                                                                                temperature=t, action_window=window, **kw)
+            assert got.shape == (full.shape[0], window), name
+            torch.testing.assert_close(got.detach(), full.detach()[:, -window:], rtol=0, atol=1e-6, msg=f"{name} {window}")
+            (got * G).sum().backward()
+            if full.detach()[:, -window:].abs().sum() > 0:
+                assert cos(h2.grad, hd.grad) >= 0.9999 and cos(w2.grad, wd.grad) >= 0.9999, (name, window)
+    with pytest.raises(ValueError):
+        model_utils.from_parallel_hidden_to_logprobs_packed_sequences(hidden, weight, tokens, cu, L, 0, V, None, action_window=L)
+
+
 def test_packed_argument_errors(cuda_device):
     lib = _lib.load()
     x = torch.zeros(8, dtype=torch.float32, device=cuda_device)
