@@ -93,11 +93,23 @@ def from_parallel_hidden_to_logprobs(
     chunk_size: Optional[int] = None,
     temperature: float = 1.0,
     fused_backend: str = "hip",
+    *,
+    action_window: Optional[int] = None,
 ) -> torch.Tensor:
-    """``hidden`` [B, S, H] + ``lm_head_weight`` [V, H] + token ids ``target`` [B, S] -> next-token logprobs [B, S-1]."""
+    """``hidden`` [B, S, H] + ``lm_head_weight`` [V, H] + token ids ``target`` [B, S] -> next-token logprobs [B, S-1].
+
+    ``action_window = n`` (an extension) returns the last ``n`` columns only, ``[B, n]``, from an LM head run on positions
+    ``S - 1 - n .. S - 2`` -- the slice the worker takes next -- instead of on all ``S`` positions."""
     if _group_size(cp_group) > 1:
         raise NotImplementedError("context parallelism is outside the one-GPU scope of the HIP fused LM-head path")
     target = target.roll(shifts=-1, dims=-1)
+    if action_window is not None:
+        n_act, S = int(action_window), hidden.shape[1]
+        if not 0 < n_act <= S - 1:
+            raise ValueError(f"action_window {action_window} does not fit sequences of length {S}")
+        hidden, target = hidden[:, S - 1 - n_act:S - 1], target[:, S - 1 - n_act:S - 1].contiguous()
+        return _fused_lm_head_logprob_apply(fused_backend, hidden, lm_head_weight, target, vocab_start_index, vocab_end_index,
+                                            n_act, tp_group, inference_only, temperature).contiguous()
     seq_len_local = hidden.shape[1]
     eff_chunk = chunk_size if (chunk_size is not None and chunk_size < seq_len_local) else seq_len_local
     logprobs = _fused_lm_head_logprob_apply(

@@ -199,9 +199,11 @@ def test_signatures_mirror_the_reference():
     assert list(inspect.signature(LinearCrossEntropy.forward).parameters) == [
         "ctx", "hidden", "weight", "labels", "temperature", "reduction", "dist_process_group"]
     # model_utils.py:713-725
-    assert list(inspect.signature(model_utils.from_parallel_hidden_to_logprobs).parameters) == [
+    dense = inspect.signature(model_utils.from_parallel_hidden_to_logprobs).parameters
+    assert list(dense)[:11] == [
         "hidden", "lm_head_weight", "target", "vocab_start_index", "vocab_end_index", "tp_group", "inference_only",
         "cp_group", "chunk_size", "temperature", "fused_backend"]
+    assert all(v.kind is inspect.Parameter.KEYWORD_ONLY and v.default is None for v in list(dense.values())[11:])
     # model_utils.py:773-789
     packed = inspect.signature(model_utils.from_parallel_hidden_to_logprobs_packed_sequences).parameters
     assert list(packed)[:15] == [

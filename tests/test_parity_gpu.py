@@ -1095,6 +1095,28 @@ def test_packed_wrapper_action_window(cuda_device):
         model_utils.from_parallel_hidden_to_logprobs_packed_sequences(hidden, weight, tokens, cu, L, 0, V, None, action_window=L)
 
 
+def test_dense_wrapper_action_window(cuda_device):
+    dev = cuda_device
+    gen = torch.Generator().manual_seed(54)
+    B, S, H, V, t = 3, 37, 128, 700, 0.7
+    hidden = torch.randn(B, S, H, generator=gen).to(torch.bfloat16).to(dev)
+    weight = (torch.randn(V, H, generator=gen) * 3 / H**0.5).to(torch.bfloat16).to(dev)
+    tokens = torch.randint(0, V, (B, S), generator=gen).to(dev)
+    for window in (1, 9, S - 1):
+        hd, wd = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
+        full = model_utils.from_parallel_hidden_to_logprobs(hd, wd, tokens, 0, V, None, temperature=t)
+        G = torch.randn(B, window, generator=gen).to(dev)
+        (full[:, -window:] * G).sum().backward()
+        h2, w2 = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
+        got = model_utils.from_parallel_hidden_to_logprobs(h2, w2, tokens, 0, V, None, temperature=t, action_window=window)
+        assert got.shape == (B, window)
+        torch.testing.assert_close(got.detach(), full.detach()[:, -window:], rtol=0, atol=1e-6)
+        (got * G).sum().backward()
+        assert cos(h2.grad, hd.grad) >= 0.9999 and cos(w2.grad, wd.grad) >= 0.9999
+    with pytest.raises(ValueError):
+        model_utils.from_parallel_hidden_to_logprobs(hidden, weight, tokens, 0, V, None, action_window=S)
+
+
 def test_packed_argument_errors(cuda_device):
     lib = _lib.load()
     x = torch.zeros(8, dtype=torch.float32, device=cuda_device)
