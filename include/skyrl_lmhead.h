@@ -81,19 +81,24 @@ int skyrl_lmhead_fwd(const void* hidden, int64_t ld_hidden, const void* weight, 
 /*
  * Backward.  Same hidden / weight / labels as the forward call; row_lse, row_pz from it (row_pz may be NULL
  * iff dentropy is NULL); dlogprobs fp32 [T] (required), dentropy fp32 [T] or NULL.
- * d_hidden: bf16 [T, H] contiguous, overwritten.  d_weight: fp32 [V, H] contiguous, overwritten, or added to
- * when accumulate_dw != 0 (gradient accumulation across micro-batches); NULL when the weight takes no gradient (a frozen
+ * d_hidden: bf16 [T, H] contiguous, overwritten.  d_weight: [V, H] contiguous; by dw_mode fp32 overwritten (SKYRL_DW_FP32),
+ * fp32 added to (SKYRL_DW_FP32_ACCUMULATE: gradient accumulation across micro-batches) or bf16 overwritten (SKYRL_DW_BF16:
+ * the fp32 sums are rounded to nearest-even in the GEMM epilogue -- grad_weight in the weight dtype as model_utils.py:428
+ * returns it, without an fp32 [V, H] buffer and a cast pass); NULL when the weight takes no gradient (a frozen
  * LM head, e.g. adapter training: autograd would drop grad_weight of model_utils.py:419-428 too) -- the dW product, a third
  * of the backward's work, is then not computed.  Both gradients are with respect to the unscaled weight / hidden: the
  * 1/temperature factor is already applied.
  * vocab_chunk: width of the dz panel in vocab columns (multiple of 256; 0 = library default: the width, with a panel of
  * at most 1.5 GiB, whose launches divide most evenly over the device's compute units).
  */
+#define SKYRL_DW_FP32 0
+#define SKYRL_DW_FP32_ACCUMULATE 1
+#define SKYRL_DW_BF16 2
 int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight,
                      const int64_t* labels, const float* row_lse, const float* row_pz,
                      const float* dlogprobs, const float* dentropy,
                      int64_t T, int64_t H, int64_t V, float rcp_temperature,
-                     void* d_hidden, float* d_weight, int accumulate_dw, int64_t vocab_chunk,
+                     void* d_hidden, void* d_weight, int dw_mode, int64_t vocab_chunk,
                      void* workspace, size_t workspace_bytes, void* stream);
 
 /*

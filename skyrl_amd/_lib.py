@@ -11,7 +11,7 @@ import os
 import threading
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libskyrl_lmhead.so")
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 _c_i64 = ctypes.c_int64
 _c_p = ctypes.c_void_p

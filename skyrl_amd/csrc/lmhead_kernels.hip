@@ -1010,7 +1010,7 @@ hipError_t launch_softce_pack(hipStream_t s, const void* student, int64_t lds_, 
 
 extern "C" {
 
-int skyrl_lmhead_version(void) { return 11; }
+int skyrl_lmhead_version(void) { return 12; }
 
 const char* skyrl_lmhead_strerror(int status) {
   switch (status) {
@@ -1090,13 +1090,14 @@ int skyrl_lmhead_fwd(const void* hidden, int64_t ld_hidden, const void* weight, 
 
 int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight, const int64_t* labels,
                      const float* row_lse, const float* row_pz, const float* dlogprobs, const float* dentropy, int64_t T,
-                     int64_t H, int64_t V, float rcp_temperature, void* d_hidden, float* d_weight, int accumulate_dw,
+                     int64_t H, int64_t V, float rcp_temperature, void* d_hidden, void* d_weight, int dw_mode,
                      int64_t vocab_chunk, void* workspace, size_t workspace_bytes, void* stream) {
   int st = check_common(hidden, ld_hidden, weight, ld_weight, labels, T, H, V, rcp_temperature);
   if (st) return st;
   if (!row_lse || !dlogprobs || !d_hidden) return SKYRL_LMHEAD_ERR_NULL;
   if (dentropy && !row_pz) return SKYRL_LMHEAD_ERR_NULL;
   if (!aligned16(d_hidden) || !aligned16(d_weight)) return SKYRL_LMHEAD_ERR_ALIGN;  // d_weight NULL: no dW wanted
+  if (dw_mode < SKYRL_DW_FP32 || dw_mode > SKYRL_DW_BF16) return SKYRL_LMHEAD_ERR_ARG;
   if (vocab_chunk < 0 || vocab_chunk % 256 != 0) return SKYRL_LMHEAD_ERR_ARG;
   const int64_t Tpad = round_up(T, 256), Vpad = round_up(V, 256);
   int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(T, H, V);
@@ -1148,7 +1149,10 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
     // dW[vc0 + v, h]  (+)= sum_t D[t, v] . hidden^T[h, t]             (A = hidden^T rows, B = D read K-major)
     const bool first = ci == 0, last = ci == nchunks - 1;
     const int64_t rows = (V - vc0) < vcw ? (V - vc0) : vcw;
-    float* dWc = d_weight ? d_weight + (size_t)vc0 * (size_t)H : (float*)nullptr;
+    // dW rows are complete within their chunk, so they can leave the GEMM epilogue in either precision.
+    const size_t dw_off = (size_t)vc0 * (size_t)H;
+    float* dWf = (d_weight && dw_mode != SKYRL_DW_BF16) ? (float*)d_weight + dw_off : (float*)nullptr;
+    uint16_t* dWb = (d_weight && dw_mode == SKYRL_DW_BF16) ? (uint16_t*)d_weight + dw_off : (uint16_t*)nullptr;
     const uint16_t* dh_out = last ? (uint16_t*)d_hidden : (uint16_t*)nullptr;
     const float* dh_in = first ? (const float*)nullptr : (const float*)w.dHacc;
     float* dh_keep = last ? (float*)nullptr : w.dHacc;
@@ -1162,7 +1166,8 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
                                nullptr, (uint16_t*)dh_out, H, dh_in, dh_keep);
     // A frozen LM head (d_weight == NULL) needs no dW: the launch then carries the dHidden tiles alone.
     const GemmArgs gw = d_weight ? make_gemm(w.Ht, Tpad + kLdPad, H, w.D, vcw + kLdPad, vcw, true, false, Tpad / BK, H, rows,
-                                             accumulate_dw ? (const float*)dWc : (const float*)nullptr, dWc, (uint16_t*)nullptr, H)
+                                             dw_mode == SKYRL_DW_FP32_ACCUMULATE ? (const float*)dWf : (const float*)nullptr, dWf,
+                                             dWb, H)
                                  : none;
     e = launch_bwd_chunk(s, dentropy != nullptr, DzArgs{}, 0, true, gh, gw);
     if (e != hipSuccess) return (int)e;

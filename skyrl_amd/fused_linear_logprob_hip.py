@@ -96,8 +96,8 @@ class LinearCrossEntropy(torch.autograd.Function):
             g = (dlogprobs.to(torch.float32) / T).expand(T).contiguous()
         q = None if dentropy is None else dentropy.reshape(-1).to(torch.float32).contiguous()
         d_hidden, d_weight = ops.lmhead_bwd_active_rows(hidden2, weight, labels1, row_lse, row_pz if q is not None else None,
-                                                        g, q, ctx.rcp_t, 0, want_dweight=ctx.needs_input_grad[1])
-        d_weight = None if d_weight is None else d_weight.to(weight.dtype)   # a frozen LM head takes no gradient
+                                                        g, q, ctx.rcp_t, 0, want_dweight=ctx.needs_input_grad[1],
+                                                        dweight_dtype=weight.dtype)   # None for a frozen LM head
         return d_hidden.view(ctx.original_hidden_shape), d_weight, None, None, None, None
 
 
@@ -150,7 +150,7 @@ class FusedLinearLogprobHip(torch.autograd.Function):
         else:
             g = grad_output.reshape(-1).to(torch.float32).contiguous()
         d_hidden, d_weight = ops.lmhead_bwd_active_rows(hidden_2d, weight_c, labels, row_lse, None, g, None, 1.0, 0,
-                                                        want_dweight=ctx.needs_input_grad[1])
-        # grad_hidden in the hidden dtype, grad_weight in the weight dtype (model_utils.py:381, 428); none for a frozen head.
-        d_weight = None if d_weight is None else d_weight.to(weight_c.dtype)
+                                                        want_dweight=ctx.needs_input_grad[1], dweight_dtype=weight_c.dtype)
+        # grad_hidden in the hidden dtype, grad_weight in the weight dtype (model_utils.py:381, 428), rounded in the GEMM
+        # epilogue; none for a frozen head.
         return d_hidden.reshape(B, S, H).to(ctx.hidden_dtype), d_weight, None, None, None, None, None, None

@@ -17,7 +17,7 @@ import torch
 
 from . import _lib
 
-__all__ = ["lmhead_fwd", "lmhead_bwd", "lmhead_bwd_hidden", "lmhead_bwd_active_rows", "fwd_workspace_bytes",
+__all__ = ["lmhead_fwd", "lmhead_bwd", "lmhead_bwd_bf16", "lmhead_bwd_hidden", "lmhead_bwd_active_rows", "fwd_workspace_bytes",
            "bwd_workspace_bytes"]
 
 
@@ -132,6 +132,37 @@ def lmhead_bwd(
     return d_hidden, d_weight
 
 
+@torch.library.custom_op("skyrl_amd::lmhead_bwd_bf16", mutates_args=())
+def lmhead_bwd_bf16(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    row_lse: torch.Tensor,
+    row_pz: Optional[torch.Tensor],
+    dlogprobs: torch.Tensor,
+    dentropy: Optional[torch.Tensor],
+    rcp_temperature: float,
+    vocab_chunk: int,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``(d_hidden bf16 [T,H], d_weight bf16 [V,H])``: the weight gradient leaves the GEMM epilogue already rounded to the
+    weight's dtype (what the autograd adapters hand back), with no fp32 ``[V, H]`` buffer and no cast pass."""
+    T, H, V = _check_operands(hidden, weight, labels)
+    dev = _require_device(hidden, weight, labels, row_lse, dlogprobs)
+    d_hidden = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    if T == 0:
+        return d_hidden, torch.zeros((V, H), dtype=torch.bfloat16, device=dev)
+    d_weight = torch.empty((V, H), dtype=torch.bfloat16, device=dev)
+    _bwd_into(_lib.load(), hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk, d_hidden,
+              d_weight, False)
+    return d_hidden, d_weight
+
+
+@lmhead_bwd_bf16.register_fake
+def _(hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk):
+    return (torch.empty_like(hidden, memory_format=torch.contiguous_format),
+            torch.empty(weight.shape, dtype=torch.bfloat16, device=weight.device))
+
+
 @torch.library.custom_op("skyrl_amd::lmhead_bwd_hidden", mutates_args=())
 def lmhead_bwd_hidden(
     hidden: torch.Tensor,
@@ -171,6 +202,7 @@ def lmhead_bwd_active_rows(
     vocab_chunk: int = 0,
     min_skip_fraction: float = 0.125,
     want_dweight: bool = True,
+    dweight_dtype: torch.dtype = torch.float32,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """``lmhead_bwd`` that first drops the tokens whose upstream gradients are all zero.
 
@@ -180,8 +212,11 @@ def lmhead_bwd_active_rows(
     backward GEMMs run on the remaining rows only: rows are gathered, the kernels run on the compact ``[T_active, H]``
     problem, and dHidden rows are scattered back into zeros.  Counting the active rows costs one host synchronisation; when
     fewer than ``min_skip_fraction`` of the rows would be dropped the dense path is used.  With ``want_dweight=False`` (the
-    weight takes no gradient) the dW product is skipped and ``None`` is returned in its place.
+    weight takes no gradient) the dW product is skipped and ``None`` is returned in its place; ``dweight_dtype`` is fp32 or
+    bf16 (rounded in the GEMM epilogue).
     """
+    if dweight_dtype not in (torch.float32, torch.bfloat16):
+        raise TypeError(f"d_weight is fp32 or bf16, not {dweight_dtype}")
     T = hidden.shape[0]
     active = dlogprobs != 0
     if dentropy is not None:
@@ -190,12 +225,12 @@ def lmhead_bwd_active_rows(
     n = int(idx.numel())
     def run(*args):
         if want_dweight:
-            return lmhead_bwd(*args)
+            return lmhead_bwd(*args) if dweight_dtype == torch.float32 else lmhead_bwd_bf16(*args)
         return lmhead_bwd_hidden(*args), None
 
     if n == 0:
         return torch.zeros_like(hidden, memory_format=torch.contiguous_format), (
-            torch.zeros(weight.shape, dtype=torch.float32, device=weight.device) if want_dweight else None)
+            torch.zeros(weight.shape, dtype=dweight_dtype, device=weight.device) if want_dweight else None)
     if T - n < min_skip_fraction * T:
         return run(hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk)
     take = lambda t: None if t is None else t.index_select(0, idx)  # noqa: E731
@@ -229,7 +264,8 @@ def _bwd_into(lib, hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy,
         st = lib.skyrl_lmhead_bwd(
             hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), labels.data_ptr(),
             row_lse.data_ptr(), _ptr(row_pz if dentropy is not None else None), dlogprobs.data_ptr(), _ptr(dentropy),
-            T, H, V, float(rcp_temperature), d_hidden.data_ptr(), _ptr(d_weight), int(bool(accumulate_dw)),
+            T, H, V, float(rcp_temperature), d_hidden.data_ptr(), _ptr(d_weight),
+            2 if (d_weight is not None and d_weight.dtype == torch.bfloat16) else int(bool(accumulate_dw)),
             int(vocab_chunk), ws.data_ptr(), ws_bytes, stream,
         )
     _lib.check(st, "skyrl_lmhead_bwd")
@@ -273,9 +309,10 @@ def _backward(ctx, d_logprobs, d_entropy, d_row_lse, d_row_pz):
     if ctx.want_entropy and d_entropy is not None:
         dent = d_entropy.to(torch.float32).contiguous()
     d_hidden, d_weight = lmhead_bwd_active_rows(hidden, weight, labels, row_lse, row_pz if dent is not None else None,
-                                                d_logprobs, dent, ctx.rcp_temperature, 0, want_dweight=ctx.needs_input_grad[1])
+                                                d_logprobs, dent, ctx.rcp_temperature, 0, want_dweight=ctx.needs_input_grad[1],
+                                                dweight_dtype=weight.dtype)
     # grad_weight is handed back in the weight's dtype, as the reference does (model_utils.py:428).
-    return d_hidden, None if d_weight is None else d_weight.to(weight.dtype), None, None, None
+    return d_hidden, d_weight, None, None, None
 
 
 lmhead_fwd.register_autograd(_backward, setup_context=_setup_context)

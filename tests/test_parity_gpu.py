@@ -1802,3 +1802,26 @@ def test_soft_ce_extreme_logits(cuda_device):
     err = (got.detach().cpu().double() - ref.detach()).abs()
     assert bool((err <= 1e-4 * ref.detach().abs() + 1e-3).all()), err.max().item()
     assert cos(d_hs.grad.float(), hs64.grad) >= GRAD_COS
+
+
+def test_weight_gradient_in_bf16_equals_the_rounded_fp32_one(cuda_device):
+    """SKYRL_DW_BF16: the GEMM epilogue rounds the fp32 sums to bf16 itself; bit-identical to casting the fp32 result, for one
+    and for several vocabulary chunks, through the functional op and the autograd adapter (which now never holds an fp32
+    [V, H] buffer)."""
+    T, H, V, t = 300, 128, 1000, 0.7
+    hidden, weight, labels, g, q = _rand(T, H, V, seed=43)
+    h, w, y, gd, qd = (x.to(cuda_device) for x in (hidden, weight, labels, g, q))
+    lp, ent, lse, pz = ops.lmhead_fwd(h, w, y, 1.0 / t, True)
+    for chunk in (0, 256):
+        dh32, dw32 = ops.lmhead_bwd(h, w, y, lse, pz, gd, qd, 1.0 / t, chunk)
+        dh16, dw16 = ops.lmhead_bwd_bf16(h, w, y, lse, pz, gd, qd, 1.0 / t, chunk)
+        assert dw16.dtype == torch.bfloat16 and torch.equal(dw16, dw32.to(torch.bfloat16)) and torch.equal(dh16, dh32)
+    hd, wd = h.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    out_lp, out_ent = linear_cross_entropy(hd, wd, y, t, "none", None)
+    ((out_lp * gd).sum() + (out_ent * qd).sum()).backward()
+    assert wd.grad.dtype == torch.bfloat16 and torch.equal(wd.grad, dw32.to(torch.bfloat16))
+    lib = _lib.load()
+    p = h.data_ptr()
+    ws = torch.empty(lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, 0), dtype=torch.uint8, device=cuda_device)
+    assert lib.skyrl_lmhead_bwd(p, H, w.data_ptr(), H, y.data_ptr(), lse.data_ptr(), None, gd.data_ptr(), None, T, H, V, 1.0,
+                                dh32.data_ptr(), dw32.data_ptr(), 3, 0, ws.data_ptr(), ws.numel(), None) == -5
