@@ -5,7 +5,7 @@
  * pointer is memory the caller owns (in practice a torch tensor's data_ptr()); the library never frees or
  * keeps it after the call returns.  All work is enqueued asynchronously on the HIP stream passed in
  * (hipStream_t as void*, NULL = the default stream).  The library allocates nothing: scratch comes in as
- * `workspace`, sized by the two *_workspace_bytes queries, so a caller can observe that no T x V buffer exists.
+ * `workspace`, sized by the *_workspace_bytes queries, so a caller can observe that no T x V buffer exists.
  *
  * Math (T tokens, H hidden, V vocab; z = (hidden . weight^T) * rcp_temperature):
  *     lse_t      = log sum_v exp z_tv
@@ -51,8 +51,11 @@ int skyrl_lmhead_version(void);
 /* Human-readable text for a status code returned by this library (never NULL). */
 const char* skyrl_lmhead_strerror(int status);
 
-/* Scratch needed by skyrl_lmhead_fwd: per-vocab-tile (max, sum-exp, sum z*exp) partials, 24 * T * ceil(V/256) bytes (T rounded up to a multiple of 64)
- * plus alignment slack.  (The reference allocates the same kind of buffers: `_max/_accu/_entropy_b [T, num_splits]`,
+/* Scratch needed by skyrl_lmhead_fwd: per-vocab-tile (max, sum-exp, sum z*exp) partials of one token block,
+ * 24 * min(T, 32768) * ceil(V/256) bytes (tokens rounded up to a multiple of 64) plus alignment slack.  The forward walks the
+ * tokens in blocks of 32768 and merges a block's partials before the next block overwrites them, so the scratch does not
+ * grow with T beyond one block (results are bit-identical to an unblocked run: block boundaries are tile boundaries).
+ * (The reference allocates the same kind of buffers for all of T: `_max/_accu/_entropy_b [T, num_splits]`,
  * fused_linear_logprob_triton.py:670-672.) */
 size_t skyrl_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V);
 

@@ -806,24 +806,25 @@ inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 constexpr int64_t kMaxExtent = (int64_t)1 << 30;
 
 // The two bf16 operands of every entry point: hidden rows [T, H] and weight rows [V, H].
+// hidden_in_blocks: the entry point walks the hidden rows in token blocks (each below 4 GiB), so only a block counts.
 int check_operands(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, int64_t T, int64_t H, int64_t V,
-                   float rcp_temperature) {
+                   float rcp_temperature, bool hidden_in_blocks = false) {
   if (!hidden || !weight) return SKYRL_LMHEAD_ERR_NULL;
   if (T < 1 || V < 1 || H < BK || H % BK != 0 || ldh < H || ldw < H) return SKYRL_LMHEAD_ERR_SHAPE;
   if (T > kMaxExtent || V > kMaxExtent || ldh > kMaxExtent || ldw > kMaxExtent) return SKYRL_LMHEAD_ERR_SHAPE;
   // The copy plan addresses an operand with 32-bit byte offsets: each operand (and each backward scratch matrix, which is
   // never larger than these two transposed) must stay below 4 GiB.
   const int64_t kMaxBytes = (int64_t)1 << 32;
-  if (T * ldh * 2 >= kMaxBytes || V * ldw * 2 >= kMaxBytes) return SKYRL_LMHEAD_ERR_SHAPE;
+  if ((hidden_in_blocks ? BN : T) * ldh * 2 >= kMaxBytes || V * ldw * 2 >= kMaxBytes) return SKYRL_LMHEAD_ERR_SHAPE;
   if (!aligned16(hidden) || !aligned16(weight) || ldh % 8 != 0 || ldw % 8 != 0) return SKYRL_LMHEAD_ERR_ALIGN;
   if (!(rcp_temperature > 0.f) || !isfinite(rcp_temperature)) return SKYRL_LMHEAD_ERR_ARG;
   return SKYRL_LMHEAD_OK;
 }
 
 int check_common(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
-                 int64_t H, int64_t V, float rcp_temperature) {
+                 int64_t H, int64_t V, float rcp_temperature, bool hidden_in_blocks = false) {
   if (!hidden || !weight || !labels) return SKYRL_LMHEAD_ERR_NULL;
-  const int st = check_operands(hidden, ldh, weight, ldw, T, H, V, rcp_temperature);
+  const int st = check_operands(hidden, ldh, weight, ldw, T, H, V, rcp_temperature, hidden_in_blocks);
   if (st == SKYRL_LMHEAD_ERR_SHAPE) return st;  // shape errors are reported before alignment errors, labels included
   if ((uintptr_t)labels & 7u) return SKYRL_LMHEAD_ERR_ALIGN;
   return st;
@@ -896,6 +897,67 @@ int64_t default_vocab_chunk(int64_t T, int64_t H, int64_t V) {
     if (vc >= Vpad || !fits) break;
   }
   return best_vc;
+}
+
+// Forward scratch: three arrays of per-part statistics for `tokens` tokens.
+size_t fwd_partials_bytes(int64_t tokens, int64_t V) {
+  const size_t nparts = (size_t)((V + BM - 1) / BM) * WAVES_M;
+  Carver c(nullptr);
+  c.take<float>(part_elems(nparts, tokens));
+  c.take<float>(part_elems(nparts, tokens));
+  c.take<float>(part_elems(nparts, tokens));
+  return (size_t)round_up((int64_t)c.off, 256);
+}
+
+// The forward walks the tokens in blocks: tokens are independent, so a block is a complete forward problem on a slice of
+// hidden / labels / outputs, and the partials of one block are merged before the next block overwrites them (launches on
+// one stream run in order).  The scratch is therefore sized by the block, not by T.  Block boundaries are multiples of the
+// 256-token tile, so every token sees the same tiles, in the same order, as in an unblocked run: results are bit-identical
+// for any block size.
+constexpr int64_t kFwdTokenBlock = 32768;
+
+// Tokens per block such that a block of hidden rows stays below the 4 GiB the copy plan can address.
+int64_t fwd_block_tokens(int64_t wanted, int64_t ld_hidden) {
+  const int64_t by_bytes = (((int64_t)1 << 32) - 1) / (ld_hidden * 2) / BN * BN;
+  int64_t b = wanted < by_bytes ? wanted : by_bytes;
+  return b < BN ? BN : b;
+}
+
+int fwd_token_blocks(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight, const int64_t* labels,
+                     int64_t T, int64_t H, int64_t V, float rcp_temperature, float* logprobs, float* entropy, float* row_lse,
+                     float* row_pz, void* scratch, int64_t block_tokens, hipStream_t s) {
+  const int tiles_m = (int)((V + BM - 1) / BM);
+  const size_t nparts = (size_t)tiles_m * WAVES_M;
+  const bool want_pz = entropy || row_pz;
+  const uint16_t* Wp = (const uint16_t*)weight;
+  for (int64_t t0 = 0; t0 < T; t0 += block_tokens) {
+    const int64_t Tb = (T - t0) < block_tokens ? (T - t0) : block_tokens;
+    const int tiles_n = (int)((Tb + BN - 1) / BN);
+    Carver c(scratch);
+    float* pmax = c.take<float>(part_elems(nparts, Tb));
+    float* psum = c.take<float>(part_elems(nparts, Tb));
+    float* ppz = c.take<float>(part_elems(nparts, Tb));
+    const uint16_t* Hp = (const uint16_t*)hidden + (size_t)t0 * (size_t)ld_hidden;
+    const dim3 grid((unsigned)(tiles_m * tiles_n)), block(NTHREADS);
+    {
+      Timed timed(kFwdTiles, s);
+      if (want_pz)
+        hipLaunchKernelGGL(lmhead_fwd_tiles<true>, grid, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)Tb, (int)H,
+                           (int)V, rcp_temperature, pmax, psum, ppz);
+      else
+        hipLaunchKernelGGL(lmhead_fwd_tiles<false>, grid, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)Tb, (int)H,
+                           (int)V, rcp_temperature, pmax, psum, ppz);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    Timed timed(kFwdMerge, s);
+    hipLaunchKernelGGL(lmhead_fwd_merge, dim3((unsigned)((Tb + kMergeTokens - 1) / kMergeTokens)), dim3(kMergeThreads), 0, s, pmax,
+                       psum, want_pz ? ppz : (float*)nullptr, (int)nparts, (int)Tb, Hp, (int)ld_hidden, Wp, (int)ld_weight,
+                       labels + t0, (int)H, (int)V, rcp_temperature, logprobs + t0, entropy ? entropy + t0 : (float*)nullptr,
+                       row_lse ? row_lse + t0 : (float*)nullptr, row_pz ? row_pz + t0 : (float*)nullptr);
+    if ((e = hipGetLastError()) != hipSuccess) return (int)e;
+  }
+  return SKYRL_LMHEAD_OK;
 }
 
 struct BwdWorkspace {
@@ -1033,12 +1095,7 @@ const char* skyrl_lmhead_strerror(int status) {
 size_t skyrl_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
   (void)H;
   if (T < 1 || V < 1 || T > kMaxExtent || V > kMaxExtent) return 0;
-  const size_t nparts = (size_t)((V + BM - 1) / BM) * WAVES_M;
-  Carver c(nullptr);
-  c.take<float>(part_elems(nparts, T));
-  c.take<float>(part_elems(nparts, T));
-  c.take<float>(part_elems(nparts, T));
-  return (size_t)round_up((int64_t)c.off, 256);
+  return fwd_partials_bytes(T < kFwdTokenBlock ? T : kFwdTokenBlock, V);
 }
 
 size_t skyrl_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t vocab_chunk) {
@@ -1052,40 +1109,13 @@ size_t skyrl_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t
 int skyrl_lmhead_fwd(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight, const int64_t* labels,
                      int64_t T, int64_t H, int64_t V, float rcp_temperature, float* logprobs, float* entropy,
                      float* row_lse, float* row_pz, void* workspace, size_t workspace_bytes, void* stream) {
-  int st = check_common(hidden, ld_hidden, weight, ld_weight, labels, T, H, V, rcp_temperature);
+  int st = check_common(hidden, ld_hidden, weight, ld_weight, labels, T, H, V, rcp_temperature, true);
   if (st) return st;
   if (!logprobs) return SKYRL_LMHEAD_ERR_NULL;
   if (!workspace || workspace_bytes < skyrl_lmhead_fwd_workspace_bytes(T, H, V)) return SKYRL_LMHEAD_ERR_WORKSPACE;
   if ((uintptr_t)workspace & 255u) return SKYRL_LMHEAD_ERR_ALIGN;
-
-  hipStream_t s = (hipStream_t)stream;
-  const int tiles_m = (int)((V + BM - 1) / BM), tiles_n = (int)((T + BN - 1) / BN);
-  const size_t nparts = (size_t)tiles_m * WAVES_M;
-  Carver c(workspace);
-  float* pmax = c.take<float>(part_elems(nparts, T));
-  float* psum = c.take<float>(part_elems(nparts, T));
-  float* ppz = c.take<float>(part_elems(nparts, T));
-  const bool want_pz = entropy || row_pz;
-  const uint16_t* Wp = (const uint16_t*)weight;
-  const uint16_t* Hp = (const uint16_t*)hidden;
-  const dim3 grid((unsigned)(tiles_m * tiles_n)), block(NTHREADS);
-  {
-    Timed timed(kFwdTiles, s);
-    if (want_pz)
-        hipLaunchKernelGGL(lmhead_fwd_tiles<true>, grid, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)T, (int)H,
-                         (int)V, rcp_temperature, pmax, psum, ppz);
-    else
-      hipLaunchKernelGGL(lmhead_fwd_tiles<false>, grid, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)T, (int)H,
-                         (int)V, rcp_temperature, pmax, psum, ppz);
-  }
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return (int)e;
-  Timed timed(kFwdMerge, s);
-  hipLaunchKernelGGL(lmhead_fwd_merge, dim3((unsigned)((T + kMergeTokens - 1) / kMergeTokens)), dim3(kMergeThreads), 0, s, pmax, psum,
-                     want_pz ? ppz : (float*)nullptr, (int)nparts, (int)T, Hp, (int)ld_hidden, Wp, (int)ld_weight, labels,
-                     (int)H, (int)V, rcp_temperature, logprobs, entropy, row_lse, row_pz);
-  e = hipGetLastError();
-  return e == hipSuccess ? SKYRL_LMHEAD_OK : (int)e;
+  return fwd_token_blocks(hidden, ld_hidden, weight, ld_weight, labels, T, H, V, rcp_temperature, logprobs, entropy, row_lse,
+                          row_pz, workspace, fwd_block_tokens(kFwdTokenBlock, ld_hidden), (hipStream_t)stream);
 }
 
 int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight, const int64_t* labels,
