@@ -43,6 +43,7 @@ extern "C" {
 #define SKYRL_LMHEAD_ERR_SHAPE (-2)     /* T, V < 1, H not a positive multiple of 64, a leading dimension < H, an operand of 4 GiB or more, a negative count */
 #define SKYRL_LMHEAD_ERR_ALIGN (-3)     /* a pointer is not 16-byte aligned or a leading dimension is not a multiple of 8 */
 #define SKYRL_LMHEAD_ERR_WORKSPACE (-4) /* workspace is NULL or smaller than the matching *_workspace_bytes() */
+#define SKYRL_LMHEAD_ERR_TOO_LARGE (-6) /* skyrl_lmhead_fwd_static_scratch only: V beyond SKYRL_LMHEAD_STATIC_SCRATCH_MAX_V */
 #define SKYRL_LMHEAD_ERR_ARG (-5)       /* rcp_temperature not finite and positive, vocab_chunk not a multiple of 256, or both sub-sequence arrays and a mask */
 
 /* ABI version of this header (bumped on any signature change). */
@@ -80,6 +81,26 @@ int skyrl_lmhead_fwd(const void* hidden, int64_t ld_hidden, const void* weight, 
                      const int64_t* labels, int64_t T, int64_t H, int64_t V, float rcp_temperature,
                      float* logprobs, float* entropy, float* row_lse, float* row_pz,
                      void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * The forward for callers that cannot allocate device memory and have no workspace to pass: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments, kernels and
+ * results (bit for bit) as skyrl_lmhead_fwd, but the partial statistics go into a fixed array of
+ * SKYRL_LMHEAD_STATIC_SCRATCH_BYTES (32 MiB) that lives in the library's own device image: every GPU the library runs on
+ * holds one until the process ends, and the call itself performs no hipMalloc / hipFree or any other allocating call.
+ * The tokens are walked in blocks whose partials fit that array (2304 tokens per block at V = 152064), so T is unlimited;
+ * a vocabulary so large that one 256-token tile does not fit, V > SKYRL_LMHEAD_STATIC_SCRATCH_MAX_V, is refused with
+ * SKYRL_LMHEAD_ERR_TOO_LARGE before anything is enqueued.  Nothing in the array has to start at zero (every partial is
+ * written before it is read).  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU -- two
+ * streams, two host threads -- race; calls on one stream are ordered and safe.
+ */
+#define SKYRL_LMHEAD_STATIC_SCRATCH_BYTES 33554432
+#define SKYRL_LMHEAD_STATIC_SCRATCH_MAX_V 1398016
+int skyrl_lmhead_fwd_static_scratch(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight,
+                                    const int64_t* labels, int64_t T, int64_t H, int64_t V, float rcp_temperature,
+                                    float* logprobs, float* entropy, float* row_lse, float* row_pz, void* stream);
+/* Size of that array, as compiled into the library (equals SKYRL_LMHEAD_STATIC_SCRATCH_BYTES). */
+size_t skyrl_lmhead_static_scratch_bytes(void);
 
 /*
  * Backward.  Same hidden / weight / labels as the forward call; row_lse, row_pz from it (row_pz may be NULL

@@ -22,6 +22,7 @@
 #include <stdint.h>
 
 #include <algorithm>
+#include <mutex>
 #include <vector>
 
 #include "../../include/skyrl_lmhead.h"
@@ -42,6 +43,12 @@ constexpr int kGroupM = LMHEAD_GROUP_M;
 constexpr int kLdPad = 64;
 
 __host__ __device__ inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+
+// Scratch of skyrl_lmhead_fwd_static_scratch, the entry point for callers that cannot allocate: one fixed array in every
+// device's memory, held until the process ends.  In host code this name is only a handle for hipGetSymbolAddress (see
+// static_scratch_of_current_device); kernels receive the looked-up address as an ordinary argument.
+constexpr size_t kStaticScratchBytes = SKYRL_LMHEAD_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char static_scratch[kStaticScratchBytes];
 
 // Partial statistics live in blocks of 64 tokens: [token block][part][64 tokens].  A wave of the tile kernel writes 64
 // contiguous bytes (16 tokens) of one part; the merge kernel reads a token block's parts as one contiguous stream, 256 bytes
@@ -960,6 +967,29 @@ int fwd_token_blocks(const void* hidden, int64_t ld_hidden, const void* weight, 
   return SKYRL_LMHEAD_OK;
 }
 
+// Address of this device's copy of the static scratch array.  Every device holds its own copy of a __device__ array at
+// its own address, so the address is looked up once per device, with that device current, and kept.
+constexpr int kMaxDevices = 64;
+void* g_static_scratch_ptr[kMaxDevices];
+std::mutex g_static_scratch_mutex;
+
+int static_scratch_of_current_device(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return SKYRL_LMHEAD_ERR_ARG;
+  std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+  if (!g_static_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(static_scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!p || ((uintptr_t)p & 255u)) return SKYRL_LMHEAD_ERR_ALIGN;
+    g_static_scratch_ptr[dev] = p;
+  }
+  *out = g_static_scratch_ptr[dev];
+  return SKYRL_LMHEAD_OK;
+}
+
 struct BwdWorkspace {
   uint16_t *Wt, *Ht, *D;
   float* dHacc;
@@ -1072,7 +1102,7 @@ hipError_t launch_softce_pack(hipStream_t s, const void* student, int64_t lds_, 
 
 extern "C" {
 
-int skyrl_lmhead_version(void) { return 12; }
+int skyrl_lmhead_version(void) { return 13; }
 
 const char* skyrl_lmhead_strerror(int status) {
   switch (status) {
@@ -1083,6 +1113,9 @@ const char* skyrl_lmhead_strerror(int status) {
              "packed-sequence calls: counts >= 0, rows == num_seqs with an attention mask";
     case SKYRL_LMHEAD_ERR_ALIGN: return "bad alignment: pointers must be 16-byte aligned, leading dimensions multiples of 8";
     case SKYRL_LMHEAD_ERR_WORKSPACE: return "workspace is NULL or too small";
+    case SKYRL_LMHEAD_ERR_TOO_LARGE:
+      return "too large for the entry point that uses the library's fixed scratch array: V exceeds "
+             "SKYRL_LMHEAD_STATIC_SCRATCH_MAX_V; use skyrl_lmhead_fwd with a caller-provided workspace";
     case SKYRL_LMHEAD_ERR_ARG:
       return "bad argument: rcp_temperature must be finite and > 0, vocab_chunk a multiple of 256; packed-sequence calls take "
              "sub-sequence arrays or an attention mask, not both";
@@ -1117,6 +1150,23 @@ int skyrl_lmhead_fwd(const void* hidden, int64_t ld_hidden, const void* weight, 
   return fwd_token_blocks(hidden, ld_hidden, weight, ld_weight, labels, T, H, V, rcp_temperature, logprobs, entropy, row_lse,
                           row_pz, workspace, fwd_block_tokens(kFwdTokenBlock, ld_hidden), (hipStream_t)stream);
 }
+
+int skyrl_lmhead_fwd_static_scratch(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight,
+                                    const int64_t* labels, int64_t T, int64_t H, int64_t V, float rcp_temperature,
+                                    float* logprobs, float* entropy, float* row_lse, float* row_pz, void* stream) {
+  int st = check_common(hidden, ld_hidden, weight, ld_weight, labels, T, H, V, rcp_temperature, true);
+  if (st) return st;
+  if (!logprobs) return SKYRL_LMHEAD_ERR_NULL;
+  // Token block: the most 256-token tiles whose partials fit the static array.
+  const int64_t block = (int64_t)(kStaticScratchBytes / fwd_partials_bytes(BN, V)) * BN;
+  if (V > SKYRL_LMHEAD_STATIC_SCRATCH_MAX_V || block < BN) return SKYRL_LMHEAD_ERR_TOO_LARGE;
+  void* scratch_ptr = nullptr;
+  if ((st = static_scratch_of_current_device(&scratch_ptr)) != SKYRL_LMHEAD_OK) return st;
+  return fwd_token_blocks(hidden, ld_hidden, weight, ld_weight, labels, T, H, V, rcp_temperature, logprobs, entropy, row_lse,
+                          row_pz, scratch_ptr, fwd_block_tokens(block, ld_hidden), (hipStream_t)stream);
+}
+
+size_t skyrl_lmhead_static_scratch_bytes(void) { return kStaticScratchBytes; }
 
 int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight, const int64_t* labels,
                      const float* row_lse, const float* row_pz, const float* dlogprobs, const float* dentropy, int64_t T,

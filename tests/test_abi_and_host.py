@@ -44,8 +44,8 @@ def test_library_is_in_tree_and_has_no_torch_dependency():
 
 
 def test_strerror_table():
-    for code in (0, -1, -2, -3, -4, -5):
-        assert _lib.strerror(code)
+    for code in (0, -1, -2, -3, -4, -5, -6):
+        assert _lib.strerror(code) and "unknown" not in _lib.strerror(code)
     assert "unknown" in _lib.strerror(-99)
 
 
@@ -89,6 +89,23 @@ def test_forward_argument_errors_are_reported_before_any_launch():
     assert _call_fwd(lib, rt=0.0) == -5
     assert _call_fwd(lib, rt=float("inf")) == -5
     assert _call_fwd(lib, rt=float("nan")) == -5
+
+
+def test_static_scratch_forward_argument_errors():
+    """The entry point without a workspace checks its operands like the ordinary forward, and its size limit, on the host."""
+    lib = _lib.load()
+
+    def call(hidden=0x1000, weight=0x2000, labels=0x3000, lp=0x4000, T=256, H=128, V=1024, ldh=None, ldw=None, rt=1.0):
+        return lib.skyrl_lmhead_fwd_static_scratch(hidden, ldh or H, weight, ldw or H, labels, T, H, V, rt, lp, None, None, None,
+                                                   None)
+
+    assert lib.skyrl_lmhead_static_scratch_bytes() == 33554432
+    assert call(hidden=None) == -1 and call(lp=None) == -1
+    assert call(H=100, ldh=104, ldw=104) == -2 and call(T=0) == -2
+    assert call(hidden=0x1008) == -3
+    assert call(rt=0.0) == -5
+    assert call(V=1398017, H=64) == -6  # a 256-token tile of partials no longer fits the 32 MiB array
+    assert call(V=300000, H=8192) == -2  # the weight limit is reported first
 
 
 def test_backward_argument_errors():
