@@ -54,7 +54,10 @@ class LinearCrossEntropy(torch.autograd.Function):
         temperature: typing.Optional[float] = 1.0,
         reduction: typing.Optional[str] = "none",
         dist_process_group: typing.Optional[dist.ProcessGroup] = None,
+        want_entropy: bool = True,
     ):
+        """``want_entropy`` (an extension; the reference always computes the entropy): with ``False`` the sum p*z accumulation is
+        skipped, the second result is ``None`` and the backward runs the kernel variant without the entropy-gradient term."""
         assert isinstance(temperature, float), f"temperature must be a float, but got {type(temperature)}"
         assert isinstance(reduction, str), f"reduction must be a str, but got {type(reduction)}"
         reduction = reduction.lower()
@@ -67,10 +70,14 @@ class LinearCrossEntropy(torch.autograd.Function):
         hidden2 = hidden.reshape(-1, hidden.shape[-1])
         labels1 = labels.reshape(-1)
         assert hidden2.shape[0] == labels1.shape[0]
+        labels1 = labels1.to(torch.int64).contiguous()  # what the kernel reads is what the backward gets back
         rcp_t = 1.0 / temperature
         with torch.no_grad():
-            logprobs, entropy, row_lse, row_pz = ops.lmhead_fwd(hidden2, weight, labels1.contiguous(), rcp_t, True)
+            logprobs, entropy, row_lse, row_pz = ops.lmhead_fwd(hidden2, weight, labels1, rcp_t, bool(want_entropy))
         ctx.save_for_backward(hidden2, weight, labels1, row_lse, row_pz)
+        # An output nobody uses arrives in backward as None, not as a tensor of zeros: an unused entropy then costs nothing.
+        ctx.set_materialize_grads(False)
+        ctx.want_entropy = bool(want_entropy)
         ctx.original_hidden_shape = original_hidden_shape
         ctx.reduction = reduction
         ctx.rcp_t = rcp_t
@@ -79,7 +86,7 @@ class LinearCrossEntropy(torch.autograd.Function):
             logprobs = logprobs.sum()
         elif reduction == "mean":
             logprobs = logprobs.mean()
-        return logprobs, entropy
+        return logprobs, (entropy if want_entropy else None)
 
     @staticmethod
     def backward(ctx, dlogprobs: torch.Tensor, dentropy: torch.Tensor):  # type: ignore[override]
@@ -94,11 +101,11 @@ class LinearCrossEntropy(torch.autograd.Function):
             g = dlogprobs.to(torch.float32).expand(T).contiguous()
         else:
             g = (dlogprobs.to(torch.float32) / T).expand(T).contiguous()
-        q = None if dentropy is None else dentropy.reshape(-1).to(torch.float32).contiguous()
+        q = None if (dentropy is None or not ctx.want_entropy) else dentropy.reshape(-1).to(torch.float32).contiguous()
         d_hidden, d_weight = ops.lmhead_bwd_active_rows(hidden2, weight, labels1, row_lse, row_pz if q is not None else None,
                                                         g, q, ctx.rcp_t, 0, want_dweight=ctx.needs_input_grad[1],
                                                         dweight_dtype=weight.dtype)   # None for a frozen LM head
-        return d_hidden.view(ctx.original_hidden_shape), d_weight, None, None, None, None
+        return d_hidden.view(ctx.original_hidden_shape), d_weight, None, None, None, None, None
 
 
 linear_cross_entropy = LinearCrossEntropy.apply
@@ -125,8 +132,8 @@ class FusedLinearLogprobHip(torch.autograd.Function):
         # Targets outside [vocab_start_index, vocab_end_index) get a label that matches no column: forward 0, backward keeps
         # -softmax * grad (fused_linear_logprob_triton.py:1876-1878, 1898-1905, 1929-1931).
         target_mask = (target < vocab_start_index) | (target >= vocab_end_index)
-        labels = torch.where(target_mask, _OOV_LABEL_SENTINEL, target - vocab_start_index).to(torch.int64).reshape(-1)
-        labels = labels.contiguous()
+        target = target.to(torch.int64)  # int32 ids: the sentinel below does not fit their dtype
+        labels = torch.where(target_mask, _OOV_LABEL_SENTINEL, target - vocab_start_index).reshape(-1).contiguous()
         # The kernel needs 2-D operands with matching dtypes: hidden follows the weight (model_utils.py:328-333).
         hidden_2d = hidden.reshape(B * S, H).to(weight.dtype).contiguous()
         weight_c = weight.contiguous()
@@ -134,6 +141,7 @@ class FusedLinearLogprobHip(torch.autograd.Function):
 
         with torch.no_grad():
             logprobs, _, row_lse, _ = ops.lmhead_fwd(hidden_2d, weight_c, labels, 1.0, False)
+        ctx.set_materialize_grads(False)
         if not inference_only:
             ctx.save_for_backward(hidden_2d, weight_c, labels, row_lse)
             ctx.shape = (B, S, H)

@@ -71,13 +71,15 @@ def _fused_lm_head_logprob_apply(
     _require_single_shard(tp_group, "_fused_lm_head_logprob_apply")
     B, S, H = hidden.shape
     target_mask = (target < vocab_start_index) | (target >= vocab_end_index)
-    labels = torch.where(target_mask, torch.iinfo(torch.int64).max, target - vocab_start_index).to(torch.int64)
+    target = target.to(torch.int64)
+    labels = torch.where(target_mask, torch.iinfo(torch.int64).max, target - vocab_start_index)
     hidden_c = hidden.to(weight.dtype)
+    # log-probabilities only: no entropy is accumulated in the forward, none differentiated in the backward
     if inference_only:
         with torch.no_grad():
-            logprobs, _ = linear_cross_entropy(hidden_c, weight.contiguous(), labels, float(temperature), "none", None)
+            logprobs, _ = linear_cross_entropy(hidden_c, weight.contiguous(), labels, float(temperature), "none", None, False)
     else:
-        logprobs, _ = linear_cross_entropy(hidden_c, weight.contiguous(), labels, float(temperature), "none", None)
+        logprobs, _ = linear_cross_entropy(hidden_c, weight.contiguous(), labels, float(temperature), "none", None, False)
     return logprobs.reshape(B, S)
 
 

@@ -257,7 +257,9 @@ def _bwd_into(lib, hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy,
             raise ValueError(f"{name} must be a contiguous fp32 tensor of shape [{T}], got {t.dtype} {tuple(t.shape)}")
     ws_bytes = int(lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, int(vocab_chunk)))
     if ws_bytes == 0:
-        raise ValueError(f"bad vocab_chunk {vocab_chunk}: must be 0 (library default) or a multiple of 256")
+        if int(vocab_chunk) < 0 or int(vocab_chunk) % 256 != 0:
+            raise ValueError(f"bad vocab_chunk {vocab_chunk}: must be 0 (library default) or a multiple of 256")
+        raise ValueError(f"no backward workspace for T={T}, H={H}, V={V}: every extent must be at least 1")
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
@@ -280,6 +282,8 @@ def lmhead_bwd_accumulate(hidden, weight, labels, row_lse, row_pz, dlogprobs, de
     if d_weight_accum.dtype != torch.float32 or d_weight_accum.shape != (V, H) or not d_weight_accum.is_contiguous():
         raise ValueError(f"d_weight_accum must be contiguous fp32 [{V},{H}]")
     d_hidden = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    if T == 0:  # an empty micro-batch adds nothing
+        return d_hidden
     _bwd_into(_lib.load(), hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk,
               d_hidden, d_weight_accum, True)
     return d_hidden
@@ -297,9 +301,14 @@ def _setup_context(ctx, inputs, output):
     ctx.save_for_backward(hidden, weight, labels, row_lse, row_pz)
     ctx.rcp_temperature = rcp_temperature
     ctx.want_entropy = want_entropy
+    ctx.set_materialize_grads(False)  # unused outputs arrive as None in _backward
 
 
 def _backward(ctx, d_logprobs, d_entropy, d_row_lse, d_row_pz):
+    if d_row_lse is not None or d_row_pz is not None:
+        # row_lse and row_pz are what the backward kernel takes back, not differentiable results: a loss built on them
+        # (a z-loss on the log-sum-exp, say) would silently get no gradient.
+        raise NotImplementedError("skyrl_amd::lmhead_fwd: row_lse and row_pz carry no gradient; only logprobs and entropy do")
     hidden, weight, labels, row_lse, row_pz = ctx.saved_tensors
     T = hidden.shape[0]
     if d_logprobs is None:

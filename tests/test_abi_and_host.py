@@ -213,8 +213,9 @@ def test_signatures_mirror_the_reference():
     assert list(inspect.signature(FusedLinearLogprobHip.forward).parameters) == [
         "ctx", "hidden", "weight", "target", "vocab_start_index", "vocab_end_index", "chunk_size", "tp_group", "inference_only"]
     # LinearCrossEntropy.forward (fused_linear_logprob_triton.py:1763-1775)
-    assert list(inspect.signature(LinearCrossEntropy.forward).parameters) == [
-        "ctx", "hidden", "weight", "labels", "temperature", "reduction", "dist_process_group"]
+    lce = inspect.signature(LinearCrossEntropy.forward).parameters
+    assert list(lce)[:7] == ["ctx", "hidden", "weight", "labels", "temperature", "reduction", "dist_process_group"]
+    assert list(lce)[7:] == ["want_entropy"] and lce["want_entropy"].default is True  # one trailing optional extension
     # model_utils.py:713-725
     dense = inspect.signature(model_utils.from_parallel_hidden_to_logprobs).parameters
     assert list(dense)[:11] == [
