@@ -34,10 +34,23 @@ if ROOT not in sys.path:
 PEAK_BF16_DENSE_FLOPS = 2.5e15  # MI355X dense bf16 MFMA
 METRIC = "fused LM-head fwd+bwd tokens/sec on 1 MI355X; % bf16 MFMA peak"
 
-# Bytes beyond L2 per lmhead_bwd_chunk launch from two `rocprofv3 --pmc` passes (FETCH_SIZE, then WRITE_SIZE), each scaled by what
-# the same counter reads for the 1 GiB copy of --copy-probe (x2048 and x1024 bytes per count).  Not measurable live; None for
-# workloads that have not been profiled.  Keyed by config name.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"qwen2.5-7b-fwdbwd": 12781769720}
+def measured_traffic(config_name: str, kernel: str):
+    """Bytes beyond L2 per launch of ``kernel`` in workload ``config_name``, or None when that workload has not been profiled.
+
+    Not measurable live: it comes from two ``rocprofv3 --pmc`` passes (FETCH_SIZE, then WRITE_SIZE), each scaled by what the
+    same counter reads for the 1 GiB copy of --copy-probe.  The summary of those passes under profiles/ ends with one line per
+    kernel, ``traffic_bytes_per_launch <workload> <kernel> <bytes>``; this reads it back, so the figure in the benchmark line
+    changes when, and only when, the profile is regenerated.  Returns ``(bytes, file name)``.
+    """
+    import glob
+
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*hbm_traffic*.txt"))):
+        with open(path) as f:
+            for line in f:
+                parts = line.split()
+                if len(parts) == 4 and parts[0] == "traffic_bytes_per_launch" and parts[1] == config_name and parts[2] == kernel:
+                    return int(float(parts[3])), os.path.basename(path)
+    return None, None
 
 
 def cpu_baseline(cfg, sample_tokens: int):
@@ -222,6 +235,7 @@ def main() -> int:
         k = kernels["lmhead_fwd_tiles"]
         dom_name, dom_ms, dom_launches, dom_flop = "lmhead_fwd_tiles", k["ms_per_step"], k["launches_per_step"], 2.0 * T * V * H
     achieved = dom_flop / (dom_ms * 1e-3) / 1e12
+    traffic, traffic_source = measured_traffic(cfg.name, dom_name)
     roofline = {
         "kernel": dom_name,
         "bound": "mfma",
@@ -229,7 +243,8 @@ def main() -> int:
         "peak": PEAK_BF16_DENSE_FLOPS / 1e12,
         "unit": "TFLOP/s",
         "frac": achieved / (PEAK_BF16_DENSE_FLOPS / 1e12),
-        "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(cfg.name),
+        "traffic": traffic,
+        "traffic_source": traffic_source,
         "flop_per_launch": dom_flop / dom_launches,
         "avg_launch_ms": dom_ms / dom_launches,
         "launches_per_step": dom_launches,

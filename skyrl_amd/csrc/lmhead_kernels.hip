@@ -26,6 +26,7 @@
 #include <vector>
 
 #include "../../include/skyrl_lmhead.h"
+#include "../../include/skyrl_lmhead_bench.h"
 #include "gemm_core.hpp"
 
 using namespace lmhead;

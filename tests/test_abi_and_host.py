@@ -14,6 +14,7 @@ from skyrl_amd.fused_linear_logprob_hip import FusedLinearLogprobHip, LinearCros
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "skyrl_lmhead.h")
+BENCH_HEADER = os.path.join(ROOT, "include", "skyrl_lmhead_bench.h")  # measurement aids, no reference counterpart
 
 
 def _read(path):
@@ -21,8 +22,8 @@ def _read(path):
         return f.read()
 
 
-def _declared_functions():
-    text = _read(HEADER)
+def _declared_functions(*headers):
+    text = "".join(_read(h) for h in (headers or (HEADER, BENCH_HEADER)))
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(skyrl_(?:lmhead|ppo|packed|approx|masked|actor|softce)_\w+)\s*\(", text)))
 
