@@ -40,7 +40,7 @@ extern "C" {
 
 #define SKYRL_LMHEAD_OK 0
 #define SKYRL_LMHEAD_ERR_NULL (-1)      /* a required pointer is NULL, or only some of seg_row / seg_col / seg_len are given */
-#define SKYRL_LMHEAD_ERR_SHAPE (-2)     /* T, V < 1, H not a positive multiple of 64, a leading dimension < H, an operand of 4 GiB or more, a negative count */
+#define SKYRL_LMHEAD_ERR_SHAPE (-2)     /* T, V < 1, H not a positive multiple of 64, a leading dimension < H, a weight (or a 32768-token block of hidden rows) of 4 GiB or more, a negative count */
 #define SKYRL_LMHEAD_ERR_ALIGN (-3)     /* a pointer is not 16-byte aligned or a leading dimension is not a multiple of 8 */
 #define SKYRL_LMHEAD_ERR_WORKSPACE (-4) /* workspace is NULL or smaller than the matching *_workspace_bytes() */
 #define SKYRL_LMHEAD_ERR_TOO_LARGE (-6) /* skyrl_lmhead_fwd_static_scratch only: V beyond SKYRL_LMHEAD_STATIC_SCRATCH_MAX_V */
@@ -60,12 +60,13 @@ const char* skyrl_lmhead_strerror(int status);
  * fused_linear_logprob_triton.py:670-672.) */
 size_t skyrl_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V);
 
-/* Scratch needed by skyrl_lmhead_bwd for a given vocab chunk width (0 = library default):
- * hidden^T bf16 [H, T'+64], fp32 dHidden partial sums (T' x H' values, kept in the kernel's accumulator order between
- * chunks), one bf16 dz panel [T', chunk+64] and, only when V is not a multiple of 64, weight^T bf16 [H, V'+64] (otherwise
- * the weight is read where it is)
- * (T', V', H' = T, V, H rounded up to 256; the 64 extra elements keep row pitches off powers of two).
- * Nothing in it scales with T * V.
+/* Scratch needed by skyrl_lmhead_bwd for a given vocab chunk width (0 = library default).  The backward walks the tokens in
+ * blocks of T_b = min(T, 32768) and every scratch matrix is sized by the block:
+ * hidden^T bf16 [H, T_b'+64], fp32 dHidden partial sums (T_b' x H' values, kept in the kernel's accumulator order between
+ * chunks), one bf16 dz panel [T_b', chunk+64] and, only when V is not a multiple of 64, weight^T bf16 [H, V'+64] (otherwise
+ * the weight is read where it is); for T > 32768 also one fp32 [V, H] matrix in which SKYRL_DW_BF16 sums dW over the blocks
+ * (T_b', V', H' = T_b, V, H rounded up to 256; the 64 extra elements keep row pitches off powers of two).
+ * The default chunk keeps the panel at or below 1.5 GiB, so nothing here grows with T * V.
  * (Stands in for the `d_logits [T, 9504]` scratch of the reference's default backward,
  * fused_linear_logprob_triton.py:1689-1748.) */
 size_t skyrl_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t vocab_chunk);
@@ -124,6 +125,26 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
                      int64_t T, int64_t H, int64_t V, float rcp_temperature,
                      void* d_hidden, void* d_weight, int dw_mode, int64_t vocab_chunk,
                      void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * The backward on the tokens that have an upstream gradient.  A token with dlogprobs == 0 (and dentropy == 0) has a zero dz
+ * row: it adds nothing to d_weight and its d_hidden row is zero.  In RL micro-batches those are the prompt and padding tokens
+ * the loss mask removes (loss_mask in workers/megatron/megatron_model_wrapper.py:607-985), often more than half of the batch; the
+ * reference runs its three backward GEMMs over them all the same (model_utils.py:383-426).  This entry point compacts them
+ * away on the device: a small kernel lists the active tokens and counts them, their hidden rows and per-token inputs are
+ * gathered into the workspace, the kernels of skyrl_lmhead_bwd run on a grid sized for T whose tiles beyond the device-side
+ * count return at once, and the d_hidden rows are scattered back (zero rows for the inactive tokens).  The host never learns
+ * the count: no synchronisation, and the call can be captured in a HIP graph.  Arguments and results as skyrl_lmhead_bwd
+ * (d_weight is bit-identical to what skyrl_lmhead_bwd computes on the compacted inputs; summing fewer zero rows may differ
+ * from the dense result in the last bit); the workspace is larger by the gathered copies, 4 * T * H + 28 * T bytes.
+ */
+size_t skyrl_lmhead_bwd_active_rows_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t vocab_chunk);
+int skyrl_lmhead_bwd_active_rows(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight,
+                                 const int64_t* labels, const float* row_lse, const float* row_pz,
+                                 const float* dlogprobs, const float* dentropy,
+                                 int64_t T, int64_t H, int64_t V, float rcp_temperature,
+                                 void* d_hidden, void* d_weight, int dw_mode, int64_t vocab_chunk,
+                                 void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * The consumer one step after the log-probabilities: the policy loss and its gradient with respect to the

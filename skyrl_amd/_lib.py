@@ -11,7 +11,7 @@ import os
 import threading
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libskyrl_lmhead.so")
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 _c_i64 = ctypes.c_int64
 _c_p = ctypes.c_void_p
@@ -33,6 +33,12 @@ SIGNATURES = {
     ),
     "skyrl_lmhead_static_scratch_bytes": (ctypes.c_size_t, []),
     "skyrl_lmhead_bwd": (
+        ctypes.c_int,
+        [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, ctypes.c_float, _c_p, _c_p,
+         ctypes.c_int, _c_i64, _c_p, ctypes.c_size_t, _c_p],
+    ),
+    "skyrl_lmhead_bwd_active_rows_workspace_bytes": (ctypes.c_size_t, [_c_i64, _c_i64, _c_i64, _c_i64]),
+    "skyrl_lmhead_bwd_active_rows": (
         ctypes.c_int,
         [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, ctypes.c_float, _c_p, _c_p,
          ctypes.c_int, _c_i64, _c_p, ctypes.c_size_t, _c_p],

@@ -293,13 +293,17 @@ struct DzArgs {
   int vc0, tiles_m, tiles_n;  // first vocab row of the chunk; tiles of the chunk panel along vocab and tokens
   uint16_t* D;                // [tiles_n * 256, ldd]  dz, token-major
   int ldd;
+  // When not NULL: the number of tokens, <= T, as a value in device memory (what a compaction kernel counted).  T then
+  // only sizes the grid: token tiles at or beyond the device-side count return at once.
+  const int* T_dev;
 };
 
 template <bool ENTGRAD>
 __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
   const uint16_t* __restrict__ W = z.W;
   const uint16_t* __restrict__ Hd = z.Hd;
-  const int ldw = z.ldw, ldh = z.ldh, T = z.T, H = z.H, V = z.V, vc0 = z.vc0, ldd = z.ldd;
+  const int ldw = z.ldw, ldh = z.ldh, H = z.H, V = z.V, vc0 = z.vc0, ldd = z.ldd;
+  const int T = z.T_dev ? __builtin_amdgcn_readfirstlane(*z.T_dev) : z.T;
   const float rcp_temp = z.rcp_temp;
   const int64_t* __restrict__ labels = z.labels;
   const float* __restrict__ row_lse = z.row_lse;
@@ -309,6 +313,7 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
   uint16_t* __restrict__ D = z.D;
   int tm, tn;
   tile_coords(id, z.tiles_m, z.tiles_n, kGroupM, tm, tn);
+  if (tn * BN >= T) return;  // only with a device-side count: this token tile holds no token (uniform over the workgroup)
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
@@ -574,23 +579,40 @@ struct GemmArgs {
   // per lane and 1 KiB contiguous per wave instruction, with no address arithmetic beyond a constant offset.
   const float* Pin;
   float* Pout;
+  // When not NULL: a token count in device memory that replaces one extent of the problem, chosen by t_role: the rows M
+  // (kTokensOnM), the columns N (kTokensOnN) or the contraction length, nk = ceil(count / 64) (kTokensOnK).  The host-side
+  // value of that extent is an upper bound that sizes the grid and the scratch; tiles beyond the count return at once.
+  const int* T_dev;
+  int t_role;
 };
+enum { kTokensOnM = 1, kTokensOnN = 2, kTokensOnK = 3 };
 
 // BKM: the B operand is K-major.  The two variants are separate instantiations of the whole tile (mainloop and
 // epilogue) so that their accumulators never meet at a join, where the register allocator would shuffle all 256 of them.
 template <bool BKM>
 __device__ __forceinline__ void gemm_tile(const GemmArgs& p, int bid, char* lds) {
-  const int M = p.M, N = p.N;
-  const int tiles_m = (M + BM - 1) / BM;
+  int M = p.M, N = p.N, nk = p.nk;
+  const int tiles_m = (M + BM - 1) / BM;  // of the host-side extents: they define the grid and the partial-sum layout
   const int tiles_n = (N + BN - 1) / BN;
   int tm, tn;
   tile_coords(bid, tiles_m, tiles_n, kGroupM, tm, tn);
+  if (p.T_dev) {
+    const int count = __builtin_amdgcn_readfirstlane(*p.T_dev);
+    if (p.t_role == kTokensOnM) M = count;
+    else if (p.t_role == kTokensOnN) N = count;
+    else nk = (count + BK - 1) / BK;
+    if (tm * BM >= M || tn * BN >= N) return;  // a tile without tokens (uniform over the workgroup)
+    // Nothing to contract: C += 0 needs no work; a C that is overwritten or converted still goes through the epilogue.
+    if (nk == 0 && !p.Cb && p.Cin == p.Cf) return;
+  }
   Operand a{p.A, p.lda, tm * BM, p.a_rows};
   Operand b{p.B, p.ldb, tn * BN, p.b_rows};
   acc_t acc;
   zero_acc(acc);
-  prefetch_first_tiles<BKM>(a, b, 0, p.nk, lds);
-  mainloop<BKM>(a, b, 0, p.nk, lds, acc);
+  if (nk > 0) {
+    prefetch_first_tiles<BKM>(a, b, 0, nk, lds);
+    mainloop<BKM>(a, b, 0, nk, lds, acc);
+  }
 
   const float* __restrict__ Cin = p.Cin;
   float* __restrict__ Cf = p.Cf;
@@ -715,9 +737,12 @@ __global__ __launch_bounds__(NTHREADS) void mfma_probe(const bf16x8* __restrict_
 }
 
 // dst[c, r] = src[r, c] for r < R, c < C;  dst[c, r] = 0 for R <= r < Rpad.  bf16 bits, 64 x 64 tiles.
+// R_dev (may be NULL): the number of valid source rows as a value in device memory, <= R.
 __global__ __launch_bounds__(256) void transpose_bf16(const uint16_t* __restrict__ src, int lds_src, int R, int C,
-                                                      uint16_t* __restrict__ dst, int ld_dst, int Rpad) {
+                                                      uint16_t* __restrict__ dst, int ld_dst, int Rpad,
+                                                      const int* __restrict__ R_dev) {
   __shared__ uint16_t tile[64][66];
+  if (R_dev) R = *R_dev;
   const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
   const int tid = threadIdx.x;
 #pragma unroll
@@ -759,17 +784,105 @@ __global__ __launch_bounds__(256) void transpose_bf16(const uint16_t* __restrict
 }
 
 // ------------------------------------------------------------------------------------------------------------
+// Row compaction for the backward.  A token whose upstream gradients are both zero has a zero dz row: it adds nothing to
+// dW and its dHidden row is zero.  In RL micro-batches those are the prompt and padding tokens the loss mask removes, often
+// more than half of the batch.  Three small kernels let the backward run on the remaining rows without the host ever
+// learning how many there are (no synchronisation, so the call can be captured in a HIP graph):
+//   compact_active_rows   one workgroup: idx[i] = i-th token with g != 0 or q != 0 (ascending), counts[0] = their number n,
+//                         counts[1 + b] = how many of them fall into block b of `block` compacted rows
+//   gather_active_rows    compacted copies of hidden rows and of the per-token inputs; zero dHidden rows for the inactive
+//   scatter_active_rows   dHidden rows of the compacted problem back to their tokens
+// The GEMM kernels take the counts from device memory (T_dev) and run on the static upper-bound grid.
+// ------------------------------------------------------------------------------------------------------------
+constexpr int kCompactThreads = 1024;
+
+__global__ __launch_bounds__(kCompactThreads) void compact_active_rows(const float* __restrict__ g, const float* __restrict__ q,
+                                                                       int T, int block, int nblocks, int* __restrict__ idx,
+                                                                       int* __restrict__ counts) {
+  __shared__ int wave_sum[kCompactThreads / 64];
+  __shared__ int carry;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (tid == 0) carry = 0;
+  __syncthreads();
+  for (int t0 = 0; t0 < T; t0 += kCompactThreads) {
+    const int t = t0 + tid;
+    const bool active = t < T && (g[t] != 0.f || (q && q[t] != 0.f));
+    const unsigned long long ballot = __ballot(active);
+    const int before = __popcll(ballot & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_sum[wave] = __popcll(ballot);
+    __syncthreads();
+    int base = carry;
+    for (int w = 0; w < wave; ++w) base += wave_sum[w];
+    if (active) idx[base + before] = t;
+    __syncthreads();
+    if (tid == 0) {
+      int total = 0;
+      for (int w = 0; w < kCompactThreads / 64; ++w) total += wave_sum[w];
+      carry += total;
+    }
+    __syncthreads();
+  }
+  const int n = carry;
+  for (int b = tid; b <= nblocks; b += kCompactThreads) {
+    if (b == 0) {
+      counts[0] = n;
+    } else {
+      const long long left = (long long)n - (long long)(b - 1) * block;
+      counts[b] = left < 0 ? 0 : (left > block ? block : (int)left);
+    }
+  }
+}
+
+// One workgroup per row r < T: as compacted row r (when r < n) it copies the inputs of token idx[r]; as token r it clears
+// d_hidden[r] -- active tokens get their row from scatter_active_rows afterwards.
+__global__ __launch_bounds__(256) void gather_active_rows(const int* __restrict__ idx, const int* __restrict__ counts,
+                                                          const uint16_t* __restrict__ hidden, int ldh, int H,
+                                                          const int64_t* __restrict__ labels, const float* __restrict__ lse,
+                                                          const float* __restrict__ pz, const float* __restrict__ g,
+                                                          const float* __restrict__ q, uint16_t* __restrict__ hidden_c,
+                                                          int64_t* __restrict__ labels_c, float* __restrict__ lse_c,
+                                                          float* __restrict__ pz_c, float* __restrict__ g_c,
+                                                          float* __restrict__ q_c, uint16_t* __restrict__ d_hidden) {
+  const int r = blockIdx.x;
+  uint16_t* zero_row = d_hidden + (size_t)r * (size_t)H;
+  for (int c = threadIdx.x * 8; c < H; c += 256 * 8) *(uint4*)(zero_row + c) = make_uint4(0, 0, 0, 0);
+  if (r >= counts[0]) return;
+  const int t = idx[r];
+  const uint16_t* src = hidden + (size_t)t * (size_t)ldh;
+  uint16_t* dst = hidden_c + (size_t)r * (size_t)H;
+  for (int c = threadIdx.x * 8; c < H; c += 256 * 8) *(uint4*)(dst + c) = *(const uint4*)(src + c);
+  if (threadIdx.x == 0) {
+    labels_c[r] = labels[t];
+    lse_c[r] = lse[t];
+    g_c[r] = g[t];
+    if (q) q_c[r] = q[t], pz_c[r] = pz[t];
+  }
+}
+
+__global__ __launch_bounds__(256) void scatter_active_rows(const int* __restrict__ idx, const int* __restrict__ counts,
+                                                           const uint16_t* __restrict__ d_hidden_c, int H,
+                                                           uint16_t* __restrict__ d_hidden) {
+  const int r = blockIdx.x;
+  if (r >= counts[0]) return;
+  const uint16_t* src = d_hidden_c + (size_t)r * (size_t)H;
+  uint16_t* dst = d_hidden + (size_t)idx[r] * (size_t)H;
+  for (int c = threadIdx.x * 8; c < H; c += 256 * 8) *(uint4*)(dst + c) = *(const uint4*)(src + c);
+}
+
+// ------------------------------------------------------------------------------------------------------------
 // Host side
 // ------------------------------------------------------------------------------------------------------------
 // Optional per-kernel timing: while a profile is open on the calling thread every launch below is bracketed by a pair of
 // HIP events on the launch stream.  Closed profiles cost one thread-local load per launch.
 enum KernelKind {
   kFwdTiles = 0, kFwdMerge, kTranspose, kBwdChunkDz, kBwdChunkGemm, kSoftCePack, kSoftCeFwdTiles, kSoftCeFinish, kSoftCeDz,
+  kCompactRows,
   kNumKernelKinds
 };
 const char* const kKernelNames[kNumKernelKinds] = {"lmhead_fwd_tiles", "lmhead_fwd_merge", "transpose_bf16",
                                                    "lmhead_bwd_chunk[dz]", "lmhead_bwd_chunk[gemm]", "softce_pack_rows",
-                                                   "softce_fwd_tiles", "softce_finish", "softce_dz_tiles"};
+                                                   "softce_fwd_tiles", "softce_finish", "softce_dz_tiles",
+                                                   "active_rows[compact+gather+scatter]"};
 struct Profile {
   struct Rec {
     int kind;
@@ -991,9 +1104,19 @@ int static_scratch_of_current_device(void** out) {
   return SKYRL_LMHEAD_OK;
 }
 
+// The backward, like the forward, walks the tokens in blocks: dHidden rows are complete within their block, dW is summed
+// over the blocks (the first block stores or adds as the caller's dw_mode says, the later ones add), and every scratch
+// matrix is sized by the block.  One block for T <= 32768, which covers every shape whose step time is quoted anywhere.
+constexpr int64_t kBwdTokenBlock = 32768;
+
 struct BwdWorkspace {
   uint16_t *Wt, *Ht, *D;
-  float* dHacc;
+  float *dHacc, *dWsum;
+  // only with row compaction (skyrl_lmhead_bwd_active_rows):
+  uint16_t *hidden_c, *d_hidden_c;
+  int64_t* labels_c;
+  float *lse_c, *pz_c, *g_c, *q_c;
+  int *idx, *counts;
   size_t bytes;
 };
 
@@ -1002,23 +1125,40 @@ struct BwdWorkspace {
 // zero-padded to whole tiles, is made in the workspace instead.
 inline bool reads_weight_in_place(int64_t V) { return V % BK == 0; }
 
-BwdWorkspace carve_bwd(void* ws, int64_t T, int64_t H, int64_t V, int64_t vc) {
-  const int64_t Tpad = round_up(T, 256), Vpad = round_up(V, 256);
+inline int64_t bwd_block_tokens(int64_t T) { return T < kBwdTokenBlock ? T : kBwdTokenBlock; }
+inline int64_t bwd_num_blocks(int64_t T) { return (T + kBwdTokenBlock - 1) / kBwdTokenBlock; }
+
+// vc: chunk width for a block of bwd_block_tokens(T) tokens.  compact: the buffers of the row-compacting entry point.
+BwdWorkspace carve_bwd(void* ws, int64_t T, int64_t H, int64_t V, int64_t vc, bool compact) {
+  const int64_t Tb = bwd_block_tokens(T), Tpad = round_up(Tb, 256), Vpad = round_up(V, 256);
   Carver c(ws);
-  BwdWorkspace w;
+  BwdWorkspace w{};
   w.Wt = reads_weight_in_place(V) ? nullptr : c.take<uint16_t>((size_t)H * (Vpad + kLdPad));
   w.Ht = c.take<uint16_t>((size_t)H * (Tpad + kLdPad));
   w.dHacc = c.take<float>((size_t)Tpad * round_up(H, 256));  // accumulator order, whole tiles
   w.D = c.take<uint16_t>((size_t)Tpad * (vc + kLdPad));
+  // Several blocks and a bf16 dW: the sum over the blocks is kept in fp32 here and rounded once, by the last block.
+  w.dWsum = bwd_num_blocks(T) > 1 ? c.take<float>((size_t)V * (size_t)H) : nullptr;
+  if (compact) {
+    w.hidden_c = c.take<uint16_t>((size_t)T * (size_t)H);
+    w.d_hidden_c = c.take<uint16_t>((size_t)T * (size_t)H);
+    w.labels_c = c.take<int64_t>((size_t)T);
+    w.lse_c = c.take<float>((size_t)T);
+    w.pz_c = c.take<float>((size_t)T);
+    w.g_c = c.take<float>((size_t)T);
+    w.q_c = c.take<float>((size_t)T);
+    w.idx = c.take<int>((size_t)T);
+    w.counts = c.take<int>((size_t)bwd_num_blocks(T) + 1);
+  }
   w.bytes = (size_t)round_up((int64_t)c.off, 256);
   return w;
 }
 
 GemmArgs make_gemm(const uint16_t* A, int64_t lda, int64_t a_rows, const uint16_t* B, int64_t ldb, int64_t b_rows, bool b_kmajor,
                    bool c_rows_m, int64_t nk, int64_t M, int64_t N, const float* Cin, float* Cf, uint16_t* Cb, int64_t ldc,
-                   const float* Pin = nullptr, float* Pout = nullptr) {
+                   const float* Pin = nullptr, float* Pout = nullptr, const int* T_dev = nullptr, int t_role = 0) {
   return GemmArgs{A,       (int)lda, (int)a_rows, B,  (int)ldb, (int)b_rows, b_kmajor ? 1 : 0, c_rows_m ? 1 : 0, (int)nk,
-                  (int)M,  (int)N,   Cin,         Cf, Cb,       (int)ldc,    Pin,              Pout};
+                  (int)M,  (int)N,   Cin,         Cf, Cb,       (int)ldc,    Pin,              Pout, T_dev, t_role};
 }
 
 unsigned gemm_tiles(const GemmArgs& g) { return (unsigned)(((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN)); }
@@ -1099,11 +1239,166 @@ hipError_t launch_softce_pack(hipStream_t s, const void* student, int64_t lds_, 
   return hipGetLastError();
 }
 
+size_t bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t vocab_chunk, bool compact) {
+  if (T < 1 || V < 1 || H < 1 || vocab_chunk < 0 || vocab_chunk % 256 != 0) return 0;
+  if (T > kMaxExtent || V > kMaxExtent || H > kMaxExtent || vocab_chunk > kMaxExtent) return 0;
+  int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(bwd_block_tokens(T), H, V);
+  if (vc > round_up(V, 256)) vc = round_up(V, 256);
+  return carve_bwd(nullptr, T, H, V, vc, compact).bytes;
+}
+
+// One token block of the backward: the vocab-chunk loop.  `Tb` tokens (an upper bound when `T_dev` points at the block's
+// count in device memory), per-token inputs and d_hidden already offset to the block.  dW of every chunk leaves the GEMM
+// epilogue as  (Cin ? Cin : 0) + product  ->  Cf (fp32) and / or Cb (bf16), each a [V, H] matrix or NULL.
+int bwd_token_block(const uint16_t* Hp, int64_t ld_hidden, const uint16_t* Wp, int64_t ld_weight, const int64_t* labels,
+                    const float* row_lse, const float* row_pz, const float* dlogprobs, const float* dentropy, int64_t Tb,
+                    const int* T_dev, int64_t H, int64_t V, float rcp_temperature, uint16_t* d_hidden, bool want_dw,
+                    const float* dw_in, float* dw_f32, uint16_t* dw_bf16, int64_t vc, const BwdWorkspace& w, hipStream_t s) {
+  const int64_t Tpad = round_up(Tb, 256), Vpad = round_up(V, 256);
+  const bool w_in_place = reads_weight_in_place(V);
+  hipError_t e;
+  if (want_dw) {  // only the dW product reads hidden^T [H, Tpad]; zero in the padding columns
+    Timed timed(kTranspose, s);
+    hipLaunchKernelGGL(transpose_bf16, dim3((unsigned)(Tpad / 64), (unsigned)(H / 64)), dim3(256), 0, s, Hp, (int)ld_hidden,
+                       (int)Tb, (int)H, w.Ht, (int)(Tpad + kLdPad), (int)Tpad, T_dev);
+    if ((e = hipGetLastError()) != hipSuccess) return (int)e;
+  }
+  const int tiles_t = (int)(Tpad / 256);
+  const int64_t nchunks = (Vpad + vc - 1) / vc;
+  auto chunk_width = [&](int64_t ci) { return (Vpad - ci * vc) < vc ? (Vpad - ci * vc) : vc; };  // multiple of 256
+  const GemmArgs none{};
+  for (int64_t ci = 0; ci < nchunks; ++ci) {
+    // dz panel of this chunk, then the two gradient GEMMs that consume it (one launch, they are independent).
+    // Carrying the next chunk's dz tiles in the GEMM launch (to fill its tail) was measured: no gain at the default chunk
+    // width, and it needs a second panel.
+    const int64_t vc0 = ci * vc, vcw = chunk_width(ci);
+    const DzArgs z{Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)Tb, (int)H, (int)V, rcp_temperature, labels, row_lse, row_pz,
+                   dlogprobs, dentropy, (int)vc0, (int)(vcw / 256), tiles_t, w.D, (int)(vcw + kLdPad), T_dev};
+    e = launch_bwd_chunk(s, dentropy != nullptr, z, (unsigned)(vcw / 256 * tiles_t), false, none, none);
+    if (e != hipSuccess) return (int)e;
+    // dHidden[t, h] (+)= sum_v D[t, v] . weight^T[h, vc0 + v]        (A = weight^T rows at k offset vc0, B = D rows)
+    // dW[vc0 + v, h]  (+)= sum_t D[t, v] . hidden^T[h, t]             (A = hidden^T rows, B = D read K-major)
+    const bool first = ci == 0, last = ci == nchunks - 1;
+    const int64_t rows = (V - vc0) < vcw ? (V - vc0) : vcw;
+    // dW rows are complete within their chunk (for this token block), so they can leave the GEMM epilogue in either precision.
+    const size_t dw_off = (size_t)vc0 * (size_t)H;
+    uint16_t* dh_out = last ? d_hidden : (uint16_t*)nullptr;
+    const float* dh_in = first ? (const float*)nullptr : (const float*)w.dHacc;
+    float* dh_keep = last ? (float*)nullptr : w.dHacc;
+    // In place: C[t, h] with A = D rows (K = vocab, contiguous), B = weight rows vc0.. read K-major; the k extent stops at V.
+    // Otherwise: C[h, t] with A = weight^T rows, B = D rows.  The partial sums are in accumulator order either way.
+    const int64_t kext = (V - vc0) < vcw ? (V - vc0) : vcw;
+    const GemmArgs gh =
+        w_in_place ? make_gemm(w.D, vcw + kLdPad, Tpad, Wp + (size_t)vc0 * (size_t)ld_weight, ld_weight, H, true, true, kext / BK, Tb,
+                               H, nullptr, nullptr, dh_out, H, dh_in, dh_keep, T_dev, kTokensOnM)
+                   : make_gemm(w.Wt + vc0, Vpad + kLdPad, H, w.D, vcw + kLdPad, Tpad, false, false, vcw / BK, H, Tb, nullptr,
+                               nullptr, dh_out, H, dh_in, dh_keep, T_dev, kTokensOnN);
+    // A frozen LM head needs no dW: the launch then carries the dHidden tiles alone.
+    const GemmArgs gw = want_dw ? make_gemm(w.Ht, Tpad + kLdPad, H, w.D, vcw + kLdPad, vcw, true, false, Tpad / BK, H, rows,
+                                            dw_in ? dw_in + dw_off : (const float*)nullptr,
+                                            dw_f32 ? dw_f32 + dw_off : (float*)nullptr,
+                                            dw_bf16 ? dw_bf16 + dw_off : (uint16_t*)nullptr, H, nullptr, nullptr, T_dev,
+                                            kTokensOnK)
+                                : none;
+    e = launch_bwd_chunk(s, dentropy != nullptr, DzArgs{}, 0, true, gh, gw);
+    if (e != hipSuccess) return (int)e;
+  }
+  return SKYRL_LMHEAD_OK;
+}
+
+int bwd_entry(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight, const int64_t* labels,
+              const float* row_lse, const float* row_pz, const float* dlogprobs, const float* dentropy, int64_t T, int64_t H,
+              int64_t V, float rcp_temperature, void* d_hidden, void* d_weight, int dw_mode, int64_t vocab_chunk,
+              void* workspace, size_t workspace_bytes, hipStream_t s, bool compact) {
+  int st = check_common(hidden, ld_hidden, weight, ld_weight, labels, T, H, V, rcp_temperature, true);
+  if (st) return st;
+  if (!row_lse || !dlogprobs || !d_hidden) return SKYRL_LMHEAD_ERR_NULL;
+  if (dentropy && !row_pz) return SKYRL_LMHEAD_ERR_NULL;
+  if (!aligned16(d_hidden) || !aligned16(d_weight)) return SKYRL_LMHEAD_ERR_ALIGN;  // d_weight NULL: no dW wanted
+  if (dw_mode < SKYRL_DW_FP32 || dw_mode > SKYRL_DW_BF16) return SKYRL_LMHEAD_ERR_ARG;
+  if (vocab_chunk < 0 || vocab_chunk % 256 != 0) return SKYRL_LMHEAD_ERR_ARG;
+  if (compact && T >= ((int64_t)1 << 31)) return SKYRL_LMHEAD_ERR_SHAPE;  // the row index list is 32-bit
+  const int64_t Tb = bwd_block_tokens(T), Tbpad = round_up(Tb, 256), Vpad = round_up(V, 256);
+  int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(Tb, H, V);
+  if (vc > Vpad) vc = Vpad;
+  // 32-bit byte offsets inside a block of hidden rows and inside the scratch matrices (weight^T, hidden^T, the dz panel)
+  if (Tb * ld_hidden * 2 >= ((int64_t)1 << 32) || H * (Vpad + kLdPad) * 2 >= ((int64_t)1 << 32) ||
+      H * (Tbpad + kLdPad) * 2 >= ((int64_t)1 << 32) || Tbpad * (vc + kLdPad) * 2 >= ((int64_t)1 << 32))
+    return SKYRL_LMHEAD_ERR_SHAPE;
+  if (!workspace || workspace_bytes < bwd_workspace_bytes(T, H, V, vc, compact)) return SKYRL_LMHEAD_ERR_WORKSPACE;
+  if ((uintptr_t)workspace & 255u) return SKYRL_LMHEAD_ERR_ALIGN;
+
+  const BwdWorkspace w = carve_bwd(workspace, T, H, V, vc, compact);
+  const uint16_t* Wp = (const uint16_t*)weight;
+  const uint16_t* Hp = (const uint16_t*)hidden;
+  const int64_t nblocks = bwd_num_blocks(T);
+  hipError_t e;
+
+  if (compact) {
+    Timed timed(kCompactRows, s);
+    hipLaunchKernelGGL(compact_active_rows, dim3(1), dim3(kCompactThreads), 0, s, dlogprobs, dentropy, (int)T, (int)Tb,
+                       (int)nblocks, w.idx, w.counts);
+    hipLaunchKernelGGL(gather_active_rows, dim3((unsigned)T), dim3(256), 0, s, (const int*)w.idx, (const int*)w.counts, Hp,
+                       (int)ld_hidden, (int)H, labels, row_lse, row_pz, dlogprobs, dentropy, w.hidden_c, w.labels_c, w.lse_c,
+                       w.pz_c, w.g_c, w.q_c, (uint16_t*)d_hidden);
+    if ((e = hipGetLastError()) != hipSuccess) return (int)e;
+  }
+  if (!reads_weight_in_place(V)) {  // weight^T [H, Vpad], zero in the padding columns
+    Timed timed(kTranspose, s);
+    hipLaunchKernelGGL(transpose_bf16, dim3((unsigned)(Vpad / 64), (unsigned)(H / 64)), dim3(256), 0, s, Wp, (int)ld_weight,
+                       (int)V, (int)H, w.Wt, (int)(Vpad + kLdPad), (int)Vpad, (const int*)nullptr);
+    if ((e = hipGetLastError()) != hipSuccess) return (int)e;
+  }
+
+  for (int64_t b = 0; b < nblocks; ++b) {
+    const int64_t t0 = b * Tb, Tcur = (T - t0) < Tb ? (T - t0) : Tb;
+    // Where dW of this block comes from and goes to.  One block: straight to the caller's matrix as dw_mode says.  Several
+    // blocks: fp32 modes add every later block to the caller's matrix; the bf16 mode sums in the fp32 scratch matrix and
+    // the last block rounds the sum into the caller's.
+    const float* dw_in = nullptr;
+    float* dw_f32 = nullptr;
+    uint16_t* dw_bf16 = nullptr;
+    if (d_weight) {
+      const bool first = b == 0, last = b == nblocks - 1;
+      if (dw_mode == SKYRL_DW_BF16) {
+        if (nblocks == 1) {
+          dw_bf16 = (uint16_t*)d_weight;
+        } else {
+          dw_in = first ? nullptr : w.dWsum;
+          if (last) dw_bf16 = (uint16_t*)d_weight; else dw_f32 = w.dWsum;
+        }
+      } else {
+        dw_f32 = (float*)d_weight;
+        dw_in = (dw_mode == SKYRL_DW_FP32_ACCUMULATE || !first) ? (const float*)d_weight : nullptr;
+      }
+    }
+    if (compact) {
+      st = bwd_token_block(w.hidden_c + (size_t)t0 * (size_t)H, H, Wp, ld_weight, w.labels_c + t0, w.lse_c + t0,
+                           dentropy ? w.pz_c + t0 : nullptr, w.g_c + t0, dentropy ? w.q_c + t0 : nullptr, Tcur,
+                           w.counts + 1 + b, H, V, rcp_temperature, w.d_hidden_c + (size_t)t0 * (size_t)H, d_weight != nullptr,
+                           dw_in, dw_f32, dw_bf16, vc, w, s);
+    } else {
+      st = bwd_token_block(Hp + (size_t)t0 * (size_t)ld_hidden, ld_hidden, Wp, ld_weight, labels + t0, row_lse + t0,
+                           row_pz ? row_pz + t0 : nullptr, dlogprobs + t0, dentropy ? dentropy + t0 : nullptr, Tcur, nullptr, H,
+                           V, rcp_temperature, (uint16_t*)d_hidden + (size_t)t0 * (size_t)H, d_weight != nullptr, dw_in, dw_f32,
+                           dw_bf16, vc, w, s);
+    }
+    if (st) return st;
+  }
+  if (compact) {
+    Timed timed(kCompactRows, s);
+    hipLaunchKernelGGL(scatter_active_rows, dim3((unsigned)T), dim3(256), 0, s, (const int*)w.idx, (const int*)w.counts,
+                       (const uint16_t*)w.d_hidden_c, (int)H, (uint16_t*)d_hidden);
+    if ((e = hipGetLastError()) != hipSuccess) return (int)e;
+  }
+  return SKYRL_LMHEAD_OK;
+}
+
 }  // namespace
 
 extern "C" {
 
-int skyrl_lmhead_version(void) { return 13; }
+int skyrl_lmhead_version(void) { return 14; }
 
 const char* skyrl_lmhead_strerror(int status) {
   switch (status) {
@@ -1133,11 +1428,11 @@ size_t skyrl_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
 }
 
 size_t skyrl_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t vocab_chunk) {
-  if (T < 1 || V < 1 || H < 1 || vocab_chunk < 0 || vocab_chunk % 256 != 0) return 0;
-  if (T > kMaxExtent || V > kMaxExtent || H > kMaxExtent || vocab_chunk > kMaxExtent) return 0;
-  int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(T, H, V);
-  if (vc > round_up(V, 256)) vc = round_up(V, 256);
-  return carve_bwd(nullptr, T, H, V, vc).bytes;
+  return bwd_workspace_bytes(T, H, V, vocab_chunk, false);
+}
+
+size_t skyrl_lmhead_bwd_active_rows_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t vocab_chunk) {
+  return bwd_workspace_bytes(T, H, V, vocab_chunk, true);
 }
 
 int skyrl_lmhead_fwd(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight, const int64_t* labels,
@@ -1173,87 +1468,17 @@ int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, 
                      const float* row_lse, const float* row_pz, const float* dlogprobs, const float* dentropy, int64_t T,
                      int64_t H, int64_t V, float rcp_temperature, void* d_hidden, void* d_weight, int dw_mode,
                      int64_t vocab_chunk, void* workspace, size_t workspace_bytes, void* stream) {
-  int st = check_common(hidden, ld_hidden, weight, ld_weight, labels, T, H, V, rcp_temperature);
-  if (st) return st;
-  if (!row_lse || !dlogprobs || !d_hidden) return SKYRL_LMHEAD_ERR_NULL;
-  if (dentropy && !row_pz) return SKYRL_LMHEAD_ERR_NULL;
-  if (!aligned16(d_hidden) || !aligned16(d_weight)) return SKYRL_LMHEAD_ERR_ALIGN;  // d_weight NULL: no dW wanted
-  if (dw_mode < SKYRL_DW_FP32 || dw_mode > SKYRL_DW_BF16) return SKYRL_LMHEAD_ERR_ARG;
-  if (vocab_chunk < 0 || vocab_chunk % 256 != 0) return SKYRL_LMHEAD_ERR_ARG;
-  const int64_t Tpad = round_up(T, 256), Vpad = round_up(V, 256);
-  int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(T, H, V);
-  if (vc > Vpad) vc = Vpad;
-  // 32-bit byte offsets inside the scratch matrices as well (weight^T, hidden^T, the dz panel)
-  if (H * (Vpad + kLdPad) * 2 >= ((int64_t)1 << 32) || H * (Tpad + kLdPad) * 2 >= ((int64_t)1 << 32) ||
-      Tpad * (vc + kLdPad) * 2 >= ((int64_t)1 << 32))
-    return SKYRL_LMHEAD_ERR_SHAPE;
-  if (!workspace || workspace_bytes < skyrl_lmhead_bwd_workspace_bytes(T, H, V, vc)) return SKYRL_LMHEAD_ERR_WORKSPACE;
-  if ((uintptr_t)workspace & 255u) return SKYRL_LMHEAD_ERR_ALIGN;
+  return bwd_entry(hidden, ld_hidden, weight, ld_weight, labels, row_lse, row_pz, dlogprobs, dentropy, T, H, V, rcp_temperature,
+                   d_hidden, d_weight, dw_mode, vocab_chunk, workspace, workspace_bytes, (hipStream_t)stream, false);
+}
 
-  hipStream_t s = (hipStream_t)stream;
-  const BwdWorkspace w = carve_bwd(workspace, T, H, V, vc);
-  const uint16_t* Wp = (const uint16_t*)weight;
-  const uint16_t* Hp = (const uint16_t*)hidden;
-  hipError_t e;
-
-  // hidden^T [H, Tpad] and, unless the weight can be read in place, weight^T [H, Vpad]; zero in the padding columns.
-  const bool w_in_place = reads_weight_in_place(V);
-  if (!w_in_place) {
-    Timed timed(kTranspose, s);
-    hipLaunchKernelGGL(transpose_bf16, dim3((unsigned)(Vpad / 64), (unsigned)(H / 64)), dim3(256), 0, s, Wp, (int)ld_weight,
-                       (int)V, (int)H, w.Wt, (int)(Vpad + kLdPad), (int)Vpad);
-  }
-  if (d_weight) {  // only the dW product reads hidden^T
-    Timed timed(kTranspose, s);
-    hipLaunchKernelGGL(transpose_bf16, dim3((unsigned)(Tpad / 64), (unsigned)(H / 64)), dim3(256), 0, s, Hp, (int)ld_hidden,
-                       (int)T, (int)H, w.Ht, (int)(Tpad + kLdPad), (int)Tpad);
-  }
-  if ((e = hipGetLastError()) != hipSuccess) return (int)e;
-
-  const int tiles_t = (int)(Tpad / 256);
-  const int64_t nchunks = (Vpad + vc - 1) / vc;
-  auto chunk_width = [&](int64_t ci) { return (Vpad - ci * vc) < vc ? (Vpad - ci * vc) : vc; };  // multiple of 256
-  auto dz_args = [&](int64_t ci) {
-    const int64_t vc0 = ci * vc, vcw = chunk_width(ci);
-    return DzArgs{Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)T, (int)H, (int)V, rcp_temperature, labels, row_lse, row_pz,
-                  dlogprobs, dentropy, (int)vc0, (int)(vcw / 256), tiles_t, w.D, (int)(vcw + kLdPad)};
-  };
-  const GemmArgs none{};
-  for (int64_t ci = 0; ci < nchunks; ++ci) {
-    // dz panel of this chunk, then the two gradient GEMMs that consume it (one launch, they are independent).
-    // Carrying the next chunk's dz tiles in the GEMM launch (to fill its tail) was measured: no gain at the default chunk
-    // width, and it needs a second panel.
-    e = launch_bwd_chunk(s, dentropy != nullptr, dz_args(ci), (unsigned)(chunk_width(ci) / 256 * tiles_t), false, none, none);
-    if (e != hipSuccess) return (int)e;
-    const int64_t vc0 = ci * vc, vcw = chunk_width(ci);
-    // dHidden[t, h] (+)= sum_v D[t, v] . weight^T[h, vc0 + v]        (A = weight^T rows at k offset vc0, B = D rows)
-    // dW[vc0 + v, h]  (+)= sum_t D[t, v] . hidden^T[h, t]             (A = hidden^T rows, B = D read K-major)
-    const bool first = ci == 0, last = ci == nchunks - 1;
-    const int64_t rows = (V - vc0) < vcw ? (V - vc0) : vcw;
-    // dW rows are complete within their chunk, so they can leave the GEMM epilogue in either precision.
-    const size_t dw_off = (size_t)vc0 * (size_t)H;
-    float* dWf = (d_weight && dw_mode != SKYRL_DW_BF16) ? (float*)d_weight + dw_off : (float*)nullptr;
-    uint16_t* dWb = (d_weight && dw_mode == SKYRL_DW_BF16) ? (uint16_t*)d_weight + dw_off : (uint16_t*)nullptr;
-    const uint16_t* dh_out = last ? (uint16_t*)d_hidden : (uint16_t*)nullptr;
-    const float* dh_in = first ? (const float*)nullptr : (const float*)w.dHacc;
-    float* dh_keep = last ? (float*)nullptr : w.dHacc;
-    // In place: C[t, h] with A = D rows (K = vocab, contiguous), B = weight rows vc0.. read K-major; the k extent stops at V.
-    // Otherwise: C[h, t] with A = weight^T rows, B = D rows.  The partial sums are in accumulator order either way.
-    const int64_t kext = (V - vc0) < vcw ? (V - vc0) : vcw;
-    const GemmArgs gh =
-        w_in_place ? make_gemm(w.D, vcw + kLdPad, Tpad, Wp + (size_t)vc0 * (size_t)ld_weight, ld_weight, H, true, true, kext / BK, T,
-                               H, nullptr, nullptr, (uint16_t*)dh_out, H, dh_in, dh_keep)
-                   : make_gemm(w.Wt + vc0, Vpad + kLdPad, H, w.D, vcw + kLdPad, Tpad, false, false, vcw / BK, H, T, nullptr,
-                               nullptr, (uint16_t*)dh_out, H, dh_in, dh_keep);
-    // A frozen LM head (d_weight == NULL) needs no dW: the launch then carries the dHidden tiles alone.
-    const GemmArgs gw = d_weight ? make_gemm(w.Ht, Tpad + kLdPad, H, w.D, vcw + kLdPad, vcw, true, false, Tpad / BK, H, rows,
-                                             dw_mode == SKYRL_DW_FP32_ACCUMULATE ? (const float*)dWf : (const float*)nullptr, dWf,
-                                             dWb, H)
-                                 : none;
-    e = launch_bwd_chunk(s, dentropy != nullptr, DzArgs{}, 0, true, gh, gw);
-    if (e != hipSuccess) return (int)e;
-  }
-  return SKYRL_LMHEAD_OK;
+int skyrl_lmhead_bwd_active_rows(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight,
+                                 const int64_t* labels, const float* row_lse, const float* row_pz, const float* dlogprobs,
+                                 const float* dentropy, int64_t T, int64_t H, int64_t V, float rcp_temperature, void* d_hidden,
+                                 void* d_weight, int dw_mode, int64_t vocab_chunk, void* workspace, size_t workspace_bytes,
+                                 void* stream) {
+  return bwd_entry(hidden, ld_hidden, weight, ld_weight, labels, row_lse, row_pz, dlogprobs, dentropy, T, H, V, rcp_temperature,
+                   d_hidden, d_weight, dw_mode, vocab_chunk, workspace, workspace_bytes, (hipStream_t)stream, true);
 }
 
 size_t skyrl_softce_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
@@ -1334,7 +1559,7 @@ int skyrl_softce_bwd(const void* student_hidden, int64_t ld_student, const void*
   if (!w_in_place) {
     Timed timed(kTranspose, s);
     hipLaunchKernelGGL(transpose_bf16, dim3((unsigned)(Vpad / 64), (unsigned)(H / 64)), dim3(256), 0, s, Wp, (int)ld_weight,
-                       (int)V, (int)H, w.Wt, (int)(Vpad + kLdPad), (int)Vpad);
+                       (int)V, (int)H, w.Wt, (int)(Vpad + kLdPad), (int)Vpad, (const int*)nullptr);
     if ((e = hipGetLastError()) != hipSuccess) return (int)e;
   }
   const int64_t nchunks = (Vpad + vc - 1) / vc;

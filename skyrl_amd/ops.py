@@ -118,8 +118,10 @@ def lmhead_bwd(
     dentropy: Optional[torch.Tensor],
     rcp_temperature: float,
     vocab_chunk: int,
+    active_rows: bool = False,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Returns ``(d_hidden bf16 [T,H], d_weight fp32 [V,H])``."""
+    """Returns ``(d_hidden bf16 [T,H], d_weight fp32 [V,H])``.  ``active_rows``: run on the tokens that have an upstream gradient
+    only (``skyrl_lmhead_bwd_active_rows``: compaction on the device, no host synchronisation)."""
     T, H, V = _check_operands(hidden, weight, labels)
     dev = _require_device(hidden, weight, labels, row_lse, dlogprobs)
     lib = _lib.load()
@@ -128,7 +130,7 @@ def lmhead_bwd(
         return d_hidden, torch.zeros((V, H), dtype=torch.float32, device=dev)
     d_weight = torch.empty((V, H), dtype=torch.float32, device=dev)
     _bwd_into(lib, hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk, d_hidden,
-              d_weight, False)
+              d_weight, False, active_rows)
     return d_hidden, d_weight
 
 
@@ -143,6 +145,7 @@ def lmhead_bwd_bf16(
     dentropy: Optional[torch.Tensor],
     rcp_temperature: float,
     vocab_chunk: int,
+    active_rows: bool = False,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """``(d_hidden bf16 [T,H], d_weight bf16 [V,H])``: the weight gradient leaves the GEMM epilogue already rounded to the
     weight's dtype (what the autograd adapters hand back), with no fp32 ``[V, H]`` buffer and no cast pass."""
@@ -153,12 +156,12 @@ def lmhead_bwd_bf16(
         return d_hidden, torch.zeros((V, H), dtype=torch.bfloat16, device=dev)
     d_weight = torch.empty((V, H), dtype=torch.bfloat16, device=dev)
     _bwd_into(_lib.load(), hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk, d_hidden,
-              d_weight, False)
+              d_weight, False, active_rows)
     return d_hidden, d_weight
 
 
 @lmhead_bwd_bf16.register_fake
-def _(hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk):
+def _(hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk, active_rows=False):
     return (torch.empty_like(hidden, memory_format=torch.contiguous_format),
             torch.empty(weight.shape, dtype=torch.bfloat16, device=weight.device))
 
@@ -174,6 +177,7 @@ def lmhead_bwd_hidden(
     dentropy: Optional[torch.Tensor],
     rcp_temperature: float,
     vocab_chunk: int,
+    active_rows: bool = False,
 ) -> torch.Tensor:
     """``d_hidden`` bf16 [T,H] alone, for a weight that takes no gradient (a frozen LM head): the dW product is skipped."""
     T, H, V = _check_operands(hidden, weight, labels)
@@ -181,12 +185,12 @@ def lmhead_bwd_hidden(
     d_hidden = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
     if T > 0:
         _bwd_into(_lib.load(), hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk,
-                  d_hidden, None, False)
+                  d_hidden, None, False, active_rows)
     return d_hidden
 
 
 @lmhead_bwd_hidden.register_fake
-def _(hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk):
+def _(hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk, active_rows=False):
     return torch.empty_like(hidden, memory_format=torch.contiguous_format)
 
 
@@ -200,49 +204,29 @@ def lmhead_bwd_active_rows(
     dentropy: Optional[torch.Tensor],
     rcp_temperature: float,
     vocab_chunk: int = 0,
-    min_skip_fraction: float = 0.125,
     want_dweight: bool = True,
     dweight_dtype: torch.dtype = torch.float32,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
-    """``lmhead_bwd`` that first drops the tokens whose upstream gradients are all zero.
+    """The backward on the tokens whose upstream gradients are not all zero -- what the autograd adapters call.
 
     A token with ``dlogprobs == 0`` (and ``dentropy == 0``) has a zero dz row: it adds nothing to dW and its dHidden row is
     zero.  In RL micro-batches those are the prompt and padding tokens the loss mask removes (``loss_mask`` in
     megatron_model_wrapper.py:607-985; half of the tokens in the Qwen2.5-1.5B benchmark configuration), so the three
-    backward GEMMs run on the remaining rows only: rows are gathered, the kernels run on the compact ``[T_active, H]``
-    problem, and dHidden rows are scattered back into zeros.  Counting the active rows costs one host synchronisation; when
-    fewer than ``min_skip_fraction`` of the rows would be dropped the dense path is used.  With ``want_dweight=False`` (the
-    weight takes no gradient) the dW product is skipped and ``None`` is returned in its place; ``dweight_dtype`` is fp32 or
-    bf16 (rounded in the GEMM epilogue).
+    backward GEMMs run on the remaining rows only.  The rows are listed, counted, gathered and scattered back by kernels
+    (``skyrl_lmhead_bwd_active_rows``): the host never reads the count, nothing synchronises, shapes are static, and the
+    call can sit inside a captured HIP graph.  With ``want_dweight=False`` (the weight takes no gradient) the dW product is
+    skipped and ``None`` is returned in its place; ``dweight_dtype`` is fp32 or bf16 (rounded in the GEMM epilogue).
     """
     if dweight_dtype not in (torch.float32, torch.bfloat16):
         raise TypeError(f"d_weight is fp32 or bf16, not {dweight_dtype}")
-    T = hidden.shape[0]
-    active = dlogprobs != 0
-    if dentropy is not None:
-        active |= dentropy != 0
-    idx = active.nonzero(as_tuple=True)[0]
-    n = int(idx.numel())
-    def run(*args):
-        if want_dweight:
-            return lmhead_bwd(*args) if dweight_dtype == torch.float32 else lmhead_bwd_bf16(*args)
-        return lmhead_bwd_hidden(*args), None
-
-    if n == 0:
-        return torch.zeros_like(hidden, memory_format=torch.contiguous_format), (
-            torch.zeros(weight.shape, dtype=dweight_dtype, device=weight.device) if want_dweight else None)
-    if T - n < min_skip_fraction * T:
-        return run(hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk)
-    take = lambda t: None if t is None else t.index_select(0, idx)  # noqa: E731
-    dh_c, d_weight = run(take(hidden), weight, take(labels), take(row_lse), take(row_pz) if dentropy is not None else None,
-                         take(dlogprobs), take(dentropy), rcp_temperature, vocab_chunk)
-    d_hidden = torch.zeros((T, hidden.shape[1]), dtype=torch.bfloat16, device=hidden.device)
-    d_hidden.index_copy_(0, idx, dh_c)
-    return d_hidden, d_weight
+    args = (hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk, True)
+    if want_dweight:
+        return lmhead_bwd(*args) if dweight_dtype == torch.float32 else lmhead_bwd_bf16(*args)
+    return lmhead_bwd_hidden(*args), None
 
 
 def _bwd_into(lib, hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk, d_hidden,
-              d_weight, accumulate_dw: bool) -> None:
+              d_weight, accumulate_dw: bool, active_rows: bool = False) -> None:
     T, H = hidden.shape
     V = weight.shape[0]
     dev = hidden.device
@@ -255,7 +239,9 @@ def _bwd_into(lib, hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy,
             continue
         if t.dtype != torch.float32 or t.shape != (T,) or not t.is_contiguous():
             raise ValueError(f"{name} must be a contiguous fp32 tensor of shape [{T}], got {t.dtype} {tuple(t.shape)}")
-    ws_bytes = int(lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, int(vocab_chunk)))
+    query = lib.skyrl_lmhead_bwd_active_rows_workspace_bytes if active_rows else lib.skyrl_lmhead_bwd_workspace_bytes
+    entry = lib.skyrl_lmhead_bwd_active_rows if active_rows else lib.skyrl_lmhead_bwd
+    ws_bytes = int(query(T, H, V, int(vocab_chunk)))
     if ws_bytes == 0:
         if int(vocab_chunk) < 0 or int(vocab_chunk) % 256 != 0:
             raise ValueError(f"bad vocab_chunk {vocab_chunk}: must be 0 (library default) or a multiple of 256")
@@ -263,14 +249,14 @@ def _bwd_into(lib, hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy,
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
-        st = lib.skyrl_lmhead_bwd(
+        st = entry(
             hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), labels.data_ptr(),
             row_lse.data_ptr(), _ptr(row_pz if dentropy is not None else None), dlogprobs.data_ptr(), _ptr(dentropy),
             T, H, V, float(rcp_temperature), d_hidden.data_ptr(), _ptr(d_weight),
             2 if (d_weight is not None and d_weight.dtype == torch.bfloat16) else int(bool(accumulate_dw)),
             int(vocab_chunk), ws.data_ptr(), ws_bytes, stream,
         )
-    _lib.check(st, "skyrl_lmhead_bwd")
+    _lib.check(st, "skyrl_lmhead_bwd_active_rows" if active_rows else "skyrl_lmhead_bwd")
 
 
 def lmhead_bwd_accumulate(hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature: float,
@@ -290,7 +276,7 @@ def lmhead_bwd_accumulate(hidden, weight, labels, row_lse, row_pz, dlogprobs, de
 
 
 @lmhead_bwd.register_fake
-def _(hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk):
+def _(hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk, active_rows=False):
     return (torch.empty_like(hidden, memory_format=torch.contiguous_format),
             torch.empty(weight.shape, dtype=torch.float32, device=weight.device))
 

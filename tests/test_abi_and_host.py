@@ -340,10 +340,16 @@ def test_default_vocab_chunk_respects_the_panel_cap():
     lib = _lib.load()
     for T, H, V in [(16384, 3584, 152064), (32768, 4096, 128256), (8192, 1536, 151936), (300, 128, 1001), (1, 64, 8),
                     (100000, 1024, 50257), (2048, 8192, 262144)]:
-        Tp, Vp, Hp = -(-T // 256) * 256, -(-V // 256) * 256, -(-H // 256) * 256
+        Tb = min(T, 32768)  # the backward walks the tokens in blocks; the scratch is sized by the block
+        Tp, Vp, Hp = -(-Tb // 256) * 256, -(-V // 256) * 256, -(-H // 256) * 256
         total = lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, 0)
         assert total == lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, 0)
         fixed = (0 if V % 64 == 0 else 2 * H * (Vp + 64)) + 2 * H * (Tp + 64) + 4 * Tp * Hp
+        if T > Tb:  # several blocks: the fp32 matrix in which a bf16 dW is summed over the blocks
+            fixed += -(-4 * V * H // 256) * 256
+        # the row-compacting variant adds the gathered copies: two [T, H] bf16 matrices and 28 bytes per token (+ counters)
+        extra = lib.skyrl_lmhead_bwd_active_rows_workspace_bytes(T, H, V, 0) - total
+        assert 4 * T * H + 28 * T <= extra <= 4 * T * H + 28 * T + 4 * (T // 32768 + 2) + 9 * 256, (T, H, V, extra)
         panel = total - fixed
         assert 0 < panel <= (3 << 29) + 2 * Tp * 64 + 4096 or panel <= 2 * Tp * (2048 + 64) + 4096, (T, H, V, panel)
         vc = (panel - 1024) // (2 * Tp) - 64          # the alignment slack is below one row

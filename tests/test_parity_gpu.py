@@ -375,8 +375,8 @@ def test_backward_skips_rows_without_upstream_gradient(cuda_device):
     assert compact[0][masked].abs().max().item() == 0.0
     assert rel_l2(compact[0].float(), dense[0].float()) < 2e-2 and rel_l2(compact[1], dense[1]) < 1e-3
     ex = O.exact_fwd_bwd(d["hidden"], d["weight"], d["labels"], 1.0, d["dlogprobs"], None)
-    assert cos(compact[0], ex["d_hidden"]) >= GRAD_COS and cos(compact[1], ex["d_weight"]) >= GRAD_COS
-    # all-zero upstream gradient: zeros, no kernel launched
+    check_grads(compact[0], compact[1], ex, "compacted")
+    # all-zero upstream gradient: zeros
     z = ops.lmhead_bwd_active_rows(h, w, y, lse, None, torch.zeros_like(g), None, 1.0, 0)
     assert z[0].abs().max().item() == 0.0 and z[1].abs().max().item() == 0.0
     # through autograd (FusedLinearLogprobHip uses the compacting path)
@@ -386,6 +386,99 @@ def test_backward_skips_rows_without_upstream_gradient(cuda_device):
     out = FusedLinearLogprobHip.apply(hd, wd, d["labels"].reshape(B, S).to(dev), 0, cfg.V, S, None, False)
     (out * g.reshape(B, S)).sum().backward()
     assert cos(hd.grad.reshape(-1, cfg.H), ex["d_hidden"]) >= GRAD_COS and cos(wd.grad, ex["d_weight"]) >= GRAD_COS
+
+
+@pytest.mark.parametrize("T,H,V,vc,keep,entgrad", [
+    (700, 128, 2048, 512, 0.4, True),     # four vocab chunks: the dHidden partial sums cross chunks under a device-side count
+    (700, 128, 2001, 0, 0.4, False),      # V not a multiple of 64: the dHidden GEMM on the transposed weight copy
+    (515, 64, 900, 256, 0.999, True),     # (nearly) everything active
+    (1000, 192, 1500, 0, 0.003, False),   # a handful of active rows: far less than one tile
+    (300, 64, 777, 0, 0.5, True),
+])
+def test_active_rows_backward_equals_the_backward_on_gathered_rows(T, H, V, vc, keep, entgrad, cuda_device):
+    """skyrl_lmhead_bwd_active_rows compacts on the device; the same compaction done here with torch indexing, followed by the
+    dense backward, must give the same bits: d_weight of the compacted problem, d_hidden rows scattered back, zeros elsewhere."""
+    dev = cuda_device
+    hidden, weight, labels, g, q = _rand(T, H, V, seed=int(1000 * keep) + T)
+    gen = torch.Generator().manual_seed(T + V)
+    active = torch.rand(T, generator=gen) < keep
+    if keep > 0.9:
+        active[:] = True
+        active[T // 2] = False
+    g = g * active
+    q = q * active if entgrad else None
+    h, w, y = hidden.to(dev), weight.to(dev), labels.to(dev)
+    gd, qd = g.to(dev), None if q is None else q.to(dev)
+    _, _, lse, pz = ops.lmhead_fwd(h, w, y, 1.0 / 0.9, True)
+    pzq = pz if entgrad else None
+    idx = active.nonzero()[:, 0].to(dev)
+    take = lambda t: None if t is None else t.index_select(0, idx)  # noqa: E731
+    for op, kw in ((ops.lmhead_bwd, {}), (ops.lmhead_bwd_bf16, {}), (ops.lmhead_bwd_hidden, {})):
+        got = op(h, w, y, lse, pzq, gd, qd, 1.0 / 0.9, vc, True)
+        want = op(take(h), w, take(y), take(lse), take(pzq), take(gd), take(qd), 1.0 / 0.9, vc)
+        got, want = (got, want) if isinstance(got, tuple) else ((got,), (want,))
+        full = torch.zeros(T, H, dtype=torch.bfloat16, device=dev)
+        full.index_copy_(0, idx, want[0])
+        assert torch.equal(got[0], full), op.__name__
+        if len(got) > 1:
+            assert torch.equal(got[1], want[1]), op.__name__
+    # and against the oracle
+    dh, dw = ops.lmhead_bwd(h, w, y, lse, pzq, gd, qd, 1.0 / 0.9, vc, True)
+    ex = O.exact_fwd_bwd(hidden, weight, labels, 0.9, g, q)
+    check_grads(dh, dw, ex, "active rows")
+    # accumulation into an existing dW goes through the same entry point
+    lib = _lib.load()
+    acc = torch.full((V, H), 0.5, dtype=torch.float32, device=dev)
+    n = lib.skyrl_lmhead_bwd_active_rows_workspace_bytes(T, H, V, vc)
+    ws = torch.empty(n, dtype=torch.uint8, device=dev)
+    dh2 = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    st = lib.skyrl_lmhead_bwd_active_rows(h.data_ptr(), H, w.data_ptr(), H, y.data_ptr(), lse.data_ptr(),
+                                          None if pzq is None else pzq.data_ptr(), gd.data_ptr(),
+                                          None if qd is None else qd.data_ptr(), T, H, V, 1.0 / 0.9, dh2.data_ptr(),
+                                          acc.data_ptr(), 1, vc, ws.data_ptr(), n, torch.cuda.current_stream().cuda_stream)
+    assert st == 0
+    torch.cuda.synchronize()
+    assert torch.equal(dh2, dh) and torch.equal(acc, dw + 0.5)
+    assert lib.skyrl_lmhead_bwd_active_rows(h.data_ptr(), H, w.data_ptr(), H, y.data_ptr(), lse.data_ptr(), None, gd.data_ptr(),
+                                            None, T, H, V, 1.0, dh2.data_ptr(), acc.data_ptr(), 1, vc, ws.data_ptr(), n - 1,
+                                            None) == -4
+
+
+def test_forward_and_backward_in_token_blocks(cuda_device):
+    """More than 32768 tokens: both passes walk the tokens in blocks.  Tokens are independent, so each block must reproduce a
+    call on that block alone bit for bit, and dW must be the blocks' dW added up -- in every dw_mode, with and without
+    row compaction."""
+    dev = cuda_device
+    T, H, V, cut = 40000, 64, 1000, 32768
+    hidden, weight, labels, g, q = _rand(T, H, V, seed=77)
+    g[torch.rand(T, generator=torch.Generator().manual_seed(5)) < 0.3] = 0.0
+    q = q * (g != 0)
+    h, w, y, gd, qd = hidden.to(dev), weight.to(dev), labels.to(dev), g.to(dev), q.to(dev)
+    out = ops.lmhead_fwd(h, w, y, 1.0, True)
+    parts = [ops.lmhead_fwd(h[a:b], w, y[a:b], 1.0, True) for a, b in ((0, cut), (cut, T))]
+    for k in range(4):
+        assert torch.equal(out[k], torch.cat([p[k] for p in parts]))
+    assert ops.fwd_workspace_bytes(T, H, V) == ops.fwd_workspace_bytes(cut, H, V)
+    lse, pz = out[2], out[3]
+    halves = [ops.lmhead_bwd(h[a:b], w, y[a:b], lse[a:b], pz[a:b], gd[a:b], qd[a:b], 1.0, 512) for a, b in ((0, cut), (cut, T))]
+    want_dh = torch.cat([p[0] for p in halves])
+    want_dw = halves[0][1] + halves[1][1]
+    for active_rows in (False, True):
+        dh, dw = ops.lmhead_bwd(h, w, y, lse, pz, gd, qd, 1.0, 512, active_rows)
+        if not active_rows:
+            assert torch.equal(dh, want_dh) and torch.equal(dw, want_dw)
+        ex_rows = torch.arange(cut - 300, cut + 300)
+        assert rel_l2(dh[ex_rows.to(dev)].float(), want_dh[ex_rows.to(dev)].float()) < 1e-2
+        assert rel_l2(dw, want_dw) < 1e-3 and worst_row(dw, want_dw) < 2e-2
+        _, dwb = ops.lmhead_bwd_bf16(h, w, y, lse, pz, gd, qd, 1.0, 512, active_rows)
+        assert torch.equal(dwb, dw.bfloat16())          # summed over the blocks in fp32, rounded once
+        acc = torch.full((V, H), -2.0, dtype=torch.float32, device=dev)
+        ops._bwd_into(_lib.load(), h, w, y, lse, pz, gd, qd, 1.0, 512, torch.empty_like(h), acc, True, active_rows)
+        assert rel_l2(acc + 2.0, dw) < 1e-5           # the same sums, added to what was there in a different order
+    ex = O.exact_fwd_bwd(hidden, weight, labels, 1.0, g, q)
+    dh, dw = ops.lmhead_bwd(h, w, y, lse, pz, gd, qd, 1.0, 0, True)
+    check_grads(dh, dw, ex, "token blocks, active rows")
+    assert (out[0].cpu().double() - ex["logprobs"]).abs().max() <= 1e-3
 
 
 def test_c_abi_called_directly(cuda_device):
@@ -1244,6 +1337,64 @@ def test_fsdp_forward_tail_from_hidden(cuda_device, packed, compute_entropy, ent
         assert out == {}
     loss.backward()
     assert cos(hd.grad, h64.grad) >= GRAD_COS and cos(wd.grad, w64.grad) >= GRAD_COS
+
+
+def test_masked_training_step_replays_from_a_hip_graph(cuda_device):
+    """Forward -> actor loss (its gradient is the backward's upstream gradient, zero on masked tokens) -> backward on the active
+    rows, captured as one HIP graph: nothing on that path reads a value back on the host.  Every replay, on new inputs and a new
+    mask (so a new number of active rows), must equal the eager step bit for bit."""
+    from types import SimpleNamespace
+
+    from skyrl_amd.policy_loss import actor_loss
+
+    dev = cuda_device
+    B, S, H, V = 3, 120, 128, 1500
+    gen = torch.Generator().manual_seed(17)
+    weight = (torch.randn(V, H, generator=gen) * 3 / H ** 0.5).bfloat16().to(dev)
+    hidden = torch.zeros(B * S, H, dtype=torch.bfloat16, device=dev)
+    labels = torch.zeros(B * S, dtype=torch.int64, device=dev)
+    old = torch.zeros(B, S, device=dev)
+    adv = torch.zeros(B, S, device=dev)
+    mask = torch.zeros(B, S, device=dev)
+    cfg = SimpleNamespace(policy_loss_type="regular", eps_clip_low=0.2, eps_clip_high=0.2, use_kl_loss=False,
+                          use_entropy_loss=False)
+
+    def step():
+        h = hidden.detach().requires_grad_(True)
+        w = weight.detach().requires_grad_(True)
+        lp, _ = linear_cross_entropy(h, w, labels, 1.0, "none", None, False)
+        loss, _ = actor_loss(lp.reshape(B, S), old, adv, cfg, mask)
+        gh, gw = torch.autograd.grad(loss, (h, w))
+        return loss.detach(), gh, gw
+
+    def refill(seed):
+        gen_ = torch.Generator().manual_seed(seed)
+        hidden.copy_(torch.randn(B * S, H, generator=gen_).bfloat16())
+        labels.copy_(torch.randint(0, V, (B * S,), generator=gen_))
+        old.copy_(torch.randn(B, S, generator=gen_) * 0.1 - 7.0)
+        adv.copy_(torch.randn(B, S, generator=gen_))
+        mask.copy_((torch.rand(B, S, generator=gen_) < 0.2 * seed).float())
+
+    refill(1)
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream(dev).wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step()
+    for seed in (2, 4, 0, 3):               # 40 %, 80 %, none and 60 % of the tokens active
+        refill(seed)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in captured]
+        want = step()
+        torch.cuda.synchronize()
+        for a, b in zip(got, want):
+            assert torch.equal(a, b)
+        assert float(got[1][(mask.reshape(-1) == 0)].abs().max() if (mask == 0).any() else 0.0) == 0.0
 
 
 def test_vocab_shards_reproduce_the_full_vocabulary(cuda_device):
