@@ -120,9 +120,9 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-mfma-probe", action="store_true")
     ap.add_argument("--skip-masked-rows", action="store_true",
-                    help="run the backward pass through skyrl_amd.ops.lmhead_bwd_active_rows, which drops the tokens whose "
-                         "upstream gradients are zero (the configurations with a response mask); value stays tokens/s over "
-                         "all T tokens, the roofline figures count the flop actually executed")
+                    help="run the backward pass through skyrl_lmhead_bwd_active_rows, which drops the tokens whose upstream "
+                         "gradients are zero on the device (the configurations with a response mask); value stays tokens/s "
+                         "over all T tokens, the roofline figures count the flop actually executed")
     ap.add_argument("--frozen-lm-head", action="store_true",
                     help="the weight takes no gradient (adapter training): d_weight = NULL, the dW product is skipped")
     ap.add_argument("--copy-probe", action="store_true",
@@ -166,7 +166,10 @@ def main() -> int:
     if cfg.backward:
         d_hidden = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
         d_weight = torch.empty(V, H, **f32)
-        ws_b = torch.empty(ops.bwd_workspace_bytes(T, H, V, args.vocab_chunk), dtype=torch.uint8, device=dev)
+        skip_rows = bool(args.skip_masked_rows)
+        bwd_query = lib.skyrl_lmhead_bwd_active_rows_workspace_bytes if skip_rows else lib.skyrl_lmhead_bwd_workspace_bytes
+        bwd_entry = lib.skyrl_lmhead_bwd_active_rows if skip_rows else lib.skyrl_lmhead_bwd
+        ws_b = torch.empty(int(bwd_query(T, H, V, args.vocab_chunk)), dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream(dev).cuda_stream
     ptr = lambda t: None if t is None else t.data_ptr()  # noqa: E731
 
@@ -178,11 +181,8 @@ def main() -> int:
                                   T, H, V, rcp_t, logprobs.data_ptr(), ptr(entropy), row_lse.data_ptr(), ptr(row_pz),
                                   ws_f.data_ptr(), ws_f.numel(), stream)
         _lib.check(st, "skyrl_lmhead_fwd")
-        if skip:
-            ops.lmhead_bwd_active_rows(hidden, weight, labels, row_lse, row_pz if q is not None else None, g, q, rcp_t,
-                                       args.vocab_chunk, want_dweight=not args.frozen_lm_head)
-        elif cfg.backward:
-            st = lib.skyrl_lmhead_bwd(hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0),
+        if cfg.backward:
+            st = bwd_entry(hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0),
                                       labels.data_ptr(), row_lse.data_ptr(), ptr(row_pz) if q is not None else None,
                                       g.data_ptr(), ptr(q), T, H, V, rcp_t, d_hidden.data_ptr(),
                                       None if args.frozen_lm_head else d_weight.data_ptr(), 0,
@@ -283,14 +283,31 @@ def main() -> int:
             "max_clock_mhz": box_khz / 1e3,
             "peak_from_box_tflops": box_cus * 4096 * box_khz * 1e3 / 1e12,
         },
+        "scratch_bytes": {"forward": ws_f.numel(), "backward": ws_b.numel() if cfg.backward else 0,
+                          "one_bf16_TxV_buffer_would_be": 2 * T * V},
         "tflops": step_roofline["achieved"],
         "pct_of_bf16_mfma_peak": 100.0 * step_roofline["frac"],
         "roofline": roofline,
         "step_roofline": step_roofline,
         "kernels": kernels,
     }
-    if not args.no_mfma_probe:
-        out["mfma_probe"] = mfma_probe(lib, dev)
+    # Each MFMA kernel against the published peak and against what the matrix pipe of this box sustains on random operands
+    # with nothing else in the loop (the power-limited ceiling of any bf16 kernel on this data).
+    kind_flop = {"lmhead_fwd_tiles": 2.0 * T * V * H}
+    if cfg.backward:
+        kind_flop["lmhead_bwd_chunk[dz]"] = 2.0 * t_active * V * H
+        kind_flop["lmhead_bwd_chunk[gemm]"] = 2.0 * (bwd_gemms - 1.0) * t_active * V * H
+    probe = None if args.no_mfma_probe else mfma_probe(lib, dev)
+    per_kernel = {}
+    for name, fl in kind_flop.items():
+        if name in kernels:
+            tf = fl / (kernels[name]["ms_per_step"] * 1e-3) / 1e12
+            per_kernel[name] = {"tflops": tf, "frac_of_peak": tf / (PEAK_BF16_DENSE_FLOPS / 1e12),
+                                "frac_of_mfma_probe_random": (tf / probe["random_operands_tflops"]) if probe else None}
+    out["mfma_kernels"] = per_kernel
+    if probe:
+        out["mfma_probe"] = probe
+        out["step_frac_of_mfma_probe_random"] = step_roofline["achieved"] / probe["random_operands_tflops"]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_sample_tokens)
     print(json.dumps(out))

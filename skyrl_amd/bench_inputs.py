@@ -27,6 +27,8 @@ class LmHeadConfig:
     layout: str = "dense"         # "dense": n_seqs x seq_len; "packed": variable lengths
     n_seqs: int = 1
     mask: str = "none"            # "none" | "prefix50" | "suffix30_90"
+    weight_scale: float = 3.0     # weight ~ N(0, (weight_scale / sqrt(H))^2)
+    upstream: str = "randn"       # "randn": dlogprobs ~ N(0,1) * mask; "minus_one": the gradient of (-logprobs).sum()
 
     @property
     def fwd_flop(self) -> float:
@@ -48,6 +50,14 @@ CONFIGS: Dict[str, LmHeadConfig] = {
         LmHeadConfig("qwen3-32b-fwd", 4, T=32768, H=5120, V=151936, backward=False, entropy=False, n_seqs=16),
     ]
 }
+
+# The long-context sweep of the reference's own harness (skyrl/benchmarks/bench_fused_linear_logprob.py:39-47, 90-97):
+# H = 2048, the vocabulary of one TP=4 shard (62080) or the full one (248320), one sequence of S tokens,
+# hidden ~ N(0,1), weight ~ N(0, 1/H), loss = (-logprobs).sum().  Not part of the five benchmark configurations; these
+# are the shapes for which the fused path exists ("what makes 262k fit", model_utils.py:289-293).
+for _i, (_s, _v) in enumerate([(65536, 62080), (262144, 62080), (65536, 248320), (262144, 248320)]):
+    _c = LmHeadConfig(f"longctx-s{_s}-v{_v}", 5 + _i, T=_s, H=2048, V=_v, entropy=False, weight_scale=1.0, upstream="minus_one")
+    CONFIGS[_c.name] = _c
 
 # Same structure (masks, temperature, packing, ragged edges) at sizes a CPU checker finishes in seconds.
 SMALL_TWINS: Dict[str, LmHeadConfig] = {
@@ -75,12 +85,18 @@ def make_inputs(cfg: LmHeadConfig, seed: Optional[int] = None) -> Dict[str, torc
     dentropy [T] fp32 (if entropy_grad), cu_seqlens [n+1] int64."""
     gen = torch.Generator().manual_seed(1000 + cfg.index if seed is None else seed)
     T, H, V = cfg.T, cfg.H, cfg.V
-    hidden = torch.randn(T, H, generator=gen, dtype=torch.float32).to(torch.bfloat16)
+    rows = max(1, (1 << 24) // H)  # generate hidden and weight in slabs: no [T,H] or [V,H] fp32 temporary
+    hidden = torch.empty(T, H, dtype=torch.bfloat16)
+    if T <= rows:  # (one draw for the sizes that existed before the slabs, so their bits stay what they were)
+        hidden.copy_(torch.randn(T, H, generator=gen, dtype=torch.float32))
+    else:
+        for r0 in range(0, T, rows):
+            r1 = min(T, r0 + rows)
+            hidden[r0:r1] = torch.randn(r1 - r0, H, generator=gen, dtype=torch.float32).to(torch.bfloat16)
     weight = torch.empty(V, H, dtype=torch.bfloat16)
-    rows = max(1, (1 << 24) // H)  # generate the weight in slabs: no [V,H] fp32 temporary
     for r0 in range(0, V, rows):
         r1 = min(V, r0 + rows)
-        weight[r0:r1] = (torch.randn(r1 - r0, H, generator=gen, dtype=torch.float32) * (3.0 / H**0.5)).to(torch.bfloat16)
+        weight[r0:r1] = (torch.randn(r1 - r0, H, generator=gen, dtype=torch.float32) * (cfg.weight_scale / H**0.5)).to(torch.bfloat16)
     labels = torch.randint(0, V, (T,), generator=gen, dtype=torch.int64)
 
     if cfg.layout == "packed":
@@ -103,7 +119,9 @@ def make_inputs(cfg: LmHeadConfig, seed: Optional[int] = None) -> Dict[str, torc
             mask[int(cu[i]) : int(cu[i]) + n - keep] = 0.0
 
     out = {"hidden": hidden, "weight": weight, "labels": labels, "mask": mask, "cu_seqlens": cu}
-    if cfg.backward:
+    if cfg.backward and cfg.upstream == "minus_one":
+        out["dlogprobs"] = -mask
+    elif cfg.backward:
         out["dlogprobs"] = torch.randn(T, generator=gen, dtype=torch.float32) * mask
     if cfg.entropy_grad:
         out["dentropy"] = torch.randn(T, generator=gen, dtype=torch.float32) * 0.01

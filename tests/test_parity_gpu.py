@@ -1546,6 +1546,17 @@ def test_full_size_forward_qwen32b(cuda_device):
     _full_size_check(CONFIGS["qwen3-32b-fwd"], cuda_device)
 
 
+def test_full_size_long_context_262k(cuda_device):
+    """One sequence of 262144 tokens at H = 2048 against one TP=4 vocabulary shard (62080 columns), the long-context point of
+    the reference's harness (skyrl/benchmarks/bench_fused_linear_logprob.py:39-47): eight token blocks in both passes, dW
+    summed over them, scratch sized by the block."""
+    cfg = CONFIGS["longctx-s262144-v62080"]
+    T, H, V = cfg.T, cfg.H, cfg.V
+    assert ops.fwd_workspace_bytes(T, H, V) == ops.fwd_workspace_bytes(32768, H, V)
+    assert ops.bwd_workspace_bytes(T, H, V) < 2 * 32768 * V // 2 + 4 * V * H + (1 << 30)  # nothing of the size of T x V (32 GB in bf16)
+    _full_size_check(cfg, cuda_device, n_rows=16, n_vocab=8)
+
+
 # ---------------------------------------------------------------------------------------------------------------------
 # MTP draft loss: soft cross-entropy from hidden states
 # ---------------------------------------------------------------------------------------------------------------------
