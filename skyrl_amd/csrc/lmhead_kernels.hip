@@ -361,6 +361,18 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
   char* stage = lds + wave * kStage;
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
+  // A token block j (16 token rows x 128 vocab, 4 KiB of the staging region) is complete after its eight i-steps; its 256
+  // 16-byte pieces (4 per lane; 16 lanes cover one token row of 256 bytes) go out in the middle of block j + 1, so that the
+  // read-back and the store issue hide behind that block's arithmetic instead of forming a tail of their own.
+  auto flush_block = [&](int j) {
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int idx = it * 64 + lane;
+      const int n = j * MT + (idx >> 4), c = idx & 15;  // token row, 8-vocab piece
+      const u32x4 v = *(const u32x4*)(stage + n * kTokRow + c * 16);
+      __builtin_nontemporal_store(v, (u32x4*)(D + (size_t)(tbase + n) * (size_t)ldd + vloc_base + c * 8));
+    }
+  };
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const float gs = gs_[j], c0 = c0_[j], c1 = c1_[j], lse2 = lse2_[j];
@@ -389,16 +401,10 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
       f32x4 v4 = {d[0], d[1], d[2], d[3]};
       const bf16x4 b4 = __builtin_convertvector(v4, bf16x4);
       *(uint2*)(stage + (j * MT + lrow) * kTokRow + vl * 2) = *(const uint2*)&b4;
+      if (i == TM / 2 - 1 && j > 0) flush_block(j - 1);
     }
   }
-  // 128 tokens x 128 vocab staged: 2048 16-byte pieces, 32 per lane; 16 lanes cover one token row (256 bytes).
-#pragma unroll
-  for (int it = 0; it < 32; ++it) {
-    const int idx = it * 64 + lane;
-    const int n = idx >> 4, c = idx & 15;  // token row, 8-vocab piece
-    const u32x4 v = *(const u32x4*)(stage + n * kTokRow + c * 16);
-    __builtin_nontemporal_store(v, (u32x4*)(D + (size_t)(tbase + n) * (size_t)ldd + vloc_base + c * 8));
-  }
+  flush_block(TN - 1);
 }
 
 
@@ -520,6 +526,15 @@ __global__ __launch_bounds__(NTHREADS) void softce_dz_tiles(const SoftCeDzArgs z
   constexpr int kStage = WN * kTokRow;
   char* stage = lds + wave * kStage;
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  auto flush_block = [&](int j) {  // as in dz_tile: a finished token block leaves while the next one is computed
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int idx = it * 64 + lane;
+      const int n = j * MT + (idx >> 4), c = idx & 15;
+      const u32x4 v = *(const u32x4*)(stage + n * kTokRow + c * 16);
+      __builtin_nontemporal_store(v, (u32x4*)(D + (size_t)(tokbase + n) * (size_t)ldd + vloc_base + c * 8));
+    }
+  };
 #pragma unroll
   for (int j = 0; j < TN / 2; ++j) {
     const float gs = gs_[j], ls2 = ls2_[j], lt2 = lt2_[j];
@@ -541,15 +556,10 @@ __global__ __launch_bounds__(NTHREADS) void softce_dz_tiles(const SoftCeDzArgs z
       f32x4 v4 = {d[0], d[1], d[2], d[3]};
       const bf16x4 b4 = __builtin_convertvector(v4, bf16x4);
       *(uint2*)(stage + (j * MT + lrow) * kTokRow + vl * 2) = *(const uint2*)&b4;
+      if (i == TM / 2 - 1 && j > 0) flush_block(j - 1);
     }
   }
-#pragma unroll
-  for (int it = 0; it < 16; ++it) {
-    const int idx = it * 64 + lane;
-    const int n = idx >> 4, c = idx & 15;
-    const u32x4 v = *(const u32x4*)(stage + n * kTokRow + c * 16);
-    __builtin_nontemporal_store(v, (u32x4*)(D + (size_t)(tokbase + n) * (size_t)ldd + vloc_base + c * 8));
-  }
+  flush_block(TN / 2 - 1);
 }
 
 // ------------------------------------------------------------------------------------------------------------
