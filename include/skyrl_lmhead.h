@@ -147,6 +147,41 @@ int skyrl_lmhead_bwd_active_rows(const void* hidden, int64_t ld_hidden, const vo
                                  void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * fp32 operands.  The reference casts hidden to the weight's dtype and forms fp32 logits when the output weight is fp32
+ * (model_utils.py:328-333; its tests cover (bf16 hidden, fp32 weight) -- "the real Megatron case" -- and (fp32, fp32),
+ * tests/backends/skyrl_train/gpu/gpu_ci/megatron/test_fused_linear_logprob.py:99-103).  The matrix pipe multiplies bf16, so
+ * an fp32 operand is given to it as a sum of bf16 terms, x = hi + lo with hi = bf16(x), lo = bf16(x - hi) (exact to 2^-17),
+ * stacked along the contraction axis; the MFMA accumulates all terms in fp32:
+ *     weight fp32, hidden bf16:   weight' = [w_hi | w_lo]         hidden' = [h | h]                 (terms = 2)
+ *     weight fp32, hidden fp32:   weight' = [w_hi | w_lo | w_hi]  hidden' = [h_hi | h_hi | h_lo]    (terms = 3)
+ * so that hidden' . weight'^T = h . w up to the dropped lo x lo products (below 2^-16 of each product; measured: log-probabilities
+ * within 1e-5 of the fp32 product at the reference's test shapes).  Nothing is down-cast silently, and no kernel is special:
+ *   skyrl_lmhead_split_operand  writes one stacked operand: src [rows, H] (fp32, or bf16 with src_is_fp32 = 0), dst bf16
+ *                               [rows, terms * H] with leading dimension ld_dst, layout one of SKYRL_SPLIT_*
+ *   skyrl_lmhead_fwd            is called on the stacked operands with H' = terms * H
+ *   skyrl_lmhead_bwd_split      is skyrl_lmhead_bwd (active_rows = 0) or skyrl_lmhead_bwd_active_rows (active_rows = 1) on the
+ *                               stacked operands: the logits are recomputed over all terms * H columns, dz is rounded to bf16
+ *                               once as always, and the two gradient GEMMs use the leading H columns (the hi terms):
+ *                               d_hidden bf16 [T, H], d_weight [V, H] by dw_mode.  Gradients therefore carry bf16 rounding of
+ *                               dz and of the multiplied operand (2^-9 per element, inside the reference's 2e-3 tolerance).
+ * Cost: the two logits GEMMs take terms times as long; the gradient GEMMs are unchanged.
+ */
+#define SKYRL_SPLIT_HI_LO 0
+#define SKYRL_SPLIT_HI_HI 1
+#define SKYRL_SPLIT_HI_LO_HI 2
+#define SKYRL_SPLIT_HI_HI_LO 3
+int skyrl_lmhead_split_operand(const void* src, int src_is_fp32, int64_t ld_src, int64_t rows, int64_t H, int layout,
+                               void* dst, int64_t ld_dst, void* stream);
+size_t skyrl_lmhead_bwd_split_workspace_bytes(int64_t T, int64_t H, int64_t terms, int64_t V, int64_t vocab_chunk,
+                                              int active_rows);
+int skyrl_lmhead_bwd_split(const void* hidden_terms, int64_t ld_hidden, const void* weight_terms, int64_t ld_weight,
+                           const int64_t* labels, const float* row_lse, const float* row_pz,
+                           const float* dlogprobs, const float* dentropy,
+                           int64_t T, int64_t H, int64_t terms, int64_t V, float rcp_temperature,
+                           void* d_hidden, void* d_weight, int dw_mode, int64_t vocab_chunk, int active_rows,
+                           void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * The consumer one step after the log-probabilities: the policy loss and its gradient with respect to the
  * log-probabilities in one pass -- what the reference computes with elementwise torch kernels plus autograd
  * (skyrl/backends/skyrl_train/utils/ppo_utils.py; safe_exp_delta / masked_mean of

@@ -11,7 +11,7 @@ import os
 import threading
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libskyrl_lmhead.so")
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 _c_i64 = ctypes.c_int64
 _c_p = ctypes.c_void_p
@@ -42,6 +42,13 @@ SIGNATURES = {
         ctypes.c_int,
         [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, ctypes.c_float, _c_p, _c_p,
          ctypes.c_int, _c_i64, _c_p, ctypes.c_size_t, _c_p],
+    ),
+    "skyrl_lmhead_split_operand": (ctypes.c_int, [_c_p, ctypes.c_int, _c_i64, _c_i64, _c_i64, ctypes.c_int, _c_p, _c_i64, _c_p]),
+    "skyrl_lmhead_bwd_split_workspace_bytes": (ctypes.c_size_t, [_c_i64, _c_i64, _c_i64, _c_i64, _c_i64, ctypes.c_int]),
+    "skyrl_lmhead_bwd_split": (
+        ctypes.c_int,
+        [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_i64, ctypes.c_float, _c_p, _c_p,
+         ctypes.c_int, _c_i64, ctypes.c_int, _c_p, ctypes.c_size_t, _c_p],
     ),
     "skyrl_ppo_policy_loss": (
         ctypes.c_int,

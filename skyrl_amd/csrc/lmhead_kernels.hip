@@ -296,6 +296,11 @@ struct DzArgs {
   // When not NULL: the number of tokens, <= T, as a value in device memory (what a compaction kernel counted).  T then
   // only sizes the grid: token tiles at or beyond the device-side count return at once.
   const int* T_dev;
+  // When not NULL (fp32 weights): for every token whose label lies in the vocabulary, its label's dz value before the
+  // rounding to bf16, fp32 [T].  That one value per token, g (1 - p) / temperature, is of order 1 where every other dz value
+  // of the row is of order p; the caller adds what the bf16 product dropped of it (label_residual_update) so that the label
+  // rows of dW keep fp32 accuracy.
+  float* label_resid;
 };
 
 template <bool ENTGRAD>
@@ -401,6 +406,11 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
       f32x4 v4 = {d[0], d[1], d[2], d[3]};
       const bf16x4 b4 = __builtin_convertvector(v4, bf16x4);
       *(uint2*)(stage + (j * MT + lrow) * kTokRow + vl * 2) = *(const uint2*)&b4;
+      if (any_label && z.label_resid) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (yrel == vl + r) z.label_resid[tbase + j * MT + lrow] = d[r];
+      }
       if (i == TM / 2 - 1 && j > 0) flush_block(j - 1);
     }
   }
@@ -794,6 +804,50 @@ __global__ __launch_bounds__(256) void transpose_bf16(const uint16_t* __restrict
 }
 
 // ------------------------------------------------------------------------------------------------------------
+// fp32 operands on the bf16 matrix pipe.  An fp32 value is the sum of bf16 terms, x = hi + lo (+ 2^-17 |x|), hi = bf16(x),
+// lo = bf16(x - hi), and a product of sums is a sum of products: stacking the terms along the contraction axis,
+//     weight fp32, hidden bf16:   [w_hi | w_lo] . [h | h]^T           = h . (w_hi + w_lo)
+//     weight fp32, hidden fp32:   [w_hi | w_lo | w_hi] . [h_hi | h_hi | h_lo]^T = h_hi . w_hi + h_hi . w_lo + h_lo . w_hi
+// turns the fp32 logits GEMM (model_utils.py:328-333: hidden is cast to the weight's dtype, the product is fp32) into the
+// ordinary bf16 GEMM with two or three times the contraction length; the MFMA accumulates all terms in fp32.  What is dropped
+// is below 2^-16 of each product.  This kernel writes one stacked operand: segment s of row r holds the hi (code 0) or lo
+// (code 1) terms of the row.
+// ------------------------------------------------------------------------------------------------------------
+__device__ __forceinline__ uint16_t bf16_rne(float x) {
+  const uint32_t u = __float_as_uint(x);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);  // NaN stays NaN
+  return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
+template <bool SRC_FP32>
+__global__ __launch_bounds__(256) void split_operand_rows(const void* __restrict__ src, int64_t ld_src, int H, int terms, int code0,
+                                                          int code1, int code2, uint16_t* __restrict__ dst, int64_t ld_dst) {
+  const int64_t r = blockIdx.x;
+  const int codes[3] = {code0, code1, code2};
+  for (int c = threadIdx.x * 4; c < H; c += 256 * 4) {
+    uint16_t hi[4], lo[4];
+    if (SRC_FP32) {
+      const float4 v = *(const float4*)((const float*)src + r * ld_src + c);
+      const float x[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        hi[k] = bf16_rne(x[k]);
+        lo[k] = bf16_rne(x[k] - __uint_as_float((uint32_t)hi[k] << 16));
+      }
+    } else {
+      const uint2 v = *(const uint2*)((const uint16_t*)src + r * ld_src + c);
+      hi[0] = (uint16_t)(v.x & 0xffffu), hi[1] = (uint16_t)(v.x >> 16), hi[2] = (uint16_t)(v.y & 0xffffu), hi[3] = (uint16_t)(v.y >> 16);
+      lo[0] = lo[1] = lo[2] = lo[3] = 0;
+    }
+    for (int s = 0; s < terms; ++s) {
+      const uint16_t* t = codes[s] ? lo : hi;
+      *(uint2*)(dst + r * ld_dst + (int64_t)s * H + c) =
+          make_uint2((uint32_t)t[0] | ((uint32_t)t[1] << 16), (uint32_t)t[2] | ((uint32_t)t[3] << 16));
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------------------
 // Row compaction for the backward.  A token whose upstream gradients are both zero has a zero dz row: it adds nothing to
 // dW and its dHidden row is zero.  In RL micro-batches those are the prompt and padding tokens the loss mask removes, often
 // more than half of the batch.  Three small kernels let the backward run on the remaining rows without the host ever
@@ -846,7 +900,7 @@ __global__ __launch_bounds__(kCompactThreads) void compact_active_rows(const flo
 // One workgroup per row r < T: as compacted row r (when r < n) it copies the inputs of token idx[r]; as token r it clears
 // d_hidden[r] -- active tokens get their row from scatter_active_rows afterwards.
 __global__ __launch_bounds__(256) void gather_active_rows(const int* __restrict__ idx, const int* __restrict__ counts,
-                                                          const uint16_t* __restrict__ hidden, int ldh, int H,
+                                                          const uint16_t* __restrict__ hidden, int ldh, int Hk, int H,
                                                           const int64_t* __restrict__ labels, const float* __restrict__ lse,
                                                           const float* __restrict__ pz, const float* __restrict__ g,
                                                           const float* __restrict__ q, uint16_t* __restrict__ hidden_c,
@@ -859,8 +913,8 @@ __global__ __launch_bounds__(256) void gather_active_rows(const int* __restrict_
   if (r >= counts[0]) return;
   const int t = idx[r];
   const uint16_t* src = hidden + (size_t)t * (size_t)ldh;
-  uint16_t* dst = hidden_c + (size_t)r * (size_t)H;
-  for (int c = threadIdx.x * 8; c < H; c += 256 * 8) *(uint4*)(dst + c) = *(const uint4*)(src + c);
+  uint16_t* dst = hidden_c + (size_t)r * (size_t)Hk;
+  for (int c = threadIdx.x * 8; c < Hk; c += 256 * 8) *(uint4*)(dst + c) = *(const uint4*)(src + c);
   if (threadIdx.x == 0) {
     labels_c[r] = labels[t];
     lse_c[r] = lse[t];
@@ -879,6 +933,34 @@ __global__ __launch_bounds__(256) void scatter_active_rows(const int* __restrict
   for (int c = threadIdx.x * 8; c < H; c += 256 * 8) *(uint4*)(dst + c) = *(const uint4*)(src + c);
 }
 
+// What the bf16 product dropped of the label's dz value d (see DzArgs::label_resid), added to the weight gradient in fp32:
+//     dW[label_t, :] += (d - bf16(d)) * h_hi[t, :]  +  d * h_lo[t, :]
+// h_lo is the third segment of a stacked fp32 hidden row (lo_offset = 2 * H) and absent (lo_offset = 0) for a bf16 hidden.
+// One workgroup per token; fp32 atomic adds, because several tokens may share a label (their order, and with it the last
+// bit of those rows, is not fixed).
+__global__ __launch_bounds__(256) void label_residual_update(const float* __restrict__ label_dz, const int64_t* __restrict__ labels,
+                                                             const uint16_t* __restrict__ hidden, int ldh, int H, int lo_offset,
+                                                             int V, const int* __restrict__ T_dev, float* __restrict__ dW) {
+  const int t = blockIdx.x;
+  if (T_dev && t >= *T_dev) return;
+  const float d = label_dz[t];
+  const int64_t y = labels[t];
+  if (d == 0.f || y < 0 || y >= (int64_t)V) return;
+  const float r = d - __uint_as_float((uint32_t)bf16_rne(d) << 16);
+  const uint16_t* hp = hidden + (size_t)t * (size_t)ldh;
+  float* wp = dW + (size_t)y * (size_t)H;
+  for (int c = threadIdx.x; c < H; c += 256) {
+    float add = r * __uint_as_float((uint32_t)hp[c] << 16);
+    if (lo_offset) add = fmaf(d, __uint_as_float((uint32_t)hp[lo_offset + c] << 16), add);
+    atomicAdd(wp + c, add);
+  }
+}
+
+__global__ __launch_bounds__(256) void zero_f32(float* __restrict__ p, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0.f;
+}
+
 // ------------------------------------------------------------------------------------------------------------
 // Host side
 // ------------------------------------------------------------------------------------------------------------
@@ -886,13 +968,13 @@ __global__ __launch_bounds__(256) void scatter_active_rows(const int* __restrict
 // HIP events on the launch stream.  Closed profiles cost one thread-local load per launch.
 enum KernelKind {
   kFwdTiles = 0, kFwdMerge, kTranspose, kBwdChunkDz, kBwdChunkGemm, kSoftCePack, kSoftCeFwdTiles, kSoftCeFinish, kSoftCeDz,
-  kCompactRows,
+  kCompactRows, kSplitOperand,
   kNumKernelKinds
 };
 const char* const kKernelNames[kNumKernelKinds] = {"lmhead_fwd_tiles", "lmhead_fwd_merge", "transpose_bf16",
                                                    "lmhead_bwd_chunk[dz]", "lmhead_bwd_chunk[gemm]", "softce_pack_rows",
                                                    "softce_fwd_tiles", "softce_finish", "softce_dz_tiles",
-                                                   "active_rows[compact+gather+scatter]"};
+                                                   "active_rows[compact+gather+scatter]", "split_operand_rows"};
 struct Profile {
   struct Rec {
     int kind;
@@ -1121,7 +1203,7 @@ constexpr int64_t kBwdTokenBlock = 32768;
 
 struct BwdWorkspace {
   uint16_t *Wt, *Ht, *D;
-  float *dHacc, *dWsum;
+  float *dHacc, *dWsum, *label_resid;
   // only with row compaction (skyrl_lmhead_bwd_active_rows):
   uint16_t *hidden_c, *d_hidden_c;
   int64_t* labels_c;
@@ -1139,7 +1221,8 @@ inline int64_t bwd_block_tokens(int64_t T) { return T < kBwdTokenBlock ? T : kBw
 inline int64_t bwd_num_blocks(int64_t T) { return (T + kBwdTokenBlock - 1) / kBwdTokenBlock; }
 
 // vc: chunk width for a block of bwd_block_tokens(T) tokens.  compact: the buffers of the row-compacting entry point.
-BwdWorkspace carve_bwd(void* ws, int64_t T, int64_t H, int64_t V, int64_t vc, bool compact) {
+// Hk: length of the logits contraction, a multiple of H when the operands are stacked bf16 terms of fp32 values.
+BwdWorkspace carve_bwd(void* ws, int64_t T, int64_t H, int64_t Hk, int64_t V, int64_t vc, bool compact) {
   const int64_t Tb = bwd_block_tokens(T), Tpad = round_up(Tb, 256), Vpad = round_up(V, 256);
   Carver c(ws);
   BwdWorkspace w{};
@@ -1149,8 +1232,9 @@ BwdWorkspace carve_bwd(void* ws, int64_t T, int64_t H, int64_t V, int64_t vc, bo
   w.D = c.take<uint16_t>((size_t)Tpad * (vc + kLdPad));
   // Several blocks and a bf16 dW: the sum over the blocks is kept in fp32 here and rounded once, by the last block.
   w.dWsum = bwd_num_blocks(T) > 1 ? c.take<float>((size_t)V * (size_t)H) : nullptr;
+  w.label_resid = Hk > H ? c.take<float>((size_t)Tpad) : nullptr;  // stacked terms: fp32 operands
   if (compact) {
-    w.hidden_c = c.take<uint16_t>((size_t)T * (size_t)H);
+    w.hidden_c = c.take<uint16_t>((size_t)T * (size_t)Hk);
     w.d_hidden_c = c.take<uint16_t>((size_t)T * (size_t)H);
     w.labels_c = c.take<int64_t>((size_t)T);
     w.lse_c = c.take<float>((size_t)T);
@@ -1249,20 +1333,21 @@ hipError_t launch_softce_pack(hipStream_t s, const void* student, int64_t lds_, 
   return hipGetLastError();
 }
 
-size_t bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t vocab_chunk, bool compact) {
-  if (T < 1 || V < 1 || H < 1 || vocab_chunk < 0 || vocab_chunk % 256 != 0) return 0;
-  if (T > kMaxExtent || V > kMaxExtent || H > kMaxExtent || vocab_chunk > kMaxExtent) return 0;
+size_t bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t vocab_chunk, bool compact, int64_t terms = 1) {
+  if (T < 1 || V < 1 || H < 1 || vocab_chunk < 0 || vocab_chunk % 256 != 0 || terms < 1 || terms > 3) return 0;
+  if (T > kMaxExtent || V > kMaxExtent || H > kMaxExtent / 4 || vocab_chunk > kMaxExtent) return 0;
   int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(bwd_block_tokens(T), H, V);
   if (vc > round_up(V, 256)) vc = round_up(V, 256);
-  return carve_bwd(nullptr, T, H, V, vc, compact).bytes;
+  return carve_bwd(nullptr, T, H, terms * H, V, vc, compact).bytes;
 }
 
-// One token block of the backward: the vocab-chunk loop.  `Tb` tokens (an upper bound when `T_dev` points at the block's
+// One token block of the backward: the vocab-chunk loop.  Hk is the contraction length of the logits recompute (H, or a
+// multiple of it for stacked bf16 terms, in which case the two gradient GEMMs use the leading H columns: the hi terms).  `Tb` tokens (an upper bound when `T_dev` points at the block's
 // count in device memory), per-token inputs and d_hidden already offset to the block.  dW of every chunk leaves the GEMM
 // epilogue as  (Cin ? Cin : 0) + product  ->  Cf (fp32) and / or Cb (bf16), each a [V, H] matrix or NULL.
 int bwd_token_block(const uint16_t* Hp, int64_t ld_hidden, const uint16_t* Wp, int64_t ld_weight, const int64_t* labels,
                     const float* row_lse, const float* row_pz, const float* dlogprobs, const float* dentropy, int64_t Tb,
-                    const int* T_dev, int64_t H, int64_t V, float rcp_temperature, uint16_t* d_hidden, bool want_dw,
+                    const int* T_dev, int64_t H, int64_t Hk, int64_t V, float rcp_temperature, uint16_t* d_hidden, bool want_dw,
                     const float* dw_in, float* dw_f32, uint16_t* dw_bf16, int64_t vc, const BwdWorkspace& w, hipStream_t s) {
   const int64_t Tpad = round_up(Tb, 256), Vpad = round_up(V, 256);
   const bool w_in_place = reads_weight_in_place(V);
@@ -1271,6 +1356,12 @@ int bwd_token_block(const uint16_t* Hp, int64_t ld_hidden, const uint16_t* Wp, i
     Timed timed(kTranspose, s);
     hipLaunchKernelGGL(transpose_bf16, dim3((unsigned)(Tpad / 64), (unsigned)(H / 64)), dim3(256), 0, s, Hp, (int)ld_hidden,
                        (int)Tb, (int)H, w.Ht, (int)(Tpad + kLdPad), (int)Tpad, T_dev);
+    if ((e = hipGetLastError()) != hipSuccess) return (int)e;
+  }
+  // fp32 operands (stacked terms) with an fp32 dW: the label's dz value keeps fp32 accuracy through a residual (DzArgs).
+  float* resid = (Hk > H && want_dw && dw_f32) ? w.label_resid : nullptr;
+  if (resid) {
+    hipLaunchKernelGGL(zero_f32, dim3((unsigned)(Tpad / 256)), dim3(256), 0, s, resid, (int)Tpad);
     if ((e = hipGetLastError()) != hipSuccess) return (int)e;
   }
   const int tiles_t = (int)(Tpad / 256);
@@ -1282,8 +1373,8 @@ int bwd_token_block(const uint16_t* Hp, int64_t ld_hidden, const uint16_t* Wp, i
     // Carrying the next chunk's dz tiles in the GEMM launch (to fill its tail) was measured: no gain at the default chunk
     // width, and it needs a second panel.
     const int64_t vc0 = ci * vc, vcw = chunk_width(ci);
-    const DzArgs z{Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)Tb, (int)H, (int)V, rcp_temperature, labels, row_lse, row_pz,
-                   dlogprobs, dentropy, (int)vc0, (int)(vcw / 256), tiles_t, w.D, (int)(vcw + kLdPad), T_dev};
+    const DzArgs z{Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)Tb, (int)Hk, (int)V, rcp_temperature, labels, row_lse, row_pz,
+                   dlogprobs, dentropy, (int)vc0, (int)(vcw / 256), tiles_t, w.D, (int)(vcw + kLdPad), T_dev, resid};
     e = launch_bwd_chunk(s, dentropy != nullptr, z, (unsigned)(vcw / 256 * tiles_t), false, none, none);
     if (e != hipSuccess) return (int)e;
     // dHidden[t, h] (+)= sum_v D[t, v] . weight^T[h, vc0 + v]        (A = weight^T rows at k offset vc0, B = D rows)
@@ -1313,15 +1404,23 @@ int bwd_token_block(const uint16_t* Hp, int64_t ld_hidden, const uint16_t* Wp, i
     e = launch_bwd_chunk(s, dentropy != nullptr, DzArgs{}, 0, true, gh, gw);
     if (e != hipSuccess) return (int)e;
   }
+  if (resid) {
+    hipLaunchKernelGGL(label_residual_update, dim3((unsigned)Tb), dim3(256), 0, s, (const float*)resid, labels, Hp, (int)ld_hidden,
+                       (int)H, Hk == 3 * H ? (int)(2 * H) : 0, (int)V, T_dev, dw_f32);
+    if ((e = hipGetLastError()) != hipSuccess) return (int)e;
+  }
   return SKYRL_LMHEAD_OK;
 }
 
 int bwd_entry(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight, const int64_t* labels,
               const float* row_lse, const float* row_pz, const float* dlogprobs, const float* dentropy, int64_t T, int64_t H,
               int64_t V, float rcp_temperature, void* d_hidden, void* d_weight, int dw_mode, int64_t vocab_chunk,
-              void* workspace, size_t workspace_bytes, hipStream_t s, bool compact) {
-  int st = check_common(hidden, ld_hidden, weight, ld_weight, labels, T, H, V, rcp_temperature, true);
+              void* workspace, size_t workspace_bytes, hipStream_t s, bool compact, int64_t terms = 1) {
+  if (terms < 1 || terms > 3 || H < 1 || H > kMaxExtent / 4) return SKYRL_LMHEAD_ERR_ARG;
+  const int64_t Hk = terms * H;
+  int st = check_common(hidden, ld_hidden, weight, ld_weight, labels, T, Hk, V, rcp_temperature, true);
   if (st) return st;
+  if (H % BK != 0) return SKYRL_LMHEAD_ERR_SHAPE;
   if (!row_lse || !dlogprobs || !d_hidden) return SKYRL_LMHEAD_ERR_NULL;
   if (dentropy && !row_pz) return SKYRL_LMHEAD_ERR_NULL;
   if (!aligned16(d_hidden) || !aligned16(d_weight)) return SKYRL_LMHEAD_ERR_ALIGN;  // d_weight NULL: no dW wanted
@@ -1332,13 +1431,13 @@ int bwd_entry(const void* hidden, int64_t ld_hidden, const void* weight, int64_t
   int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(Tb, H, V);
   if (vc > Vpad) vc = Vpad;
   // 32-bit byte offsets inside a block of hidden rows and inside the scratch matrices (weight^T, hidden^T, the dz panel)
-  if (Tb * ld_hidden * 2 >= ((int64_t)1 << 32) || H * (Vpad + kLdPad) * 2 >= ((int64_t)1 << 32) ||
+  if (Tb * ld_hidden * 2 >= ((int64_t)1 << 32) || Tb * Hk * 2 >= ((int64_t)1 << 32) || H * (Vpad + kLdPad) * 2 >= ((int64_t)1 << 32) ||
       H * (Tbpad + kLdPad) * 2 >= ((int64_t)1 << 32) || Tbpad * (vc + kLdPad) * 2 >= ((int64_t)1 << 32))
     return SKYRL_LMHEAD_ERR_SHAPE;
-  if (!workspace || workspace_bytes < bwd_workspace_bytes(T, H, V, vc, compact)) return SKYRL_LMHEAD_ERR_WORKSPACE;
+  if (!workspace || workspace_bytes < bwd_workspace_bytes(T, H, V, vc, compact, terms)) return SKYRL_LMHEAD_ERR_WORKSPACE;
   if ((uintptr_t)workspace & 255u) return SKYRL_LMHEAD_ERR_ALIGN;
 
-  const BwdWorkspace w = carve_bwd(workspace, T, H, V, vc, compact);
+  const BwdWorkspace w = carve_bwd(workspace, T, H, Hk, V, vc, compact);
   const uint16_t* Wp = (const uint16_t*)weight;
   const uint16_t* Hp = (const uint16_t*)hidden;
   const int64_t nblocks = bwd_num_blocks(T);
@@ -1349,8 +1448,8 @@ int bwd_entry(const void* hidden, int64_t ld_hidden, const void* weight, int64_t
     hipLaunchKernelGGL(compact_active_rows, dim3(1), dim3(kCompactThreads), 0, s, dlogprobs, dentropy, (int)T, (int)Tb,
                        (int)nblocks, w.idx, w.counts);
     hipLaunchKernelGGL(gather_active_rows, dim3((unsigned)T), dim3(256), 0, s, (const int*)w.idx, (const int*)w.counts, Hp,
-                       (int)ld_hidden, (int)H, labels, row_lse, row_pz, dlogprobs, dentropy, w.hidden_c, w.labels_c, w.lse_c,
-                       w.pz_c, w.g_c, w.q_c, (uint16_t*)d_hidden);
+                       (int)ld_hidden, (int)Hk, (int)H, labels, row_lse, row_pz, dlogprobs, dentropy, w.hidden_c, w.labels_c,
+                       w.lse_c, w.pz_c, w.g_c, w.q_c, (uint16_t*)d_hidden);
     if ((e = hipGetLastError()) != hipSuccess) return (int)e;
   }
   if (!reads_weight_in_place(V)) {  // weight^T [H, Vpad], zero in the padding columns
@@ -1383,14 +1482,14 @@ int bwd_entry(const void* hidden, int64_t ld_hidden, const void* weight, int64_t
       }
     }
     if (compact) {
-      st = bwd_token_block(w.hidden_c + (size_t)t0 * (size_t)H, H, Wp, ld_weight, w.labels_c + t0, w.lse_c + t0,
+      st = bwd_token_block(w.hidden_c + (size_t)t0 * (size_t)Hk, Hk, Wp, ld_weight, w.labels_c + t0, w.lse_c + t0,
                            dentropy ? w.pz_c + t0 : nullptr, w.g_c + t0, dentropy ? w.q_c + t0 : nullptr, Tcur,
-                           w.counts + 1 + b, H, V, rcp_temperature, w.d_hidden_c + (size_t)t0 * (size_t)H, d_weight != nullptr,
+                           w.counts + 1 + b, H, Hk, V, rcp_temperature, w.d_hidden_c + (size_t)t0 * (size_t)H, d_weight != nullptr,
                            dw_in, dw_f32, dw_bf16, vc, w, s);
     } else {
       st = bwd_token_block(Hp + (size_t)t0 * (size_t)ld_hidden, ld_hidden, Wp, ld_weight, labels + t0, row_lse + t0,
                            row_pz ? row_pz + t0 : nullptr, dlogprobs + t0, dentropy ? dentropy + t0 : nullptr, Tcur, nullptr, H,
-                           V, rcp_temperature, (uint16_t*)d_hidden + (size_t)t0 * (size_t)H, d_weight != nullptr, dw_in, dw_f32,
+                           Hk, V, rcp_temperature, (uint16_t*)d_hidden + (size_t)t0 * (size_t)H, d_weight != nullptr, dw_in, dw_f32,
                            dw_bf16, vc, w, s);
     }
     if (st) return st;
@@ -1408,7 +1507,7 @@ int bwd_entry(const void* hidden, int64_t ld_hidden, const void* weight, int64_t
 
 extern "C" {
 
-int skyrl_lmhead_version(void) { return 14; }
+int skyrl_lmhead_version(void) { return 15; }
 
 const char* skyrl_lmhead_strerror(int status) {
   switch (status) {
@@ -1489,6 +1588,48 @@ int skyrl_lmhead_bwd_active_rows(const void* hidden, int64_t ld_hidden, const vo
                                  void* stream) {
   return bwd_entry(hidden, ld_hidden, weight, ld_weight, labels, row_lse, row_pz, dlogprobs, dentropy, T, H, V, rcp_temperature,
                    d_hidden, d_weight, dw_mode, vocab_chunk, workspace, workspace_bytes, (hipStream_t)stream, true);
+}
+
+size_t skyrl_lmhead_bwd_split_workspace_bytes(int64_t T, int64_t H, int64_t terms, int64_t V, int64_t vocab_chunk,
+                                              int active_rows) {
+  return bwd_workspace_bytes(T, H, V, vocab_chunk, active_rows != 0, terms);
+}
+
+int skyrl_lmhead_bwd_split(const void* hidden_terms, int64_t ld_hidden, const void* weight_terms, int64_t ld_weight,
+                           const int64_t* labels, const float* row_lse, const float* row_pz, const float* dlogprobs,
+                           const float* dentropy, int64_t T, int64_t H, int64_t terms, int64_t V, float rcp_temperature,
+                           void* d_hidden, void* d_weight, int dw_mode, int64_t vocab_chunk, int active_rows, void* workspace,
+                           size_t workspace_bytes, void* stream) {
+  return bwd_entry(hidden_terms, ld_hidden, weight_terms, ld_weight, labels, row_lse, row_pz, dlogprobs, dentropy, T, H, V,
+                   rcp_temperature, d_hidden, d_weight, dw_mode, vocab_chunk, workspace, workspace_bytes, (hipStream_t)stream,
+                   active_rows != 0, terms);
+}
+
+int skyrl_lmhead_split_operand(const void* src, int src_is_fp32, int64_t ld_src, int64_t rows, int64_t H, int layout, void* dst,
+                               int64_t ld_dst, void* stream) {
+  if (!src || !dst) return SKYRL_LMHEAD_ERR_NULL;
+  int terms, codes[3] = {0, 0, 0};
+  switch (layout) {
+    case SKYRL_SPLIT_HI_LO: terms = 2, codes[1] = 1; break;
+    case SKYRL_SPLIT_HI_HI: terms = 2; break;
+    case SKYRL_SPLIT_HI_LO_HI: terms = 3, codes[1] = 1; break;
+    case SKYRL_SPLIT_HI_HI_LO: terms = 3, codes[2] = 1; break;
+    default: return SKYRL_LMHEAD_ERR_ARG;
+  }
+  if (rows < 1 || rows > kMaxExtent || H < 4 || H % 4 != 0 || H > kMaxExtent / 4 || ld_src < H || ld_dst < terms * H ||
+      ld_src > kMaxExtent || ld_dst > kMaxExtent)
+    return SKYRL_LMHEAD_ERR_SHAPE;
+  if (!aligned16(src) || !aligned16(dst) || ld_src % 4 != 0 || ld_dst % 8 != 0) return SKYRL_LMHEAD_ERR_ALIGN;
+  hipStream_t s = (hipStream_t)stream;
+  Timed timed(kSplitOperand, s);
+  if (src_is_fp32)
+    hipLaunchKernelGGL(split_operand_rows<true>, dim3((unsigned)rows), dim3(256), 0, s, src, ld_src, (int)H, terms, codes[0],
+                       codes[1], codes[2], (uint16_t*)dst, ld_dst);
+  else
+    hipLaunchKernelGGL(split_operand_rows<false>, dim3((unsigned)rows), dim3(256), 0, s, src, ld_src, (int)H, terms, codes[0],
+                       codes[1], codes[2], (uint16_t*)dst, ld_dst);
+  const hipError_t e = hipGetLastError();
+  return e == hipSuccess ? SKYRL_LMHEAD_OK : (int)e;
 }
 
 size_t skyrl_softce_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {

@@ -105,7 +105,7 @@ class LinearCrossEntropy(torch.autograd.Function):
         d_hidden, d_weight = ops.lmhead_bwd_active_rows(hidden2, weight, labels1, row_lse, row_pz if q is not None else None,
                                                         g, q, ctx.rcp_t, 0, want_dweight=ctx.needs_input_grad[1],
                                                         dweight_dtype=weight.dtype)   # None for a frozen LM head
-        return d_hidden.view(ctx.original_hidden_shape), d_weight, None, None, None, None, None
+        return d_hidden.to(hidden2.dtype).view(ctx.original_hidden_shape), d_weight, None, None, None, None, None
 
 
 linear_cross_entropy = LinearCrossEntropy.apply
@@ -135,7 +135,7 @@ class FusedLinearLogprobHip(torch.autograd.Function):
         target = target.to(torch.int64)  # int32 ids: the sentinel below does not fit their dtype
         labels = torch.where(target_mask, _OOV_LABEL_SENTINEL, target - vocab_start_index).reshape(-1).contiguous()
         # The kernel needs 2-D operands with matching dtypes: hidden follows the weight (model_utils.py:328-333).
-        hidden_2d = hidden.reshape(B * S, H).to(weight.dtype).contiguous()
+        hidden_2d = ops.hidden_for_weight(hidden.reshape(B * S, H), weight).contiguous()
         weight_c = weight.contiguous()
         assert local_vocab == weight_c.shape[0]
 

@@ -73,7 +73,7 @@ def _fused_lm_head_logprob_apply(
     target_mask = (target < vocab_start_index) | (target >= vocab_end_index)
     target = target.to(torch.int64)
     labels = torch.where(target_mask, torch.iinfo(torch.int64).max, target - vocab_start_index)
-    hidden_c = hidden.to(weight.dtype)
+    hidden_c = ops.hidden_for_weight(hidden, weight)
     # log-probabilities only: no entropy is accumulated in the forward, none differentiated in the backward
     if inference_only:
         with torch.no_grad():
@@ -240,7 +240,7 @@ def _fused_vocab_parallel_entropy_from_hidden(
     B, S, H = hidden.shape
     with torch.no_grad():
         labels = torch.full((B * S,), torch.iinfo(torch.int64).max, dtype=torch.int64, device=hidden.device)
-        _, entropy, _, _ = ops.lmhead_fwd(hidden.reshape(B * S, H).to(lm_head_weight.dtype).contiguous(),
+        _, entropy, _, _ = ops.lmhead_fwd(ops.hidden_for_weight(hidden.reshape(B * S, H), lm_head_weight).contiguous(),
                                           lm_head_weight.contiguous(), labels, 1.0 / float(temperature), True)
     return entropy.reshape(B, S)
 
@@ -304,6 +304,6 @@ def fused_logprobs_and_entropy_from_hidden(
     ``entropy_requires_grad`` (workers/worker.py:976-986, 1058-1065).
     """
     B, S, H = hidden.shape
-    lp, ent = linear_cross_entropy(hidden.to(lm_head_weight.dtype), lm_head_weight.contiguous(), target.reshape(B, S),
+    lp, ent = linear_cross_entropy(ops.hidden_for_weight(hidden, lm_head_weight), lm_head_weight.contiguous(), target.reshape(B, S),
                                    float(temperature), "none", None)
     return lp.reshape(B, S), ent.reshape(B, S)

@@ -17,6 +17,7 @@ from typing import List, Optional, Tuple, Union
 
 import torch
 
+from . import ops
 from .fused_linear_logprob_hip import linear_cross_entropy
 from .model_utils import _fused_lm_head_logprob_apply
 
@@ -80,7 +81,7 @@ def action_log_probs_from_hidden(
 
     output = {}
     if compute_entropy:
-        hidden = last_hidden_state.to(lm_head_weight.dtype)
+        hidden = ops.hidden_for_weight(last_hidden_state, lm_head_weight)
         log_probs, entropy = linear_cross_entropy(hidden, lm_head_weight.contiguous(), rolled.contiguous(), float(temperature),
                                                   "none", None)
         log_probs, entropy = log_probs.reshape(tokens.shape), entropy.reshape(tokens.shape)
@@ -120,7 +121,7 @@ def _action_rows_only(last_hidden_state, lm_head_weight, rolled, batch, seqlen, 
     else:
         src, present = flat, None
     H = last_hidden_state.shape[-1]
-    rows = last_hidden_state.reshape(-1, H).index_select(0, src).to(lm_head_weight.dtype).unsqueeze(0)
+    rows = ops.hidden_for_weight(last_hidden_state.reshape(-1, H).index_select(0, src), lm_head_weight).unsqueeze(0)
     labels = rolled.reshape(-1).index_select(0, src).unsqueeze(0).contiguous()
     output = {}
     if compute_entropy:

@@ -17,7 +17,7 @@ import torch
 
 from . import _lib
 
-__all__ = ["lmhead_fwd", "lmhead_bwd", "lmhead_bwd_bf16", "lmhead_bwd_hidden", "lmhead_bwd_active_rows", "fwd_workspace_bytes",
+__all__ = ["hidden_for_weight", "lmhead_fwd", "lmhead_bwd", "lmhead_bwd_bf16", "lmhead_bwd_hidden", "lmhead_bwd_active_rows", "fwd_workspace_bytes",
            "bwd_workspace_bytes"]
 
 
@@ -38,9 +38,10 @@ def _check_operands(hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Te
     if hidden.dim() != 2 or weight.dim() != 2 or labels.dim() != 1:
         raise ValueError(f"expected hidden [T,H], weight [V,H], labels [T]; got {tuple(hidden.shape)}, "
                          f"{tuple(weight.shape)}, {tuple(labels.shape)}")
-    if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
-        raise TypeError(f"the HIP path computes in bf16: hidden and weight must be torch.bfloat16, got {hidden.dtype} and "
-                        f"{weight.dtype} (cast explicitly if a down-cast is intended)")
+    if (hidden.dtype, weight.dtype) not in _DTYPE_TERMS:
+        raise TypeError(f"hidden / weight must be (bf16, bf16), (bf16, fp32) or (fp32, fp32) -- the reference casts hidden to the "
+                        f"weight's dtype (model_utils.py:328-333) -- got {hidden.dtype} and {weight.dtype}; an fp32 hidden with a "
+                        "bf16 weight would be a down-cast: do it explicitly if it is intended")
     if labels.dtype != torch.int64:
         raise TypeError(f"labels must be int64, got {labels.dtype}")
     T, H = hidden.shape
@@ -50,6 +51,44 @@ def _check_operands(hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Te
     if hidden.stride(1) != 1 or weight.stride(1) != 1 or not labels.is_contiguous():
         raise ValueError("hidden and weight must have unit stride in the last dimension and labels must be contiguous")
     return int(T), int(H), int(V)
+
+
+# Number of bf16 terms per product for each (hidden, weight) dtype pair: 1 = the native bf16 path; 2 = fp32 weight as
+# [w_hi | w_lo] against [h | h]; 3 = both fp32, [w_hi | w_lo | w_hi] against [h_hi | h_hi | h_lo].
+_DTYPE_TERMS = {(torch.bfloat16, torch.bfloat16): 1, (torch.bfloat16, torch.float32): 2, (torch.float32, torch.float32): 3}
+_SPLIT_HI_LO, _SPLIT_HI_HI, _SPLIT_HI_LO_HI, _SPLIT_HI_HI_LO = 0, 1, 2, 3
+
+
+def _bf16_terms(hidden: torch.Tensor, weight: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, int]:
+    """The operands as the kernels take them: bf16, stacked hi / lo terms along the contraction axis when the weight is fp32
+    (``skyrl_lmhead_split_operand``).  Nothing is down-cast: the fp32 logits are reproduced to about 2^-16 of each product."""
+    terms = _DTYPE_TERMS[(hidden.dtype, weight.dtype)]
+    if terms == 1:
+        return hidden, weight, 1
+    lib = _lib.load()
+    T, H = hidden.shape
+    V = weight.shape[0]
+    dev = hidden.device
+    h2 = torch.empty((T, terms * H), dtype=torch.bfloat16, device=dev)
+    w2 = torch.empty((V, terms * H), dtype=torch.bfloat16, device=dev)
+    h_layout, w_layout = (_SPLIT_HI_HI, _SPLIT_HI_LO) if terms == 2 else (_SPLIT_HI_HI_LO, _SPLIT_HI_LO_HI)
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        if T > 0:
+            _lib.check(lib.skyrl_lmhead_split_operand(hidden.data_ptr(), int(hidden.dtype == torch.float32), hidden.stride(0), T, H,
+                                                      h_layout, h2.data_ptr(), terms * H, stream), "skyrl_lmhead_split_operand")
+        _lib.check(lib.skyrl_lmhead_split_operand(weight.data_ptr(), 1, weight.stride(0), V, H, w_layout, w2.data_ptr(),
+                                                  terms * H, stream), "skyrl_lmhead_split_operand")
+    return h2, w2, terms
+
+
+def hidden_for_weight(hidden: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """``hidden`` as the reference's ``hidden.to(weight.dtype)`` needs it (model_utils.py:328-333) without a cast that changes
+    nothing: a bf16 hidden stays bf16 next to an fp32 weight (the up-cast is exact, and two bf16 terms per product are cheaper
+    than three); an fp32 hidden next to a bf16 weight is cast down, as the reference does."""
+    if hidden.dtype == torch.bfloat16 and weight.dtype == torch.float32:
+        return hidden
+    return hidden.to(weight.dtype)
 
 
 def fwd_workspace_bytes(T: int, H: int, V: int) -> int:
@@ -88,10 +127,11 @@ def lmhead_fwd(
     row_pz = torch.empty(T if want_entropy else 0, **f32)
     ws_bytes = int(lib.skyrl_lmhead_fwd_workspace_bytes(T, H, V))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    hidden, weight, terms = _bf16_terms(hidden, weight)
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
         st = lib.skyrl_lmhead_fwd(
-            hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), labels.data_ptr(), T, H, V,
+            hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), labels.data_ptr(), T, terms * H, V,
             float(rcp_temperature), logprobs.data_ptr(), _ptr(entropy if want_entropy else None), row_lse.data_ptr(),
             _ptr(row_pz if want_entropy else None), ws.data_ptr(), ws_bytes, stream,
         )
@@ -162,7 +202,7 @@ def lmhead_bwd_bf16(
 
 @lmhead_bwd_bf16.register_fake
 def _(hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk, active_rows=False):
-    return (torch.empty_like(hidden, memory_format=torch.contiguous_format),
+    return (torch.empty(hidden.shape, dtype=torch.bfloat16, device=hidden.device),
             torch.empty(weight.shape, dtype=torch.bfloat16, device=weight.device))
 
 
@@ -191,7 +231,7 @@ def lmhead_bwd_hidden(
 
 @lmhead_bwd_hidden.register_fake
 def _(hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk, active_rows=False):
-    return torch.empty_like(hidden, memory_format=torch.contiguous_format)
+    return torch.empty(hidden.shape, dtype=torch.bfloat16, device=hidden.device)
 
 
 def lmhead_bwd_active_rows(
@@ -239,24 +279,24 @@ def _bwd_into(lib, hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy,
             continue
         if t.dtype != torch.float32 or t.shape != (T,) or not t.is_contiguous():
             raise ValueError(f"{name} must be a contiguous fp32 tensor of shape [{T}], got {t.dtype} {tuple(t.shape)}")
-    query = lib.skyrl_lmhead_bwd_active_rows_workspace_bytes if active_rows else lib.skyrl_lmhead_bwd_workspace_bytes
-    entry = lib.skyrl_lmhead_bwd_active_rows if active_rows else lib.skyrl_lmhead_bwd
-    ws_bytes = int(query(T, H, V, int(vocab_chunk)))
+    terms = _DTYPE_TERMS[(hidden.dtype, weight.dtype)]
+    ws_bytes = int(lib.skyrl_lmhead_bwd_split_workspace_bytes(T, H, terms, V, int(vocab_chunk), int(bool(active_rows))))
     if ws_bytes == 0:
         if int(vocab_chunk) < 0 or int(vocab_chunk) % 256 != 0:
             raise ValueError(f"bad vocab_chunk {vocab_chunk}: must be 0 (library default) or a multiple of 256")
         raise ValueError(f"no backward workspace for T={T}, H={H}, V={V}: every extent must be at least 1")
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    hidden, weight, terms = _bf16_terms(hidden, weight)  # recomputed rather than kept from the forward: a pass over W, no 2x copy held
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
-        st = entry(
+        st = lib.skyrl_lmhead_bwd_split(
             hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), labels.data_ptr(),
             row_lse.data_ptr(), _ptr(row_pz if dentropy is not None else None), dlogprobs.data_ptr(), _ptr(dentropy),
-            T, H, V, float(rcp_temperature), d_hidden.data_ptr(), _ptr(d_weight),
+            T, H, terms, V, float(rcp_temperature), d_hidden.data_ptr(), _ptr(d_weight),
             2 if (d_weight is not None and d_weight.dtype == torch.bfloat16) else int(bool(accumulate_dw)),
-            int(vocab_chunk), ws.data_ptr(), ws_bytes, stream,
+            int(vocab_chunk), int(bool(active_rows)), ws.data_ptr(), ws_bytes, stream,
         )
-    _lib.check(st, "skyrl_lmhead_bwd_active_rows" if active_rows else "skyrl_lmhead_bwd")
+    _lib.check(st, "skyrl_lmhead_bwd_split")
 
 
 def lmhead_bwd_accumulate(hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature: float,
@@ -277,7 +317,7 @@ def lmhead_bwd_accumulate(hidden, weight, labels, row_lse, row_pz, dlogprobs, de
 
 @lmhead_bwd.register_fake
 def _(hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk, active_rows=False):
-    return (torch.empty_like(hidden, memory_format=torch.contiguous_format),
+    return (torch.empty(hidden.shape, dtype=torch.bfloat16, device=hidden.device),
             torch.empty(weight.shape, dtype=torch.float32, device=weight.device))
 
 
@@ -306,8 +346,8 @@ def _backward(ctx, d_logprobs, d_entropy, d_row_lse, d_row_pz):
     d_hidden, d_weight = lmhead_bwd_active_rows(hidden, weight, labels, row_lse, row_pz if dent is not None else None,
                                                 d_logprobs, dent, ctx.rcp_temperature, 0, want_dweight=ctx.needs_input_grad[1],
                                                 dweight_dtype=weight.dtype)
-    # grad_weight is handed back in the weight's dtype, as the reference does (model_utils.py:428).
-    return d_hidden, d_weight, None, None, None
+    # grad_hidden in the hidden dtype, grad_weight in the weight's dtype, as the reference does (model_utils.py:381, 428).
+    return d_hidden.to(hidden.dtype), d_weight, None, None, None
 
 
 lmhead_fwd.register_autograd(_backward, setup_context=_setup_context)

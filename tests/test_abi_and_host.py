@@ -109,6 +109,31 @@ def test_static_scratch_forward_argument_errors():
     assert call(V=300000, H=8192) == -2  # the weight limit is reported first
 
 
+def test_split_operand_argument_errors():
+    """fp32 operands as stacked bf16 terms: layouts, shapes and alignment are checked on the host."""
+    lib = _lib.load()
+    p, q = 0x10000, 0x20000
+    assert lib.skyrl_lmhead_split_operand(None, 1, 128, 4, 128, 0, q, 256, None) == -1
+    assert lib.skyrl_lmhead_split_operand(p, 1, 128, 4, 128, 7, q, 256, None) == -5      # no such layout
+    assert lib.skyrl_lmhead_split_operand(p, 1, 128, 4, 128, 0, q, 128, None) == -2      # destination rows too short for 2 terms
+    assert lib.skyrl_lmhead_split_operand(p, 1, 128, 4, 128, 2, q, 256, None) == -2      # ... for 3 terms
+    assert lib.skyrl_lmhead_split_operand(p, 1, 64, 4, 128, 0, q, 256, None) == -2       # source rows shorter than H
+    assert lib.skyrl_lmhead_split_operand(p, 1, 128, 0, 128, 0, q, 256, None) == -2
+    assert lib.skyrl_lmhead_split_operand(p + 4, 1, 128, 4, 128, 0, q, 256, None) == -3
+    assert lib.skyrl_lmhead_split_operand(p, 1, 130, 4, 128, 0, q, 256, None) == -3
+    T, H, V = 300, 128, 1000
+    base = lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, 0)
+    assert lib.skyrl_lmhead_bwd_split_workspace_bytes(T, H, 1, V, 0, 0) == base           # one term: the ordinary backward
+    # more terms only lengthen the logits GEMM; the scratch grows by one fp32 per (padded) token, the label residuals
+    assert lib.skyrl_lmhead_bwd_split_workspace_bytes(T, H, 3, V, 0, 0) == base + 512 * 4
+    assert lib.skyrl_lmhead_bwd_split_workspace_bytes(T, H, 1, V, 0, 1) == lib.skyrl_lmhead_bwd_active_rows_workspace_bytes(T, H, V, 0)
+    assert lib.skyrl_lmhead_bwd_split_workspace_bytes(T, H, 4, V, 0, 0) == 0
+    args = (p, 3 * H, p, 3 * H, p, p, None, p, None, T, H)
+    tail = (V, 1.0, p, p, 0, 0, 0, p, 1 << 40, None)
+    assert lib.skyrl_lmhead_bwd_split(*args, 0, *tail) == -5 and lib.skyrl_lmhead_bwd_split(*args, 4, *tail) == -5
+    assert lib.skyrl_lmhead_bwd_split(p, 2 * H, p, 3 * H, p, p, None, p, None, T, H, 3, *tail) == -2   # hidden rows hold 2 of 3 terms
+
+
 def test_backward_argument_errors():
     lib = _lib.load()
 
@@ -187,7 +212,9 @@ def test_ops_refuse_cpu_tensors_and_wrong_dtypes():
     with pytest.raises(RuntimeError, match="no CPU implementation"):
         ops.lmhead_fwd(h, w, y, 1.0, True)
     with pytest.raises(TypeError, match="bf16"):
-        ops.lmhead_fwd(h.float(), w, y, 1.0, True)
+        ops.lmhead_fwd(h.float(), w, y, 1.0, True)        # fp32 hidden with a bf16 weight would be a silent down-cast
+    with pytest.raises(TypeError, match="bf16"):
+        ops.lmhead_fwd(h.half(), w.half(), y, 1.0, True)
     with pytest.raises(TypeError, match="int64"):
         ops.lmhead_fwd(h, w, y.int(), 1.0, True)
     with pytest.raises(ValueError):

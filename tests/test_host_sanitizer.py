@@ -36,11 +36,17 @@ DRIVER = textwrap.dedent("""
     for T, H, V, vc in itertools.product(big, (64, 896, 3584, 1 << 20), (5, 1000, 152064, 1 << 31, 1 << 40), (0, 256, 49152, 1 << 40)):
         lib.skyrl_lmhead_fwd_workspace_bytes(T, H, V); lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, vc)
         lib.skyrl_softce_fwd_workspace_bytes(T, H, V); lib.skyrl_softce_bwd_workspace_bytes(T, H, V, vc)
+        lib.skyrl_lmhead_bwd_active_rows_workspace_bytes(T, H, V, vc)
+        for terms in (1, 2, 3, 1 << 40): lib.skyrl_lmhead_bwd_split_workspace_bytes(T, H, terms, V, vc, 1)
     p = 0x10000
     for T, H, V in itertools.product(big, (64, 3584, 1 << 20), (5, 152064, 1 << 31, 1 << 40)):
         ld = H
         assert lib.skyrl_lmhead_fwd(p, ld, p, ld, p, T, H, V, 1.0, p, None, None, None, p, 16, None) < 0
         assert lib.skyrl_lmhead_bwd(p, ld, p, ld, p, p, None, p, None, T, H, V, 1.0, p, p, 0, 0, p, 16, None) < 0
+        assert lib.skyrl_lmhead_bwd_active_rows(p, ld, p, ld, p, p, None, p, None, T, H, V, 1.0, p, p, 0, 0, p, 16, None) < 0
+        assert lib.skyrl_lmhead_bwd_split(p, 3 * ld, p, 3 * ld, p, p, None, p, None, T, H, 3, V, 1.0, p, p, 0, 0, 1, p, 16, None) < 0
+        assert lib.skyrl_lmhead_fwd_static_scratch(p, ld, p, ld, p, T, H, V, float("nan"), p, None, None, None, None) < 0
+        assert lib.skyrl_lmhead_split_operand(p, 1, ld, T, H, 3, p, 2 * ld, None) < 0
         assert lib.skyrl_softce_fwd(p, ld, p, ld, p, ld, T, T, 1, H, V, 1.0, p, p, p, p, 16, None) < 0
         assert lib.skyrl_softce_bwd(p, ld, p, ld, p, ld, p, p, p, T, T, 1, H, V, 1.0, p, 0, p, 16, None) < 0
     assert lib.skyrl_ppo_policy_loss(p, p, p, None, None, 0, 0.2, 0.2, 3.0, 0, p, None, None, None) < 0

@@ -288,6 +288,59 @@ def test_adapter_corner_cases(cuda_device):
         lse3.square().sum().backward()
 
 
+@pytest.mark.parametrize("with_oov_targets", [False, True])
+@pytest.mark.parametrize("hidden_dtype", [torch.bfloat16, torch.float32])
+def test_fp32_weight_matches_the_fp32_product(hidden_dtype, with_oov_targets, cuda_device):
+    """The reference's dtype matrix (tests/backends/skyrl_train/gpu/gpu_ci/megatron/test_fused_linear_logprob.py:89-118): an fp32
+    output weight with a bf16 or an fp32 hidden, same shapes, same upstream gradient, same tolerances -- log-probabilities
+    1e-5, grad_hidden 2e-3, grad_weight 2e-3 against logits materialised in fp32 -- and results in the reference's dtypes.
+    Here the fp32 operands reach the bf16 matrix pipe as stacked hi / lo terms."""
+    dev = cuda_device
+    B, S, V, H = 4, 32, 4096, 256
+    gen = torch.Generator().manual_seed(0)
+    hidden = torch.randn(B, S, H, generator=gen).to(hidden_dtype)
+    weight = torch.randn(V, H, generator=gen) * H ** -0.5
+    target = torch.randint(0, V + 1024 if with_oov_targets else V, (B, S), generator=gen)
+    g = torch.linspace(0.5, 1.5, steps=B * S).reshape(B, S)          # the reference's non-uniform upstream gradient
+    h = hidden.to(dev).requires_grad_(True)
+    w = weight.to(dev).requires_grad_(True)
+    out = FusedLinearLogprobHip.apply(h, w, target.to(dev), 0, V, 64, None, False)
+    out.backward(g.to(dev))
+    assert out.dtype == torch.float32 and h.grad.dtype == hidden_dtype and w.grad.dtype == torch.float32
+    # materialised fp32 logits + autograd, as the reference's own check does (hidden cast to the weight's dtype)
+    hr = hidden.float().clone().requires_grad_(True)
+    wr = weight.clone().requires_grad_(True)
+    logits = hr @ wr.t()
+    in_vocab = target < V
+    ref = torch.log_softmax(logits, -1).gather(-1, target.clamp(max=V - 1)[..., None])[..., 0] * in_vocab
+    # targets outside the shard: forward 0, backward keeps -softmax * g (model_utils.py:337, 405-411), the gradient of -lse * g
+    lse = torch.logsumexp(logits, -1)
+    ((ref - (~in_vocab) * lse) * g).sum().backward()
+    torch.testing.assert_close(out.cpu(), ref.detach(), atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(h.grad.cpu().float(), hr.grad, atol=2e-3, rtol=2e-3)
+    torch.testing.assert_close(w.grad.cpu(), wr.grad, atol=2e-3, rtol=2e-3)
+    # the verl interface with temperature and a grad-carrying entropy, against the fp64 statement
+    q = torch.randn(B * S, generator=gen) * 0.1
+    h2 = hidden.reshape(-1, H).to(dev).requires_grad_(True)
+    w2 = weight.to(dev).requires_grad_(True)
+    labels = torch.where(in_vocab, target, SENTINEL).reshape(-1)
+    lp, ent = linear_cross_entropy(h2, w2, labels.to(dev), 0.7, "none")
+    (lp * g.reshape(-1).to(dev) + ent * q.to(dev)).sum().backward()
+    ex = O.exact_fwd_bwd(hidden.reshape(-1, H), weight, labels, 0.7, g.reshape(-1), q)
+    lp_err = float((lp.detach().cpu().double() - ex["logprobs"]).abs().max())
+    ent_err = float(((ent.detach().cpu().double() - ex["entropy"]).abs() / ex["entropy"].abs()).max())
+    assert lp_err <= 5e-5 and ent_err <= 2e-5, (lp_err, ent_err)
+    check_grads(h2.grad, w2.grad, ex, "fp32 weight, entropy gradient")
+    # rows without upstream gradient are dropped on this path too
+    gm = g.reshape(-1).clone()
+    gm[::2] = 0
+    _, _, lse_d, _ = ops.lmhead_fwd(h2.detach(), w2.detach(), labels.to(dev), 1.0, False)
+    dense = ops.lmhead_bwd(h2.detach(), w2.detach(), labels.to(dev), lse_d, None, gm.to(dev), None, 1.0, 0)
+    compact = ops.lmhead_bwd(h2.detach(), w2.detach(), labels.to(dev), lse_d, None, gm.to(dev), None, 1.0, 0, True)
+    assert float(compact[0][::2].abs().max()) == 0.0 and torch.equal(compact[0][1::2], dense[0][1::2])
+    assert rel_l2(compact[1], dense[1]) < 1e-5
+
+
 def test_extreme_logits(cuda_device):
     # one dominant logit -> logprob, entropy -> 0; all logits very negative -> the split merge must not underflow
     T, H, V = 40, 64, 700
