@@ -316,9 +316,12 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
   const float* __restrict__ dlogprobs = z.dlogprobs;
   const float* __restrict__ dentropy = z.dentropy;
   uint16_t* __restrict__ D = z.D;
+  // With a device-side count the tiles that hold tokens are numbered 0 .. tiles_m * ceil(T / 256) - 1, so that the hardware's
+  // round-robin of workgroup ids over the XCDs spreads exactly those; the other workgroups of the (static) grid return at once.
+  const int tiles_n = z.T_dev ? (T + BN - 1) / BN : z.tiles_n;
+  if (id >= z.tiles_m * tiles_n) return;
   int tm, tn;
-  tile_coords(id, z.tiles_m, z.tiles_n, kGroupM, tm, tn);
-  if (tn * BN >= T) return;  // only with a device-side count: this token tile holds no token (uniform over the workgroup)
+  tile_coords(id, z.tiles_m, tiles_n, kGroupM, tm, tn);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
@@ -612,19 +615,22 @@ enum { kTokensOnM = 1, kTokensOnN = 2, kTokensOnK = 3 };
 template <bool BKM>
 __device__ __forceinline__ void gemm_tile(const GemmArgs& p, int bid, char* lds) {
   int M = p.M, N = p.N, nk = p.nk;
-  const int tiles_m = (M + BM - 1) / BM;  // of the host-side extents: they define the grid and the partial-sum layout
-  const int tiles_n = (N + BN - 1) / BN;
-  int tm, tn;
-  tile_coords(bid, tiles_m, tiles_n, kGroupM, tm, tn);
   if (p.T_dev) {
     const int count = __builtin_amdgcn_readfirstlane(*p.T_dev);
     if (p.t_role == kTokensOnM) M = count;
     else if (p.t_role == kTokensOnN) N = count;
     else nk = (count + BK - 1) / BK;
-    if (tm * BM >= M || tn * BN >= N) return;  // a tile without tokens (uniform over the workgroup)
     // Nothing to contract: C += 0 needs no work; a C that is overwritten or converted still goes through the epilogue.
     if (nk == 0 && !p.Cb && p.Cin == p.Cf) return;
   }
+  // Tiles of the extents in force: with a device-side count the tiles that hold tokens are numbered from 0, so that the
+  // round-robin of workgroup ids over the XCDs spreads exactly those, and the rest of the (static) grid returns at once.  The
+  // partial sums that cross vocab chunks are laid out by the same numbering (the count does not change between chunks).
+  const int tiles_m = (M + BM - 1) / BM;
+  const int tiles_n = (N + BN - 1) / BN;
+  if (bid >= tiles_m * tiles_n) return;
+  int tm, tn;
+  tile_coords(bid, tiles_m, tiles_n, kGroupM, tm, tn);
   Operand a{p.A, p.lda, tm * BM, p.a_rows};
   Operand b{p.B, p.ldb, tn * BN, p.b_rows};
   acc_t acc;
