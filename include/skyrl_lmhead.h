@@ -221,13 +221,22 @@ int skyrl_lmhead_bwd_split(const void* hidden_terms, int64_t ld_hidden, const vo
  *     loss = -r A keep, keep = 0 where the probability moved too far in the advantage's direction -- TV: p - p_old >
  *     eps_clip_high (A > 0) or p_old - p > eps_clip_low (A < 0); KL: the binary KL of p_old to p exceeds the same thresholds
  *     (the two arguments carry delta_low and delta_high); out3[1] counts keep == 0.
- * Not covered: clip_cov and kl_cov (a random subset / a top-k over the whole batch). */
+ * The two covariance-based types (skyrl_ppo_policy_loss only).  Which tokens they single out is decided from the whole batch
+ * on the host side, as the reference does (a random subset drawn with the host's generator / a top-k computed on the CPU);
+ * the per-token decision comes in through loss_weight:
+ *   CLIP_COV (compute_policy_loss_clip_cov, :938-999): the clipped surrogate of REGULAR on the unclamped ratio exp(logprobs -
+ *     old_logprobs), times loss_weight = 0 for the tokens the covariance rule removes, 1 elsewhere; out3[1] counts clipped tokens.
+ *   KL_COV (compute_policy_loss_kl_cov, :1002-1053): loss = -exp(logprobs - old_logprobs) A + clip_ratio_c |logprobs - old_logprobs|
+ *     where loss_weight = 1 (the selected tokens; clip_ratio_c carries ppo_kl_coef), the plain importance-sampling term
+ *     elsewhere; loss_weight does not scale the loss here; out3[1] counts selected tokens. */
 #define SKYRL_POLICY_LOSS_GSPO 4
 #define SKYRL_POLICY_LOSS_SAPO 5
 #define SKYRL_POLICY_LOSS_CISPO 6
 #define SKYRL_POLICY_LOSS_ROLLOUT_IS 7
 #define SKYRL_POLICY_LOSS_DPPO_TV 8
 #define SKYRL_POLICY_LOSS_DPPO_KL 9
+#define SKYRL_POLICY_LOSS_CLIP_COV 10
+#define SKYRL_POLICY_LOSS_KL_COV 11
 int skyrl_ppo_policy_loss(const float* logprobs, const float* old_logprobs, const float* advantages,
                           const float* loss_mask, const float* loss_weight, int64_t T,
                           float eps_clip_low, float eps_clip_high, float clip_ratio_c, int loss_type,

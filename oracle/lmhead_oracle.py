@@ -33,6 +33,10 @@ What pins each function (all in ``tests/test_oracle.py``; none of them re-types 
     limits that tie them to pinned functions (GSPO on rows of one token is the clipped surrogate; DPPO with nothing masked
     and SAPO's gate near r = 1 are the importance-sampling surrogate; CISPO and rollout-IS agree inside the interval), and
     fp64 central finite differences of the surrogate with the stop-gradient factors held fixed.
+  * clip-cov and kl-cov losses: the selection counted and listed by hand on a 2 x 4 batch (which tokens are candidates, how
+    many are drawn, the top-k by sorting the hand-computed covariance terms), the limit in which every candidate is drawn
+    (so that the random permutation cannot matter), loss values token by token with ``math``, and fp64 central finite
+    differences with the selection held fixed.  CISPO's ratio diagnostics: hand values with and without a mask.
   * approximate KL: hand values at d = 0, ln 2, -1 and in both clamps; the identities the estimators are built on --
     under x ~ p the expectation of k1 and of k3 is KL(p || q) exactly, summed by brute force over a small alphabet and
     compared with ``torch.nn.functional.kl_div`` -- and k3 ~ k2 for small differences; the trainer's reduction against a
@@ -567,6 +571,62 @@ def dppo_policy_loss(log_probs, mu_log_probs, advantages, dppo_type: str, delta_
         else:
             raise ValueError(f"Unknown DPPO type: {dppo_type}. Must be 'binary_tv' or 'binary_kl'.")
     return _reduce(-(ratio * advantages * keep), loss_mask), masked_mean((keep == 0).to(log_probs.dtype), loss_mask).detach()
+
+
+def cispo_ratio_diagnostics(log_probs, behaviour_log_probs, eps_clip_low: float, eps_clip_high: float, loss_mask=None):
+    """ppo_utils.py:790-815: the four ``cispo/ratio_*`` metrics -- masked means of the ratio and of the clamped ratio, and the
+    largest / smallest ratio among the unmasked tokens (among all tokens when there is no mask or the mask is empty)."""
+    ratio = _safe_ratio(log_probs, behaviour_log_probs).detach()
+    clamped = torch.clamp(ratio, 1 - eps_clip_low, 1 + eps_clip_high)
+    active = ratio[loss_mask.bool()] if (loss_mask is not None and bool(loss_mask.any())) else ratio
+    return {"cispo/ratio_mean": float(masked_mean(ratio, loss_mask)), "cispo/ratio_clamped_mean": float(masked_mean(clamped, loss_mask)),
+            "cispo/ratio_max": float(active.max()), "cispo/ratio_min": float(active.min())}
+
+
+def clip_cov_policy_loss(log_probs, old_log_probs, advantages, eps_clip_low: float, eps_clip_high: float, clip_ratio: float,
+                         clip_cov_lb: float, clip_cov_ub: float, loss_mask: torch.Tensor):
+    """ppo_utils.py:938-999.  The clipped surrogate on the unclamped ratio (:962-967); among the unmasked tokens that the clip
+    did not catch and whose covariance term (A - mean A)(logp - mean logp) lies strictly inside (lb, ub) (:970-978),
+    ``max(int(clip_ratio * sum mask), 1)`` are drawn with ``torch.randperm`` -- the global CPU generator (:977-982) -- and their
+    loss is removed (:987-996).  Returns ``(loss, fraction of unmasked tokens removed, the 0/1 factor)``."""
+    ratio = torch.exp(log_probs - old_log_probs)
+    pg1 = -advantages * ratio
+    pg2 = -advantages * torch.clamp(ratio, 1 - eps_clip_low, 1 + eps_clip_high)
+    clip_by_origin = (pg2 > pg1) & (loss_mask > 0)
+    cov_all = ((advantages - masked_mean(advantages, loss_mask)) * (log_probs - masked_mean(log_probs.detach(), loss_mask))).detach().clone()
+    cov_all[loss_mask == 0] = -torch.inf
+    cov_all[clip_by_origin] = -torch.inf
+    clip_num = max(int(clip_ratio * loss_mask.sum().item()), 1)
+    candidates = torch.nonzero((cov_all < clip_cov_ub) & (cov_all > clip_cov_lb) & (loss_mask > 0))
+    corr = torch.ones_like(advantages)
+    if len(candidates) > 0:
+        perm = torch.randperm(len(candidates))
+        chosen = candidates[perm[: min(clip_num, len(candidates))]]
+        corr[chosen[:, 0], chosen[:, 1]] = 0
+    clip_frac = masked_mean((corr == 0).to(log_probs.dtype), loss_mask)
+    return _reduce(torch.maximum(pg1, pg2) * corr, loss_mask), clip_frac.detach(), corr
+
+
+def kl_cov_policy_loss(log_probs, old_log_probs, advantages, kl_cov_frac: float, ppo_kl_coef: float, loss_mask: torch.Tensor):
+    """ppo_utils.py:1002-1053.  The importance-sampling surrogate -A r; the ``max(1, int(n * kl_cov_frac))`` unmasked tokens
+    with the largest covariance term -- means over the unmasked tokens, computed on the CPU in the inputs' dtype (:1027-1036) --
+    pay ``ppo_kl_coef * |logp - old|`` on top (:1038-1047).  Returns ``(loss, the 0/1 selector)``."""
+    delta = log_probs - old_log_probs
+    ratio = torch.exp(delta)
+    pg = -advantages * ratio
+    pg_kl = pg + ppo_kl_coef * delta.abs()
+    valid = loss_mask > 0
+    idx = torch.nonzero(valid.reshape(-1), as_tuple=True)[0]
+    adv_v = advantages[valid].detach().reshape(-1).cpu()
+    lp_v = log_probs[valid].detach().reshape(-1).cpu()
+    selector = torch.zeros(advantages.numel(), dtype=log_probs.dtype)
+    if len(adv_v) > 0:
+        cov = (adv_v - adv_v.mean()) * (lp_v - lp_v.mean())
+        k = max(1, int(len(cov) * kl_cov_frac))
+        top = torch.topk(cov, min(k, len(cov)), largest=True).indices
+        selector[idx[top]] = 1.0
+    selector = selector.reshape(advantages.shape)
+    return _reduce(torch.where(selector > 0, pg_kl, pg), loss_mask), selector
 
 
 def cross_entropy_loss(log_probs: torch.Tensor, loss_mask: Optional[torch.Tensor] = None) -> torch.Tensor:

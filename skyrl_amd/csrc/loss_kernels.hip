@@ -51,6 +51,22 @@ __device__ __forceinline__ void policy_term(int type, float lp, float old, float
     stat = ratio;
     return;
   }
+  if (type == SKYRL_POLICY_LOSS_KL_COV) {  // c = ppo_kl_coef, row_lr = this token's selector (1: the |log-ratio| penalty applies)
+    const float delta = lp - old, ratio = expf(delta);
+    loss = -(ratio * A) + c * row_lr * fabsf(delta);
+    dloss = -(ratio * A) + c * row_lr * (delta > 0.f ? 1.f : (delta < 0.f ? -1.f : 0.f));
+    stat = row_lr;
+    return;
+  }
+  if (type == SKYRL_POLICY_LOSS_CLIP_COV) {  // the clipped surrogate on the unclamped ratio; the selection comes in as the weight
+    const float ratio = expf(lp - old);
+    const float pg1 = -A * ratio, pg2 = -A * fminf(fmaxf(ratio, lo), hi);
+    const float d1 = pg1, d2 = (ratio >= lo && ratio <= hi) ? pg1 : 0.f;
+    loss = fmaxf(pg1, pg2);
+    dloss = pg1 > pg2 ? d1 : (pg1 < pg2 ? d2 : 0.5f * (d1 + d2));
+    stat = pg2 > pg1 ? 1.f : 0.f;
+    return;
+  }
   // safe_exp_delta: the log-ratio clamped to +-20; the clamp passes the gradient on its closed interval
   const float delta = lp - old;
   float ratio = expf(fminf(fmaxf(delta, -20.f), 20.f));
@@ -120,7 +136,7 @@ __device__ __forceinline__ void policy_term(int type, float lp, float old, float
 // The interval parameters of a type: clip types take (1 - eps_low, 1 + eps_high), the others their two values as given.
 __device__ __forceinline__ bool is_interval_type(int type) {
   return type == SKYRL_POLICY_LOSS_REGULAR || type == SKYRL_POLICY_LOSS_DUAL_CLIP || type == SKYRL_POLICY_LOSS_GSPO ||
-         type == SKYRL_POLICY_LOSS_CISPO || type == SKYRL_POLICY_LOSS_ROLLOUT_IS;
+         type == SKYRL_POLICY_LOSS_CISPO || type == SKYRL_POLICY_LOSS_ROLLOUT_IS || type == SKYRL_POLICY_LOSS_CLIP_COV;
 }
 
 // Workgroup b sums tokens [b * slice, (b + 1) * slice) in a fixed order and writes its three sums to out[k * out_stride + b]:
@@ -137,9 +153,11 @@ __global__ __launch_bounds__(1024) void policy_loss_kernel(const float* __restri
   for (int64_t t = t0 + threadIdx.x; t < t1; t += blockDim.x) {
     float loss, dloss, stat;
     const bool ce = type == SKYRL_POLICY_LOSS_CROSS_ENTROPY;  // reads neither old nor adv
-    policy_term(type, lp[t], ce ? 0.f : old[t], ce ? 0.f : adv[t], lo, hi, clip_c, 0.f, loss, dloss, stat);
+    const bool selector = type == SKYRL_POLICY_LOSS_KL_COV;  // the weight array selects tokens instead of scaling the loss
+    policy_term(type, lp[t], ce ? 0.f : old[t], ce ? 0.f : adv[t], lo, hi, clip_c, (selector && weight) ? weight[t] : 0.f, loss,
+                dloss, stat);
     const float m = mask ? mask[t] : 1.f;
-    const float w = weight ? m * weight[t] : m;
+    const float w = (weight && !selector) ? m * weight[t] : m;
     s_loss += loss * w;
     s_clip += stat * m;
     s_mask += m;
@@ -396,6 +414,7 @@ bool interval_type(int t) {
 // Types that read their two parameters need them finite (SAPO's temperatures also non-zero); the dual clip its third.
 bool valid_loss_params(int t, float a, float b, float c) {
   if (t == SKYRL_POLICY_LOSS_CROSS_ENTROPY || t == SKYRL_POLICY_LOSS_IMPORTANCE_SAMPLING) return true;
+  if (t == SKYRL_POLICY_LOSS_KL_COV) return finite(c);
   if (!finite(a) || !finite(b)) return false;
   if (t == SKYRL_POLICY_LOSS_SAPO && (a == 0.f || b == 0.f)) return false;
   return t != SKYRL_POLICY_LOSS_DUAL_CLIP || finite(c);
@@ -409,7 +428,8 @@ int skyrl_ppo_policy_loss(const float* logprobs, const float* old_logprobs, cons
                           const float* loss_weight, int64_t T, float eps_clip_low, float eps_clip_high, float clip_ratio_c,
                           int loss_type, float* out3, float* dlogprobs, float* partials, void* stream) {
   // the sequence-level type needs rows: it is part of skyrl_actor_loss only
-  if (!valid_loss_type(loss_type) || loss_type == SKYRL_POLICY_LOSS_GSPO) return SKYRL_LMHEAD_ERR_ARG;
+  const bool cov_type = loss_type == SKYRL_POLICY_LOSS_CLIP_COV || loss_type == SKYRL_POLICY_LOSS_KL_COV;  // this entry point only
+  if ((!valid_loss_type(loss_type) && !cov_type) || loss_type == SKYRL_POLICY_LOSS_GSPO) return SKYRL_LMHEAD_ERR_ARG;
   const bool needs_old = loss_type != SKYRL_POLICY_LOSS_CROSS_ENTROPY;
   if (!logprobs || !out3 || (needs_old && (!old_logprobs || !advantages))) return SKYRL_LMHEAD_ERR_NULL;
   if (T < 1) return SKYRL_LMHEAD_ERR_SHAPE;

@@ -25,7 +25,9 @@ loss by an importance ratio that does not depend on the policy's log-probabiliti
 with the trainer's own helper and pass the ratio as ``loss_weight`` and the thinned mask as ``loss_mask``.  Computing them
 from ``rollout_logprobs`` is outside this module: the losses raise when the config switches a correction on, and otherwise
 use ``rollout_logprobs`` only where the loss itself is anchored on them (rollout-IS, DPPO, CISPO with the rollout anchor).
-The two covariance-based types (clip_cov, kl_cov) pick a random subset / a top-k over the whole batch and are not here.
+The two covariance-based types pick their tokens from the whole batch exactly as the reference does -- ``clip_cov`` a random
+subset drawn with ``torch.randperm`` on the host's generator, ``kl_cov`` a top-k computed on the CPU -- and hand the
+per-token decision to the same fused kernel (``compute_policy_loss_clip_cov``, ``compute_policy_loss_kl_cov``, :938-1053).
 """
 
 from __future__ import annotations
@@ -39,10 +41,11 @@ from .ops import _require_device
 
 __all__ = ["ppo_policy_loss", "cross_entropy_loss", "importance_sampling_loss", "sapo_policy_loss", "gspo_policy_loss",
            "compute_policy_loss_cispo", "rollout_is_policy_loss", "dppo_policy_loss", "compute_approx_kl", "approx_kl_loss",
-           "masked_mean", "actor_loss", "ppo_policy_loss_terms"]
+           "masked_mean", "actor_loss", "ppo_policy_loss_terms", "compute_policy_loss_clip_cov", "compute_policy_loss_kl_cov"]
 
 LOSS_REGULAR, LOSS_DUAL_CLIP, LOSS_CROSS_ENTROPY, LOSS_IMPORTANCE_SAMPLING = 0, 1, 2, 3
 LOSS_GSPO, LOSS_SAPO, LOSS_CISPO, LOSS_ROLLOUT_IS, LOSS_DPPO_TV, LOSS_DPPO_KL = 4, 5, 6, 7, 8, 9
+LOSS_CLIP_COV, LOSS_KL_COV = 10, 11
 
 
 def _get(obj: Any, name: str, default: Any = None) -> Any:
@@ -271,10 +274,88 @@ def compute_policy_loss_cispo(log_probs, old_log_probs, advantages, config, loss
                               loss_weight=None, sync_metrics: bool = True) -> Tuple[torch.Tensor, Dict[str, Any]]:
     """Clipped importance-weight policy optimisation (reference ``compute_policy_loss_cispo``, ppo_utils.py:732-821):
     ``-A stopgrad(clamp(r, 1 - cispo_eps_clip_low, 1 + cispo_eps_clip_high)) log_probs`` with the ratio anchored as
-    ``config.cispo.cispo_anchor`` says.  Returns ``clip_ratio``; the reference's four ``cispo/ratio_*`` diagnostics are not
-    computed."""
-    return _elementwise_loss("cispo", log_probs, old_log_probs, advantages, config, loss_mask, rollout_logprobs, loss_weight,
-                             sync_metrics)
+    ``config.cispo.cispo_anchor`` says.  Returns ``clip_ratio`` and the reference's four ``cispo/ratio_*`` diagnostics
+    (:790-815: masked means of the ratio and of the clamped ratio, extremes over the unmasked tokens), which are monitoring
+    values outside the loss kernel; as floats, or as 0-dim tensors with ``sync_metrics=False`` (the extremes are then taken
+    with the masked tokens neutralised instead of selected, so nothing waits for a count)."""
+    loss, metrics = _elementwise_loss("cispo", log_probs, old_log_probs, advantages, config, loss_mask, rollout_logprobs,
+                                      loss_weight, sync_metrics)
+    _, lo, hi, _, behaviour = _type_parameters(config, "cispo", rollout_logprobs, old_log_probs)
+    with torch.no_grad():
+        ratio = torch.clamp(log_probs.detach().float() - behaviour.float(), -20.0, 20.0).exp()
+        clamped = ratio.clamp(1.0 - lo, 1.0 + hi)
+        if loss_mask is None:
+            mean, cmean, rmax, rmin = ratio.mean(), clamped.mean(), ratio.max(), ratio.min()
+        else:
+            m = loss_mask.float()
+            count = m.sum()
+            denom = count.clamp(min=1.0)
+            mean, cmean = (ratio * m).sum() / denom, (clamped * m).sum() / denom
+            active = m > 0
+            some = count > 0   # an empty mask: the extremes over all tokens, as the reference's else branch
+            rmax = torch.where(some, torch.where(active, ratio, ratio.new_full((), -torch.inf)).max(), ratio.max())
+            rmin = torch.where(some, torch.where(active, ratio, ratio.new_full((), torch.inf)).min(), ratio.min())
+    extra = {"cispo/ratio_mean": mean, "cispo/ratio_clamped_mean": cmean, "cispo/ratio_max": rmax, "cispo/ratio_min": rmin}
+    metrics.update({k: (v.item() if sync_metrics else v) for k, v in extra.items()})
+    return loss, metrics
+
+
+def compute_policy_loss_clip_cov(log_probs, old_log_probs, advantages, config, loss_mask=None, rollout_logprobs=None
+                                 ) -> Tuple[torch.Tensor, Dict[str, Any]]:
+    """Clip-Cov (reference ``compute_policy_loss_clip_cov``, ppo_utils.py:938-999): the clipped surrogate on the unclamped
+    ratio, with the loss of a random subset of tokens removed -- tokens the clip did not catch whose covariance term
+    ``(A - mean A)(logp - mean logp)`` lies inside ``(clip_cov_lb, clip_cov_ub)``, ``max(int(clip_ratio * sum mask), 1)`` of them,
+    drawn with ``torch.randperm`` on the global CPU generator exactly as the reference draws them (same generator state, same
+    tokens).  The selection is batch-level host logic there and here (it reads a count and a permutation back); value,
+    gradient and sums then come from the fused kernel with the selection as its per-token weight.  ``loss_mask`` is required,
+    as in the reference."""
+    cc = _get(config, "clip_cov")
+    ratio_frac, lb, ub = float(_get(cc, "clip_ratio")), float(_get(cc, "clip_cov_lb")), float(_get(cc, "clip_cov_ub"))
+    eps_low, eps_high = float(config.eps_clip_low), float(config.eps_clip_high)
+    with torch.no_grad():
+        lp, old, adv, mask = log_probs.detach(), old_log_probs, advantages, loss_mask
+        r = torch.exp(lp - old)
+        pg1 = -adv * r
+        pg2 = -adv * torch.clamp(r, 1 - eps_low, 1 + eps_high)
+        clip_by_origin = (pg2 > pg1) & (mask > 0)
+        denom = mask.sum().clamp(min=1.0)
+        cov_all = (adv - (adv * mask).sum() / denom) * (lp - (lp * mask).sum() / denom)
+        cov_all[mask == 0] = -torch.inf
+        cov_all[clip_by_origin] = -torch.inf
+        clip_num = max(int(ratio_frac * mask.sum().item()), 1)
+        candidates = torch.nonzero((cov_all < ub) & (cov_all > lb) & (mask > 0))
+        corr = torch.ones_like(adv, dtype=torch.float32)
+        if len(candidates) > 0:
+            perm = torch.randperm(len(candidates))
+            chosen = candidates[perm[: min(clip_num, len(candidates))].to(candidates.device)]
+            corr[tuple(chosen[:, k] for k in range(chosen.shape[1]))] = 0
+        clip_frac = ((corr == 0).float() * mask).sum() / denom
+    loss, _ = _PolicyLoss.apply(log_probs, old_log_probs, advantages, loss_mask, corr, eps_low, eps_high, 0.0, LOSS_CLIP_COV)
+    return loss, {"clip_ratio": clip_frac.item()}
+
+
+def compute_policy_loss_kl_cov(log_probs, old_log_probs, advantages, config, loss_mask=None, rollout_logprobs=None
+                               ) -> Tuple[torch.Tensor, Dict[str, Any]]:
+    """KL-Cov (reference ``compute_policy_loss_kl_cov``, ppo_utils.py:1002-1053): the importance-sampling surrogate, plus
+    ``ppo_kl_coef * |logp - old|`` on the ``max(1, int(n * kl_cov_frac))`` unmasked tokens with the largest covariance term.
+    The top-k is taken on the CPU from the unmasked values, as the reference takes it (:1027-1036), so that ties and rounding
+    fall the same way; the selector then goes to the fused kernel, which returns value and gradient."""
+    kc = _get(config, "kl_cov")
+    frac, coef = float(_get(kc, "kl_cov_frac")), float(_get(kc, "ppo_kl_coef"))
+    with torch.no_grad():
+        valid = loss_mask > 0
+        idx = torch.nonzero(valid.reshape(-1), as_tuple=True)[0]
+        adv_v = advantages[valid].detach().reshape(-1).cpu()
+        lp_v = log_probs[valid].detach().reshape(-1).cpu()
+        selector = torch.zeros(advantages.numel(), dtype=torch.float32, device=log_probs.device)
+        if len(adv_v) > 0:
+            cov = (adv_v - adv_v.mean()) * (lp_v - lp_v.mean())
+            k = max(1, int(len(cov) * frac))
+            top = torch.topk(cov, min(k, len(cov)), largest=True).indices
+            selector[idx[top.to(idx.device)]] = 1.0
+    loss, _ = _PolicyLoss.apply(log_probs, old_log_probs, advantages, loss_mask, selector.reshape(advantages.shape), 0.0, 0.0, coef,
+                                LOSS_KL_COV)
+    return loss, {"clip_ratio": 0.0}   # not applicable to KL-Cov: the reference reports 0.0 (:1052)
 
 
 def rollout_is_policy_loss(log_probs, old_log_probs, advantages, config, loss_mask=None, rollout_logprobs=None, *,

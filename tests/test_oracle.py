@@ -570,6 +570,91 @@ def test_cispo_and_rollout_is_by_hand():
     assert a[0] == pytest.approx(b[0]) and a[2] == pytest.approx(b[2]) and a[1] == b[1] == 0.0
 
 
+def test_cov_losses_by_hand():
+    """clip-cov and kl-cov (ppo_utils.py:938-1053) on a 2 x 4 batch whose selection can be listed by hand."""
+    ln = math.log
+    old = _t([[-1.0] * 4, [-1.0] * 4])
+    # ratios 1, 2, 1/2, 1 | 1, 1, 3, 1
+    lp = _t([[-1.0, ln(2) - 1, ln(0.5) - 1, -1.0], [-1.0, -1.0, ln(3) - 1, -1.0]])
+    adv = _t([[1.0, 1.0, -2.0, 3.0], [-1.0, 2.0, 1.0, 0.5]])
+    mask = _t([[1.0, 1.0, 1.0, 0.0], [1.0, 1.0, 1.0, 1.0]])
+    # clipped by the surrogate with [0.8, 1.2]: (0,1) ratio 2 with A > 0, (0,2) ratio 1/2 with A < 0, (1,2) ratio 3 with A > 0
+    m = mask.bool()
+    mean_a, mean_l = float(adv[m].mean()), float(lp[m].mean())
+    cov = {(i, j): (float(adv[i, j]) - mean_a) * (float(lp[i, j]) - mean_l) for i in range(2) for j in range(4)}
+    candidates = [ij for ij in cov if ij not in [(0, 1), (0, 2), (1, 2), (0, 3)]]            # unmasked and not clipped
+    inside = [ij for ij in candidates if -0.2 < cov[ij] < 0.3]
+    assert sorted(candidates) == [(0, 0), (1, 0), (1, 1), (1, 3)] and len(inside) >= 2
+    # a clip ratio large enough to draw every candidate inside the bounds: the permutation cannot matter
+    x = lp.clone().requires_grad_(True)
+    loss, frac, corr = O.clip_cov_policy_loss(x, old, adv, 0.2, 0.2, 1.0, -0.2, 0.3, mask)
+    want_corr = torch.ones(2, 4, dtype=torch.float64)
+    for ij in inside:
+        want_corr[ij] = 0.0
+    assert torch.equal(corr, want_corr) and float(frac) == pytest.approx(len(inside) / 7)
+    tok = lambda i, j: max(-float(adv[i, j]) * math.exp(float(lp[i, j]) + 1), -float(adv[i, j]) * min(max(math.exp(float(lp[i, j]) + 1), 0.8), 1.2))  # noqa: E731
+    want = sum(tok(i, j) * float(want_corr[i, j]) * float(mask[i, j]) for i in range(2) for j in range(4))
+    assert loss.item() == pytest.approx(want)
+    loss.backward()
+    # gradient: -A r where the unclipped branch is active, the loss kept and the token unmasked; 0 elsewhere
+    for (i, j), c in cov.items():
+        live = (i, j) in candidates and want_corr[i, j] == 1.0
+        assert float(x.grad[i, j]) == pytest.approx(-float(adv[i, j]) * math.exp(float(lp[i, j]) + 1) if live else 0.0)
+    # clip_ratio = 0.3: int(0.3 * 7) = 2 tokens are drawn from the candidates inside the bounds, whichever the generator picks
+    torch.manual_seed(3)
+    _, frac, corr = O.clip_cov_policy_loss(lp, old, adv, 0.2, 0.2, 0.3, -10.0, 10.0, mask)
+    removed = [(i, j) for i in range(2) for j in range(4) if corr[i, j] == 0]
+    assert len(removed) == 2 and set(removed) <= set(candidates) and float(frac) == pytest.approx(2 / 7)
+    torch.manual_seed(3)
+    perm = torch.randperm(4)                                     # the draw the function makes: candidates in row-major order
+    assert sorted(removed) == sorted(sorted(candidates)[k] for k in perm[:2].tolist())
+    # a clip ratio that rounds to zero still draws one token; no candidate inside the bounds draws none
+    assert int((O.clip_cov_policy_loss(lp, old, adv, 0.2, 0.2, 0.01, -10.0, 10.0, mask)[2] == 0).sum()) == 1
+    assert int((O.clip_cov_policy_loss(lp, old, adv, 0.2, 0.2, 1.0, 50.0, 60.0, mask)[2] == 0).sum()) == 0
+
+    # kl-cov: the top int(7 * 0.3) = 2 unmasked tokens by covariance pay coef * |log-ratio| on top of -A r
+    order = sorted((ij for ij in cov if ij != (0, 3)), key=lambda ij: -cov[ij])
+    x = lp.clone().requires_grad_(True)
+    loss, sel = O.kl_cov_policy_loss(x, old, adv, 0.3, 0.5, mask)
+    assert sorted((i, j) for i in range(2) for j in range(4) if sel[i, j] == 1) == sorted(order[:2])
+    want = 0.0
+    for i in range(2):
+        for j in range(4):
+            d = float(lp[i, j]) + 1.0
+            want += float(mask[i, j]) * (-float(adv[i, j]) * math.exp(d) + (0.5 * abs(d) if (i, j) in order[:2] else 0.0))
+    assert loss.item() == pytest.approx(want)
+    loss.backward()
+    for i in range(2):
+        for j in range(4):
+            d = float(lp[i, j]) + 1.0
+            sign = (d > 0) - (d < 0)
+            gw = float(mask[i, j]) * (-float(adv[i, j]) * math.exp(d) + (0.5 * sign if (i, j) in order[:2] else 0.0))
+            assert float(x.grad[i, j]) == pytest.approx(gw)
+    # a fraction that rounds to zero still selects one token; finite differences with the selection held fixed
+    assert int(O.kl_cov_policy_loss(lp, old, adv, 0.01, 0.5, mask)[1].sum()) == 1
+    eps = 1e-6
+    for (i, j) in [(0, 1), (1, 2), (1, 3)]:
+        up, dn = lp.clone(), lp.clone()
+        up[i, j] += eps
+        dn[i, j] -= eps
+        fd = (float(O.kl_cov_policy_loss(up, old, adv, 0.3, 0.5, mask)[0]) - float(O.kl_cov_policy_loss(dn, old, adv, 0.3, 0.5, mask)[0])) / (2 * eps)
+        assert fd == pytest.approx(float(x.grad[i, j]), rel=1e-5, abs=1e-6)
+    # with nothing selected to pay (coef 0) it is the importance-sampling surrogate pinned above
+    assert float(O.kl_cov_policy_loss(lp, old, adv, 0.3, 0.0, mask)[0]) == pytest.approx(float(O.importance_sampling_loss(lp, old, adv, mask)[0]))
+
+
+def test_cispo_ratio_diagnostics_by_hand():
+    ln = math.log
+    lp, old = _t([ln(2) - 1, ln(3) - 1, ln(0.5) - 1, -1.0]), _t([-1.0] * 4)     # ratios 2, 3, 1/2, 1
+    d = O.cispo_ratio_diagnostics(lp, old, 0.25, 1.5)                           # clamp to [0.75, 2.5]
+    assert d["cispo/ratio_mean"] == pytest.approx(6.5 / 4) and d["cispo/ratio_clamped_mean"] == pytest.approx((2 + 2.5 + 0.75 + 1) / 4)
+    assert d["cispo/ratio_max"] == pytest.approx(3.0) and d["cispo/ratio_min"] == pytest.approx(0.5)
+    d = O.cispo_ratio_diagnostics(lp, old, 0.25, 1.5, _t([1.0, 0.0, 0.0, 1.0]))  # the masked extremes do not count
+    assert d["cispo/ratio_mean"] == pytest.approx(1.5) and d["cispo/ratio_max"] == pytest.approx(2.0) and d["cispo/ratio_min"] == pytest.approx(1.0)
+    d = O.cispo_ratio_diagnostics(lp, old, 0.25, 1.5, _t([0.0] * 4))             # an empty mask: extremes over all tokens, means 0
+    assert d["cispo/ratio_mean"] == 0.0 and d["cispo/ratio_max"] == pytest.approx(3.0) and d["cispo/ratio_min"] == pytest.approx(0.5)
+
+
 def test_dppo_by_hand():
     ln = math.log
     # probabilities now / behaviour: (0.5, 0.2), (0.2, 0.5), (0.5, 0.2), (0.2, 0.5), (0.3, 0.2)

@@ -785,6 +785,118 @@ def test_further_policy_losses_match_oracle(kind, masked, cuda_device):
     assert err <= 2e-5 * max(1.0, want_grad.abs().max().item()), f"actor-loss gradient max abs err {err}"
 
 
+def _cov_case(seed=47, B=6, S=203):
+    from types import SimpleNamespace
+
+    gen = torch.Generator().manual_seed(seed)
+    lp = (torch.randn(B, S, generator=gen) * 0.7 - 1.5).clamp(max=-0.02)
+    old = lp + torch.randn(B, S, generator=gen) * 0.3
+    adv = torch.randn(B, S, generator=gen)
+    mask = (torch.rand(B, S, generator=gen) > 0.3).float()
+    mask[1] = 0
+    cfg = SimpleNamespace(policy_loss_type="clip_cov", eps_clip_low=0.2, eps_clip_high=0.25, loss_reduction="sequence_mean",
+                          clip_cov=SimpleNamespace(clip_ratio=0.05, clip_cov_lb=0.05, clip_cov_ub=2.0),
+                          kl_cov=SimpleNamespace(kl_cov_frac=0.1, ppo_kl_coef=0.7))
+    return lp, old, adv, mask, cfg
+
+
+def test_clip_cov_policy_loss_matches_oracle(cuda_device):
+    """The clip-cov loss (ppo_utils.py:938-999): same tokens drawn as the oracle draws from the same generator state, same
+    loss, removed fraction and gradient.  Tokens whose candidate decision is within 1e-4 of a bound in fp64 are masked out."""
+    from skyrl_amd import policy_loss as PL
+
+    lp, old, adv, mask, cfg = _cov_case()
+    cc = cfg.clip_cov
+    m64 = mask.double()
+    cov = (adv.double() - O.masked_mean(adv.double(), m64)) * (lp.double() - O.masked_mean(lp.double(), m64))
+    ratio = (lp.double() - old.double()).exp()
+    fragile = ((cov - cc.clip_cov_lb).abs() < 1e-4) | ((cov - cc.clip_cov_ub).abs() < 1e-4) | \
+              ((ratio - 0.8).abs() < 1e-4) | ((ratio - 1.25).abs() < 1e-4)
+    mask = torch.where(fragile, torch.zeros(()), mask)
+    m64 = mask.double()
+    cov = (adv.double() - O.masked_mean(adv.double(), m64)) * (lp.double() - O.masked_mean(lp.double(), m64))
+    assert not bool((((cov - cc.clip_cov_lb).abs() < 5e-5) | ((cov - cc.clip_cov_ub).abs() < 5e-5))[mask > 0].any())
+    x = lp.double().requires_grad_(True)
+    torch.manual_seed(11)
+    ref, ref_frac, corr = O.clip_cov_policy_loss(x, old.double(), adv.double(), cfg.eps_clip_low, cfg.eps_clip_high, cc.clip_ratio,
+                                                 cc.clip_cov_lb, cc.clip_cov_ub, m64)
+    ref.backward()
+    removed = int((corr == 0).sum())
+    assert removed == max(int(cc.clip_ratio * float(mask.sum())), 1)      # enough candidates: the draw is a strict subset
+    to = lambda t: t.to(cuda_device)  # noqa: E731
+    d = to(lp).requires_grad_(True)
+    torch.manual_seed(11)
+    loss, metrics = PL.compute_policy_loss_clip_cov(d, to(old), to(adv), cfg, to(mask))
+    loss.backward()
+    scale = max(abs(ref.item()), 1e3)
+    assert abs(loss.item() - ref.item()) <= 5e-6 * scale, (loss.item(), ref.item())
+    assert metrics["clip_ratio"] == pytest.approx(ref_frac.item(), abs=1e-6)
+    err = (d.grad.double().cpu() - x.grad).abs().max().item()
+    assert err <= 1e-5 * max(1.0, x.grad.abs().max().item()), f"gradient max abs err {err}"
+    # exactly the drawn tokens, the masked ones and the ones the clip catches carry no gradient
+    assert bool((d.grad.cpu()[(corr == 0) | (mask == 0)] == 0).all())
+    # another generator state draws other tokens
+    torch.manual_seed(12)
+    d2 = to(lp).requires_grad_(True)
+    PL.compute_policy_loss_clip_cov(d2, to(old), to(adv), cfg, to(mask))[0].backward()
+    assert not torch.equal(d2.grad == 0, d.grad == 0)
+    # no candidate inside the bounds: the clipped surrogate on the unclamped ratio
+    cfg.clip_cov.clip_cov_lb, cfg.clip_cov.clip_cov_ub = 500.0, 600.0
+    x = lp.double().requires_grad_(True)
+    ref, ref_frac, _ = O.clip_cov_policy_loss(x, old.double(), adv.double(), 0.2, 0.25, cc.clip_ratio, 500.0, 600.0, m64)
+    loss, metrics = PL.compute_policy_loss_clip_cov(to(lp), to(old), to(adv), cfg, to(mask))
+    assert abs(loss.item() - ref.item()) <= 5e-6 * scale and metrics["clip_ratio"] == 0.0 == ref_frac.item()
+
+
+def test_kl_cov_policy_loss_matches_oracle(cuda_device):
+    """The kl-cov loss (ppo_utils.py:1002-1053): the same top-k tokens as the oracle, loss and gradient."""
+    from skyrl_amd import policy_loss as PL
+
+    lp, old, adv, mask, cfg = _cov_case(seed=53)
+    kc = cfg.kl_cov
+    old[0, 0] = lp[0, 0]                                          # a log-ratio of exactly zero: |.| has subgradient 0 there
+    x = lp.double().requires_grad_(True)
+    ref, sel = O.kl_cov_policy_loss(x, old.double(), adv.double(), kc.kl_cov_frac, kc.ppo_kl_coef, mask.double())
+    ref.backward()
+    k = max(1, int(float((mask > 0).sum()) * kc.kl_cov_frac))
+    assert int(sel.sum()) == k
+    # the k-th and (k+1)-th covariance terms are far enough apart for fp32 to order them alike
+    valid = mask > 0
+    c = ((adv.double()[valid] - adv.double()[valid].mean()) * (lp.double()[valid] - lp.double()[valid].mean())).sort(descending=True).values
+    assert float(c[k - 1] - c[k]) > 1e-5
+    to = lambda t: t.to(cuda_device)  # noqa: E731
+    d = to(lp).requires_grad_(True)
+    loss, metrics = PL.compute_policy_loss_kl_cov(d, to(old), to(adv), cfg, to(mask))
+    loss.backward()
+    assert metrics == {"clip_ratio": 0.0}
+    assert abs(loss.item() - ref.item()) <= 5e-6 * max(abs(ref.item()), 1e3)
+    err = (d.grad.double().cpu() - x.grad).abs().max().item()
+    assert err <= 1e-5 * max(1.0, x.grad.abs().max().item()), f"gradient max abs err {err}"
+    # with a zero coefficient it is the importance-sampling loss of the same kernel, bit for bit
+    cfg.kl_cov.ppo_kl_coef = 0.0
+    a, _ = PL.compute_policy_loss_kl_cov(to(lp), to(old), to(adv), cfg, to(mask))
+    b, _ = PL.importance_sampling_loss(to(lp), to(old), to(adv), None, to(mask))
+    assert a.item() == pytest.approx(b.item(), rel=1e-6)
+
+
+@pytest.mark.parametrize("masked", ["none", "some", "empty"])
+def test_cispo_ratio_diagnostics_match_oracle(masked, cuda_device):
+    from skyrl_amd import policy_loss as PL
+
+    lp, old, adv, mask, _weight, cfg, *_ = _further_loss_case("cispo", masked == "some")
+    if masked == "empty":
+        mask = torch.zeros_like(lp)
+    m64 = None if mask is None else mask.double()
+    want = O.cispo_ratio_diagnostics(lp.double(), old.double(), cfg.cispo.cispo_eps_clip_low, cfg.cispo.cispo_eps_clip_high, m64)
+    to = lambda t: None if t is None else t.to(cuda_device)  # noqa: E731
+    _, metrics = PL.compute_policy_loss_cispo(to(lp), to(old), to(adv), cfg, to(mask))
+    _, lazy = PL.compute_policy_loss_cispo(to(lp), to(old), to(adv), cfg, to(mask), sync_metrics=False)
+    for key, value in want.items():
+        assert metrics[key] == pytest.approx(value, rel=1e-5, abs=1e-9), key
+        assert isinstance(lazy[key], torch.Tensor) and lazy[key].item() == metrics[key]
+    assert want["cispo/ratio_max"] == pytest.approx(math.exp(20.0)) or masked == "some"   # the clamp of the log-ratio at +-20
+
+
 def test_further_policy_losses_argument_handling(cuda_device):
     from types import SimpleNamespace
 
