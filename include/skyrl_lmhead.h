@@ -341,8 +341,8 @@ int skyrl_packed_gather_grad(const float* d_out, const int64_t* cu_seqlens, int6
  * skyrl_softce_bwd writes d_student_hidden [T, H] bf16 = sum_v dloss[t] * (softmax(z_s) - softmax(z_t))_v / temperature *
  * weight[v] (soft_ce.py:146-151 followed by the output layer's input gradient).  The teacher and the weight get no gradient:
  * the reference detaches both (soft_ce.py:16-19, mtp/adapter.py:51-56).  Workspaces: 256-byte aligned device memory of at
- * least the queried size (0 = bad arguments); vocab_chunk as in skyrl_lmhead_bwd.  Not covered: the top-k variant
- * (draft_soft_ce_topk, soft_ce.py:243-341) and more than one vocabulary shard.
+ * least the queried size (0 = bad arguments); vocab_chunk as in skyrl_lmhead_bwd.  Not covered: more than one vocabulary
+ * shard.
  */
 size_t skyrl_softce_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V);
 size_t skyrl_softce_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t vocab_chunk);
@@ -354,6 +354,35 @@ int skyrl_softce_bwd(const void* student_hidden, int64_t ld_student, const void*
                      const void* weight, int64_t ld_weight, const float* lse_student, const float* lse_teacher,
                      const float* dloss, int64_t T, int64_t seq_len, int64_t shift, int64_t H, int64_t V, float rcp_temperature,
                      void* d_student_hidden, int64_t vocab_chunk, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- top-k draft loss from hidden states ----------------------------------------------------------------------------
+ * Stands in for draft_soft_ce_topk / _VocabParallelTopkSoftCE (skyrl/backends/skyrl_train/mtp/soft_ce.py:243-341) on one
+ * vocabulary shard, together with the two output-layer products in front of it: only the teacher's k largest logits of a
+ * token are distilled, teacher and student renormalised over those k columns.
+ *
+ * skyrl_lmhead_topk_logits stands in for `teacher_logits.topk(k, dim=-1)` (:273) on logits = hidden . weight^T *
+ * rcp_temperature that are never stored: values [T, k] fp32 and columns [T, k] int32, best first; among equal values the
+ * lower column comes first.  1 <= k <= min(V, 1024).  The workspace (256-byte aligned, at least the queried size, 0 = bad
+ * arguments) does not grow with T * V: at most 16384 tokens x 8192 candidate slots of 8 bytes.
+ *
+ * skyrl_softce_topk_fwd: token b * seq_len + s takes the teacher's list of token b * seq_len + (s + shift) % seq_len (the roll
+ * of the [B, S, k] result, :276-279), gathers the student's logits at those columns (k dot products of student_hidden[t] with
+ * weight rows, :282), and writes loss [T] = -sum_j softmax(teacher)_j log softmax(student)_j (:285-300), coef [T, k] =
+ * softmax(student) - softmax(teacher) (:309) and the columns [T, k] it used -- the O(T * k) state the backward needs.
+ * skyrl_softce_topk_bwd writes d_student_hidden [T, H] bf16 = dloss[t] * rcp_temperature * sum_j coef[t, j] * weight[columns
+ * [t, j]] (the scatter of :309-312 followed by the output layer's input gradient).  Teacher and weight get no gradient.
+ */
+size_t skyrl_lmhead_topk_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t k);
+int skyrl_lmhead_topk_logits(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight, int64_t T, int64_t H,
+                             int64_t V, int64_t k, float rcp_temperature, float* values, int32_t* columns, void* workspace,
+                             size_t workspace_bytes, void* stream);
+int skyrl_softce_topk_fwd(const void* student_hidden, int64_t ld_student, const void* weight, int64_t ld_weight,
+                          const float* teacher_values, const int32_t* teacher_columns, int64_t T, int64_t seq_len, int64_t shift,
+                          int64_t H, int64_t V, int64_t k, float rcp_temperature, float* loss, float* coef, int32_t* columns,
+                          void* stream);
+int skyrl_softce_topk_bwd(const void* weight, int64_t ld_weight, const float* coef, const int32_t* columns, const float* dloss,
+                          int64_t T, int64_t H, int64_t V, int64_t k, float rcp_temperature, void* d_student_hidden,
+                          int64_t ld_d_student, void* stream);
 
 #ifdef __cplusplus
 }

@@ -49,6 +49,11 @@ What pins each function (all in ``tests/test_oracle.py``; none of them re-types 
     against ``torch.distributions`` / ``torch.nn.functional.kl_div``, the limits "teacher = student -> entropy" (the
     reference's known answer, test_soft_ce.py:248-284) and "one-hot teacher -> -log q(label)" (the pinned log-probability),
     and the gradient softmax(student) - softmax(teacher) (test_soft_ce.py:171-181) by fp64 finite differences.
+  * MTP top-k soft cross-entropy: a per-token Python loop that picks the k largest teacher logits with ``sorted`` and sums
+    the loss with ``math``; the limit k = V, where it is the full soft cross-entropy pinned above; the roll of the small
+    [B, S, k] lists against a pre-rolled teacher (the reference's own check, test_soft_ce.py:122-144); the restated custom
+    backward against autograd of the forward and fp64 finite differences, and its at most k non-zero columns per token
+    (test_soft_ce.py:147-156).
 No function is left "parity unpinned".
 """
 
@@ -806,3 +811,51 @@ def draft_soft_ce_from_hidden(student_hidden, teacher_hidden, weight, mask, mtp_
     student_logits = student_hidden @ w.t()
     teacher_logits = build_teacher_logits(teacher_hidden.detach() @ w.t(), mtp_layer_number)
     return draft_soft_ce(student_logits, teacher_logits, mask, global_normalization_factor)
+
+
+def soft_ce_topk_per_token(student_logits: torch.Tensor, teacher_logits: torch.Tensor, k: int, roll_shift: int = 0):
+    """mtp/soft_ce.py:258-305 (``_VocabParallelTopkSoftCE.forward`` with a group of one): the teacher's ``min(k, V)`` largest
+    logits per position, the small ``[B, S, k]`` lists rolled left by ``roll_shift``, the student's logits gathered at those
+    columns, both softmaxes over the k columns only.  Returns ``(per_token_loss, q_student, p_teacher, columns)``; autograd
+    differentiates the loss through the gather."""
+    up = torch.float64 if student_logits.dtype == torch.float64 else torch.float32
+    k_eff = min(int(k), teacher_logits.shape[-1])
+    t_vals, t_idx = teacher_logits.detach().topk(k_eff, dim=-1)
+    if roll_shift:
+        t_vals = torch.roll(t_vals, shifts=-int(roll_shift), dims=1)
+        t_idx = torch.roll(t_idx, shifts=-int(roll_shift), dims=1)
+    t_vals = t_vals.to(up)
+    s_vals = student_logits.gather(-1, t_idx).to(up)
+    t_exp = (t_vals - t_vals.max(dim=-1, keepdim=True).values).exp()
+    t_p = t_exp / t_exp.sum(dim=-1, keepdim=True)
+    s_shift = s_vals - s_vals.max(dim=-1, keepdim=True).values
+    s_denom = s_shift.exp().sum(dim=-1, keepdim=True)
+    q_s = s_shift.exp() / s_denom
+    s_logp = s_shift - s_denom.log()
+    return -(t_p * s_logp).sum(dim=-1), q_s, t_p, t_idx
+
+
+def soft_ce_topk_backward(q_student, p_teacher, columns, grad_output, vocab_size: int) -> torch.Tensor:
+    """mtp/soft_ce.py:307-315: ``(softmax(student) - softmax(teacher)) * grad`` scattered to the k columns, zero elsewhere."""
+    grad_topk = (q_student - p_teacher) * grad_output.unsqueeze(-1)
+    grad = torch.zeros(*columns.shape[:-1], vocab_size, dtype=grad_topk.dtype)
+    grad.scatter_(-1, columns, grad_topk)
+    return grad
+
+
+def draft_soft_ce_topk(student_logits, teacher_logits, mask, k: int, global_normalization_factor=None, roll_shift: int = 0):
+    """mtp/soft_ce.py:318-341 with the reduction of :154-159."""
+    assert not teacher_logits.requires_grad, "MTP draft loss: teacher_logits must be detached"
+    per_token = soft_ce_topk_per_token(student_logits, teacher_logits, k, roll_shift)[0]
+    if global_normalization_factor is not None:
+        return (per_token * mask).sum() / global_normalization_factor.clamp(min=1.0)
+    return masked_mean(per_token, mask)
+
+
+def draft_soft_ce_topk_from_hidden(student_hidden, teacher_hidden, weight, mask, k: int, global_normalization_factor=None,
+                                   roll_shift: int = 0):
+    """Both hidden states through the shared, detached output layer (mtp/adapter.py:51-64), the teacher un-rolled, then
+    ``draft_soft_ce_topk`` with the MTP depth as ``roll_shift`` (megatron_model_wrapper.py passes ``mtp_layer_number + 1``)."""
+    w = weight.detach()
+    return draft_soft_ce_topk(student_hidden @ w.t(), teacher_hidden.detach() @ w.t(), mask, k, global_normalization_factor,
+                              roll_shift)

@@ -11,7 +11,7 @@ import os
 import threading
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libskyrl_lmhead.so")
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 _c_i64 = ctypes.c_int64
 _c_p = ctypes.c_void_p
@@ -77,6 +77,20 @@ SIGNATURES = {
         ctypes.c_int,
         [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, ctypes.c_float,
          _c_p, _c_i64, _c_p, ctypes.c_size_t, _c_p],
+    ),
+    "skyrl_lmhead_topk_workspace_bytes": (ctypes.c_size_t, [_c_i64, _c_i64, _c_i64, _c_i64]),
+    "skyrl_lmhead_topk_logits": (
+        ctypes.c_int,
+        [_c_p, _c_i64, _c_p, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, ctypes.c_float, _c_p, _c_p, _c_p, ctypes.c_size_t, _c_p],
+    ),
+    "skyrl_softce_topk_fwd": (
+        ctypes.c_int,
+        [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, ctypes.c_float, _c_p, _c_p, _c_p,
+         _c_p],
+    ),
+    "skyrl_softce_topk_bwd": (
+        ctypes.c_int,
+        [_c_p, _c_i64, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_i64, ctypes.c_float, _c_p, _c_i64, _c_p],
     ),
     "skyrl_lmhead_mfma_probe": (ctypes.c_int, [_c_p, ctypes.c_int, ctypes.c_int, _c_p, _c_p]),
     "skyrl_lmhead_device_info": (ctypes.c_int, [ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]),

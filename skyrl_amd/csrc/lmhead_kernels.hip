@@ -28,6 +28,7 @@
 #include "../../include/skyrl_lmhead.h"
 #include "../../include/skyrl_lmhead_bench.h"
 #include "gemm_core.hpp"
+#include "topk_kernels.hpp"
 
 using namespace lmhead;
 
@@ -974,13 +975,15 @@ __global__ __launch_bounds__(256) void zero_f32(float* __restrict__ p, int n) {
 // HIP events on the launch stream.  Closed profiles cost one thread-local load per launch.
 enum KernelKind {
   kFwdTiles = 0, kFwdMerge, kTranspose, kBwdChunkDz, kBwdChunkGemm, kSoftCePack, kSoftCeFwdTiles, kSoftCeFinish, kSoftCeDz,
-  kCompactRows, kSplitOperand,
+  kCompactRows, kSplitOperand, kTopkFilter, kTopkSelect, kTopkRows, kTopkBwdRows,
   kNumKernelKinds
 };
 const char* const kKernelNames[kNumKernelKinds] = {"lmhead_fwd_tiles", "lmhead_fwd_merge", "transpose_bf16",
                                                    "lmhead_bwd_chunk[dz]", "lmhead_bwd_chunk[gemm]", "softce_pack_rows",
                                                    "softce_fwd_tiles", "softce_finish", "softce_dz_tiles",
-                                                   "active_rows[compact+gather+scatter]", "split_operand_rows"};
+                                                   "active_rows[compact+gather+scatter]", "split_operand_rows",
+                                                   "topk_filter_tiles", "topk_select", "topk_softce_rows",
+                                                   "topk_softce_bwd_rows"};
 struct Profile {
   struct Rec {
     int kind;
@@ -1339,6 +1342,38 @@ hipError_t launch_softce_pack(hipStream_t s, const void* student, int64_t lds_, 
   return hipGetLastError();
 }
 
+
+// Top-k logits from hidden states.  Tokens are walked in blocks of at most 16384 and the vocabulary in chunks of 1024, 2048,
+// 4096 and then 8192 columns: the first chunk passes every logit (no threshold yet), and from then on a logit passes with
+// probability k / (columns seen so far) on exchangeable columns, so that short early chunks keep the candidate lists short.
+// A candidate list holds a whole chunk (cap columns per token), which makes the filter exact for any data: in the worst
+// case -- logits ascending with the column -- every logit is a candidate and the select kernel does all the work.
+constexpr int64_t kTopkTokenBlock = 16384;
+constexpr int64_t kTopkFirstChunk = 1024, kTopkMaxChunk = 8192;
+
+struct TopkWorkspace {
+  unsigned *cnt, *have;
+  float* thr;
+  topk::key_t *best, *cand;
+  int64_t block_tokens, cap;
+  size_t bytes;
+};
+
+TopkWorkspace carve_topk(void* ws, int64_t T, int64_t V, int64_t k) {
+  TopkWorkspace w;
+  w.block_tokens = T < kTopkTokenBlock ? T : kTopkTokenBlock;
+  const int64_t vpad = round_up(V, 256);
+  w.cap = vpad < kTopkMaxChunk ? vpad : kTopkMaxChunk;
+  Carver c(ws);
+  w.cnt = c.take<unsigned>((size_t)w.block_tokens);
+  w.have = c.take<unsigned>((size_t)w.block_tokens);
+  w.thr = c.take<float>((size_t)w.block_tokens);
+  w.best = c.take<topk::key_t>((size_t)w.block_tokens * (size_t)k);
+  w.cand = c.take<topk::key_t>((size_t)w.block_tokens * (size_t)w.cap);
+  w.bytes = (size_t)round_up((int64_t)c.off, 256);
+  return w;
+}
+
 size_t bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t vocab_chunk, bool compact, int64_t terms = 1) {
   if (T < 1 || V < 1 || H < 1 || vocab_chunk < 0 || vocab_chunk % 256 != 0 || terms < 1 || terms > 3) return 0;
   if (T > kMaxExtent || V > kMaxExtent || H > kMaxExtent / 4 || vocab_chunk > kMaxExtent) return 0;
@@ -1513,7 +1548,7 @@ int bwd_entry(const void* hidden, int64_t ld_hidden, const void* weight, int64_t
 
 extern "C" {
 
-int skyrl_lmhead_version(void) { return 15; }
+int skyrl_lmhead_version(void) { return 16; }
 
 const char* skyrl_lmhead_strerror(int status) {
   switch (status) {
@@ -1746,6 +1781,110 @@ int skyrl_softce_bwd(const void* student_hidden, int64_t ld_student, const void*
     if (e != hipSuccess) return (int)e;
   }
   return SKYRL_LMHEAD_OK;
+}
+
+
+size_t skyrl_lmhead_topk_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t k) {
+  if (T < 1 || V < 1 || H < 1 || k < 1 || k > V || k > topk::kMaxK) return 0;
+  if (T > kMaxExtent || V > kMaxExtent || H > kMaxExtent) return 0;
+  return carve_topk(nullptr, T, V, k).bytes;
+}
+
+int skyrl_lmhead_topk_logits(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight, int64_t T, int64_t H,
+                             int64_t V, int64_t k, float rcp_temperature, float* values, int32_t* columns, void* workspace,
+                             size_t workspace_bytes, void* stream) {
+  int st = check_operands(hidden, ld_hidden, weight, ld_weight, T, H, V, rcp_temperature, true);
+  if (st) return st;
+  if (!values || !columns) return SKYRL_LMHEAD_ERR_NULL;
+  if (k < 1 || k > V || k > topk::kMaxK) return SKYRL_LMHEAD_ERR_ARG;
+  if (!workspace || workspace_bytes < skyrl_lmhead_topk_workspace_bytes(T, H, V, k)) return SKYRL_LMHEAD_ERR_WORKSPACE;
+  if ((uintptr_t)workspace & 255u) return SKYRL_LMHEAD_ERR_ALIGN;
+
+  hipStream_t s = (hipStream_t)stream;
+  const TopkWorkspace w = carve_topk(workspace, T, V, k);
+  const int64_t block_tokens = fwd_block_tokens(w.block_tokens, ld_hidden);
+  const uint16_t* Wp = (const uint16_t*)weight;
+  const size_t select_lds = (size_t)topk::kSelectWaves * (size_t)k * sizeof(topk::key_t);
+  hipError_t e;
+  for (int64_t t0 = 0; t0 < T; t0 += block_tokens) {
+    const int64_t Tb = (T - t0) < block_tokens ? (T - t0) : block_tokens;
+    const int tiles_n = (int)((Tb + BN - 1) / BN);
+    const uint16_t* Hp = (const uint16_t*)hidden + (size_t)t0 * (size_t)ld_hidden;
+    hipLaunchKernelGGL(topk::topk_reset, dim3((unsigned)((Tb + 255) / 256)), dim3(256), 0, s, (int)Tb, w.have, w.thr, w.cnt);
+    if ((e = hipGetLastError()) != hipSuccess) return (int)e;
+    int64_t width = kTopkFirstChunk;
+    for (int64_t v0 = 0; v0 < V;) {
+      const int64_t chunk = width < w.cap ? width : w.cap;
+      const int64_t vrows = (V - v0) < chunk ? (V - v0) : chunk;
+      const bool last = v0 + vrows >= V;
+      topk::FilterArgs a{Wp + (size_t)v0 * (size_t)ld_weight, (int)ld_weight, Hp, (int)ld_hidden, (int)Tb, (int)H, (int)vrows,
+                         (int)v0, rcp_temperature, (int)((vrows + BM - 1) / BM), tiles_n, kGroupM, w.thr, w.cnt, w.cand,
+                         (int)w.cap};
+      {
+        Timed timed(kTopkFilter, s);
+        hipLaunchKernelGGL(topk::topk_filter_tiles, dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(NTHREADS), 0, s, a);
+      }
+      if ((e = hipGetLastError()) != hipSuccess) return (int)e;
+      {
+        Timed timed(kTopkSelect, s);
+        hipLaunchKernelGGL(topk::topk_select, dim3((unsigned)((Tb + topk::kSelectWaves - 1) / topk::kSelectWaves)),
+                           dim3(64 * topk::kSelectWaves), select_lds, s, (int)Tb, (int)k, w.best, w.have, w.thr, w.cnt, w.cand,
+                           (int)w.cap, last ? values + (size_t)t0 * (size_t)k : (float*)nullptr,
+                           last ? columns + (size_t)t0 * (size_t)k : (int32_t*)nullptr);
+      }
+      if ((e = hipGetLastError()) != hipSuccess) return (int)e;
+      v0 += vrows;
+      width *= 2;
+    }
+  }
+  return SKYRL_LMHEAD_OK;
+}
+
+namespace {
+int check_topk_rows(const void* weight, int64_t ld_weight, int64_t T, int64_t H, int64_t V, int64_t k, float rcp_temperature) {
+  if (!weight) return SKYRL_LMHEAD_ERR_NULL;
+  if (T < 1 || V < 1 || H < 8 || H % 8 != 0 || ld_weight < H || k < 1 || k > V || k > topk::kMaxK) return SKYRL_LMHEAD_ERR_SHAPE;
+  if (T > kMaxExtent || V > kMaxExtent || H > kMaxExtent || ld_weight > kMaxExtent) return SKYRL_LMHEAD_ERR_SHAPE;
+  if (!aligned16(weight) || ld_weight % 8 != 0) return SKYRL_LMHEAD_ERR_ALIGN;
+  if (!(rcp_temperature > 0.f) || !isfinite(rcp_temperature)) return SKYRL_LMHEAD_ERR_ARG;
+  return SKYRL_LMHEAD_OK;
+}
+}  // namespace
+
+int skyrl_softce_topk_fwd(const void* student_hidden, int64_t ld_student, const void* weight, int64_t ld_weight,
+                          const float* teacher_values, const int32_t* teacher_columns, int64_t T, int64_t seq_len, int64_t shift,
+                          int64_t H, int64_t V, int64_t k, float rcp_temperature, float* loss, float* coef, int32_t* columns,
+                          void* stream) {
+  int st = check_topk_rows(weight, ld_weight, T, H, V, k, rcp_temperature);
+  if (st) return st;
+  if (!student_hidden || !teacher_values || !teacher_columns || !loss || !coef || !columns) return SKYRL_LMHEAD_ERR_NULL;
+  if (ld_student < H || ld_student > kMaxExtent || seq_len < 1 || T % seq_len != 0 || shift < 0) return SKYRL_LMHEAD_ERR_SHAPE;
+  if (!aligned16(student_hidden) || ld_student % 8 != 0) return SKYRL_LMHEAD_ERR_ALIGN;
+  hipStream_t s = (hipStream_t)stream;
+  Timed timed(kTopkRows, s);
+  hipLaunchKernelGGL(topk::topk_softce_rows, dim3((unsigned)T), dim3(topk::kRowThreads), (size_t)(2 * k + 4) * sizeof(float), s,
+                     (const uint16_t*)student_hidden, (int)ld_student, (const uint16_t*)weight, (int)ld_weight, teacher_values,
+                     teacher_columns, (int)T, (int)seq_len, (int)(shift % seq_len), (int)H, (int)V, (int)k, rcp_temperature, loss,
+                     coef, columns);
+  const hipError_t e = hipGetLastError();
+  return e == hipSuccess ? SKYRL_LMHEAD_OK : (int)e;
+}
+
+int skyrl_softce_topk_bwd(const void* weight, int64_t ld_weight, const float* coef, const int32_t* columns, const float* dloss,
+                          int64_t T, int64_t H, int64_t V, int64_t k, float rcp_temperature, void* d_student_hidden,
+                          int64_t ld_d_student, void* stream) {
+  int st = check_topk_rows(weight, ld_weight, T, H, V, k, rcp_temperature);
+  if (st) return st;
+  if (!coef || !columns || !dloss || !d_student_hidden) return SKYRL_LMHEAD_ERR_NULL;
+  if (ld_d_student < H || ld_d_student > kMaxExtent) return SKYRL_LMHEAD_ERR_SHAPE;
+  if (!aligned16(d_student_hidden) || ld_d_student % 8 != 0) return SKYRL_LMHEAD_ERR_ALIGN;
+  hipStream_t s = (hipStream_t)stream;
+  Timed timed(kTopkBwdRows, s);
+  hipLaunchKernelGGL(topk::topk_softce_bwd_rows, dim3((unsigned)T), dim3(topk::kRowThreads), (size_t)(2 * k) * sizeof(float), s,
+                     (const uint16_t*)weight, (int)ld_weight, coef, columns, dloss, (int)H, (int)V, (int)k, rcp_temperature,
+                     (uint16_t*)d_student_hidden, (int)ld_d_student);
+  const hipError_t e = hipGetLastError();
+  return e == hipSuccess ? SKYRL_LMHEAD_OK : (int)e;
 }
 
 int skyrl_lmhead_mfma_probe(const void* operands, int workgroups, int iters, float* sink, void* stream) {

@@ -13,7 +13,11 @@ chunking with recomputation (:162-197).  Here the loss and its gradient come str
   logits and ``mtp_layer_number`` in place of a pre-rolled teacher;
 * ``shift_mask_for_mtp`` (:37-79) -- the mask roll the caller applies, same signature and results.
 
-No ``[T, V]`` tensor exists at any point; the top-k variant (``draft_soft_ce_topk``) is not part of this module.
+* ``topk_logits_from_hidden``, ``soft_ce_topk_from_hidden``, ``draft_soft_ce_topk_from_hidden`` -- the top-k variant
+  (``draft_soft_ce_topk`` / ``_VocabParallelTopkSoftCE``, :243-341): the teacher's k largest logits per token straight from
+  its hidden states, the student's logits at those columns as k gathered dot products, loss and gradient over the k columns.
+
+No ``[T, V]`` tensor exists at any point.
 """
 
 from __future__ import annotations
@@ -25,7 +29,9 @@ import torch
 from . import _lib
 from .ops import _require_device
 
-__all__ = ["soft_ce_from_hidden", "draft_soft_ce_from_hidden", "shift_mask_for_mtp", "softce_fwd", "softce_bwd"]
+__all__ = ["soft_ce_from_hidden", "draft_soft_ce_from_hidden", "shift_mask_for_mtp", "softce_fwd", "softce_bwd",
+           "topk_logits_from_hidden", "soft_ce_topk_from_hidden", "draft_soft_ce_topk_from_hidden", "topk_logits",
+           "softce_topk_fwd", "softce_topk_bwd"]
 
 
 def _check(student: torch.Tensor, teacher: torch.Tensor, weight: torch.Tensor, seq_len: int) -> Tuple[int, int, int]:
@@ -168,6 +174,167 @@ def draft_soft_ce_from_hidden(
             and torch.distributed.get_world_size(vocab_parallel_group) > 1:
         raise NotImplementedError("the fused soft cross-entropy covers one vocabulary shard")
     per_token = soft_ce_from_hidden(student_hidden, teacher_hidden, weight, shift=mtp_layer_number + 1, vocab_chunk=vocab_chunk)
+    mask = mask.to(per_token.dtype)
+    if global_normalization_factor is not None:
+        return (per_token * mask).sum() / global_normalization_factor.clamp(min=1.0)
+    return (per_token * mask).sum() / mask.sum().clamp(min=1.0)
+
+
+@torch.library.custom_op("skyrl_amd::topk_logits", mutates_args=())
+def topk_logits(hidden: torch.Tensor, weight: torch.Tensor, k: int, rcp_temperature: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``(values [T, k] fp32, columns [T, k] int32)``: the k largest entries of every row of ``hidden @ weight.T *
+    rcp_temperature``, best first, the lower column first among equal values.  bf16 operands, ``1 <= k <= min(V, 1024)``."""
+    T, H, V = _check(hidden, hidden, weight, 1)
+    dev = _require_device(hidden, weight)
+    lib = _lib.load()
+    ws_bytes = int(lib.skyrl_lmhead_topk_workspace_bytes(T, H, V, int(k)))
+    if ws_bytes == 0:
+        raise ValueError(f"bad k {k}: must be between 1 and min(V, 1024) = {min(V, 1024)}")
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    values = torch.empty((T, k), dtype=torch.float32, device=dev)
+    columns = torch.empty((T, k), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        st = lib.skyrl_lmhead_topk_logits(hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), T, H, V, int(k),
+                                          float(rcp_temperature), values.data_ptr(), columns.data_ptr(), ws.data_ptr(), ws.numel(),
+                                          torch.cuda.current_stream(dev).cuda_stream)
+    _lib.check(st, "skyrl_lmhead_topk_logits")
+    return values, columns
+
+
+@topk_logits.register_fake
+def _(hidden, weight, k, rcp_temperature):
+    T = hidden.shape[0]
+    return hidden.new_empty((T, k), dtype=torch.float32), hidden.new_empty((T, k), dtype=torch.int32)
+
+
+@torch.library.custom_op("skyrl_amd::softce_topk_fwd", mutates_args=())
+def softce_topk_fwd(student_hidden: torch.Tensor, weight: torch.Tensor, teacher_values: torch.Tensor, teacher_columns: torch.Tensor,
+                    seq_len: int, shift: int, rcp_temperature: float) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``(loss [T] fp32, coef [T, k] fp32, columns [T, k] int32)`` for bf16 ``student_hidden [T, H]``, ``weight [V, H]`` and the
+    teacher's top-k lists; token ``b * seq_len + s`` is scored against the list of token ``b * seq_len + (s + shift) mod seq_len``."""
+    T, H, V = _check(student_hidden, student_hidden, weight, seq_len)
+    dev = _require_device(student_hidden, weight, teacher_values, teacher_columns)
+    k = int(teacher_values.shape[1]) if teacher_values.dim() == 2 else 0
+    if (teacher_values.shape != (T, k) or teacher_columns.shape != (T, k) or teacher_values.dtype != torch.float32
+            or teacher_columns.dtype != torch.int32 or not teacher_values.is_contiguous() or not teacher_columns.is_contiguous()):
+        raise ValueError(f"teacher_values must be contiguous fp32 [{T}, k] and teacher_columns contiguous int32 [{T}, k]")
+    lib = _lib.load()
+    loss = torch.empty(T, dtype=torch.float32, device=dev)
+    coef = torch.empty((T, k), dtype=torch.float32, device=dev)
+    columns = torch.empty((T, k), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        st = lib.skyrl_softce_topk_fwd(student_hidden.data_ptr(), student_hidden.stride(0), weight.data_ptr(), weight.stride(0),
+                                       teacher_values.data_ptr(), teacher_columns.data_ptr(), T, int(seq_len), int(shift), H, V, k,
+                                       float(rcp_temperature), loss.data_ptr(), coef.data_ptr(), columns.data_ptr(),
+                                       torch.cuda.current_stream(dev).cuda_stream)
+    _lib.check(st, "skyrl_softce_topk_fwd")
+    return loss, coef, columns
+
+
+@softce_topk_fwd.register_fake
+def _(student_hidden, weight, teacher_values, teacher_columns, seq_len, shift, rcp_temperature):
+    T = student_hidden.shape[0]
+    return (student_hidden.new_empty(T, dtype=torch.float32), torch.empty_like(teacher_values), torch.empty_like(teacher_columns))
+
+
+@torch.library.custom_op("skyrl_amd::softce_topk_bwd", mutates_args=())
+def softce_topk_bwd(weight: torch.Tensor, coef: torch.Tensor, columns: torch.Tensor, dloss: torch.Tensor,
+                    rcp_temperature: float) -> torch.Tensor:
+    """d loss / d student_hidden, bf16 ``[T, H]``, from what ``softce_topk_fwd`` kept and the upstream gradient ``dloss [T]``."""
+    T, k = int(coef.shape[0]), int(coef.shape[1])
+    V, H = int(weight.shape[0]), int(weight.shape[1])
+    dev = _require_device(weight, coef, columns, dloss)
+    if weight.dtype != torch.bfloat16 or weight.stride(1) != 1:
+        raise TypeError("weight must be bf16 with unit stride in the last dimension")
+    if (coef.dtype != torch.float32 or columns.dtype != torch.int32 or columns.shape != coef.shape or not coef.is_contiguous()
+            or not columns.is_contiguous() or dloss.dtype != torch.float32 or dloss.shape != (T,) or not dloss.is_contiguous()):
+        raise ValueError("coef fp32 [T, k], columns int32 [T, k] and dloss fp32 [T] must be contiguous")
+    lib = _lib.load()
+    d_student = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    with torch.cuda.device(dev):
+        st = lib.skyrl_softce_topk_bwd(weight.data_ptr(), weight.stride(0), coef.data_ptr(), columns.data_ptr(), dloss.data_ptr(), T, H,
+                                       V, k, float(rcp_temperature), d_student.data_ptr(), H, torch.cuda.current_stream(dev).cuda_stream)
+    _lib.check(st, "skyrl_softce_topk_bwd")
+    return d_student
+
+
+@softce_topk_bwd.register_fake
+def _(weight, coef, columns, dloss, rcp_temperature):
+    return weight.new_empty((coef.shape[0], weight.shape[1]))
+
+
+class _SoftCETopk(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, student_hidden, teacher_hidden, weight, k, seq_len, shift, rcp_temperature):
+        values, columns = topk_logits(teacher_hidden, weight, k, rcp_temperature)
+        loss, coef, used = softce_topk_fwd(student_hidden, weight, values, columns, seq_len, shift, rcp_temperature)
+        ctx.save_for_backward(weight, coef, used)
+        ctx.rcp_temperature = rcp_temperature
+        return loss
+
+    @staticmethod
+    def backward(ctx, dloss):
+        weight, coef, used = ctx.saved_tensors
+        return (softce_topk_bwd(weight, coef, used, dloss.to(torch.float32).contiguous(), ctx.rcp_temperature), None, None, None,
+                None, None, None)
+
+
+def topk_logits_from_hidden(hidden: torch.Tensor, weight: torch.Tensor, k: int, *, temperature: float = 1.0
+                            ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``(hidden @ weight.T / temperature).topk(min(k, V), dim=-1)`` without the logits: values fp32 and indices int64 of shape
+    ``hidden.shape[:-1] + (k,)``.  Not differentiable (the reference takes the top-k of a detached teacher, soft_ce.py:273)."""
+    H = hidden.shape[-1]
+    k_eff = min(int(k), int(weight.shape[0]))
+    with torch.no_grad():
+        values, columns = topk_logits(hidden.detach().reshape(-1, H).to(torch.bfloat16).contiguous(), weight.detach().to(torch.bfloat16),
+                                      k_eff, 1.0 / float(temperature))
+    shape = tuple(hidden.shape[:-1]) + (k_eff,)
+    return values.reshape(shape), columns.reshape(shape).to(torch.int64)
+
+
+def soft_ce_topk_from_hidden(student_hidden: torch.Tensor, teacher_hidden: torch.Tensor, weight: torch.Tensor, k: int, *,
+                             shift: int = 0, temperature: float = 1.0) -> torch.Tensor:
+    """Per-token top-k soft cross-entropy ``[B, S]`` (fp32): the teacher's ``min(k, V)`` largest logits of position ``s + shift``
+    (``roll(teacher, -shift, dims=1)``) and the student's logits at the same columns, both renormalised over those columns
+    (``_VocabParallelTopkSoftCE.forward``, soft_ce.py:258-305, one vocabulary shard).  Differentiable with respect to
+    ``student_hidden`` only; the gradient touches the k columns alone (:307-315)."""
+    assert not teacher_hidden.requires_grad, "MTP draft loss: teacher_hidden must be detached"
+    assert not weight.requires_grad, "MTP draft loss: the output weight must be detached"
+    if student_hidden.shape != teacher_hidden.shape:
+        raise ValueError(f"student {tuple(student_hidden.shape)} and teacher {tuple(teacher_hidden.shape)} differ in shape")
+    if student_hidden.dim() not in (2, 3):
+        raise ValueError("hidden states must be [B, S, H] or [T, H]")
+    if int(k) < 1:
+        raise ValueError(f"k must be positive, got {k}")
+    H = student_hidden.shape[-1]
+    seq_len = student_hidden.shape[-2]
+    out_shape = student_hidden.shape[:-1]
+    if student_hidden.numel() == 0:
+        return student_hidden.new_zeros(out_shape, dtype=torch.float32) + 0.0 * student_hidden.sum()
+    flat = lambda t: t.reshape(-1, H).to(torch.bfloat16).contiguous()  # noqa: E731
+    loss = _SoftCETopk.apply(flat(student_hidden), flat(teacher_hidden), weight.to(torch.bfloat16), min(int(k), int(weight.shape[0])),
+                             int(seq_len), int(shift), 1.0 / float(temperature))
+    return loss.reshape(out_shape)
+
+
+def draft_soft_ce_topk_from_hidden(
+    student_hidden: torch.Tensor,
+    teacher_hidden: torch.Tensor,
+    weight: torch.Tensor,
+    mask: torch.Tensor,
+    k: int,
+    global_normalization_factor: Optional[torch.Tensor] = None,
+    vocab_parallel_group=None,
+    roll_shift: int = 0,
+) -> torch.Tensor:
+    """Masked-mean top-k soft cross-entropy, the scalar ``draft_soft_ce_topk(student_logits, teacher_logits, mask, k,
+    global_normalization_factor, vocab_parallel_group, roll_shift)`` returns (soft_ce.py:318-341), with the hidden states that
+    feed the shared output layer in place of the two logits tensors.  ``teacher_hidden`` is the un-rolled policy hidden state
+    and ``roll_shift`` the MTP depth roll, as there."""
+    if vocab_parallel_group is not None and torch.distributed.is_initialized() \
+            and torch.distributed.get_world_size(vocab_parallel_group) > 1:
+        raise NotImplementedError("the fused top-k soft cross-entropy covers one vocabulary shard")
+    per_token = soft_ce_topk_from_hidden(student_hidden, teacher_hidden, weight, k, shift=roll_shift)
     mask = mask.to(per_token.dtype)
     if global_normalization_factor is not None:
         return (per_token * mask).sum() / global_normalization_factor.clamp(min=1.0)

@@ -1025,3 +1025,57 @@ def test_build_teacher_logits_and_hidden_chain():
     assert got.item() == pytest.approx(total / n)
     got.backward()
     assert w.grad is None and hs.grad is not None                      # the output weight is detached
+
+
+def test_soft_ce_topk_by_brute_force_and_its_limits():
+    """The top-k draft loss (mtp/soft_ce.py:243-341): selection by ``sorted``, sums with ``math``; k = V is the full soft
+    cross-entropy; rolling the small lists equals pre-rolling the teacher; custom backward = autograd = finite differences."""
+    gen = torch.Generator().manual_seed(5)
+    B, S, V, k = 2, 6, 11, 4
+    student = torch.randn(B, S, V, generator=gen, dtype=torch.float64)
+    teacher = torch.randn(B, S, V, generator=gen, dtype=torch.float64)
+    x = student.clone().requires_grad_(True)
+    per_token, q_s, t_p, cols = O.soft_ce_topk_per_token(x, teacher, k)
+    for b in range(B):
+        for s in range(S):
+            best = sorted(range(V), key=lambda v: -float(teacher[b, s, v]))[:k]
+            assert sorted(cols[b, s].tolist()) == sorted(best)
+            zt = [float(teacher[b, s, v]) for v in best]
+            zs = [float(student[b, s, v]) for v in best]
+            pt = [math.exp(z) / sum(math.exp(u) for u in zt) for z in zt]
+            logq = [z - math.log(sum(math.exp(u) for u in zs)) for z in zs]
+            assert float(per_token[b, s].detach()) == pytest.approx(-sum(p * lq for p, lq in zip(pt, logq)), rel=1e-12)
+    # k >= V: every column is kept and the loss is the full soft cross-entropy
+    full = O.soft_ce_topk_per_token(student, teacher, V + 3)[0]
+    assert torch.allclose(full, O.soft_ce_per_token(student, teacher), rtol=1e-12, atol=1e-12)
+    # roll_shift on the un-rolled teacher = top-k of the pre-rolled teacher (the reference's own check, test_soft_ce.py:122-144)
+    for shift in (1, 2, 5):
+        a = O.soft_ce_topk_per_token(student, teacher, k, roll_shift=shift)[0]
+        b_ = O.soft_ce_topk_per_token(student, torch.roll(teacher, shifts=-shift, dims=1), k)[0]
+        assert torch.equal(a, b_)
+    # gradient: the restated custom backward, autograd through the gather, and central finite differences
+    g = torch.randn(B, S, generator=gen, dtype=torch.float64)
+    (per_token * g).sum().backward()
+    custom = O.soft_ce_topk_backward(q_s.detach(), t_p, cols, g, V)
+    assert torch.allclose(x.grad, custom, rtol=1e-12, atol=1e-14)
+    assert int((custom != 0).sum(-1).max()) <= k and int((custom != 0).sum(-1).min()) == k
+    eps = 1e-6
+    for (b, s, v) in [(0, 0, int(cols[0, 0, 0])), (1, 3, int(cols[1, 3, 2])), (1, 5, int(cols[1, 5, 3]))]:
+        up, dn = student.clone(), student.clone()
+        up[b, s, v] += eps
+        dn[b, s, v] -= eps
+        fd = ((O.soft_ce_topk_per_token(up, teacher, k)[0] - O.soft_ce_topk_per_token(dn, teacher, k)[0]) * g).sum() / (2 * eps)
+        assert float(fd) == pytest.approx(float(custom[b, s, v]), rel=1e-6, abs=1e-9)
+    # the reductions, and the call chain from hidden states
+    mask = torch.ones(B, S, dtype=torch.float64)
+    mask[0, 4:] = 0
+    pt = O.soft_ce_topk_per_token(student, teacher, k, roll_shift=1)[0]
+    assert float(O.draft_soft_ce_topk(student, teacher, mask, k, roll_shift=1)) == pytest.approx(float((pt * mask).sum() / 10))
+    assert float(O.draft_soft_ce_topk(student, teacher, mask, k, torch.tensor(40.0), roll_shift=1)) == pytest.approx(float((pt * mask).sum() / 40))
+    H = 5
+    hs, ht = torch.randn(B, S, H, generator=gen, dtype=torch.float64), torch.randn(B, S, H, generator=gen, dtype=torch.float64)
+    w = torch.randn(V, H, generator=gen, dtype=torch.float64)
+    assert float(O.draft_soft_ce_topk_from_hidden(hs, ht, w, mask, k, roll_shift=2)) == pytest.approx(
+        float(O.draft_soft_ce_topk(hs @ w.t(), ht @ w.t(), mask, k, roll_shift=2)))
+    with pytest.raises(AssertionError):
+        O.draft_soft_ce_topk(student, teacher.clone().requires_grad_(True), mask, k)
