@@ -28,6 +28,33 @@ _OOV_LABEL_SENTINEL = torch.iinfo(torch.int64).max
 _REDUCTIONS = ("none", "sum", "mean")
 
 
+class BackwardEnum:
+    """The backward methods verl's kernels offer (``fused_linear_logprob_triton.py:185-195``).  One of them is built here:
+    ``_Split_Dlogits_N`` -- d_logits formed one vocabulary chunk at a time and fed to two GEMMs -- which is also the
+    reference's default and the only one SkyRL ever selects (:206, :213-216)."""
+
+    _Total_Fuse_MN = 0
+    _Total_Separate = 1
+    _Split_Dlogits_N = 2
+    _Split_Dlogits_M = 3
+
+
+def set_backward_method(backward_method: int) -> None:
+    """Counterpart of ``set_backward_method`` (``fused_linear_logprob_triton.py:213-216``).  Accepts the method that is built
+    and refuses the others: ``_Total_Fuse_MN`` needs fp32 atomic adds of whole ``[256, H]`` tiles (280 GB of them at the 7B
+    shape), ``_Total_Separate`` stores the full ``[T, V]`` d_logits, ``_Split_Dlogits_M`` re-reads the weight once per token
+    split."""
+    if backward_method != BackwardEnum._Split_Dlogits_N:
+        raise NotImplementedError(
+            f"backward method {backward_method!r}: the HIP path builds BackwardEnum._Split_Dlogits_N (value 2) only")
+
+
+# Counterpart of the reference's module flag (``fused_linear_logprob_triton.py:603-611``), which switches fp32 operands from
+# tf32 to IEEE products in its tests.  There is no reduced-precision route for fp32 operands here -- an fp32 weight always
+# enters the matrix pipe as exact hi + lo bf16 terms -- so the flag is accepted and changes nothing.
+FORCE_FP32_IEEE_PRECISION = False
+
+
 def _group_size(group: Optional[dist.ProcessGroup]) -> int:
     if group is None or not (dist.is_available() and dist.is_initialized()):
         return 1

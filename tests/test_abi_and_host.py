@@ -286,6 +286,20 @@ def test_backend_validation():
             model_utils.validate_fused_backend(bad)
 
 
+def test_backward_method_knobs_mirror_the_reference():
+    """``BackwardEnum`` / ``set_backward_method`` / ``FORCE_FP32_IEEE_PRECISION`` (fused_linear_logprob_triton.py:185-216,
+    603-611): the built method is accepted, the others are refused by name, the precision flag exists and is off."""
+    from skyrl_amd import fused_linear_logprob_hip as F
+
+    assert (F.BackwardEnum._Total_Fuse_MN, F.BackwardEnum._Total_Separate, F.BackwardEnum._Split_Dlogits_N,
+            F.BackwardEnum._Split_Dlogits_M) == (0, 1, 2, 3)
+    F.set_backward_method(F.BackwardEnum._Split_Dlogits_N)
+    for other in (F.BackwardEnum._Total_Fuse_MN, F.BackwardEnum._Total_Separate, F.BackwardEnum._Split_Dlogits_M):
+        with pytest.raises(NotImplementedError):
+            F.set_backward_method(other)
+    assert F.FORCE_FP32_IEEE_PRECISION is False
+
+
 def test_packed_index_helpers_match_brute_force():
     cu = torch.tensor([0, 4, 5, 12, 12, 20])
     _, tok, si, so, sl = model_utils._packed_sequence_indices(cu, 20, torch.device("cpu"))
