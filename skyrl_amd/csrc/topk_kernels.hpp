@@ -80,23 +80,53 @@ __global__ __launch_bounds__(NTHREADS) void topk_filter_tiles(const FilterArgs a
     const int t = tn * BN + wn * WN + j * MT + lrow;
     th[j] = t < a.T ? a.thr[t] : INFINITY;  // rows past the last token never pass
   }
+  // A lane holds 32 logits of each of its eight tokens.  First sweep: how many of them pass (a wave-wide vote on the largest
+  // of four skips the blocks in which nothing does -- nearly all of them once a threshold exists; rounding is monotone and
+  // s > 0, so the scaled maximum is the maximum of the scaled values).  Then one atomic add per lane and token reserves that
+  // many slots of the token's list -- eight independent atomics in flight, one round trip per tile -- and a second sweep
+  // stores the keys.  The accumulators are only read, so both sweeps see the same values.
+  const bool ragged = vbase + WM > a.vrows;
+  int hits[TN];
+  unsigned long long voted[TN];  // bit i: block i of token column j has a passing logit somewhere in the wave
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    hits[j] = 0;
+    voted[j] = 0;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const float m4 = fmaxf(fmaxf(acc[i][j][0], acc[i][j][1]), fmaxf(acc[i][j][2], acc[i][j][3])) * s;
+      if (__any(m4 >= th[j])) {
+        voted[j] |= 1ull << i;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int vr = vbase + i * MT + kq * 4 + r;
+          hits[j] += (acc[i][j][r] * s >= th[j] && (!ragged || vr < a.vrows)) ? 1 : 0;
+        }
+      }
+    }
+  }
+  unsigned base[TN];
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int t = tn * BN + wn * WN + j * MT + lrow;
+    base[j] = hits[j] > 0 ? atomicAdd(a.cnt + t, (unsigned)hits[j]) : 0u;
+  }
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    if (voted[j] == 0) continue;  // wave-uniform
+    const int t = tn * BN + wn * WN + j * MT + lrow;
+    key_t* list = a.cand + (size_t)t * (size_t)a.cap;
+    unsigned slot = base[j];
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      // rounding is monotone and s > 0, so the scaled maximum is the maximum of the scaled values: one multiplication and one
-      // comparison decide for four logits
-      const float m4 = fmaxf(fmaxf(acc[i][j][0], acc[i][j][1]), fmaxf(acc[i][j][2], acc[i][j][3])) * s;
-      if (__any(m4 >= th[j])) {
+      if (!((voted[j] >> i) & 1)) continue;  // wave-uniform
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float z = acc[i][j][r] * s;
-          const int vr = vbase + i * MT + kq * 4 + r;
-          if (z >= th[j] && vr < a.vrows) {
-            const unsigned slot = atomicAdd(a.cnt + t, 1u);
-            if (slot < (unsigned)a.cap) a.cand[(size_t)t * (size_t)a.cap + slot] = make_key(z, a.v0 + vr);
-          }
+      for (int r = 0; r < 4; ++r) {
+        const float z = acc[i][j][r] * s;
+        const int vr = vbase + i * MT + kq * 4 + r;
+        if (z >= th[j] && (!ragged || vr < a.vrows)) {
+          if (slot < (unsigned)a.cap) list[slot] = make_key(z, a.v0 + vr);
+          ++slot;
         }
       }
     }
