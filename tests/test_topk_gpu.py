@@ -85,6 +85,26 @@ def test_topk_logits_ties_and_the_worst_case_order_bit_exact(cuda_device):
     assert np.array_equal(idx.cpu().numpy(), order) and torch.equal(vals.cpu(), z.gather(-1, torch.from_numpy(order)))
 
 
+def test_topk_logits_in_token_blocks_and_with_strided_rows(cuda_device):
+    """More tokens than one block of 16384 (the per-token scratch is reused by the second block), hidden rows and weight rows
+    with a pitch larger than H: bit-identical to the calls on contiguous halves."""
+    T, H, V, k = 16384 + 300, 64, 1500, 8
+    hidden, weight = _operands(T, H, V, seed=21)
+    wide_h = torch.zeros(T, H + 24, dtype=torch.bfloat16, device=cuda_device)
+    wide_h[:, :H] = hidden.to(cuda_device)
+    wide_w = torch.zeros(V, H + 8, dtype=torch.bfloat16, device=cuda_device)
+    wide_w[:, :H] = weight.to(cuda_device)
+    vals, idx = M.topk_logits(wide_h[:, :H], wide_w[:, :H], k, 1.0)
+    h, w = hidden.to(cuda_device), weight.to(cuda_device)
+    a_vals, a_idx = M.topk_logits(h[:16384], w, k, 1.0)
+    b_vals, b_idx = M.topk_logits(h[16384:].contiguous(), w, k, 1.0)
+    assert torch.equal(vals, torch.cat([a_vals, b_vals])) and torch.equal(idx, torch.cat([a_idx, b_idx]))
+    z = hidden[-300:].double() @ weight.double().t()
+    want = z.topk(k + 1, dim=-1)
+    clear = (want.values[:, k - 1] - want.values[:, k]) > 1e-4
+    assert torch.equal(idx[-300:].cpu().long().sort(-1).values[clear], want.indices[:, :k].sort(-1).values[clear])
+
+
 def test_topk_logits_are_reproducible(cuda_device):
     hidden, weight = _operands(700, 128, 12000, seed=3)
     h, w = hidden.to(cuda_device), weight.to(cuda_device)
