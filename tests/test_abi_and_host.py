@@ -65,6 +65,16 @@ def test_workspace_queries():
     assert bwd < 2 * T * V
     assert lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, 100) == 0  # not a multiple of 256
     assert lib.skyrl_lmhead_fwd_workspace_bytes(0, H, V) == 0
+    # top-k: a candidate list of one chunk (8192 slots of 8 bytes) and k running keys per token of a 16384-token block,
+    # whatever T and V are beyond that
+    k = 32
+    topk = lib.skyrl_lmhead_topk_workspace_bytes(T, H, V, k)
+    assert 8 * T * (8192 + k) <= topk <= 8 * T * (8192 + k) + 12 * T + 4096
+    assert lib.skyrl_lmhead_topk_workspace_bytes(16 * T, H, 2 * V, k) == topk
+    assert lib.skyrl_lmhead_topk_workspace_bytes(T, H, 1000, k) < topk // 7      # a vocabulary below one chunk
+    for bad_k in (0, 1025, -1):
+        assert lib.skyrl_lmhead_topk_workspace_bytes(T, H, V, bad_k) == 0
+    assert lib.skyrl_lmhead_topk_workspace_bytes(T, H, 20, 21) == 0              # k beyond the vocabulary
 
 
 def _call_fwd(lib, **kw):

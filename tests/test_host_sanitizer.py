@@ -38,6 +38,7 @@ DRIVER = textwrap.dedent("""
         lib.skyrl_softce_fwd_workspace_bytes(T, H, V); lib.skyrl_softce_bwd_workspace_bytes(T, H, V, vc)
         lib.skyrl_lmhead_bwd_active_rows_workspace_bytes(T, H, V, vc)
         for terms in (1, 2, 3, 1 << 40): lib.skyrl_lmhead_bwd_split_workspace_bytes(T, H, terms, V, vc, 1)
+        for k in (1, 32, 1024, 1025, 1 << 40): lib.skyrl_lmhead_topk_workspace_bytes(T, H, V, k)
     p = 0x10000
     for T, H, V in itertools.product(big, (64, 3584, 1 << 20), (5, 152064, 1 << 31, 1 << 40)):
         ld = H
@@ -49,6 +50,10 @@ DRIVER = textwrap.dedent("""
         assert lib.skyrl_lmhead_split_operand(p, 1, ld, T, H, 3, p, 2 * ld, None) < 0
         assert lib.skyrl_softce_fwd(p, ld, p, ld, p, ld, T, T, 1, H, V, 1.0, p, p, p, p, 16, None) < 0
         assert lib.skyrl_softce_bwd(p, ld, p, ld, p, ld, p, p, p, T, T, 1, H, V, 1.0, p, 0, p, 16, None) < 0
+        for k in (1, 5, 1 << 40):
+            assert lib.skyrl_lmhead_topk_logits(p, ld, p, ld, T, H, V, k, 1.0, p, p, p, 16, None) < 0
+            assert lib.skyrl_softce_topk_fwd(p, ld, p, ld, p, p, T, 0, 1, H, V, k, 1.0, p, p, p, None) < 0
+            assert lib.skyrl_softce_topk_bwd(p, ld, p, p, p, T, H, V, k, 1.0, p, 0, None) < 0
     assert lib.skyrl_ppo_policy_loss(p, p, p, None, None, 0, 0.2, 0.2, 3.0, 0, p, None, None, None) < 0
     assert lib.skyrl_actor_loss(p, p, p, None, None, None, None, 1 << 40, 1 << 40, 0, 0.2, 0.2, 3.0, 3, 1.0, 1.0, 0.0, 0.0, p, p,
                                 None, None, None) < 0
