@@ -384,6 +384,31 @@ int skyrl_softce_topk_bwd(const void* weight, int64_t ld_weight, const float* co
                           int64_t T, int64_t H, int64_t V, int64_t k, float rcp_temperature, void* d_student_hidden,
                           int64_t ld_d_student, void* stream);
 
+/* ---- the same statistics from materialised logits -------------------------------------------------------------------
+ * For callers that hold a [T, V] logits matrix: the FSDP worker's forward tail -- logprobs_from_logits / _v2 / _flash_attn
+ * (skyrl/backends/skyrl_train/utils/torch_utils.py:115-177) and chunked_entropy_from_logits (:58-111) -- and the
+ * logits-input autograd functions DistributedLogprob / ChunkedDistributedLogprob (distributed/megatron/model_utils.py:66-272)
+ * and _VocabParallelEntropy (:1316-1345) on one vocabulary shard.  One pass over the matrix per call; nothing of size T * V is
+ * allocated or saved (the reference keeps an fp32 softmax of the whole matrix for its backward, model_utils.py:91-104).
+ *
+ * logits: bf16 or fp32 (logits_dtype), row r at logits + r * ld_logits elements; rows and pitches that allow 16-byte loads
+ * take the fast path, any other alignment works.  labels int64 [T] (NULL when no log-probability is wanted); a label outside
+ * [0, V) gives log-probability 0 and, in the backward, no one-hot term (model_utils.py:83-99, 111-137).
+ * skyrl_logits_fwd writes any of logprobs / entropy / row_lse / row_pz (fp32 [T], NULL = not wanted), computed on
+ * logits * rcp_temperature (the worker divides its logits by the temperature in place first, workers/model_wrapper.py:334).
+ * skyrl_logits_bwd writes dlogits (same dtype as the logits; leading dimension ld_dlogits)
+ *   = ( dlogprobs * (onehot - p) - dentropy * p * (y - row_pz) ) * rcp_temperature,  p = exp(y - row_lse),  y = logits * rcp_temperature
+ * dlogits may be the logits pointer itself with the same leading dimension -- the gradient then overwrites the logits, as the
+ * flash-attn cross-entropy does with inplace_backward=True (torch_utils.py:131-152) -- or a buffer that does not overlap them.
+ * Rows whose upstream gradients are both zero are written as zeros without being read. */
+#define SKYRL_LOGITS_BF16 0
+#define SKYRL_LOGITS_F32 1
+int skyrl_logits_fwd(const void* logits, int logits_dtype, int64_t ld_logits, const int64_t* labels, int64_t T, int64_t V,
+                     float rcp_temperature, float* logprobs, float* entropy, float* row_lse, float* row_pz, void* stream);
+int skyrl_logits_bwd(const void* logits, int logits_dtype, int64_t ld_logits, const int64_t* labels, const float* row_lse,
+                     const float* row_pz, const float* dlogprobs, const float* dentropy, int64_t T, int64_t V,
+                     float rcp_temperature, void* dlogits, int64_t ld_dlogits, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -54,6 +54,10 @@ What pins each function (all in ``tests/test_oracle.py``; none of them re-types 
     [B, S, k] lists against a pre-rolled teacher (the reference's own check, test_soft_ce.py:122-144); the restated custom
     backward against autograd of the forward and fp64 finite differences, and its at most k non-zero columns per token
     (test_soft_ce.py:147-156).
+  * logits-input functions (``logprobs_from_logits_v2``, ``DistributedLogprob`` forward / backward): ``torch.distributions.
+    Categorical.log_prob``, the uniform-logits known answer ``-ln V``, autograd of ``log_softmax`` + ``gather`` in fp64 for the
+    hand-written backward, its row sums (zero for a target inside the shard, ``-g`` outside), and the reference's own
+    out-of-shard semantics (forward 0, backward keeps ``-softmax * g``).
 No function is left "parity unpinned".
 """
 
@@ -859,3 +863,36 @@ def draft_soft_ce_topk_from_hidden(student_hidden, teacher_hidden, weight, mask,
     w = weight.detach()
     return draft_soft_ce_topk(student_hidden @ w.t(), teacher_hidden.detach() @ w.t(), mask, k, global_normalization_factor,
                               roll_shift)
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# Logits-input functions: the FSDP worker's log-probabilities and the Megatron path's materialised-logits autograd functions
+# ----------------------------------------------------------------------------------------------------------------------
+def logprobs_from_logits_v2(logits: torch.Tensor, labels: torch.Tensor) -> torch.Tensor:
+    """skyrl/backends/skyrl_train/utils/torch_utils.py:156-177: fp32 / fp64 logits -> gathered logit minus ``logsumexp`` row by
+    row; bf16 logits -> per-row ``log_softmax`` + ``gather`` (in bf16)."""
+    if logits.dtype in (torch.float32, torch.float64):
+        picked = torch.gather(logits, dim=-1, index=labels.unsqueeze(-1)).squeeze(-1)
+        return picked - torch.stack([torch.logsumexp(row, dim=-1) for row in logits])
+    rows = [torch.log_softmax(r, dim=-1).gather(dim=-1, index=y.unsqueeze(-1)).squeeze(-1) for r, y in zip(logits, labels)]
+    return torch.stack(rows)
+
+
+def distributed_logprob_forward(logits: torch.Tensor, target: torch.Tensor, vocab_start: int, vocab_end: int):
+    """MU:73-106 (``DistributedLogprob.forward``) on one shard: fp32 (or wider) copy of the logits, a1's log-softmax, gather at
+    the re-based target, 0 for targets outside the shard.  Returns ``(logprobs, softmax, target_mask, masked_target)``."""
+    target_mask, masked_target = _mask_targets(target, vocab_start, vocab_end)
+    wide = logits.to(torch.float64 if logits.dtype == torch.float64 else torch.float32)
+    log_probs = distributed_log_softmax(wide)
+    softmax = log_probs.exp()
+    picked = torch.gather(log_probs, -1, masked_target.unsqueeze(-1)).squeeze(-1)
+    picked[target_mask] = 0.0
+    return picked, softmax, target_mask, masked_target
+
+
+def distributed_logprob_backward(softmax: torch.Tensor, target_mask: torch.Tensor, masked_target: torch.Tensor,
+                                 grad_output: torch.Tensor) -> torch.Tensor:
+    """MU:108-137 (``DistributedLogprob.backward``): ``(onehot * in_shard - softmax) * grad``."""
+    V = softmax.size(-1)
+    is_chosen = (~target_mask).unsqueeze(-1) * torch.nn.functional.one_hot(masked_target, num_classes=V)
+    return (is_chosen.to(softmax.dtype) - softmax) * grad_output.unsqueeze(-1)

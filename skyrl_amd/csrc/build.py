@@ -14,7 +14,7 @@ import tempfile
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_NAME = "libskyrl_lmhead.so"
-SOURCES = ["lmhead_kernels.hip", "packed_kernels.hip", "loss_kernels.hip"]
+SOURCES = ["lmhead_kernels.hip", "packed_kernels.hip", "loss_kernels.hip", "logits_kernels.hip"]
 # -packed-fp32-ops off: the compiler must not form v_pk_{add,mul,fma}_f32 from the scalar fp32 epilogue code.
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -54,6 +54,10 @@ DRIVER = textwrap.dedent("""
             assert lib.skyrl_lmhead_topk_logits(p, ld, p, ld, T, H, V, k, 1.0, p, p, p, 16, None) < 0
             assert lib.skyrl_softce_topk_fwd(p, ld, p, ld, p, p, T, 0, 1, H, V, k, 1.0, p, p, p, None) < 0
             assert lib.skyrl_softce_topk_bwd(p, ld, p, p, p, T, H, V, k, 1.0, p, 0, None) < 0
+    for T, V, ld in itertools.product(big, (1, 152064, (1 << 31) - 1, 1 << 31, 1 << 40), (0, 152064, 1 << 40, 1 << 62)):
+        assert lib.skyrl_logits_fwd(p, 7, ld, p, T, V, 1.0, p, None, None, None, None) < 0
+        assert lib.skyrl_logits_fwd(p + 1, 0, ld, p, T, V, 1.0, p, None, None, None, None) < 0
+        assert lib.skyrl_logits_bwd(p, 1, ld, p, p, None, p, None, T, V, 1.0, p + 2, ld, None) < 0
     assert lib.skyrl_ppo_policy_loss(p, p, p, None, None, 0, 0.2, 0.2, 3.0, 0, p, None, None, None) < 0
     assert lib.skyrl_actor_loss(p, p, p, None, None, None, None, 1 << 40, 1 << 40, 0, 0.2, 0.2, 3.0, 3, 1.0, 1.0, 0.0, 0.0, p, p,
                                 None, None, None) < 0

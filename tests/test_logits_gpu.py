@@ -1,0 +1,274 @@
+"""GPU parity of the logits-input kernels (skyrl_logits_fwd / skyrl_logits_bwd and their reference-shaped wrappers) against
+the oracle's restatements of logprobs_from_logits_v2, chunked_entropy_from_logits (skyrl/backends/skyrl_train/utils/
+torch_utils.py:58-177), DistributedLogprob (distributed/megatron/model_utils.py:66-138) and the entropy gradient of
+_VocabParallelEntropy (:1316-1345), computed in fp64 from the same bf16 / fp32 logits.
+
+Tolerances: log-probabilities 1e-4 absolute and entropy 1e-4 relative on fp32 logits (2e-2 / 1e-2 are the path's stated bounds);
+gradients 1e-5 relative to the row's largest entry for fp32 logits, half a bf16 ulp of it for bf16 logits.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import math
+
+import pytest
+import torch
+
+from oracle import lmhead_oracle as O
+from skyrl_amd import _lib, torch_utils as TU
+
+pytestmark = pytest.mark.gpu
+
+ERR_NULL, ERR_SHAPE, ERR_ALIGN, ERR_ARG = -1, -2, -3, -5   # include/skyrl_lmhead.h
+
+
+def _case(T, V, dtype, seed, scale=3.0):
+    gen = torch.Generator().manual_seed(seed)
+    logits = (torch.randn(T, V, generator=gen) * scale).to(dtype)
+    labels = torch.randint(0, V, (T,), generator=gen)
+    g = torch.randn(T, generator=gen)
+    q = torch.randn(T, generator=gen) * 0.1
+    return logits, labels, g, q
+
+
+def _exact(logits, labels, g, q, temperature):
+    """fp64 values and gradient of sum(g * logprob + q * entropy) for logits / temperature."""
+    x = logits.double().requires_grad_(True)
+    lsm = torch.log_softmax(x / temperature, -1)
+    lp = lsm.gather(-1, labels[:, None])[:, 0]
+    ent = torch.distributions.Categorical(logits=x / temperature).entropy()
+    (lp * g.double() + ent * q.double()).sum().backward()
+    return lp.detach(), ent.detach(), x.grad
+
+
+@pytest.mark.parametrize("T,V,dtype,temperature", [
+    (37, 5000, torch.float32, 1.0),
+    (130, 20011, torch.bfloat16, 0.7),     # a vocabulary that is not a multiple of a 16-byte piece
+    (5, 151936, torch.bfloat16, 1.0),      # a full-size row
+    (64, 7, torch.float32, 1.3),           # rows shorter than one piece
+    (3, 2049, torch.bfloat16, 1.0),
+    (1, 1, torch.float32, 1.0),
+])
+def test_logits_forward_and_backward_match_fp64(T, V, dtype, temperature, cuda_device):
+    logits, labels, g, q = _case(T, V, dtype, seed=T + V)
+    want_lp, want_ent, want_grad = _exact(logits, labels, g, q, temperature)
+    d, y = logits.to(cuda_device), labels.to(cuda_device)
+    lp, ent, lse, pz = TU.logits_fwd(d, y, 1.0 / temperature, True)
+    assert (lp.cpu().double() - want_lp).abs().max() <= 1e-4
+    assert ((ent.cpu().double() - want_ent).abs() / want_ent.abs().clamp_min(1e-3)).max() <= 1e-4
+    assert (lse.cpu().double() - torch.logsumexp(logits.double() / temperature, -1)).abs().max() <= 1e-4
+    grad = TU.logits_bwd(d, y, lse, pz, g.to(cuda_device), q.to(cuda_device), 1.0 / temperature)
+    assert grad.dtype == dtype and grad.shape == (T, V)
+    # errors are measured against the size of the row's terms g / temperature and p * g / temperature, not against their
+    # difference: where the label's probability is close to 1 the two nearly cancel, in any fp32 evaluation
+    row_scale = torch.maximum(want_grad.abs().amax(-1, keepdim=True), ((g.abs() + q.abs()) / temperature).double()[:, None]).clamp_min(1e-30)
+    tol = 1e-5 if dtype == torch.float32 else 2.0 ** -8
+    assert ((grad.cpu().double() - want_grad).abs() / row_scale).max() <= tol
+    # the gradient written over the logits themselves is the same, bit for bit
+    clone = d.clone()
+    TU.logits_bwd_(clone, y, lse, pz, g.to(cuda_device), q.to(cuda_device), 1.0 / temperature)
+    assert torch.equal(clone, grad)
+    # log-probability alone (no entropy statistics), entropy alone (no labels)
+    lp2, ent2, lse2, _ = TU.logits_fwd(d, y, 1.0 / temperature, False)
+    assert torch.equal(lp2, lp) and torch.equal(lse2, lse) and float(ent2.abs().max()) == 0.0
+    lp3, ent3, _, _ = TU.logits_fwd(d, None, 1.0 / temperature, True)
+    assert torch.equal(ent3, ent) and float(lp3.abs().max()) == 0.0
+
+
+def test_logits_rows_that_do_not_allow_vector_loads_and_strided_rows(cuda_device):
+    """A row pitch that is not a multiple of 16 bytes, a base that is not 16-byte aligned, rows with padding between them."""
+    T, V = 33, 3001
+    logits, labels, g, q = _case(T, V, torch.bfloat16, seed=4)
+    want_lp, want_ent, want_grad = _exact(logits, labels, g, q, 1.0)
+    padded = torch.zeros(T, V + 7, dtype=torch.bfloat16, device=cuda_device)      # pitch 3008 * 2 bytes: 16-byte pieces
+    padded[:, :V] = logits.to(cuda_device)
+    odd = torch.zeros(T * (V + 3) + 1, dtype=torch.bfloat16, device=cuda_device)[1:].reshape(T, V + 3)   # 2-byte aligned base
+    odd[:, :V] = logits.to(cuda_device)
+    y, gd, qd = labels.to(cuda_device), g.to(cuda_device), q.to(cuda_device)
+    ref = None
+    for view in (padded[:, :V], odd[:, :V]):
+        lp, ent, lse, pz = TU.logits_fwd(view, y, 1.0, True)
+        assert (lp.cpu().double() - want_lp).abs().max() <= 1e-4 and (ent.cpu().double() - want_ent).abs().max() <= 1e-3
+        grad = TU.logits_bwd(view, y, lse, pz, gd, qd, 1.0)
+        row_scale = want_grad.abs().amax(-1, keepdim=True)
+        assert ((grad.cpu().double() - want_grad).abs() / row_scale).max() <= 2.0 ** -8
+        if ref is not None:   # the two load paths add the same numbers in different orders
+            assert (lp - ref[0]).abs().max() <= 1e-5 and (grad.float() - ref[1].float()).abs().max() <= 2.0 ** -8 * float(row_scale.max())
+        ref = (lp, grad)
+        before = view.clone()
+        TU.logits_bwd_(view, y, lse, pz, gd, qd, 1.0)                # in place into a strided view: the padding stays untouched
+        assert torch.equal(view, grad)
+    assert float(padded[:, V:].abs().max()) == 0.0 and float(odd[:, V:].abs().max()) == 0.0 and before.shape == (T, V)
+
+
+def test_logits_extreme_rows(cuda_device):
+    """Rows of equal logits (-ln V), a row with one dominant logit, very negative rows (no underflow to log 0), -inf entries
+    (masked vocabulary: probability exactly 0), rows without upstream gradient (exact zeros)."""
+    V = 4099
+    rows = torch.zeros(6, V)
+    rows[1, 17] = 80.0
+    rows[2] = -300.0                                                    # exp(-300) is 0 in fp32: a maximum that started at 0 would give log 0
+    rows[3] = torch.linspace(-50, 50, V)
+    rows[4, ::2] = -math.inf
+    rows[5] = torch.randn(V, generator=torch.Generator().manual_seed(0)) * 10
+    labels = torch.tensor([5, 17, 9, V - 1, 1, 3])
+    d = rows.to(cuda_device)
+    lp, ent, lse, pz = TU.logits_fwd(d, labels.to(cuda_device), 1.0, True)
+    want_lp = torch.log_softmax(rows.double(), -1).gather(-1, labels[:, None])[:, 0]
+    want_ent = torch.distributions.Categorical(logits=rows.double()).entropy()
+    assert torch.isfinite(lp).all() and torch.isfinite(ent).all()
+    assert (lp.cpu().double() - want_lp).abs().max() <= 1e-4 and (ent.cpu().double() - want_ent).abs().max() <= 1e-4
+    assert lp[0].item() == pytest.approx(-math.log(V), abs=1e-5) and ent[0].item() == pytest.approx(math.log(V), abs=1e-5)
+    assert lp[2].item() == pytest.approx(-math.log(V), abs=1e-4)
+    assert ent[4].item() == pytest.approx(math.log((V - 1) // 2), abs=1e-5)
+    g = torch.tensor([1.0, -2.0, 0.5, 0.0, 1.0, 0.0], device=cuda_device)
+    grad = TU.logits_bwd(d, labels.to(cuda_device), lse, None, g, None, 1.0)
+    assert float(grad[3].abs().max()) == 0.0 and float(grad[5].abs().max()) == 0.0
+    assert float(grad[4, ::2].abs().max()) == 0.0                       # masked columns get no gradient
+    assert torch.isfinite(grad).all()
+    assert grad.sum(-1).abs().max() <= 1e-4                              # rows of (onehot - p) * g sum to zero
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_reference_shaped_wrappers_match_oracle(dtype, cuda_device):
+    gen = torch.Generator().manual_seed(3)
+    B, S, V = 3, 41, 2500
+    logits = (torch.randn(B, S, V, generator=gen) * 2).to(dtype)
+    labels = torch.randint(0, V, (B, S), generator=gen)
+    mask = (torch.rand(B, S, generator=gen) > 0.3).to(dtype)
+    d, y = logits.to(cuda_device), labels.to(cuda_device)
+    want = O.logprobs_from_logits_v2(logits.double(), labels)
+    got = TU.logprobs_from_logits(d, y, inplace_backward=False)
+    assert got.dtype == torch.float32 and got.shape == (B, S) and (got.cpu().double() - want).abs().max() <= 1e-4
+    v2 = TU.logprobs_from_logits_v2(d, y)
+    assert v2.dtype == dtype and (v2.cpu().double() - want).abs().max() <= (1e-4 if dtype == torch.float32 else 0.05)
+    if dtype == torch.bfloat16:      # inside the error ball of the reference's own bf16 path around the exact value
+        ref_bf16 = O.logprobs_from_logits_v2(logits, labels)
+        assert (v2.cpu().double() - want).abs().max() <= (ref_bf16.double() - want).abs().max() + 1e-6
+    ent_want = O.chunked_entropy_from_logits(logits.double(), mask.double())
+    ent = TU.chunked_entropy_from_logits(d, attention_mask=mask.to(cuda_device), chunk_size=7)
+    assert ent.dtype == dtype and not ent.requires_grad
+    assert (ent.cpu().double() - ent_want).abs().max() <= (1e-4 if dtype == torch.float32 else 0.05)
+    assert bool((ent.cpu()[mask == 0] == 0).all())
+    with pytest.raises(ValueError):
+        TU.chunked_entropy_from_logits(d, attention_mask=mask.to(cuda_device)[:, :-1])
+    with pytest.raises(ValueError):
+        TU.chunked_entropy_from_logits(d, chunk_size=0)
+    # gradients through autograd: out of place, and in place over a non-leaf logits tensor
+    g = torch.randn(B, S, generator=gen)
+    x = logits.double().requires_grad_(True)
+    (O.logprobs_from_logits_v2(x, labels) * g.double()).sum().backward()
+    leaf = d.clone().requires_grad_(True)
+    (TU.logprobs_from_logits(leaf, y, inplace_backward=False) * g.to(cuda_device)).sum().backward()
+    scale = x.grad.abs().amax(-1, keepdim=True)
+    tol = 1e-5 if dtype == torch.float32 else 2.0 ** -8
+    assert ((leaf.grad.cpu().double() - x.grad).abs() / scale).max() <= tol
+    leaf2 = d.clone().requires_grad_(True)
+    mid = leaf2 * 1.0                                                     # what a model's output is: not a leaf
+    (TU.logprobs_from_logits(mid, y, inplace_backward=True) * g.to(cuda_device)).sum().backward()
+    assert torch.equal(leaf2.grad, leaf.grad) and torch.equal(mid.detach(), leaf.grad)   # the logits now hold their gradient
+    # entropy with gradient, and both outputs of one pass
+    leaf3 = d.clone().requires_grad_(True)
+    ent_g = TU.chunked_entropy_from_logits(leaf3, requires_grad=True)
+    (ent_g.float() * g.to(cuda_device)).sum().backward()
+    x2 = logits.double().requires_grad_(True)
+    (torch.distributions.Categorical(logits=x2).entropy() * g.double()).sum().backward()
+    scale2 = x2.grad.abs().amax(-1, keepdim=True)
+    assert ((leaf3.grad.cpu().double() - x2.grad).abs() / scale2).max() <= (1e-5 if dtype == torch.float32 else 2.0 ** -7)
+    both_lp, both_ent = TU.logprobs_and_entropy_from_logits(d, y, temperature=0.6)
+    assert (both_lp.cpu().double() - O.logprobs_from_logits_v2(logits.double() / 0.6, labels)).abs().max() <= 1e-4
+    assert (both_ent.cpu().double() - O.chunked_entropy_from_logits(logits.double() / 0.6)).abs().max() <= 1e-4
+
+
+def test_distributed_logprob_adapters_match_oracle(cuda_device):
+    gen = torch.Generator().manual_seed(8)
+    B, S, V, start = 2, 33, 1800, 500
+    logits = torch.randn(B, S, V, generator=gen).bfloat16()
+    target = torch.randint(start, start + V, (B, S), generator=gen)
+    target[0, :4] = torch.tensor([0, start - 1, start + V, 10 ** 9])       # outside the shard on either side
+    g = torch.randn(B, S, generator=gen)
+    lp_want, softmax, tmask, masked = O.distributed_logprob_forward(logits.double(), target, start, start + V)
+    grad_want = O.distributed_logprob_backward(softmax, tmask, masked, g.double())
+    for chunked in (False, True):
+        leaf = logits.to(cuda_device).requires_grad_(True)
+        if chunked:
+            lp = TU.ChunkedDistributedLogprob.apply(leaf, target.to(cuda_device), start, start + V, 8, None, False)
+        else:
+            lp = TU.DistributedLogprob.apply(leaf, target.to(cuda_device), start, start + V, None, False)
+        assert lp.dtype == torch.float32 and lp.shape == (B, S)
+        assert (lp.cpu().double() - lp_want).abs().max() <= 1e-4 and bool((lp.cpu()[tmask] == 0).all())
+        (lp * g.to(cuda_device)).sum().backward()
+        assert leaf.grad.dtype == torch.bfloat16
+        scale = grad_want.abs().amax(-1, keepdim=True)
+        assert ((leaf.grad.cpu().double() - grad_want).abs() / scale).max() <= 2.0 ** -8
+    with torch.no_grad():
+        out = TU.DistributedLogprob.apply(logits.to(cuda_device), target.to(cuda_device), start, start + V, None, True)
+    assert torch.equal(out, lp.detach())
+    rolled_want = O.distributed_logprob_forward(logits.double(), target.roll(-1, -1), start, start + V)[0][:, :-1]
+    got = TU.from_parallel_logits_to_logprobs(logits.to(cuda_device), target.to(cuda_device), start, start + V, None, inference_only=True)
+    assert got.shape == (B, S - 1) and (got.cpu().double() - rolled_want).abs().max() <= 1e-4
+
+
+def test_logits_c_abi_argument_errors(cuda_device):
+    lib = _lib.load()
+    T, V = 8, 640
+    x = torch.randn(T, V, device=cuda_device)
+    y = torch.zeros(T, dtype=torch.int64, device=cuda_device)
+    out = torch.empty(T, device=cuda_device)
+    p = lambda t: t.data_ptr()  # noqa: E731
+    fwd = lambda **kw: lib.skyrl_logits_fwd(kw.get("logits", p(x)), kw.get("dtype", 1), kw.get("ld", V), kw.get("labels", p(y)), kw.get("T", T),  # noqa: E731
+                                            V, kw.get("rt", 1.0), kw.get("lp", p(out)), None, None, None, None)
+    assert fwd() == 0
+    assert fwd(logits=ctypes.c_void_p(0)) == ERR_NULL and fwd(labels=None) == ERR_NULL and fwd(lp=None) == ERR_NULL
+    assert fwd(dtype=2) == ERR_ARG and fwd(rt=0.0) == ERR_ARG and fwd(rt=float("nan")) == ERR_ARG
+    assert fwd(ld=V - 1) == ERR_SHAPE and fwd(T=0) == ERR_SHAPE
+    assert fwd(logits=p(x) + 2) == ERR_ALIGN
+    grad = torch.empty(T, V, device=cuda_device)
+    bwd = lambda dst, ldd, g=p(out): lib.skyrl_logits_bwd(p(x), 1, V, p(y), p(out), None, g, None, T, V, 1.0, dst, ldd, None)  # noqa: E731
+    assert bwd(p(grad), V) == 0 and bwd(p(x), V) == 0                     # apart, or exactly in place
+    assert bwd(p(x) + 4 * V, V) == ERR_ARG                                # overlapping the logits any other way
+    assert bwd(p(grad), V - 1) == ERR_SHAPE and bwd(None, V) == ERR_NULL and bwd(p(grad), V, None) == ERR_NULL
+    torch.cuda.synchronize()
+
+
+def test_logits_ops_opcheck(cuda_device):
+    x = torch.randn(12, 300, device=cuda_device).bfloat16()
+    y = torch.randint(0, 300, (12,), device=cuda_device)
+    torch.library.opcheck(TU.logits_fwd, (x, y, 1.0, True), test_utils=("test_schema", "test_faketensor"))
+    lp, ent, lse, pz = TU.logits_fwd(x, y, 1.0, True)
+    torch.library.opcheck(TU.logits_bwd, (x, y, lse, pz, lp, ent, 1.0), test_utils=("test_schema", "test_faketensor"))
+    torch.library.opcheck(TU.logits_bwd_, (x.clone(), y, lse, pz, lp, ent, 1.0), test_utils=("test_schema", "test_faketensor"))
+
+
+def test_logits_full_size_properties(cuda_device):
+    """16384 rows of 152064 bf16 logits (4.6 GiB): sampled rows against fp64, the entropy bounds, rows of the gradient that
+    sum to zero, nothing of the matrix's size allocated by the forward or by the in-place backward."""
+    T, V = 16384, 152064
+    gen = torch.Generator(device=cuda_device).manual_seed(0)
+    logits = torch.empty(T, V, dtype=torch.bfloat16, device=cuda_device)
+    for r in range(0, T, 2048):
+        logits[r:r + 2048] = (torch.randn(2048, V, device=cuda_device, generator=gen) * 3).bfloat16()
+    labels = torch.randint(0, V, (T,), device=cuda_device, generator=gen)
+    g = torch.randn(T, device=cuda_device, generator=gen)
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    lp, ent, lse, pz = TU.logits_fwd(logits, labels, 1.0, True)
+    torch.cuda.synchronize()
+    assert torch.cuda.max_memory_allocated() - base < (1 << 20)
+    rows = torch.randperm(T, generator=torch.Generator().manual_seed(1))[:16].to(cuda_device)
+    z = logits[rows].double()
+    want_lp = torch.log_softmax(z, -1).gather(-1, labels[rows][:, None])[:, 0]
+    assert (lp[rows].double() - want_lp).abs().max() <= 1e-4
+    assert (ent[rows].double() - torch.distributions.Categorical(logits=z).entropy()).abs().max() <= 1e-4
+    assert bool((lp <= 0).all()) and bool((ent >= 0).all()) and bool((ent <= math.log(V) + 1e-3).all())
+    want_grad = (torch.nn.functional.one_hot(labels[rows], V) - torch.softmax(z, -1)) * g[rows].double()[:, None]
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    TU.logits_bwd_(logits, labels, lse, None, g, None, 1.0)
+    torch.cuda.synchronize()
+    assert torch.cuda.max_memory_allocated() - base < (1 << 20)
+    got = logits[rows].double()
+    assert ((got - want_grad).abs() / want_grad.abs().amax(-1, keepdim=True)).max() <= 2.0 ** -8
+    assert bool(torch.isfinite(logits[:512]).all())

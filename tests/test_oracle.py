@@ -1079,3 +1079,37 @@ def test_soft_ce_topk_by_brute_force_and_its_limits():
         float(O.draft_soft_ce_topk(hs @ w.t(), ht @ w.t(), mask, k, roll_shift=2)))
     with pytest.raises(AssertionError):
         O.draft_soft_ce_topk(student, teacher.clone().requires_grad_(True), mask, k)
+
+
+def test_logits_input_functions_against_library_distributions():
+    """logprobs_from_logits_v2 (torch_utils.py:156-177) and DistributedLogprob (model_utils.py:66-138) on one shard."""
+    gen = torch.Generator().manual_seed(9)
+    B, S, V = 2, 5, 13
+    logits = torch.randn(B, S, V, generator=gen, dtype=torch.float64) * 2
+    labels = torch.randint(0, V, (B, S), generator=gen)
+    want = torch.distributions.Categorical(logits=logits).log_prob(labels)
+    assert torch.allclose(O.logprobs_from_logits_v2(logits, labels), want, rtol=1e-12, atol=1e-12)
+    assert torch.allclose(O.logprobs_from_logits_v2(logits.float(), labels).double(), want, atol=1e-5)
+    bf = O.logprobs_from_logits_v2(logits.bfloat16(), labels)
+    assert bf.dtype == torch.bfloat16 and torch.allclose(bf.double(), want, atol=0.1)
+    flat = O.logprobs_from_logits_v2(torch.zeros(3, 2, V, dtype=torch.float64), labels[:, :2].repeat(2, 1)[:3])
+    assert torch.allclose(flat, torch.full((3, 2), -math.log(V), dtype=torch.float64))
+    # DistributedLogprob on a shard [3, 3 + V): targets re-based, outside -> 0 forward and -softmax * g backward
+    target = labels + 3
+    target[0, 1], target[1, 4] = 1, 3 + V
+    lp, softmax, mask, masked = O.distributed_logprob_forward(logits, target, 3, 3 + V)
+    inside = ~mask
+    assert mask.sum() == 2 and bool((lp[mask] == 0).all())
+    # the reference's log-softmax takes the row sum through fp32 (model_utils.py:52-60): fp32 accuracy even on fp64 logits
+    assert torch.allclose(lp[inside], want[inside], atol=1e-6)
+    assert torch.allclose(softmax, torch.softmax(logits, -1), atol=1e-6)
+    g = torch.randn(B, S, generator=gen, dtype=torch.float64)
+    grad = O.distributed_logprob_backward(softmax, mask, masked, g)
+    x = logits.clone().requires_grad_(True)
+    picked = torch.log_softmax(x, -1).gather(-1, masked.unsqueeze(-1)).squeeze(-1) * inside
+    (picked * g).sum().backward()
+    # autograd of the masked closed form gives the in-shard rows; out-of-shard rows keep -softmax * g in the reference
+    assert torch.allclose(grad[inside], x.grad[inside], atol=1e-6)
+    assert torch.allclose(grad[mask], -(torch.softmax(logits, -1) * g.unsqueeze(-1))[mask], atol=1e-6)
+    assert torch.allclose(grad.sum(-1)[inside], torch.zeros(int(inside.sum()), dtype=torch.float64), atol=1e-6)
+    assert torch.allclose(grad.sum(-1)[mask], -g[mask], atol=1e-6)
