@@ -26,7 +26,8 @@ from .ops import _require_device as _require_device_all
 
 __all__ = ["logprobs_from_logits", "logprobs_from_logits_v2", "logprobs_from_logits_flash_attn", "chunked_entropy_from_logits",
            "logprobs_and_entropy_from_logits", "DistributedLogprob", "ChunkedDistributedLogprob",
-           "from_parallel_logits_to_logprobs", "logits_fwd", "logits_bwd", "logits_bwd_"]
+           "from_parallel_logits_to_logprobs", "vocab_parallel_entropy", "vocab_parallel_entropy_weighted_sum",
+           "vocab_parallel_entropy_packed_sequences", "logits_fwd", "logits_bwd", "logits_bwd_"]
 
 _DTYPES = {torch.bfloat16: 0, torch.float32: 1}
 
@@ -270,3 +271,64 @@ def from_parallel_logits_to_logprobs(vocab_parallel_logits: torch.Tensor, target
     rolled = target.roll(shifts=-1, dims=-1)
     logprobs = DistributedLogprob.apply(vocab_parallel_logits, rolled, vocab_start_index, vocab_end_index, tp_group, inference_only)
     return logprobs.contiguous()[:, :-1]
+
+
+def _check_entropy_chunking(chunk_size: Optional[int], chunk_memory_mb: int) -> None:
+    """The argument errors of ``_resolve_vocab_entropy_chunk_size`` (model_utils.py:1352-1385).  The chunking itself bounds
+    fp32 temporaries that do not exist here, so valid values change nothing."""
+    if chunk_size is not None and chunk_size < 0:
+        raise ValueError(f"chunk_size must be non-negative or None, got {chunk_size}")
+    if chunk_size is not None and chunk_memory_mb <= 0:
+        raise ValueError(f"chunk_memory_mb must be positive, got {chunk_memory_mb}")
+
+
+def vocab_parallel_entropy(vocab_parallel_logits: torch.Tensor, chunk_size: Optional[int] = None, chunk_memory_mb: int = 512
+                           ) -> torch.Tensor:
+    """Reference ``vocab_parallel_entropy`` / ``_VocabParallelEntropy`` (model_utils.py:1316-1410) on one vocabulary shard:
+    entropy of ``softmax(logits)`` per position, shape ``logits.shape[:-1]``, in the logits' dtype, with the gradient
+    ``softmax * (sum softmax * logits - logits) * grad`` (:1337-1345) recomputed from the logits in the backward instead of
+    kept as a second tensor of the logits' size."""
+    _check_entropy_chunking(chunk_size, chunk_memory_mb)
+    shape = vocab_parallel_logits.shape[:-1]
+    _, ent = _FromLogits.apply(_flat(vocab_parallel_logits), None, 1.0, True, False)
+    return ent.reshape(shape).to(vocab_parallel_logits.dtype)
+
+
+def vocab_parallel_entropy_weighted_sum(vocab_parallel_logits: torch.Tensor, weights: torch.Tensor, chunk_size: Optional[int] = None,
+                                        chunk_memory_mb: int = 512) -> torch.Tensor:
+    """Reference ``vocab_parallel_entropy_weighted_sum`` (model_utils.py:1413-1440): ``sum(entropy * weights)``.  Rows whose
+    weight is zero cost nothing in the backward (their gradient rows are written as zeros without reading the logits)."""
+    return (vocab_parallel_entropy(vocab_parallel_logits, chunk_size, chunk_memory_mb) * weights).sum()
+
+
+def vocab_parallel_entropy_packed_sequences(vocab_parallel_logits: torch.Tensor, cu_seqlens_padded: torch.Tensor, unpacked_seqlen: int,
+                                            num_actions: int, attention_mask: torch.Tensor, loss_mask: Optional[torch.Tensor],
+                                            cp_group: Any, sub_seq_lengths: Optional[list] = None, chunk_size: Optional[int] = None,
+                                            chunk_memory_mb: int = 512) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Reference ``vocab_parallel_entropy_packed_sequences`` (model_utils.py:1001-1087) without context parallelism:
+    ``(entropy, entropy_for_loss)``, the action-token mean of the per-token entropy of packed logits ``[1, T, V]``; the first
+    is detached, the second carries the gradient.  The reference brings the ``[B, unpacked_seqlen - 1]`` action weights to
+    the packed stream with boolean-mask indexing and one ``.item()``; here the per-token entropy goes the other way through
+    the (differentiable) scatter-back kernel and the weighted mean is taken in the ``[B, unpacked_seqlen - 1]`` layout -- the
+    same sums, no host synchronisation."""
+    from .model_utils import _packed_subseq_row_indices_offsets_and_lens
+    from .packed import packed_scatter_logprobs
+
+    _require_single_shard(cp_group, "vocab_parallel_entropy_packed_sequences (context parallelism)")
+    entropy_tokens = vocab_parallel_entropy(vocab_parallel_logits, chunk_size, chunk_memory_mb).reshape(-1).float()
+    device = entropy_tokens.device
+    batch_size, cols = attention_mask.shape[0], unpacked_seqlen - 1
+    with torch.no_grad():
+        action_weights = torch.zeros((batch_size, cols), dtype=torch.float32, device=device)
+        action_weights[:, -num_actions:] = 1.0 if loss_mask is None else loss_mask.to(device=device, dtype=torch.float32)
+        cu = cu_seqlens_padded.to(device=device, dtype=torch.long)
+        if sub_seq_lengths is not None:
+            rows, row_offs, seq_lens = _packed_subseq_row_indices_offsets_and_lens(cu, sub_seq_lengths, device)
+            layout = dict(seg_row=rows, seg_col=row_offs, seg_len=seq_lens)
+        else:
+            layout = dict(attention_mask=attention_mask.to(device=device, dtype=torch.bool))
+        landed = packed_scatter_logprobs(torch.ones_like(entropy_tokens), cu, batch_size, cols, **layout)
+        count = (landed * action_weights).sum().clamp(min=1.0)
+    entropy_bs = packed_scatter_logprobs(entropy_tokens.contiguous(), cu, batch_size, cols, **layout)
+    entropy_for_loss = ((entropy_bs * action_weights).sum() / count).to(vocab_parallel_logits.dtype)
+    return entropy_for_loss.detach().clone(), entropy_for_loss

@@ -272,3 +272,75 @@ def test_logits_full_size_properties(cuda_device):
     got = logits[rows].double()
     assert ((got - want_grad).abs() / want_grad.abs().amax(-1, keepdim=True)).max() <= 2.0 ** -8
     assert bool(torch.isfinite(logits[:512]).all())
+
+
+def test_vocab_parallel_entropy_wrappers_match_library(cuda_device):
+    """vocab_parallel_entropy / _weighted_sum (model_utils.py:1316-1440): values and the gradient
+    softmax * (sum softmax * logits - logits) * grad, against torch.distributions in fp64."""
+    gen = torch.Generator().manual_seed(12)
+    S, V = 57, 3000
+    logits = (torch.randn(1, S, V, generator=gen) * 2).bfloat16()
+    weights = (torch.rand(S, generator=gen) > 0.4).float()
+    x = logits.double().requires_grad_(True)
+    ent64 = torch.distributions.Categorical(logits=x).entropy()
+    (ent64[0] * weights.double()).sum().backward()
+    leaf = logits.to(cuda_device).requires_grad_(True)
+    ent = TU.vocab_parallel_entropy(leaf, chunk_size=0, chunk_memory_mb=64)
+    assert ent.shape == (1, S) and ent.dtype == torch.bfloat16
+    assert (ent.detach().cpu().double() - ent64.detach()).abs().max() <= 0.05
+    total = TU.vocab_parallel_entropy_weighted_sum(leaf, weights.to(cuda_device), chunk_size=16)
+    total.backward()
+    scale = x.grad.abs().amax(-1, keepdim=True).clamp_min(1e-30)
+    assert ((leaf.grad.cpu().double() - x.grad).abs() / scale)[0][weights > 0].max() <= 2.0 ** -7
+    assert float(leaf.grad[0][(weights == 0).to(cuda_device)].abs().max()) == 0.0
+    with pytest.raises(ValueError):
+        TU.vocab_parallel_entropy(leaf, chunk_size=-1)
+    with pytest.raises(ValueError):
+        TU.vocab_parallel_entropy(leaf, chunk_size=0, chunk_memory_mb=0)
+
+
+@pytest.mark.parametrize("layout", ["attention_mask", "sub_sequences"])
+@pytest.mark.parametrize("with_loss_mask", [False, True])
+def test_vocab_parallel_entropy_packed_sequences_matches_oracle(layout, with_loss_mask, cuda_device):
+    """The packed action-token entropy on materialised logits (model_utils.py:1001-1087): value and gradient against the
+    oracle's restatement of the reference's packed-weight route applied to fp64 entropies."""
+    import numpy as np
+
+    gen = torch.Generator().manual_seed(34)
+    V = 900
+    if layout == "attention_mask":
+        L, num_actions = 40, 17
+        real = [40, 23, 31, 5, 1]
+        am = torch.zeros(len(real), L, dtype=torch.long)
+        am[0] = 1
+        am[1, L - 23:] = 1
+        am[2, :31] = 1
+        am[3, 10:15] = 1
+        am[4, L - 1] = 1
+        padded = [r + (-r) % 8 for r in real]
+        sub = None
+    else:
+        L, num_actions = 48, 30
+        sub = [[9, 1, 14], [20, 6], [33]]
+        padded = [16, 8, 16, 24, 8, 40]
+        am = torch.ones(len(sub), L, dtype=torch.long)
+    B = am.shape[0]
+    cu = torch.tensor([0] + list(np.cumsum(padded)))
+    T = int(cu[-1])
+    logits = (torch.randn(1, T, V, generator=gen) * 2).float()
+    loss_mask = (torch.rand(B, num_actions, generator=gen) > 0.35).float() if with_loss_mask else None
+    x = logits.double().requires_grad_(True)
+    ent64 = torch.distributions.Categorical(logits=x).entropy().squeeze(0)
+    want, want_loss = O.packed_action_entropy(ent64, cu, L, num_actions, am, None if loss_mask is None else loss_mask.double(), sub)
+    want_loss.backward()
+    to = lambda t: None if t is None else t.to(cuda_device)  # noqa: E731
+    leaf = logits.to(cuda_device).requires_grad_(True)
+    got, got_loss = TU.vocab_parallel_entropy_packed_sequences(leaf, to(cu), L, num_actions, to(am), to(loss_mask), None,
+                                                               sub_seq_lengths=sub, chunk_size=0)
+    assert got.dim() == 0 and not got.requires_grad and got_loss.requires_grad
+    assert want.item() > 0.5
+    assert got.item() == pytest.approx(want.item(), rel=1e-4) and got_loss.item() == pytest.approx(want.item(), rel=1e-4)
+    got_loss.backward()
+    err = (leaf.grad.cpu().double() - x.grad).abs().max().item()
+    assert err <= 1e-5 * x.grad.abs().max().item(), err
+    assert bool(((leaf.grad.cpu() != 0).any(-1) == (x.grad != 0).any(-1)).all())       # the same tokens carry gradient
