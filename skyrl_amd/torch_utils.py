@@ -26,7 +26,7 @@ from .ops import _require_device as _require_device_all
 
 __all__ = ["logprobs_from_logits", "logprobs_from_logits_v2", "logprobs_from_logits_flash_attn", "chunked_entropy_from_logits",
            "logprobs_and_entropy_from_logits", "DistributedLogprob", "ChunkedDistributedLogprob",
-           "from_parallel_logits_to_logprobs", "vocab_parallel_entropy", "vocab_parallel_entropy_weighted_sum",
+           "from_parallel_logits_to_logprobs", "from_parallel_logits_to_logprobs_packed_sequences", "vocab_parallel_entropy", "vocab_parallel_entropy_weighted_sum",
            "vocab_parallel_entropy_packed_sequences", "logits_fwd", "logits_bwd", "logits_bwd_"]
 
 _DTYPES = {torch.bfloat16: 0, torch.float32: 1}
@@ -271,6 +271,38 @@ def from_parallel_logits_to_logprobs(vocab_parallel_logits: torch.Tensor, target
     rolled = target.roll(shifts=-1, dims=-1)
     logprobs = DistributedLogprob.apply(vocab_parallel_logits, rolled, vocab_start_index, vocab_end_index, tp_group, inference_only)
     return logprobs.contiguous()[:, :-1]
+
+
+def from_parallel_logits_to_logprobs_packed_sequences(vocab_parallel_logits: torch.Tensor, target: torch.Tensor,
+                                                      cu_seqlens_padded: torch.Tensor, unpacked_seqlen: int, vocab_start_index: int,
+                                                      vocab_end_index: int, group: Any, inference_only: bool = False, cp_group: Any = None,
+                                                      chunk_size: Optional[int] = None, attention_mask: Optional[torch.Tensor] = None,
+                                                      sub_seq_lengths: Optional[list] = None) -> torch.Tensor:
+    """Reference ``from_parallel_logits_to_logprobs_packed_sequences`` (model_utils.py:566-710) without context parallelism:
+    packed logits ``[1, T, V]`` and packed targets ``[1, T]`` -> ``[batch, unpacked_seqlen - 1]`` fp32.  Every token is scored
+    against its successor inside its own sequence (one index kernel), the log-probabilities come from the one-pass logits
+    kernel, and the scatter back to rows is one kernel per direction instead of boolean-mask indexing."""
+    from .model_utils import _packed_subseq_row_indices_offsets_and_lens
+    from .packed import packed_next_token_labels, packed_scatter_logprobs
+
+    _require_single_shard(cp_group, "from_parallel_logits_to_logprobs_packed_sequences (context parallelism)")
+    target = target.squeeze(0)
+    device = target.device
+    batch_size = len(sub_seq_lengths) if sub_seq_lengths is not None else cu_seqlens_padded.shape[0] - 1
+    cu = cu_seqlens_padded.to(device=device, dtype=torch.long)
+    rolled = packed_next_token_labels(target.to(torch.long).contiguous(), cu).unsqueeze(0)
+    if sub_seq_lengths is not None:
+        rows, row_offs, seq_lens = _packed_subseq_row_indices_offsets_and_lens(cu, sub_seq_lengths, device)
+        layout = dict(seg_row=rows, seg_col=row_offs, seg_len=seq_lens)
+    elif attention_mask is not None:
+        layout = dict(attention_mask=attention_mask.to(device=device, dtype=torch.bool))
+    else:
+        layout = {}
+    probs = DistributedLogprob.apply(vocab_parallel_logits, rolled, vocab_start_index, vocab_end_index, group, inference_only)
+    probs = probs.contiguous().squeeze(0)
+    if probs.dim() != 1:
+        raise ValueError(f"Expected probs to be 1D after squeezing, but got shape {probs.shape}.")
+    return packed_scatter_logprobs(probs, cu, batch_size, unpacked_seqlen - 1, **layout)
 
 
 def _check_entropy_chunking(chunk_size: Optional[int], chunk_memory_mb: int) -> None:

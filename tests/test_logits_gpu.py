@@ -344,3 +344,41 @@ def test_vocab_parallel_entropy_packed_sequences_matches_oracle(layout, with_los
     err = (leaf.grad.cpu().double() - x.grad).abs().max().item()
     assert err <= 1e-5 * x.grad.abs().max().item(), err
     assert bool(((leaf.grad.cpu() != 0).any(-1) == (x.grad != 0).any(-1)).all())       # the same tokens carry gradient
+
+
+def test_packed_logits_wrapper_all_layouts_with_gradient(cuda_device):
+    """from_parallel_logits_to_logprobs_packed_sequences (model_utils.py:566-710) end to end -- labels kernel, logits kernel,
+    scatter kernel -- in the three layouts, against the oracle's statement of the same pipeline (per-sequence roll, the
+    materialised-logits log-probability, scatter-back), values and gradient."""
+    dev = cuda_device
+    V = 515
+    gen = torch.Generator().manual_seed(52)
+    true_lens = [9, 1, 17, 13, 6]
+    padded = [10, 2, 17, 16, 6]
+    cu = torch.cat([torch.zeros(1, dtype=torch.long), torch.tensor(padded).cumsum(0)])
+    T = int(cu[-1])
+    logits = (torch.randn(1, T, V, generator=gen) * 2).float()
+    tokens = torch.randint(0, V, (1, T), generator=gen)
+    rolled = O.packed_rolled_targets(tokens[0], cu)
+    L = 20
+    am = torch.zeros(len(true_lens), L, dtype=torch.bool)
+    for b, n in enumerate(true_lens):
+        am[b, L - n:] = True
+    sub = [[9, 1], [17], [13, 6]]
+    cases = {"plain": (dict(), len(padded), L), "mask": (dict(attention_mask=am), len(padded), L),
+             "sub": (dict(sub_seq_lengths=sub), len(sub), 30)}
+    for name, (kw, rows, seqlen) in cases.items():
+        x = logits.double().requires_grad_(True)
+        probs = O.distributed_logprob_forward(x, rolled[None], 0, V)[0][0]
+        want = O.packed_scatter_back(probs, cu, rows, seqlen, **kw)
+        G = torch.randn(want.shape, generator=gen)
+        (want * G.double()).sum().backward()
+        leaf = logits.to(dev).requires_grad_(True)
+        dkw = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in kw.items()}
+        got = TU.from_parallel_logits_to_logprobs_packed_sequences(leaf, tokens.to(dev), cu.to(dev), seqlen, 0, V, None, **dkw)
+        assert got.shape == want.shape and got.dtype == torch.float32, name
+        assert (got.detach().cpu().double() - want.detach()).abs().max() <= 1e-4, name
+        assert torch.equal(got.detach().cpu() == 0, want.detach() == 0), name
+        (got * G.to(dev)).sum().backward()
+        err = (leaf.grad.cpu().double() - x.grad).abs().max().item()
+        assert err <= 1e-5 * max(1.0, x.grad.abs().max().item()), (name, err)
