@@ -78,7 +78,7 @@ __global__ __launch_bounds__(NTHREADS) void topk_filter_tiles(const FilterArgs a
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int t = tn * BN + wn * WN + j * MT + lrow;
-    th[j] = t < a.T ? a.thr[t] : INFINITY;  // rows past the last token never pass
+    th[j] = t < a.T ? a.thr[t] : NAN;  // rows past the last token never pass: every comparison with NaN is false
   }
   // A lane holds 32 logits of each of its eight tokens.  First sweep: how many of them pass (a wave-wide vote on the largest
   // of four skips the blocks in which nothing does -- nearly all of them once a threshold exists; rounding is monotone and

@@ -105,6 +105,24 @@ def test_topk_logits_in_token_blocks_and_with_strided_rows(cuda_device):
     assert torch.equal(idx[-300:].cpu().long().sort(-1).values[clear], want.indices[:, :k].sort(-1).values[clear])
 
 
+def test_topk_logits_with_infinite_logits_in_a_ragged_tile(cuda_device):
+    """The last token of a ragged token tile has logits of +-inf: the tile's padding rows repeat that token and must not
+    reach any list; the token's own list holds the first k columns of +inf."""
+    T, H, V, k = 300, 64, 1300, 4
+    hidden, weight = _operands(T, H, V, seed=5)
+    hidden[T - 1] = 0
+    hidden[T - 1, 0] = 3.0e38
+    weight[:, 0] = torch.where(torch.arange(V) % 3 == 0, 2.0, -2.0).bfloat16()
+    vals, idx = M.topk_logits_from_hidden(hidden.to(cuda_device), weight.to(cuda_device), k)
+    assert torch.isinf(vals[T - 1]).all() and bool((vals[T - 1] > 0).all()) and idx[T - 1].tolist() == [0, 3, 6, 9]
+    z = hidden[: T - 1].double() @ weight.double().t()
+    want = z.topk(k + 1, dim=-1)
+    clear = (want.values[:, k - 1] - want.values[:, k]) > 1e-4
+    assert torch.equal(idx[: T - 1].cpu().sort(-1).values[clear], want.indices[:, :k].sort(-1).values[clear])
+    again = M.topk_logits_from_hidden(hidden.to(cuda_device), weight.to(cuda_device), k)
+    assert torch.equal(again[1], idx)
+
+
 def test_topk_logits_are_reproducible(cuda_device):
     hidden, weight = _operands(700, 128, 12000, seed=3)
     h, w = hidden.to(cuda_device), weight.to(cuda_device)
@@ -266,4 +284,4 @@ def test_topk_full_size_properties(cuda_device):
         zt = teacher[tt].double() @ weight.double().t()
         zs = student[t].detach().double() @ weight.double().t()
         want = O.soft_ce_topk_per_token(zs[None, None].cpu(), zt[None, None].cpu(), k)[0]
-        assert float(loss.reshape(-1)[t]) == pytest.approx(float(want), abs=5e-3)
+        assert float(loss.detach().reshape(-1)[t]) == pytest.approx(float(want), abs=5e-3)
