@@ -285,3 +285,46 @@ def test_topk_full_size_properties(cuda_device):
         zs = student[t].detach().double() @ weight.double().t()
         want = O.soft_ce_topk_per_token(zs[None, None].cpu(), zt[None, None].cpu(), k)[0]
         assert float(loss.detach().reshape(-1)[t]) == pytest.approx(float(want), abs=5e-3)
+
+
+def test_topk_draft_loss_replays_from_a_hip_graph(cuda_device):
+    """The top-k entry points launch kernels and nothing else (the per-token counters are cleared by a kernel, not by a
+    memset), so a forward + backward of the draft loss can be captured; three replays on new inputs, with eager work in
+    between, each reproduce the eager result bit for bit."""
+    T, S, H, V, k = 320, 80, 128, 3000, 16
+    gen = torch.Generator().manual_seed(5)
+    weight = (torch.randn(V, H, generator=gen) * 3 / H ** 0.5).bfloat16().to(cuda_device)
+    student = torch.zeros(T, H, dtype=torch.bfloat16, device=cuda_device)
+    teacher = torch.zeros(T, H, dtype=torch.bfloat16, device=cuda_device)
+    g = torch.zeros(T, device=cuda_device)
+
+    def step():
+        values, columns = M.topk_logits(teacher, weight, k, 1.0)
+        loss, coef, used = M.softce_topk_fwd(student, weight, values, columns, S, 1, 1.0)
+        return values, columns, loss, M.softce_topk_bwd(weight, coef, used, g, 1.0)
+
+    def refill(seed):
+        gen_ = torch.Generator().manual_seed(seed)
+        student.copy_(torch.randn(T, H, generator=gen_).bfloat16())
+        teacher.copy_(torch.randn(T, H, generator=gen_).bfloat16())
+        g.copy_(torch.randn(T, generator=gen_))
+
+    refill(0)
+    side = torch.cuda.Stream(device=cuda_device)
+    side.wait_stream(torch.cuda.current_stream(cuda_device))
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream(cuda_device).wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step()
+    for seed in (1, 2, 3):
+        refill(seed)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in captured]
+        want = step()
+        torch.cuda.synchronize()
+        for a, b in zip(got, want):
+            assert torch.equal(a, b)
