@@ -426,3 +426,26 @@ def test_logits_entry_points_replay_from_a_hip_graph(cuda_device):
         torch.cuda.synchronize()
         for a, b in zip(got, want):
             assert torch.equal(a, b)
+
+
+def test_logits_random_shapes_against_fp64(cuda_device):
+    """Thirty random (T, V, dtype, temperature, row pitch) cases, ragged ends and unaligned pitches included."""
+    rng = torch.Generator().manual_seed(2024)
+    for case in range(30):
+        T = int(torch.randint(1, 70, (1,), generator=rng))
+        V = int(torch.randint(1, 9000, (1,), generator=rng))
+        dtype = torch.bfloat16 if case % 2 else torch.float32
+        temperature = float(torch.rand(1, generator=rng)) * 1.5 + 0.3
+        pad = int(torch.randint(0, 9, (1,), generator=rng))
+        logits, labels, g, q = _case(T, V, dtype, seed=1000 + case)
+        want_lp, want_ent, want_grad = _exact(logits, labels, g, q, temperature)
+        wide = torch.zeros(T, V + pad, dtype=dtype, device=cuda_device)
+        wide[:, :V] = logits.to(cuda_device)
+        view, y = wide[:, :V], labels.to(cuda_device)
+        lp, ent, lse, pz = TU.logits_fwd(view, y, 1.0 / temperature, True)
+        tag = (case, T, V, dtype, pad)
+        assert (lp.cpu().double() - want_lp).abs().max() <= 1e-4, tag
+        assert (ent.cpu().double() - want_ent).abs().max() <= 1e-4 * max(1.0, float(want_ent.max())), tag
+        grad = TU.logits_bwd(view, y, lse, pz, g.to(cuda_device), q.to(cuda_device), 1.0 / temperature)
+        scale = torch.maximum(want_grad.abs().amax(-1, keepdim=True), ((g.abs() + q.abs()) / temperature).double()[:, None])
+        assert ((grad.cpu().double() - want_grad).abs() / scale).max() <= (1e-5 if dtype == torch.float32 else 2.0 ** -8), tag

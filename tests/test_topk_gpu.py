@@ -62,6 +62,25 @@ def test_topk_logits_match_fp64(T, H, V, k, temperature, cuda_device):
     assert torch.equal(got_sets[clear], want_sets[clear])
 
 
+def test_topk_logits_random_shapes(cuda_device):
+    """Twenty random (T, H, V, k) cases: the column sets of fp64 wherever fp64 separates the k-th from the (k+1)-th logit."""
+    rng = torch.Generator().manual_seed(77)
+    for case in range(20):
+        T = int(torch.randint(1, 600, (1,), generator=rng))
+        H = 64 * int(torch.randint(1, 5, (1,), generator=rng))
+        V = int(torch.randint(2, 12000, (1,), generator=rng))
+        k = int(torch.randint(1, min(V, 200), (1,), generator=rng))
+        hidden, weight = _operands(T, H, V, seed=500 + case)
+        z = hidden.double() @ weight.double().t()
+        want = z.topk(k + 1, dim=-1)
+        clear = (want.values[:, k - 1] - want.values[:, k]) > 1e-4
+        vals, idx = M.topk_logits_from_hidden(hidden.to(cuda_device), weight.to(cuda_device), k)
+        tag = (case, T, H, V, k)
+        assert torch.equal(idx.cpu().sort(-1).values[clear], want.indices[:, :k].sort(-1).values[clear]), tag
+        assert (vals.cpu().double() - z.gather(-1, idx.cpu())).abs().max() <= 1e-4 * max(1.0, float(z.abs().max())), tag
+        assert bool((vals[:, 1:] <= vals[:, :-1]).all()), tag
+
+
 def test_topk_logits_ties_and_the_worst_case_order_bit_exact(cuda_device):
     """Logits that are exact in bf16 and ascend with the column -- every logit is a candidate in every chunk, the worst case of
     the filter -- with many equal values: equal values come out lower column first, results bit-exact."""
