@@ -21,7 +21,7 @@ from . import ops
 from .fused_linear_logprob_hip import linear_cross_entropy
 from .model_utils import _fused_lm_head_logprob_apply
 
-__all__ = ["action_log_probs_from_hidden"]
+__all__ = ["action_log_probs_from_hidden", "action_log_probs_from_logits"]
 
 
 def _pad_back(values: torch.Tensor, nnz_indices: torch.Tensor, batch: int, seqlen: int) -> torch.Tensor:
@@ -97,6 +97,58 @@ def action_log_probs_from_hidden(
     else:
         log_probs = _fused_lm_head_logprob_apply("hip", last_hidden_state, lm_head_weight, rolled, 0, V, tokens.shape[1], None,
                                                  not torch.is_grad_enabled(), float(temperature))
+    if packed:
+        log_probs = _pad_back(log_probs.reshape(-1), nnz_indices, batch, seqlen)
+    action_log_probs = log_probs[:, -num_actions - 1 : -1]
+    return (action_log_probs, output) if return_output else action_log_probs
+
+
+def action_log_probs_from_logits(
+    logits_BSV: torch.Tensor,
+    sequences: torch.Tensor,
+    num_actions: Union[int, List[int]],
+    attention_mask: Optional[torch.Tensor] = None,
+    temperature: float = 1.0,
+    return_output: bool = False,
+    compute_entropy: bool = False,
+    entropy_requires_grad: bool = True,
+    nnz_indices: Optional[torch.Tensor] = None,
+    inplace_backward: bool = True,
+) -> Union[torch.Tensor, Tuple[torch.Tensor, dict]]:
+    """The same tail for a worker that keeps its ``[B, S, V]`` logits (``[1, nnz, V]`` with the padding removed): lines
+    333-393 of the reference's ``HFModelWrapper.forward`` as they stand, with the temperature division (:334), the
+    log-probability (:337-341) and the entropy (:358-386) taken from ONE pass over the logits instead of an in-place division
+    and six to eight elementwise passes, and the backward written over the logits' own storage (``inplace_backward``, what
+    the reference gets from flash-attn's cross-entropy when it is installed, torch_utils.py:131-152).  The logits themselves
+    are left undivided.  Entropy in the logits' dtype, as the reference returns it (torch_utils.py:92)."""
+    from .torch_utils import _FromLogits, _flat
+
+    if isinstance(num_actions, list):
+        if len(num_actions) != 1:
+            raise NotImplementedError("per-row num_actions is not supported (the reference slices with a numpy array here, "
+                                      "which torch rejects as well)")
+        num_actions = num_actions[0]
+    batch, seqlen = sequences.shape
+    packed = nnz_indices is not None
+    tokens = sequences.reshape(-1)[nnz_indices.to(torch.long)].unsqueeze(0) if packed else sequences
+    if logits_BSV.shape[:2] != tokens.shape:
+        raise ValueError(f"logits {tuple(logits_BSV.shape)} do not match the token stream {tuple(tokens.shape)}")
+    rolled = torch.roll(tokens, shifts=-1, dims=1)
+    log_probs, entropy = _FromLogits.apply(_flat(logits_BSV), rolled.reshape(-1).to(torch.int64).contiguous(),
+                                           1.0 / float(temperature), bool(compute_entropy), bool(inplace_backward))
+    log_probs = log_probs.reshape(tokens.shape)
+    output = {}
+    if compute_entropy:
+        entropy = entropy.reshape(tokens.shape).to(logits_BSV.dtype)
+        if not entropy_requires_grad:
+            entropy = entropy.detach()
+        if packed:
+            entropy = _pad_back(entropy.reshape(-1), nnz_indices, batch, seqlen)
+        elif attention_mask is not None:
+            if attention_mask.shape != entropy.shape:
+                raise ValueError(f"attention_mask shape {tuple(attention_mask.shape)} does not match {tuple(entropy.shape)}")
+            entropy = entropy * attention_mask
+        output["entropy"] = entropy
     if packed:
         log_probs = _pad_back(log_probs.reshape(-1), nnz_indices, batch, seqlen)
     action_log_probs = log_probs[:, -num_actions - 1 : -1]

@@ -449,3 +449,57 @@ def test_logits_random_shapes_against_fp64(cuda_device):
         grad = TU.logits_bwd(view, y, lse, pz, g.to(cuda_device), q.to(cuda_device), 1.0 / temperature)
         scale = torch.maximum(want_grad.abs().amax(-1, keepdim=True), ((g.abs() + q.abs()) / temperature).double()[:, None])
         assert ((grad.cpu().double() - want_grad).abs() / scale).max() <= (1e-5 if dtype == torch.float32 else 2.0 ** -8), tag
+
+
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("compute_entropy,entropy_grad", [(False, False), (True, False), (True, True)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_fsdp_forward_tail_from_logits(cuda_device, packed, compute_entropy, entropy_grad, dtype):
+    """action_log_probs_from_logits against the reference's forward tail (workers/model_wrapper.py:291, 333-393, restated in
+    the oracle) on the same logits in fp64: values, shapes, the zero padding, the gradient into the logits -- out of place
+    and written over a non-leaf logits tensor."""
+    from skyrl_amd.model_wrapper import action_log_probs_from_logits
+    dev = cuda_device
+    gen = torch.Generator().manual_seed(61)
+    B, S, V, A, t = 3, 24, 700, 7, 0.8
+    seqs = torch.randint(0, V, (B, S), generator=gen)
+    am = torch.ones(B, S, dtype=torch.long)
+    am[0, :5] = 0
+    am[1, :2] = 0
+    nnz = am.flatten().nonzero().flatten() if packed else None
+    n_tok = int(am.sum()) if packed else B * S
+    logits = (torch.randn(1 if packed else B, n_tok if packed else S, V, generator=gen) * 2).to(dtype)
+    x = logits.double().requires_grad_(True)
+    want_alp, want_ent = O.hf_wrapper_tail(x, seqs, A, am.double(), t, nnz_indices=nnz)
+    G = torch.randn(B, A, generator=gen).double()
+    Q = torch.randn(B, S, generator=gen).double() * 0.1
+    ((want_alp * G).sum() + ((want_ent * Q).sum() if entropy_grad else 0.0)).backward()
+    grads = []
+    for inplace in (False, True):
+        leaf = logits.to(dev).requires_grad_(True)
+        mid = leaf * 1.0
+        alp, out = action_log_probs_from_logits(mid, seqs.to(dev), A, am.to(dev), t, return_output=True,
+                                                compute_entropy=compute_entropy, entropy_requires_grad=entropy_grad,
+                                                nnz_indices=None if nnz is None else nnz.to(dev), inplace_backward=inplace)
+        assert alp.shape == (B, A) and alp.dtype == torch.float32
+        assert (alp.detach().cpu().double() - want_alp.detach()).abs().max() <= 1e-4
+        loss = (alp * G.float().to(dev)).sum()
+        if compute_entropy:
+            ent = out["entropy"]
+            assert ent.shape == (B, S) and ent.dtype == dtype and ent.requires_grad == entropy_grad
+            assert (ent.detach().cpu().double() - want_ent.detach()).abs().max() <= (1e-4 if dtype == torch.float32 else 0.05)
+            assert bool((ent.detach().cpu()[am == 0] == 0).all())
+            if entropy_grad:
+                loss = loss + (ent.float() * Q.float().to(dev)).sum()
+        else:
+            assert out == {}
+        loss.backward()
+        grads.append(leaf.grad.clone())
+        if inplace:
+            assert torch.equal(mid.detach(), leaf.grad)       # the logits' storage now holds the gradient
+    assert torch.equal(grads[0], grads[1])
+    scale = x.grad.abs().amax(-1, keepdim=True).clamp_min(1e-6)
+    live = x.grad.abs().amax(-1) > 0
+    tol = 1e-4 if dtype == torch.float32 else 2.0 ** -6        # bf16: the entropy reaches the loss rounded to bf16
+    assert ((grads[0].cpu().double() - x.grad).abs() / scale)[live].max() <= tol
+    assert float(grads[0].cpu()[~live].abs().max() if bool((~live).any()) else 0.0) == 0.0
