@@ -1804,7 +1804,7 @@ int skyrl_lmhead_topk_logits(const void* hidden, int64_t ld_hidden, const void* 
   const TopkWorkspace w = carve_topk(workspace, T, V, k);
   const int64_t block_tokens = fwd_block_tokens(w.block_tokens, ld_hidden);
   const uint16_t* Wp = (const uint16_t*)weight;
-  const size_t select_lds = (size_t)topk::kSelectWaves * (size_t)k * sizeof(topk::key_t);
+  const size_t select_lds = (size_t)topk::kSelectWaves * (size_t)(k + topk::kSelectStage) * sizeof(topk::key_t);
   hipError_t e;
   for (int64_t t0 = 0; t0 < T; t0 += block_tokens) {
     const int64_t Tb = (T - t0) < block_tokens ? (T - t0) : block_tokens;

@@ -145,18 +145,24 @@ __device__ __forceinline__ key_t wave_min_key(key_t v) {
 
 constexpr int kSelectWaves = 4;
 constexpr int kMaxK = 1024;
+constexpr int kSelectStage = 1024;   // candidates one bulk round takes into LDS, behind the list
+constexpr int kSelectBulkMin = 96;   // fewer candidates than this are inserted one by one
 
 // best: [T, k] running lists (unordered), have: [T] entries of the list that are filled.  One wave per token; the list lives
-// in LDS while the wave works on it.  With `final_vals` the finished list is written out best first.
+// in LDS while the wave works on it.  Many candidates (the first chunks, a large k, adversarial data) are merged in bulk: up to
+// kSelectStage of them are put behind the list, a bisection over the key bits finds a threshold that exactly k keys reach
+// (keys are unique, so one exists; a pass over the keys per bit, usually 20 to 30 bits until the count is exact), and the keys
+// that reach it are compacted to the front in place.  A few candidates are inserted one by one, each replacing the worst
+// entry.  With `final_vals` the finished list is written out best first.
 __global__ __launch_bounds__(64 * kSelectWaves) void topk_select(int T, int k, key_t* __restrict__ best, unsigned* __restrict__ have,
                                                                  float* __restrict__ thr, unsigned* __restrict__ cnt,
                                                                  const key_t* __restrict__ cand, int cap,
                                                                  float* __restrict__ final_vals, int* __restrict__ final_idx) {
-  extern __shared__ key_t sm_list[];  // kSelectWaves * k keys
+  extern __shared__ key_t sm_list[];  // kSelectWaves * (k + kSelectStage) keys
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int t = blockIdx.x * kSelectWaves + wave;
   if (t >= T) return;  // whole waves leave; no barrier below
-  key_t* list = sm_list + (size_t)wave * (size_t)k;
+  key_t* list = sm_list + (size_t)wave * (size_t)(k + kSelectStage);
   key_t* gl = best + (size_t)t * (size_t)k;
   int n_have = (int)have[t];
   for (int e = lane; e < n_have; e += 64) list[e] = gl[e];
@@ -180,10 +186,46 @@ __global__ __launch_bounds__(64 * kSelectWaves) void topk_select(int T, int k, k
     const unsigned long long owner = __ballot(pos >= 0);
     worst_pos = __shfl(pos, (int)__ffsll((long long)owner) - 1, 64);
   };
+  const key_t* cl = cand + (size_t)t * (size_t)cap;
+  int done = 0;
+  while (n - done >= kSelectBulkMin) {
+    const int take = (n - done) < kSelectStage ? (n - done) : kSelectStage;
+    for (int e = lane; e < take; e += 64) list[n_have + e] = cl[done + e];
+    lds_fence();
+    const int M = n_have + take;
+    done += take;
+    if (M <= k) {
+      n_have = M;
+      continue;
+    }
+    key_t reach = 0;  // grows bit by bit while at least k keys reach it; done when exactly k do
+    for (int b = 63; b >= 0; --b) {
+      const key_t trial = reach | ((key_t)1 << b);
+      int c = 0;
+      for (int e = lane; e < M; e += 64) c += list[e] >= trial ? 1 : 0;
+#pragma unroll
+      for (int o = 32; o >= 1; o >>= 1) c += __shfl_xor(c, o, 64);
+      if (c >= k) {
+        reach = trial;
+        if (c == k) break;
+      }
+    }
+    int w = 0;  // in-place compaction: a step reads 64 entries and writes at or below where it read
+    for (int base = 0; base < M; base += 64) {
+      const int e = base + lane;
+      const key_t x = e < M ? list[e] : 0;
+      const bool keep = e < M && x >= reach;
+      const unsigned long long mask = __ballot(keep);
+      lds_fence();
+      if (keep) list[w + __popcll(mask & (((key_t)1 << lane) - 1))] = x;
+      w += (int)__popcll(mask);
+      lds_fence();
+    }
+    n_have = k;
+  }
   if (n_have == k) find_worst();
 
-  const key_t* cl = cand + (size_t)t * (size_t)cap;
-  for (int c0 = 0; c0 < n; c0 += 64) {
+  for (int c0 = done; c0 < n; c0 += 64) {
     const bool in = c0 + lane < n;
     const key_t c = in ? cl[c0 + lane] : 0;
     unsigned long long pending = __ballot(in && (n_have < k || c > worst));
