@@ -41,7 +41,8 @@ from .ops import _require_device
 
 __all__ = ["ppo_policy_loss", "cross_entropy_loss", "importance_sampling_loss", "sapo_policy_loss", "gspo_policy_loss",
            "compute_policy_loss_cispo", "rollout_is_policy_loss", "dppo_policy_loss", "compute_approx_kl", "approx_kl_loss",
-           "masked_mean", "actor_loss", "ppo_policy_loss_terms", "compute_policy_loss_clip_cov", "compute_policy_loss_kl_cov"]
+           "masked_mean", "actor_loss", "ppo_policy_loss_terms", "compute_policy_loss_clip_cov", "compute_policy_loss_kl_cov",
+           "POLICY_LOSS_FUNCTIONS", "get_policy_loss"]
 
 LOSS_REGULAR, LOSS_DUAL_CLIP, LOSS_CROSS_ENTROPY, LOSS_IMPORTANCE_SAMPLING = 0, 1, 2, 3
 LOSS_GSPO, LOSS_SAPO, LOSS_CISPO, LOSS_ROLLOUT_IS, LOSS_DPPO_TV, LOSS_DPPO_KL = 4, 5, 6, 7, 8, 9
@@ -657,3 +658,28 @@ def actor_loss(
     metrics = {"policy_loss": out6[1], "policy_kl": out6[4], "policy_entropy": out6[5],
                ("importance_ratio" if loss_type == LOSS_IMPORTANCE_SAMPLING else "clip_ratio"): stat}
     return loss, metrics
+
+
+# The names under which the reference registers its policy losses (``PolicyLossRegistry.repopulate_registry``,
+# ppo_utils.py:497-515), each with the function of this module that has the same signature:
+# ``PolicyLossRegistry.register(name, POLICY_LOSS_FUNCTIONS[name])`` puts the fused loss in the reference's place.
+POLICY_LOSS_FUNCTIONS = {
+    "regular": ppo_policy_loss,
+    "dual_clip": ppo_policy_loss,
+    "gspo": gspo_policy_loss,
+    "cispo": compute_policy_loss_cispo,
+    "clip_cov": compute_policy_loss_clip_cov,
+    "kl_cov": compute_policy_loss_kl_cov,
+    "sapo": sapo_policy_loss,
+    "cross_entropy": cross_entropy_loss,
+    "importance_sampling": importance_sampling_loss,
+    "dppo": dppo_policy_loss,
+    "rollout_is": rollout_is_policy_loss,
+}
+
+
+def get_policy_loss(name: str):
+    """The fused loss registered under ``name`` in the reference (``PolicyLossRegistry.get``, ppo_utils.py:444-452)."""
+    if name not in POLICY_LOSS_FUNCTIONS:
+        raise ValueError(f"Unknown policy loss '{name}'. Available: {sorted(POLICY_LOSS_FUNCTIONS)}")
+    return POLICY_LOSS_FUNCTIONS[name]

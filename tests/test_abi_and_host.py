@@ -310,6 +310,23 @@ def test_backward_method_knobs_mirror_the_reference():
     assert F.FORCE_FP32_IEEE_PRECISION is False
 
 
+def test_policy_loss_names_are_the_reference_registry_names():
+    """ppo_utils.py:497-515: the eleven names of PolicyLossRegistry.repopulate_registry, each with six positional arguments
+    (log_probs, old_log_probs, advantages, config, loss_mask, rollout_logprobs)."""
+    import inspect
+
+    from skyrl_amd import policy_loss as PL
+
+    assert sorted(PL.POLICY_LOSS_FUNCTIONS) == sorted(["regular", "dual_clip", "gspo", "cispo", "clip_cov", "kl_cov", "sapo",
+                                                       "cross_entropy", "importance_sampling", "dppo", "rollout_is"])
+    for name, fn in PL.POLICY_LOSS_FUNCTIONS.items():
+        params = list(inspect.signature(fn).parameters)
+        assert params[:6] == ["log_probs", "old_log_probs", "advantages", "config", "loss_mask", "rollout_logprobs"], name
+        assert PL.get_policy_loss(name) is fn
+    with pytest.raises(ValueError):
+        PL.get_policy_loss("nope")
+
+
 def test_packed_index_helpers_match_brute_force():
     cu = torch.tensor([0, 4, 5, 12, 12, 20])
     _, tok, si, so, sl = model_utils._packed_sequence_indices(cu, 20, torch.device("cpu"))
