@@ -384,6 +384,33 @@ int skyrl_softce_topk_bwd(const void* weight, int64_t ld_weight, const float* co
                           int64_t T, int64_t H, int64_t V, int64_t k, float rcp_temperature, void* d_student_hidden,
                           int64_t ld_d_student, void* stream);
 
+/* ---- off-policy correction from the rollout engine's log-probabilities -------------------------------------------------
+ * Stands in for compute_off_policy_correction (skyrl/backends/skyrl_train/utils/off_policy_correction_utils.py:257-348) and
+ * the four functions it combines (compute_tis_ratio :24-72, compute_outlier_token_mask :75-134, compute_token_mask :137-188,
+ * compute_sequence_mask :191-254), which the policy losses apply to their per-token loss (apply_off_policy_correction,
+ * :351-391; ppo_utils.py:581, 653, 722, 815, 857, 929).  It depends on old_log_probs and rollout_logprobs only, never on the
+ * policy's current log-probabilities, so it carries no gradient.
+ *   old_log_probs, rollout_logprobs, loss_mask: fp32 [rows, cols] (loss_mask NULL = all ones).
+ *   tis_type: 0 off, 1 "token" (weight min(r, tis_cap)), 2 "sequence" (the row's product ratio, capped).
+ *   seq_metric: 0 off, 1 "geometric", 2 "product", with bounds seq_low / seq_high (geo_mask_* / product_mask_*).
+ *   outlier_low / outlier_high: pointers to the thresholds, NULL = not set (either alone switches the outlier filter on);
+ *   token_low / token_high: the per-token hard mask, on only when both are given.
+ * Outputs (each may be NULL): keep [rows, cols] in {0, 1} -- loss_mask * keep is the mask the reference returns; tis
+ * [rows, cols] (a row's value repeated for "sequence"; ones when tis_type is 0); weight = tis * keep, the per-token factor
+ * to hand to the policy-loss entry points as loss_weight together with the ORIGINAL loss_mask (the reference counts its
+ * clip statistic with the original mask and sums the loss with the new one).  metrics: SKYRL_OFF_POLICY_METRICS floats --
+ * 0 is_ratio_mean, 1 is_ratio_std, 2 is_ratio_max, 3 is_ratio_min, 4 outlier_seq_masked_ratio, 5 outlier_seq_over_high_ratio,
+ * 6 outlier_seq_under_low_ratio, 7 token_mask_ratio, 8 tis_token_clip_high_ratio, 9 tis_seq_clip_high_ratio, 10-12 the
+ * sequence mask's masked / over_high / under_low ratios -- added over the rows in a fixed order.  row_stats: scratch of
+ * rows * SKYRL_OFF_POLICY_ROW_STATS floats.  Two launches, no synchronisation. */
+#define SKYRL_OFF_POLICY_ROW_STATS 20
+#define SKYRL_OFF_POLICY_METRICS 16
+int skyrl_off_policy_correction(const float* old_log_probs, const float* rollout_logprobs, const float* loss_mask, int64_t rows,
+                                int64_t cols, int tis_type, float tis_cap, int seq_metric, float seq_low, float seq_high,
+                                const float* outlier_low, const float* outlier_high, const float* token_low,
+                                const float* token_high, float* keep_out, float* tis_out, float* weight_out, float* metrics,
+                                float* row_stats, void* stream);
+
 /* ---- the same statistics from materialised logits -------------------------------------------------------------------
  * For callers that hold a [T, V] logits matrix: the FSDP worker's forward tail -- logprobs_from_logits / _v2 / _flash_attn
  * (skyrl/backends/skyrl_train/utils/torch_utils.py:115-177) and chunked_entropy_from_logits (:58-111) -- and the

@@ -58,6 +58,9 @@ What pins each function (all in ``tests/test_oracle.py``; none of them re-types 
     Categorical.log_prob``, the uniform-logits known answer ``-ln V``, autograd of ``log_softmax`` + ``gather`` in fp64 for the
     hand-written backward, its row sums (zero for a target inside the shard, ``-g`` outside), and the reference's own
     out-of-shard semantics (forward 0, backward keeps ``-softmax * g``).
+  * off-policy correction: every step on a 3 x 4 batch whose ratios are powers of two, each mask, weight and metric
+    written down by hand, and the order of the steps (a row removed as an outlier no longer counts in the token-mask and
+    TIS statistics and has sequence ratio 1; the sequence mask sees the tokens the token mask left).
 No function is left "parity unpinned".
 """
 
@@ -896,3 +899,82 @@ def distributed_logprob_backward(softmax: torch.Tensor, target_mask: torch.Tenso
     V = softmax.size(-1)
     is_chosen = (~target_mask).unsqueeze(-1) * torch.nn.functional.one_hot(masked_target, num_classes=V)
     return (is_chosen.to(softmax.dtype) - softmax) * grad_output.unsqueeze(-1)
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# Off-policy correction from the rollout engine's log-probabilities
+# ----------------------------------------------------------------------------------------------------------------------
+OPC = "skyrl/backends/skyrl_train/utils/off_policy_correction_utils.py"
+
+
+def _cfg(cfg, name):
+    return cfg.get(name) if isinstance(cfg, dict) else getattr(cfg, name, None)
+
+
+def off_policy_correction(old_log_probs: torch.Tensor, rollout_logprobs: torch.Tensor, loss_mask: torch.Tensor, cfg):
+    """OPC:257-348 with the helpers it calls (:24-254), in its order: is-ratio metrics on the incoming mask; outlier rows
+    (any unmasked token's ratio beyond a threshold removes the row); the per-token hard mask (both bounds needed); the
+    truncated importance weight, per token or per sequence, on the mask left so far; the sequence mask (geometric mean or
+    product of the ratios outside its bounds removes the row).  Returns ``(tis_ratio | None, metrics, loss_mask)``."""
+    tis_type, seq_metric = _cfg(cfg, "tis_ratio_type"), _cfg(cfg, "sequence_mask_metric")
+    out_lo, out_hi = _cfg(cfg, "outlier_token_is_threshold_low"), _cfg(cfg, "outlier_token_is_threshold_high")
+    tok_lo, tok_hi = _cfg(cfg, "token_mask_is_threshold_low"), _cfg(cfg, "token_mask_is_threshold_high")
+    use_outlier, use_token = out_lo is not None or out_hi is not None, tok_lo is not None and tok_hi is not None
+    if tis_type is None and seq_metric is None and not use_outlier and not use_token:
+        return None, {}, loss_mask
+    delta = old_log_probs - rollout_logprobs
+    ratio = torch.clamp(delta, -20.0, 20.0).exp()
+    rows = float(ratio.shape[0])
+    m = {"is_ratio_mean": float(masked_mean(ratio, loss_mask)), "is_ratio_std": float((ratio * loss_mask).std()),
+         "is_ratio_max": float((ratio * loss_mask).max()), "is_ratio_min": float((ratio * loss_mask).min())}
+    mask = loss_mask
+    if use_outlier:
+        live = mask > 0
+        over = (ratio > out_hi) & live if out_hi is not None else torch.zeros_like(live)
+        under = (ratio < out_lo) & live if out_lo is not None else torch.zeros_like(live)
+        ok = ((~over & ~under) | ~live).all(dim=-1, keepdim=True)
+        m["outlier_seq_masked_ratio"] = float((~ok).sum() / rows)
+        m["outlier_seq_over_high_ratio"] = float(over.any(dim=-1).sum() / rows)
+        m["outlier_seq_under_low_ratio"] = float(under.any(dim=-1).sum() / rows)
+        mask = mask * ok.to(mask.dtype)
+    if use_token:
+        inside = (ratio >= tok_lo) & (ratio <= tok_hi)
+        m["token_mask_ratio"] = float(((~inside) & (mask > 0)).sum() / (mask > 0).sum().clamp(min=1))
+        mask = mask * (inside | (mask == 0)).to(mask.dtype)
+    tis = None
+    if tis_type == "token":
+        cap = _cfg(cfg, "token_tis_ratio_clip_high")
+        m["tis_token_clip_high_ratio"] = float(((ratio > cap) & (mask > 0)).sum() / (mask > 0).sum().clamp(min=1))
+        tis = torch.clamp(ratio, max=cap)
+    elif tis_type == "sequence":
+        cap = _cfg(cfg, "sequence_tis_ratio_clip_high")
+        seq = torch.clamp((delta * mask).sum(dim=-1, keepdim=True), -20.0, 20.0).exp()
+        m["tis_seq_clip_high_ratio"] = float((seq > cap).sum() / rows)
+        tis = torch.clamp(seq, max=cap)
+    elif tis_type is not None:
+        raise ValueError(f"Unknown tis_ratio_type: {tis_type}")
+    if seq_metric in ("geometric", "product"):
+        total = (delta * mask).sum(dim=-1, keepdim=True)
+        if seq_metric == "geometric":
+            value = torch.clamp(total / mask.sum(dim=-1, keepdim=True).clamp(min=1.0), -20.0, 20.0).exp()
+            lo, hi, name = _cfg(cfg, "geo_mask_low"), _cfg(cfg, "geo_mask_high"), "geo_sequence_mask"
+        else:
+            value = torch.clamp(total, -20.0, 20.0).exp()
+            lo, hi, name = _cfg(cfg, "product_mask_low"), _cfg(cfg, "product_mask_high"), "product_sequence_mask"
+        over, under = value > hi, value < lo
+        m[f"{name}_masked_ratio"] = float((over | under).sum() / rows)
+        m[f"{name}_over_high_ratio"] = float(over.sum() / rows)
+        m[f"{name}_under_low_ratio"] = float(under.sum() / rows)
+        mask = mask * (~over & ~under).to(mask.dtype)
+    elif seq_metric is not None:
+        raise ValueError(f"Unknown sequence_mask_metric: {seq_metric}")
+    return tis, m, mask
+
+
+def apply_off_policy_correction(loss, old_log_probs, rollout_logprobs, loss_mask, cfg):
+    """OPC:351-391: the per-token loss times the weight (when there is one), the new mask, the metrics; nothing without
+    rollout log-probabilities."""
+    if rollout_logprobs is None:
+        return loss, loss_mask, {}
+    tis, metrics, mask = off_policy_correction(old_log_probs, rollout_logprobs, loss_mask, cfg)
+    return (loss if tis is None else loss * tis), mask, metrics

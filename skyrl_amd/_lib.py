@@ -11,7 +11,7 @@ import os
 import threading
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libskyrl_lmhead.so")
-ABI_VERSION = 17
+ABI_VERSION = 18
 
 _c_i64 = ctypes.c_int64
 _c_p = ctypes.c_void_p
@@ -92,6 +92,11 @@ SIGNATURES = {
         ctypes.c_int,
         [_c_p, _c_i64, _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_i64, ctypes.c_float, _c_p, _c_i64, _c_p],
     ),
+    "skyrl_off_policy_correction": (
+        ctypes.c_int,
+        [_c_p, _c_p, _c_p, _c_i64, _c_i64, ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_float,
+         ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float),
+         ctypes.POINTER(ctypes.c_float), _c_p, _c_p, _c_p, _c_p, _c_p, _c_p]),
     "skyrl_logits_fwd": (
         ctypes.c_int, [_c_p, ctypes.c_int, _c_i64, _c_p, _c_i64, _c_i64, ctypes.c_float, _c_p, _c_p, _c_p, _c_p, _c_p]),
     "skyrl_logits_bwd": (

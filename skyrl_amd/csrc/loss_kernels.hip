@@ -405,6 +405,142 @@ __global__ __launch_bounds__(256) void actor_loss_dentropy_kernel(const ActorLos
   a.dent[i] = a.mask ? c * a.mask[i] : c;
 }
 
+
+// ------------------------------------------------------------------------------------------------------------
+// Off-policy correction from the rollout engine's log-probabilities (utils/off_policy_correction_utils.py:257-348, the
+// steps in the reference's order), one workgroup per row of [B, S]:
+//   r = exp(clamp(old - rollout, -20, 20)) per token
+//   1. outlier rows (:75-134):  a row with any unmasked token whose r > high or r < low loses its whole mask
+//   2. token mask (:137-188):   unmasked tokens with r outside [low, high] lose their mask
+//   3. TIS weight (:24-72):     "token": min(r, cap);  "sequence": min(exp(clamp(sum (old - rollout) * mask)), cap) of the row
+//   4. sequence mask (:191-254): "geometric": exp(clamp(sum (old - rollout) * mask / max(sum mask, 1))) outside [low, high],
+//                                "product": the row's product ratio outside [low, high] -> the row loses its mask
+// Steps 3 and 4 see the mask that steps 1 and 2 left.  Outputs: keep [B, S] in {0, 1} (mask_out = mask * keep is what the
+// reference returns), tis [B, S] (the row's value repeated for "sequence"), weight = tis * keep (what multiplies a
+// per-token loss next to the ORIGINAL mask: the reference's losses count their clip statistic with the original mask and
+// sum the loss with the new one, ppo_utils.py:570-587), and SKYRL_OFF_POLICY_ROW_STATS floats per row from which a one-workgroup kernel forms the
+// reference's metrics in a fixed order.
+// ------------------------------------------------------------------------------------------------------------
+struct OffPolicyArgs {
+  const float *old, *rollout, *mask;  // mask may be NULL (all ones)
+  int64_t rows, cols;
+  int tis_type, seq_metric;           // 0 = off; tis 1 token, 2 sequence; metric 1 geometric, 2 product
+  float tis_cap, seq_low, seq_high;
+  int use_outlier_low, use_outlier_high, use_token_mask;
+  float outlier_low, outlier_high, token_low, token_high;
+  float *keep_out, *tis_out, *weight_out;  // each may be NULL
+  float *row_stats, *metrics;              // [rows, SKYRL_OFF_POLICY_ROW_STATS], [SKYRL_OFF_POLICY_METRICS]
+};
+enum {
+  kOpSumRatioMask = 0, kOpSumMask, kOpSumX, kOpSumXX, kOpMaxX, kOpMinX, kOpRowInvalid, kOpRowOver, kOpRowUnder, kOpValidTokens,
+  kOpMaskedTokens, kOpTokens2, kOpCapped, kOpSeqCapped, kOpSeqOver, kOpSeqUnder, kOpSeqMasked,
+  kOpRowStats = SKYRL_OFF_POLICY_ROW_STATS
+};
+static_assert(kOpSeqMasked < kOpRowStats, "row statistics do not fit their slots");
+
+__device__ __forceinline__ float block_max(float v, float* red) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float s = red[0];
+  for (int k = 1; k < kRowThreads / 64; ++k) s = fmaxf(s, red[k]);
+  return s;
+}
+
+__global__ __launch_bounds__(kRowThreads) void off_policy_rows_kernel(const OffPolicyArgs a) {
+  __shared__ float red[kRowThreads / 64];
+  const int64_t row0 = (int64_t)blockIdx.x * a.cols;
+  const bool outlier = a.use_outlier_low || a.use_outlier_high;
+  float s_rm = 0.f, s_m = 0.f, s_x = 0.f, s_xx = 0.f, mx = -INFINITY, mn = INFINITY;
+  float over = 0.f, under = 0.f, pos = 0.f, oob = 0.f, dm2 = 0.f, m2s = 0.f, pos2 = 0.f, capped = 0.f;
+  for (int64_t c = threadIdx.x; c < a.cols; c += kRowThreads) {
+    const float delta = a.old[row0 + c] - a.rollout[row0 + c];
+    const float r = expf(fminf(fmaxf(delta, -20.f), 20.f));
+    const float m = a.mask ? a.mask[row0 + c] : 1.f;
+    const float x = r * m;
+    s_rm += x, s_m += m, s_x += x, s_xx += x * x;
+    mx = fmaxf(mx, x), mn = fminf(mn, x);
+    const bool live = m > 0.f;
+    if (a.use_outlier_high && live && r > a.outlier_high) over = 1.f;
+    if (a.use_outlier_low && live && r < a.outlier_low) under = 1.f;
+    const bool in_bounds = !a.use_token_mask || (r >= a.token_low && r <= a.token_high);
+    pos += live ? 1.f : 0.f;
+    oob += (live && !in_bounds) ? 1.f : 0.f;
+    const float m2 = (in_bounds || m == 0.f) ? m : 0.f;  // the mask after step 2, if the row survives step 1
+    dm2 = fmaf(delta, m2, dm2);
+    m2s += m2;
+    pos2 += m2 > 0.f ? 1.f : 0.f;
+    capped += (a.tis_type == 1 && m2 > 0.f && r > a.tis_cap) ? 1.f : 0.f;
+  }
+  s_rm = block_sum(s_rm, red), s_m = block_sum(s_m, red), s_x = block_sum(s_x, red), s_xx = block_sum(s_xx, red);
+  mx = block_max(mx, red), mn = -block_max(-mn, red);
+  over = block_max(over, red), under = block_max(under, red);
+  pos = block_sum(pos, red), oob = block_sum(oob, red), dm2 = block_sum(dm2, red), m2s = block_sum(m2s, red);
+  pos2 = block_sum(pos2, red), capped = block_sum(capped, red);
+  const bool valid = !(outlier && (over > 0.f || under > 0.f));
+  if (!valid) pos = 0.f, oob = 0.f, dm2 = 0.f, m2s = 0.f, pos2 = 0.f, capped = 0.f;  // the row's mask is gone from step 1 on
+  const float seq_ratio = expf(fminf(fmaxf(dm2, -20.f), 20.f));
+  float tis_row = 1.f, seq_capped = 0.f;
+  if (a.tis_type == 2) {
+    seq_capped = seq_ratio > a.tis_cap ? 1.f : 0.f;
+    tis_row = fminf(seq_ratio, a.tis_cap);
+  }
+  float seq_over = 0.f, seq_under = 0.f;
+  if (a.seq_metric) {
+    const float v = a.seq_metric == 1 ? expf(fminf(fmaxf(dm2 / fmaxf(m2s, 1.f), -20.f), 20.f)) : seq_ratio;
+    seq_over = v > a.seq_high ? 1.f : 0.f;
+    seq_under = v < a.seq_low ? 1.f : 0.f;
+  }
+  const bool keep_row = valid && seq_over == 0.f && seq_under == 0.f;
+  for (int64_t c = threadIdx.x; c < a.cols; c += kRowThreads) {
+    const float delta = a.old[row0 + c] - a.rollout[row0 + c];
+    const float r = expf(fminf(fmaxf(delta, -20.f), 20.f));
+    const float m = a.mask ? a.mask[row0 + c] : 1.f;
+    const bool in_bounds = !a.use_token_mask || (r >= a.token_low && r <= a.token_high);
+    const float keep = (keep_row && (in_bounds || m == 0.f)) ? 1.f : 0.f;
+    const float tis = a.tis_type == 1 ? fminf(r, a.tis_cap) : tis_row;
+    if (a.keep_out) a.keep_out[row0 + c] = keep;
+    if (a.tis_out) a.tis_out[row0 + c] = tis;
+    if (a.weight_out) a.weight_out[row0 + c] = tis * keep;
+  }
+  if (threadIdx.x == 0) {
+    float* st = a.row_stats + (int64_t)blockIdx.x * kOpRowStats;
+    st[kOpSumRatioMask] = s_rm, st[kOpSumMask] = s_m, st[kOpSumX] = s_x, st[kOpSumXX] = s_xx, st[kOpMaxX] = mx, st[kOpMinX] = mn;
+    st[kOpRowInvalid] = valid ? 0.f : 1.f, st[kOpRowOver] = over, st[kOpRowUnder] = under;
+    st[kOpValidTokens] = pos, st[kOpMaskedTokens] = oob, st[kOpTokens2] = pos2, st[kOpCapped] = capped;
+    st[kOpSeqCapped] = seq_capped, st[kOpSeqOver] = seq_over, st[kOpSeqUnder] = seq_under;
+    st[kOpSeqMasked] = (seq_over > 0.f || seq_under > 0.f) ? 1.f : 0.f;
+  }
+}
+
+// metrics: 0 is_ratio_mean, 1 is_ratio_std, 2 is_ratio_max, 3 is_ratio_min, 4 outlier_seq_masked_ratio, 5 outlier_seq_over_high_ratio,
+// 6 outlier_seq_under_low_ratio, 7 token_mask_ratio, 8 tis_token_clip_high_ratio, 9 tis_seq_clip_high_ratio,
+// 10 sequence-mask masked ratio, 11 its over-high ratio, 12 its under-low ratio.  Rows are added in order, in fp64.
+__global__ __launch_bounds__(64) void off_policy_finish_kernel(const OffPolicyArgs a) {
+  if (threadIdx.x != 0) return;
+  double s[kOpRowStats];
+  for (int k = 0; k < kOpRowStats; ++k) s[k] = 0.0;
+  double mx = -INFINITY, mn = INFINITY;
+  for (int64_t r = 0; r < a.rows; ++r) {
+    const float* st = a.row_stats + r * kOpRowStats;
+    for (int k = 0; k < kOpRowStats; ++k) s[k] += (double)st[k];
+    mx = fmax(mx, (double)st[kOpMaxX]), mn = fmin(mn, (double)st[kOpMinX]);
+  }
+  const double n = (double)a.rows * (double)a.cols, rows = (double)a.rows;
+  float* o = a.metrics;
+  o[0] = (float)(s[kOpSumRatioMask] / fmax(s[kOpSumMask], 1.0));
+  o[1] = (float)sqrt(fmax((s[kOpSumXX] - s[kOpSumX] * s[kOpSumX] / n) / (n - 1.0), 0.0));  // unbiased, as Tensor.std()
+  o[2] = (float)mx, o[3] = (float)mn;
+  o[4] = (float)(s[kOpRowInvalid] / rows), o[5] = (float)(s[kOpRowOver] / rows), o[6] = (float)(s[kOpRowUnder] / rows);
+  o[7] = (float)(s[kOpMaskedTokens] / fmax(s[kOpValidTokens], 1.0));
+  o[8] = (float)(s[kOpCapped] / fmax(s[kOpTokens2], 1.0));
+  o[9] = (float)(s[kOpSeqCapped] / rows);
+  o[10] = (float)(s[kOpSeqMasked] / rows), o[11] = (float)(s[kOpSeqOver] / rows), o[12] = (float)(s[kOpSeqUnder] / rows);
+  o[13] = o[14] = o[15] = 0.f;
+}
+
 bool finite(float x) { return std::isfinite(x); }
 bool valid_loss_type(int t) { return t >= SKYRL_POLICY_LOSS_REGULAR && t <= SKYRL_POLICY_LOSS_DPPO_KL; }
 bool interval_type(int t) {
@@ -497,6 +633,34 @@ int skyrl_masked_mean(const float* values, const float* mask, int64_t rows, int6
   hipLaunchKernelGGL(masked_mean_rows_kernel, dim3((unsigned)rows), dim3(kRowThreads), 0, (hipStream_t)stream, values, mask, cols,
                      means, dvalues);
   return (int)hipGetLastError();
+}
+
+int skyrl_off_policy_correction(const float* old_log_probs, const float* rollout_logprobs, const float* loss_mask, int64_t rows,
+                                int64_t cols, int tis_type, float tis_cap, int seq_metric, float seq_low, float seq_high,
+                                const float* outlier_low, const float* outlier_high, const float* token_low,
+                                const float* token_high, float* keep_out, float* tis_out, float* weight_out, float* metrics,
+                                float* row_stats, void* stream) {
+  if (!old_log_probs || !rollout_logprobs || !metrics || !row_stats) return SKYRL_LMHEAD_ERR_NULL;
+  if (rows < 1 || cols < 1 || rows > ((int64_t)1 << 31) - 1 || cols > ((int64_t)1 << 40)) return SKYRL_LMHEAD_ERR_SHAPE;
+  if (tis_type < 0 || tis_type > 2 || seq_metric < 0 || seq_metric > 2) return SKYRL_LMHEAD_ERR_ARG;
+  if ((tis_type && !finite(tis_cap)) || (seq_metric && (!finite(seq_low) || !finite(seq_high)))) return SKYRL_LMHEAD_ERR_ARG;
+  for (const float* p : {outlier_low, outlier_high, token_low, token_high})
+    if (p && !finite(*p)) return SKYRL_LMHEAD_ERR_ARG;
+  OffPolicyArgs a{};
+  a.old = old_log_probs, a.rollout = rollout_logprobs, a.mask = loss_mask, a.rows = rows, a.cols = cols;
+  a.tis_type = tis_type, a.seq_metric = seq_metric, a.tis_cap = tis_cap, a.seq_low = seq_low, a.seq_high = seq_high;
+  a.use_outlier_low = outlier_low != nullptr, a.use_outlier_high = outlier_high != nullptr;
+  a.use_token_mask = token_low != nullptr && token_high != nullptr;  // the token mask needs both bounds (:18-21)
+  a.outlier_low = outlier_low ? *outlier_low : 0.f, a.outlier_high = outlier_high ? *outlier_high : 0.f;
+  a.token_low = a.use_token_mask ? *token_low : 0.f, a.token_high = a.use_token_mask ? *token_high : 0.f;
+  a.keep_out = keep_out, a.tis_out = tis_out, a.weight_out = weight_out, a.row_stats = row_stats, a.metrics = metrics;
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(off_policy_rows_kernel, dim3((unsigned)rows), dim3(kRowThreads), 0, s, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return (int)e;
+  hipLaunchKernelGGL(off_policy_finish_kernel, dim3(1), dim3(64), 0, s, a);
+  e = hipGetLastError();
+  return e == hipSuccess ? SKYRL_LMHEAD_OK : (int)e;
 }
 
 }  // extern "C"

@@ -20,11 +20,12 @@ computes each with a chain of elementwise torch kernels and lets autograd derive
 value, statistics and gradient, so the upstream gradient of ``skyrl_lmhead_bwd`` is ready without another pass over the
 ``[B, S]`` tensors and, with ``sync_metrics=False``, without a host synchronisation.
 
-Off-policy correction (``apply_off_policy_correction``, off_policy_correction_utils.py:351-385) multiplies the per-token
-loss by an importance ratio that does not depend on the policy's log-probabilities and may thin the loss mask: compute both
-with the trainer's own helper and pass the ratio as ``loss_weight`` and the thinned mask as ``loss_mask``.  Computing them
-from ``rollout_logprobs`` is outside this module: the losses raise when the config switches a correction on, and otherwise
-use ``rollout_logprobs`` only where the loss itself is anchored on them (rollout-IS, DPPO, CISPO with the rollout anchor).
+Off-policy correction (``apply_off_policy_correction``, off_policy_correction_utils.py:351-391): the six losses that end with
+it in the reference (regular / dual clip, SAPO, GSPO, CISPO, rollout-IS, DPPO) end with it here -- when the config
+switches a correction on and ``rollout_logprobs`` are given, ``skyrl_amd.off_policy_correction`` computes the truncated
+importance weight and the thinned mask in two launches and their product joins ``loss_weight``; the metrics of the
+correction are added to the loss's metrics under the reference's names.  A weight computed elsewhere can still be passed as
+``loss_weight``.
 The two covariance-based types pick their tokens from the whole batch exactly as the reference does -- ``clip_cov`` a random
 subset drawn with ``torch.randperm`` on the host's generator, ``kl_cov`` a top-k computed on the CPU -- and hand the
 per-token decision to the same fused kernel (``compute_policy_loss_clip_cov``, ``compute_policy_loss_kl_cov``, :938-1053).
@@ -58,20 +59,20 @@ def _get(obj: Any, name: str, default: Any = None) -> Any:
     return getattr(obj, name, default)
 
 
-def _reject_off_policy_correction(config: Any, rollout_logprobs: Optional[torch.Tensor]) -> None:
-    """The reference corrects only when rollout log-probabilities are given and one of the config's switches is on
-    (off_policy_correction_utils.py:285-305, 388-391)."""
-    opc = _get(config, "off_policy_correction")
-    if rollout_logprobs is None or opc is None:
-        return
-    on = (_get(opc, "tis_ratio_type") is not None or _get(opc, "sequence_mask_metric") is not None
-          or _get(opc, "outlier_token_is_threshold_low") is not None
-          or _get(opc, "outlier_token_is_threshold_high") is not None
-          or (_get(opc, "token_mask_is_threshold_low") is not None and _get(opc, "token_mask_is_threshold_high") is not None))
-    if on:
-        raise NotImplementedError(
-            "off-policy correction from rollout_logprobs is not part of the fused loss; compute the importance ratio and the "
-            "thinned mask with the trainer's own helper and pass them as loss_weight and loss_mask")
+def _with_off_policy_correction(config: Any, old_log_probs, rollout_logprobs, loss_mask, loss_weight, sync_metrics: bool):
+    """The reference's losses end with ``apply_off_policy_correction(loss, old_log_probs, rollout_logprobs, loss_mask,
+    config.off_policy_correction)`` (ppo_utils.py:581, 653, 722, 815, 857, 929): the per-token loss times the truncated
+    importance weight, summed over the thinned mask, while their clip statistic was counted with the original mask.  Here
+    the correction's per-token factor ``tis * keep`` joins ``loss_weight`` and the original mask stays the kernel's mask.
+    Returns ``(loss_weight, the correction's metrics)``; nothing changes when the reference would not correct."""
+    from .off_policy_correction import correction_weight
+
+    weight, metrics = correction_weight(config, old_log_probs, rollout_logprobs, loss_mask, sync_metrics)
+    if weight is None:
+        return loss_weight, metrics
+    return (weight if loss_weight is None else loss_weight.to(torch.float32) * weight), metrics
+
+
 KL_ESTIMATORS = {"k1": 0, "abs": 1, "k2": 2, "k3": 3}
 _LOSS_PARTIALS = 256  # SKYRL_POLICY_LOSS_PARTIALS of the header
 
@@ -168,13 +169,13 @@ def ppo_policy_loss(
     """
     loss_type = getattr(config, "policy_loss_type", "regular")
     assert loss_type in ["regular", "dual_clip"], "loss_type must be either 'regular' or 'dual_clip'"
-    _reject_off_policy_correction(config, rollout_logprobs)
+    loss_weight, extra = _with_off_policy_correction(config, old_log_probs, rollout_logprobs, loss_mask, loss_weight, sync_metrics)
     dual = loss_type == "dual_clip"
     loss, sums = _PolicyLoss.apply(log_probs, old_log_probs, advantages, loss_mask, loss_weight, float(config.eps_clip_low),
                                    float(config.eps_clip_high), float(getattr(config, "clip_ratio_c", 0.0)) if dual else 0.0,
                                    LOSS_DUAL_CLIP if dual else LOSS_REGULAR)
     clip_ratio = sums[1] / sums[2].clamp(min=1.0)
-    return loss, {"clip_ratio": clip_ratio.item() if sync_metrics else clip_ratio}
+    return loss, {"clip_ratio": clip_ratio.item() if sync_metrics else clip_ratio, **extra}
 
 
 def cross_entropy_loss(
@@ -254,11 +255,11 @@ _POLICY_LOSS_NAMES = ("regular", "dual_clip", "cross_entropy", "importance_sampl
 
 def _elementwise_loss(name: str, log_probs, old_log_probs, advantages, config, loss_mask, rollout_logprobs, loss_weight,
                       sync_metrics: bool):
-    _reject_off_policy_correction(config, rollout_logprobs)
     loss_type, a, b, c, behaviour = _type_parameters(config, name, rollout_logprobs, old_log_probs)
+    loss_weight, extra = _with_off_policy_correction(config, old_log_probs, rollout_logprobs, loss_mask, loss_weight, sync_metrics)
     loss, sums = _PolicyLoss.apply(log_probs, behaviour, advantages, loss_mask, loss_weight, a, b, c, loss_type)
     clip_ratio = sums[1] / sums[2].clamp(min=1.0)
-    return loss, {"clip_ratio": clip_ratio.item() if sync_metrics else clip_ratio}
+    return loss, {"clip_ratio": clip_ratio.item() if sync_metrics else clip_ratio, **extra}
 
 
 def sapo_policy_loss(log_probs, old_log_probs, advantages, config, loss_mask=None, rollout_logprobs=None, *,
@@ -266,9 +267,10 @@ def sapo_policy_loss(log_probs, old_log_probs, advantages, config, loss_mask=Non
     """Soft adaptive policy optimisation (reference ``sapo_policy_loss``, ppo_utils.py:590-660): the gate
     ``sigmoid(tau (r - 1)) 4 / tau`` replaces the clipped ratio, ``tau = config.sapo.tau_pos`` where the advantage is
     positive, ``tau_neg`` elsewhere.  ``clip_ratio`` is 0.0 as in the reference."""
-    loss, _ = _elementwise_loss("sapo", log_probs, old_log_probs, advantages, config, loss_mask, rollout_logprobs, loss_weight,
-                                False)
-    return loss, {"clip_ratio": 0.0}
+    loss, metrics = _elementwise_loss("sapo", log_probs, old_log_probs, advantages, config, loss_mask, rollout_logprobs, loss_weight,
+                                      True)
+    metrics["clip_ratio"] = 0.0
+    return loss, metrics
 
 
 def compute_policy_loss_cispo(log_probs, old_log_probs, advantages, config, loss_mask=None, rollout_logprobs=None, *,
@@ -382,13 +384,13 @@ def gspo_policy_loss(log_probs, old_log_probs, advantages, config, loss_mask=Non
     """Group sequence policy optimisation, token-level variant (reference ``gspo_policy_loss``, ppo_utils.py:663-729): the
     clipped surrogate with every token's ratio replaced by its sequence's, ``exp(min(masked row mean of the log-ratio,
     10))``.  ``log_probs`` is ``[B, S]``; the rows are the sequences."""
-    _reject_off_policy_correction(config, rollout_logprobs)
     if log_probs.dim() < 2:
         raise ValueError("gspo_policy_loss needs [B, S] inputs: the importance weight is a row mean")
+    loss_weight, extra = _with_off_policy_correction(config, old_log_probs, rollout_logprobs, loss_mask, loss_weight, sync_metrics)
     scalars = (LOSS_GSPO, float(config.eps_clip_low), float(config.eps_clip_high), 0.0, 3, 1.0, 1.0, 0.0, 0.0)
     loss, out6 = _ActorLoss.apply(log_probs, None, (old_log_probs, advantages, loss_mask, loss_weight, None), scalars)
     clip_ratio = out6[2] / out6[3].clamp(min=1.0)
-    return loss, {"clip_ratio": clip_ratio.item() if sync_metrics else clip_ratio}
+    return loss, {"clip_ratio": clip_ratio.item() if sync_metrics else clip_ratio, **extra}
 
 
 # ----------------------------------------------------------------------------------------------------------------------
@@ -638,8 +640,10 @@ def actor_loss(
     and ``clip_ratio`` (``importance_ratio`` for the importance-sampling loss).
     """
     name = getattr(config, "policy_loss_type", "regular")
-    _reject_off_policy_correction(config, rollout_logprobs)
     loss_type, a, b, c, behaviour = _type_parameters(config, name, rollout_logprobs, old_log_probs)
+    extra: Dict[str, Any] = {}
+    if name not in ("cross_entropy", "importance_sampling"):   # the two losses the reference never corrects (:1056-1142)
+        loss_weight, extra = _with_off_policy_correction(config, old_log_probs, rollout_logprobs, loss_mask, loss_weight, False)
     use_kl = bool(getattr(config, "use_kl_loss", False))
     if use_kl and base_log_probs is None:
         raise ValueError("use_kl_loss needs base_log_probs")
@@ -656,7 +660,7 @@ def actor_loss(
     loss, out6 = _ActorLoss.apply(log_probs, entropy, consts, scalars)
     stat = out6[2] / (out6[3] if loss_type == LOSS_IMPORTANCE_SAMPLING else out6[3].clamp(min=1.0))
     metrics = {"policy_loss": out6[1], "policy_kl": out6[4], "policy_entropy": out6[5],
-               ("importance_ratio" if loss_type == LOSS_IMPORTANCE_SAMPLING else "clip_ratio"): stat}
+               ("importance_ratio" if loss_type == LOSS_IMPORTANCE_SAMPLING else "clip_ratio"): stat, **extra}
     return loss, metrics
 
 

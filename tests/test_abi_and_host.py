@@ -25,7 +25,7 @@ def _read(path):
 def _declared_functions(*headers):
     text = "".join(_read(h) for h in (headers or (HEADER, BENCH_HEADER)))
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(skyrl_(?:lmhead|ppo|packed|approx|masked|actor|softce|logits)_\w+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(skyrl_(?:lmhead|ppo|packed|approx|masked|actor|softce|logits|off)_\w+)\s*\(", text)))
 
 
 def test_library_exports_every_declared_symbol():
@@ -195,10 +195,13 @@ def test_ppo_policy_loss_mirror_contract():
     cfg = SimpleNamespace(policy_loss_type="regular", eps_clip_low=0.2, eps_clip_high=0.2, clip_ratio_c=3.0)
     with pytest.raises(AssertionError):
         ppo_policy_loss(x, x, x, SimpleNamespace(policy_loss_type="gspo", eps_clip_low=0.2, eps_clip_high=0.2))
-    # rollout log-probabilities are used for off-policy correction only: refused when the config switches one on,
-    # ignored (as in the reference) when it does not
+    # rollout log-probabilities are used for off-policy correction only: computed on the device when the config switches one
+    # on (a cap that is missing is named), ignored (as in the reference) when it does not
     cfg.off_policy_correction = SimpleNamespace(tis_ratio_type="token")
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(ValueError, match="token_tis_ratio_clip_high"):
+        ppo_policy_loss(x, x, x, cfg, rollout_logprobs=x)
+    cfg.off_policy_correction = SimpleNamespace(tis_ratio_type="token", token_tis_ratio_clip_high=2.0)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
         ppo_policy_loss(x, x, x, cfg, rollout_logprobs=x)
     cfg.off_policy_correction = {"tis_ratio_type": None, "sequence_mask_metric": None}
     with pytest.raises(RuntimeError, match="no CPU implementation"):

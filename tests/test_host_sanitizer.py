@@ -59,6 +59,11 @@ DRIVER = textwrap.dedent("""
         assert lib.skyrl_logits_fwd(p + 1, 0, ld, p, T, V, 1.0, p, None, None, None, None) < 0
         assert lib.skyrl_logits_bwd(p, 1, ld, p, p, None, p, None, T, V, 1.0, p + 2, ld, None) < 0
     assert lib.skyrl_ppo_policy_loss(p, p, p, None, None, 0, 0.2, 0.2, 3.0, 0, p, None, None, None) < 0
+    for rows, cols in itertools.product((0, 1 << 31, 1 << 40), (0, 5, 1 << 41)):
+        assert lib.skyrl_off_policy_correction(p, p, None, rows, cols, 1, 2.0, 0, 0.0, 0.0, None, None, None, None, p, p, p, p, p, None) < 0
+    assert lib.skyrl_off_policy_correction(p, p, None, 4, 4, 3, 2.0, 0, 0.0, 0.0, None, None, None, None, p, p, p, p, p, None) < 0
+    assert lib.skyrl_off_policy_correction(p, p, None, 4, 4, 1, float("inf"), 0, 0.0, 0.0, None, None, None, None, p, p, p, p, p, None) < 0
+    assert lib.skyrl_off_policy_correction(p, p, None, 4, 4, 0, 0.0, 0, 0.0, 0.0, None, None, None, None, p, p, p, None, p, None) < 0
     assert lib.skyrl_actor_loss(p, p, p, None, None, None, None, 1 << 40, 1 << 40, 0, 0.2, 0.2, 3.0, 3, 1.0, 1.0, 0.0, 0.0, p, p,
                                 None, None, None) < 0
     assert lib.skyrl_approx_kl(p, p, None, 1 << 40, 4, 3, None, p, p, 0, None, None) < 0

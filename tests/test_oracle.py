@@ -1113,3 +1113,85 @@ def test_logits_input_functions_against_library_distributions():
     assert torch.allclose(grad[mask], -(torch.softmax(logits, -1) * g.unsqueeze(-1))[mask], atol=1e-6)
     assert torch.allclose(grad.sum(-1)[inside], torch.zeros(int(inside.sum()), dtype=torch.float64), atol=1e-6)
     assert torch.allclose(grad.sum(-1)[mask], -g[mask], atol=1e-6)
+
+
+def _opc_cfg(**kw):
+    from types import SimpleNamespace
+
+    base = dict(tis_ratio_type=None, token_tis_ratio_clip_high=2.0, sequence_tis_ratio_clip_high=5.0, sequence_mask_metric=None,
+                geo_mask_high=1.01, geo_mask_low=0.99, product_mask_high=2.0, product_mask_low=0.5,
+                outlier_token_is_threshold_low=None, outlier_token_is_threshold_high=None,
+                token_mask_is_threshold_low=None, token_mask_is_threshold_high=None)
+    base.update(kw)
+    return SimpleNamespace(**base)
+
+
+def _opc_batch():
+    """Ratios old / rollout that are powers of two, so that every product and threshold decision can be read off."""
+    ratio = _t([[1.0, 2.0, 0.5, 4.0], [1.0, 8.0, 1.0, 1.0], [0.25, 1.0, 2.0, 1.0]])
+    mask = _t([[1.0, 1.0, 1.0, 0.0], [1.0, 1.0, 1.0, 1.0], [1.0, 0.0, 1.0, 1.0]])
+    rollout = _t([[-1.0, -2.0, -0.5, -3.0]] * 3)
+    return rollout + ratio.log(), rollout, mask, ratio
+
+
+def test_off_policy_correction_by_hand():
+    """off_policy_correction_utils.py:24-391 on a 3 x 4 batch: masks, weights and metrics of every step written down by hand,
+    and the order of the steps."""
+    import statistics
+
+    old, rollout, mask, ratio = _opc_batch()
+    assert O.off_policy_correction(old, rollout, mask, _opc_cfg()) == (None, {}, mask)
+    # outlier rows: row 1 holds an 8 (> 6); the 4 of row 0 is masked and does not count
+    tis, m, out = O.off_policy_correction(old, rollout, mask, _opc_cfg(outlier_token_is_threshold_high=6.0))
+    assert tis is None and torch.equal(out, _t([[1, 1, 1, 0], [0, 0, 0, 0], [1, 0, 1, 1]]))
+    assert m["outlier_seq_masked_ratio"] == pytest.approx(1 / 3) and m["outlier_seq_over_high_ratio"] == pytest.approx(1 / 3)
+    assert m["outlier_seq_under_low_ratio"] == 0.0
+    x = [1, 2, .5, 0, 1, 8, 1, 1, .25, 0, 2, 1]                      # ratio * mask, all twelve entries
+    assert m["is_ratio_mean"] == pytest.approx(17.75 / 10) and m["is_ratio_std"] == pytest.approx(statistics.stdev(x))
+    assert m["is_ratio_max"] == pytest.approx(8.0) and m["is_ratio_min"] == 0.0
+    _, m, out = O.off_policy_correction(old, rollout, mask, _opc_cfg(outlier_token_is_threshold_low=0.3))
+    assert torch.equal(out, _t([[1, 1, 1, 0], [1, 1, 1, 1], [0, 0, 0, 0]])) and m["outlier_seq_under_low_ratio"] == pytest.approx(1 / 3)
+    # + the per-token hard mask [0.4, 3]: of the six tokens the outlier step left, the 0.25 of row 2 goes
+    both = dict(outlier_token_is_threshold_high=6.0, token_mask_is_threshold_low=0.4, token_mask_is_threshold_high=3.0)
+    _, m, out = O.off_policy_correction(old, rollout, mask, _opc_cfg(**both))
+    assert torch.equal(out, _t([[1, 1, 1, 0], [0, 0, 0, 0], [0, 0, 1, 1]])) and m["token_mask_ratio"] == pytest.approx(1 / 6)
+    # one bound alone does not switch the token mask on
+    assert O.off_policy_correction(old, rollout, mask, _opc_cfg(token_mask_is_threshold_low=0.4))[0:2] == (None, {})
+    # + token-level TIS capped at 1.5: two of the five tokens still alive exceed it
+    tis, m, _ = O.off_policy_correction(old, rollout, mask, _opc_cfg(tis_ratio_type="token", token_tis_ratio_clip_high=1.5, **both))
+    assert torch.allclose(tis, _t([[1, 1.5, .5, 1.5], [1, 1.5, 1, 1], [.25, 1, 1.5, 1]])) and m["tis_token_clip_high_ratio"] == pytest.approx(0.4)
+    # sequence-level TIS on the same masks: products 1, 1 (the removed row) and 2; without the other steps row 1 has 8
+    tis, m, _ = O.off_policy_correction(old, rollout, mask, _opc_cfg(tis_ratio_type="sequence", sequence_tis_ratio_clip_high=1.5, **both))
+    assert torch.allclose(tis, _t([[1.0], [1.0], [1.5]])) and m["tis_seq_clip_high_ratio"] == pytest.approx(1 / 3)
+    tis, m, out = O.off_policy_correction(old, rollout, mask, _opc_cfg(tis_ratio_type="sequence"))
+    assert torch.allclose(tis, _t([[1.0], [5.0], [0.5]])) and m["tis_seq_clip_high_ratio"] == pytest.approx(1 / 3) and torch.equal(out, mask)
+    half = mask.clone()
+    half[0, 1] = 0.5                                                # a fractional mask weighs the log-ratio: 2 ** 0.5 * 0.5
+    tis, _, _ = O.off_policy_correction(old, rollout, half, _opc_cfg(tis_ratio_type="sequence"))
+    assert float(tis[0]) == pytest.approx(2 ** -0.5)
+    # sequence masks on the masks the first two steps left: geometric means 1, 1, sqrt 2; products 1, 1, 2
+    _, m, out = O.off_policy_correction(old, rollout, mask, _opc_cfg(sequence_mask_metric="geometric", geo_mask_low=0.9, geo_mask_high=1.3, **both))
+    assert torch.equal(out, _t([[1, 1, 1, 0], [0, 0, 0, 0], [0, 0, 0, 0]]))
+    assert (m["geo_sequence_mask_masked_ratio"], m["geo_sequence_mask_over_high_ratio"], m["geo_sequence_mask_under_low_ratio"]) == \
+        (pytest.approx(1 / 3), pytest.approx(1 / 3), 0.0)
+    _, m, out = O.off_policy_correction(old, rollout, mask, _opc_cfg(sequence_mask_metric="geometric", geo_mask_low=1.05, geo_mask_high=1.3, **both))
+    assert float(out.sum()) == 0.0 and m["geo_sequence_mask_masked_ratio"] == 1.0 and m["geo_sequence_mask_under_low_ratio"] == pytest.approx(2 / 3)
+    _, m, out = O.off_policy_correction(old, rollout, mask, _opc_cfg(sequence_mask_metric="product", product_mask_low=0.5, product_mask_high=1.5, **both))
+    assert torch.equal(out, _t([[1, 1, 1, 0], [0, 0, 0, 0], [0, 0, 0, 0]])) and m["product_sequence_mask_over_high_ratio"] == pytest.approx(1 / 3)
+    _, m, out = O.off_policy_correction(old, rollout, mask, _opc_cfg(sequence_mask_metric="product", product_mask_low=0.6, product_mask_high=6.0))
+    assert torch.equal(out, _t([[1, 1, 1, 0], [0, 0, 0, 0], [0, 0, 0, 0]]))          # products 1, 8, 0.5 without the other steps
+    assert m["product_sequence_mask_under_low_ratio"] == pytest.approx(1 / 3) and m["product_sequence_mask_masked_ratio"] == pytest.approx(2 / 3)
+    # the clamp of the log-ratio at +-20, unknown names, and the wrapper on a per-token loss
+    far = old.clone()
+    far[0, 0] += 50.0
+    tis, _, _ = O.off_policy_correction(far, rollout, mask, _opc_cfg(tis_ratio_type="token", token_tis_ratio_clip_high=1e30))
+    assert float(tis[0, 0]) == pytest.approx(math.exp(20.0))
+    with pytest.raises(ValueError):
+        O.off_policy_correction(old, rollout, mask, _opc_cfg(tis_ratio_type="rows"))
+    with pytest.raises(ValueError):
+        O.off_policy_correction(old, rollout, mask, _opc_cfg(sequence_mask_metric="median"))
+    loss = _t([[1.0, 2.0, 3.0, 4.0]] * 3)
+    got, got_mask, m = O.apply_off_policy_correction(loss, old, rollout, mask, _opc_cfg(tis_ratio_type="token", token_tis_ratio_clip_high=1.5, **both))
+    assert torch.allclose(got, loss * _t([[1, 1.5, .5, 1.5], [1, 1.5, 1, 1], [.25, 1, 1.5, 1]])) and "token_mask_ratio" in m
+    assert torch.equal(got_mask, _t([[1, 1, 1, 0], [0, 0, 0, 0], [0, 0, 1, 1]]))
+    assert O.apply_off_policy_correction(loss, old, None, mask, _opc_cfg(tis_ratio_type="token")) == (loss, mask, {})

@@ -909,9 +909,14 @@ def test_further_policy_losses_argument_handling(cuda_device):
                           off_policy_correction=SimpleNamespace(tis_ratio_type="token", sequence_mask_metric=None))
     with pytest.raises(AssertionError):                          # the rollout anchor needs rollout log-probabilities
         PL.compute_policy_loss_cispo(x, x, x, cfg)
-    with pytest.raises(NotImplementedError):                     # a correction switched on is not silently skipped
-        PL.ppo_policy_loss(x, x, x, SimpleNamespace(policy_loss_type="regular", eps_clip_low=0.2, eps_clip_high=0.2,
-                                                    off_policy_correction=cfg.off_policy_correction), None, x)
+    # a correction switched on is applied, not skipped: old / rollout = e^0.5 on every token, capped at 1.5
+    tis_cfg = SimpleNamespace(policy_loss_type="regular", eps_clip_low=0.2, eps_clip_high=0.2,
+                              off_policy_correction=SimpleNamespace(tis_ratio_type="token", token_tis_ratio_clip_high=1.5,
+                                                                    sequence_mask_metric=None))
+    loss, m = PL.ppo_policy_loss(x, x, x, tis_cfg, None, x - 0.5)
+    assert loss.item() == pytest.approx(16.0 * 1.5) and m["tis_token_clip_high_ratio"] == 1.0
+    with pytest.raises(ValueError):                              # the rollout anchor already is the correction: TIS would double-count
+        PL.compute_policy_loss_cispo(x, x, x, cfg, None, x)
     cfg.off_policy_correction.tis_ratio_type = None
     loss, m = PL.compute_policy_loss_cispo(x, x + 9.0, x, cfg, None, x)   # ratio 1 against the rollout anchor
     assert loss.item() == pytest.approx(-16.0) and m["clip_ratio"] == 0.0
