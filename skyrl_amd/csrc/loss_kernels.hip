@@ -519,14 +519,29 @@ __global__ __launch_bounds__(kRowThreads) void off_policy_rows_kernel(const OffP
 // 6 outlier_seq_under_low_ratio, 7 token_mask_ratio, 8 tis_token_clip_high_ratio, 9 tis_seq_clip_high_ratio,
 // 10 sequence-mask masked ratio, 11 its over-high ratio, 12 its under-low ratio.  Rows are added in order, in fp64.
 __global__ __launch_bounds__(64) void off_policy_finish_kernel(const OffPolicyArgs a) {
+  // lane l adds rows l, l + 64, ... in order; lane 0 then adds the 64 partial sums in lane order: a fixed order for any rows
+  __shared__ double part[64][kOpRowStats];
+  __shared__ double part_max[64], part_min[64];
+  {
+    double s[kOpRowStats];
+    for (int k = 0; k < kOpRowStats; ++k) s[k] = 0.0;
+    double mx = -INFINITY, mn = INFINITY;
+    for (int64_t r = threadIdx.x; r < a.rows; r += 64) {
+      const float* st = a.row_stats + r * kOpRowStats;
+      for (int k = 0; k < kOpRowStats; ++k) s[k] += (double)st[k];
+      mx = fmax(mx, (double)st[kOpMaxX]), mn = fmin(mn, (double)st[kOpMinX]);
+    }
+    for (int k = 0; k < kOpRowStats; ++k) part[threadIdx.x][k] = s[k];
+    part_max[threadIdx.x] = mx, part_min[threadIdx.x] = mn;
+  }
+  __syncthreads();
   if (threadIdx.x != 0) return;
   double s[kOpRowStats];
   for (int k = 0; k < kOpRowStats; ++k) s[k] = 0.0;
   double mx = -INFINITY, mn = INFINITY;
-  for (int64_t r = 0; r < a.rows; ++r) {
-    const float* st = a.row_stats + r * kOpRowStats;
-    for (int k = 0; k < kOpRowStats; ++k) s[k] += (double)st[k];
-    mx = fmax(mx, (double)st[kOpMaxX]), mn = fmin(mn, (double)st[kOpMinX]);
+  for (int l = 0; l < 64; ++l) {
+    for (int k = 0; k < kOpRowStats; ++k) s[k] += part[l][k];
+    mx = fmax(mx, part_max[l]), mn = fmin(mn, part_min[l]);
   }
   const double n = (double)a.rows * (double)a.cols, rows = (double)a.rows;
   float* o = a.metrics;
