@@ -546,7 +546,8 @@ __global__ __launch_bounds__(64) void off_policy_finish_kernel(const OffPolicyAr
   const double n = (double)a.rows * (double)a.cols, rows = (double)a.rows;
   float* o = a.metrics;
   o[0] = (float)(s[kOpSumRatioMask] / fmax(s[kOpSumMask], 1.0));
-  o[1] = (float)sqrt(fmax((s[kOpSumXX] - s[kOpSumX] * s[kOpSumX] / n) / (n - 1.0), 0.0));  // unbiased, as Tensor.std()
+  // unbiased, as Tensor.std(): NaN for a single element
+  o[1] = n > 1.0 ? (float)sqrt(fmax((s[kOpSumXX] - s[kOpSumX] * s[kOpSumX] / n) / (n - 1.0), 0.0)) : NAN;
   o[2] = (float)mx, o[3] = (float)mn;
   o[4] = (float)(s[kOpRowInvalid] / rows), o[5] = (float)(s[kOpRowOver] / rows), o[6] = (float)(s[kOpRowUnder] / rows);
   o[7] = (float)(s[kOpMaskedTokens] / fmax(s[kOpValidTokens], 1.0));

@@ -20,6 +20,7 @@ from skyrl_amd import policy_loss as PL
 
 pytestmark = pytest.mark.gpu
 
+ERR_NULL, ERR_SHAPE, ERR_ARG = -1, -2, -5   # include/skyrl_lmhead.h
 THRESHOLDS = (0.5, 0.7, 0.9, 1.1, 1.5, 2.0, 3.0)
 
 
@@ -221,3 +222,139 @@ def test_actor_loss_ends_with_the_correction(cuda_device):
     cfg.policy_loss_type = "cross_entropy"
     a, m = PL.actor_loss(to(lp), to(old), to(adv), cfg, to(mask), rollout_logprobs=to(rollout))
     assert "token_mask_ratio" not in m and a.item() == pytest.approx(float(-(lp * mask).sum()), rel=1e-5)
+
+
+@pytest.mark.filterwarnings("ignore:std\\(\\)")   # one element: Tensor.std() is NaN and says so
+@pytest.mark.parametrize("rows,cols", [(1, 1), (1, 7), (3, 1), (2, 255), (5, 256), (4, 257), (1, 5000), (33, 1023), (7, 2049)])
+def test_off_policy_correction_row_shapes(rows, cols, cuda_device):
+    """Rows shorter than, equal to and longer than a workgroup's sweep, with every step on; every row is its own case."""
+    gen = torch.Generator().manual_seed(rows * 10007 + cols)
+    rollout = torch.randn(rows, cols, generator=gen) * 0.5 - 1.0
+    delta = torch.randn(rows, cols, generator=gen) * (0.3 / max(1.0, cols ** 0.5))        # row sums of order 0.3
+    delta[0, 0] += 0.8
+    mask = (torch.rand(rows, cols, generator=gen) > 0.25).float()
+    mask[0, 0] = 1
+    ratio = delta.double().exp()
+    for th in THRESHOLDS:
+        delta = torch.where((ratio / th - 1).abs() < 1e-4, delta + 3e-4, delta)
+    for name in ("everything_token", "everything_sequence"):
+        cfg = _cfg(**CASES[name])
+        old = rollout + delta
+        if not _rows_are_decided_alike(old, rollout, mask, cfg):
+            old = rollout + delta * 1.01
+            assert _rows_are_decided_alike(old, rollout, mask, cfg)
+        want_tis, want_metrics, want_mask = O.off_policy_correction(old.double(), rollout.double(), mask.double(), cfg)
+        tis, metrics, new_mask = OPC.compute_off_policy_correction(old.to(cuda_device), rollout.to(cuda_device), mask.to(cuda_device), cfg)
+        assert torch.equal(new_mask.cpu().double(), want_mask), name
+        assert torch.allclose(tis.cpu().double(), want_tis, rtol=2e-5), name
+        for key, value in want_metrics.items():
+            assert metrics[key] == pytest.approx(value, rel=5e-5, abs=1e-6, nan_ok=True), (name, key)
+
+
+def test_off_policy_correction_leading_dimensions_and_dtypes(cuda_device):
+    """[B, G, S] inputs are rows of S; bf16 / fp64 inputs are read as fp32 and the weight comes back in the inputs' dtype."""
+    old, rollout, mask = _batch(B=12, S=40, seed=21)
+    cfg = _cfg(**CASES["everything_token"])
+    flat = OPC.compute_off_policy_correction(old.to(cuda_device), rollout.to(cuda_device), mask.to(cuda_device), cfg)
+    cube = OPC.compute_off_policy_correction(*(t.reshape(3, 4, 40).to(cuda_device) for t in (old, rollout, mask)), cfg)
+    assert cube[0].shape == (3, 4, 40) and torch.equal(cube[0].reshape(12, 40), flat[0]) and torch.equal(cube[2].reshape(12, 40), flat[2])
+    assert cube[1] == flat[1]
+    seq = OPC.compute_off_policy_correction(*(t.reshape(3, 4, 40).to(cuda_device) for t in (old, rollout, mask)), _cfg(**CASES["tis_sequence"]))
+    assert seq[0].shape == (3, 4, 1)
+    wide = OPC.compute_off_policy_correction(old.double().to(cuda_device), rollout.double().to(cuda_device), mask.double().to(cuda_device), cfg)
+    assert wide[0].dtype == torch.float64 and wide[2].dtype == torch.float64 and torch.equal(wide[2].float(), flat[2])
+    # a non-contiguous view gives what its contiguous copy gives
+    view = OPC.compute_off_policy_correction(old.to(cuda_device).t().contiguous().t(), rollout.to(cuda_device), mask.to(cuda_device), cfg)
+    assert torch.equal(view[0], flat[0]) and view[1] == flat[1]
+
+
+def test_off_policy_c_abi_argument_errors(cuda_device):
+    import ctypes
+
+    from skyrl_amd import _lib
+    lib = _lib.load()
+    rows, cols = 4, 16
+    old = torch.zeros(rows, cols, device=cuda_device)
+    out = torch.empty(rows, cols, device=cuda_device)
+    metrics = torch.empty(16, device=cuda_device)
+    stats = torch.empty(rows * 20, device=cuda_device)
+    f = lambda v: ctypes.byref(ctypes.c_float(v))  # noqa: E731
+
+    def call(old_p=old.data_ptr(), roll_p=old.data_ptr(), r=rows, c=cols, tis=1, cap=2.0, seq=0, lo=0.0, hi=0.0, ol=None, oh=None,
+             tl=None, th=None, metrics_p=metrics.data_ptr(), stats_p=stats.data_ptr()):
+        return lib.skyrl_off_policy_correction(old_p, roll_p, None, r, c, tis, cap, seq, lo, hi, ol, oh, tl, th, out.data_ptr(), None, None,
+                                               metrics_p, stats_p, torch.cuda.current_stream(cuda_device).cuda_stream)
+
+    assert call() == 0                                           # optional outputs may be left out
+    torch.cuda.synchronize()
+    assert bool((out == 1).all()) and metrics[0].item() == 1.0   # equal log-probabilities: ratio 1, nothing removed
+    assert call(old_p=None) == ERR_NULL and call(roll_p=None) == ERR_NULL
+    assert call(metrics_p=None) == ERR_NULL and call(stats_p=None) == ERR_NULL
+    assert call(r=0) == ERR_SHAPE and call(c=0) == ERR_SHAPE
+    assert call(r=1 << 31) == ERR_SHAPE
+    assert call(tis=3) == ERR_ARG and call(seq=-1) == ERR_ARG
+    assert call(cap=float("nan")) == ERR_ARG and call(seq=1, lo=float("inf")) == ERR_ARG
+    assert call(oh=f(float("nan"))) == ERR_ARG and call(tl=f(float("inf")), th=f(1.0)) == ERR_ARG
+    assert call(tis=0, cap=float("nan")) == 0                    # a cap that nothing reads is not checked
+    torch.cuda.synchronize()
+
+
+def test_off_policy_correction_full_size_properties(cuda_device):
+    """4.2 M tokens (1024 rows of 4096): what must hold whatever the data -- keep is 0 or 1 and constant 0 on a removed row,
+    weight = tis * keep, the token weight is min(ratio, cap) bit for bit, the metrics agree with torch reductions of the
+    outputs, a second call returns the same bits, and applying the thinned mask again removes nothing more."""
+    rows, cols = 1024, 4096
+    gen = torch.Generator(device=cuda_device).manual_seed(77)
+    rollout = torch.randn(rows, cols, device=cuda_device, generator=gen) * 0.7 - 1.5
+    old = rollout + torch.randn(rows, cols, device=cuda_device, generator=gen) * 0.02
+    old[::7, 5] += 1.0                                           # outlier tokens in every seventh row
+    mask = (torch.rand(rows, cols, device=cuda_device, generator=gen) > 0.4).float()
+    mask[::7, 5] = 1
+    cfg = _cfg(tis_ratio_type="token", token_tis_ratio_clip_high=1.02, outlier_token_is_threshold_high=2.0,
+               token_mask_is_threshold_low=0.97, token_mask_is_threshold_high=1.03)
+    keep, tis, weight, m = OPC.off_policy_correction_terms(old, rollout, mask, 1, 1.02, 0, 0.0, 0.0, None, 2.0, 0.97, 1.03)
+    assert bool(((keep == 0) | (keep == 1)).all()) and torch.equal(weight, tis * keep)
+    ratio = (old - rollout).clamp(-20, 20).exp()
+    assert torch.allclose(tis, ratio.clamp(max=1.02), rtol=2e-6)
+    assert bool((keep[::7] == 0).all())                          # rows with an outlier token are removed whole
+    other = torch.ones(rows, dtype=torch.bool, device=cuda_device)
+    other[::7] = False
+    inside = ((ratio >= 0.97) & (ratio <= 1.03)).float()
+    clear = ((ratio / 0.97 - 1).abs() > 1e-5) & ((ratio / 1.03 - 1).abs() > 1e-5) & (mask > 0)   # two exp() may differ in the last bit
+    assert torch.equal(keep[other][clear[other]], inside[other][clear[other]])
+    assert bool((keep[other][mask[other] == 0] == 1).all())     # tokens outside the mask are not judged
+    metrics = OPC.compute_off_policy_correction(old, rollout, mask, cfg)[1]
+    assert metrics["outlier_seq_masked_ratio"] == pytest.approx(len(range(0, rows, 7)) / rows)
+    assert metrics["is_ratio_max"] == pytest.approx(float((ratio * mask).max()), rel=1e-5)
+    assert metrics["is_ratio_mean"] == pytest.approx(float((ratio.double() * mask).sum() / mask.sum()), rel=1e-5)
+    kept_rows = mask[other].double()
+    assert metrics["token_mask_ratio"] == pytest.approx(float(((1 - inside[other].double()) * kept_rows).sum() / kept_rows.sum().clamp(min=1)), rel=1e-4)
+    again = OPC.off_policy_correction_terms(old, rollout, mask, 1, 1.02, 0, 0.0, 0.0, None, 2.0, 0.97, 1.03)
+    assert all(torch.equal(a, b) for a, b in zip((keep, tis, weight, m), again))
+    twice = OPC.off_policy_correction_terms(old, rollout, mask * keep, 1, 1.02, 0, 0.0, 0.0, None, 2.0, 0.97, 1.03)
+    assert torch.equal(twice[0] * mask * keep, mask * keep)
+
+
+def test_off_policy_correction_replays_from_a_hip_graph(cuda_device):
+    """The two launches hold no memset and no allocation of the library's own: captured once, replayed on new data with eager
+    work and synchronisations in between, every replay equals the eager result bit for bit."""
+    old0, rollout0, mask0 = (t.to(cuda_device) for t in _batch(B=16, S=300, seed=31))
+    args = (1, 1.5, 1, 0.9, 1.1, None, 3.0, 0.7, 1.5)
+    old, rollout, mask = old0.clone(), rollout0.clone(), mask0.clone()
+    side = torch.cuda.Stream(device=cuda_device)
+    side.wait_stream(torch.cuda.current_stream(cuda_device))
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            OPC.off_policy_correction_terms(old, rollout, mask, *args)
+    torch.cuda.current_stream(cuda_device).wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = OPC.off_policy_correction_terms(old, rollout, mask, *args)
+    for seed in (32, 33, 34):
+        o, r, k = (t.to(cuda_device) for t in _batch(B=16, S=300, seed=seed))
+        old.copy_(o), rollout.copy_(r), mask.copy_(k)
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = OPC.off_policy_correction_terms(o, r, k, *args)
+        torch.cuda.synchronize()
+        assert all(torch.equal(a, b) for a, b in zip(captured, eager)), seed
