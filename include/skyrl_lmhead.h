@@ -290,6 +290,17 @@ int skyrl_masked_mean(const float* values, const float* mask, int64_t rows, int6
                       void* stream);
 
 /*
+ * compute_minibatch_rollout_logprob_diff_metrics (workers/worker_utils.py:34-58), the drift statistics both trainers log per
+ * micro-batch (workers/worker.py:1124-1126, megatron_model_wrapper.py:982-984): over n fp32 tokens, with d = |logprobs -
+ * rollout_logprobs| and m = loss_mask (NULL: every token counts, plain means),
+ *     out4 = { sum d m / max(sum m, 1),  sum d^2 m / max(sum m, 1),  max d m,  min d m }.
+ * partials: fp32 scratch of 5 * SKYRL_POLICY_LOSS_PARTIALS elements.  Two launches, no read-back; the sums are added in a
+ * fixed order (bit-reproducible); a NaN reaches all four results, as with the torch reductions.
+ */
+int skyrl_logprob_diff_metrics(const float* logprobs, const float* rollout_logprobs, const float* loss_mask, int64_t n, float* out4,
+                               float* partials, void* stream);
+
+/*
  * Packed-sequence front end: the label of every token of a packed [T] stream is its successor inside its own sequence,
  *     labels[t] = tokens[cu[s] + (t - cu[s] + 1) mod (cu[s+1] - cu[s])],   s = the sequence with cu[s] <= t < cu[s+1]
  * (next_offsets / rolled_targets_full of from_parallel_hidden_to_logprobs_packed_sequences,

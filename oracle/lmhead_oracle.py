@@ -61,6 +61,7 @@ What pins each function (all in ``tests/test_oracle.py``; none of them re-types 
   * off-policy correction: every step on a 3 x 4 batch whose ratios are powers of two, each mask, weight and metric
     written down by hand, and the order of the steps (a row removed as an outlier no longer counts in the token-mask and
     TIS statistics and has sequence ratio 1; the sequence mask sees the tokens the token mask left).
+  * log-probability drift statistics: a six-token case worked out by hand, with a mask, with fractional weights and without.
 No function is left "parity unpinned".
 """
 
@@ -978,3 +979,15 @@ def apply_off_policy_correction(loss, old_log_probs, rollout_logprobs, loss_mask
         return loss, loss_mask, {}
     tis, metrics, mask = off_policy_correction(old_log_probs, rollout_logprobs, loss_mask, cfg)
     return (loss if tis is None else loss * tis), mask, metrics
+
+
+def minibatch_rollout_logprob_diff_metrics(action_log_probs, rollout_logprobs, loss_mask):
+    """workers/worker_utils.py:34-58: nothing without rollout log-probabilities; else the masked mean of the absolute
+    difference and of its square, and the largest and smallest masked absolute difference."""
+    if rollout_logprobs is None:
+        return {}
+    diff = (action_log_probs - rollout_logprobs).abs()
+    weighted = diff if loss_mask is None else diff * loss_mask
+    prefix = "minibatch_rollout_logprobs_abs_diff"
+    return {f"{prefix}_mean": float(masked_mean(diff, loss_mask)), f"{prefix}_sq_mean": float(masked_mean(diff * diff, loss_mask)),
+            f"{prefix}_max": float(weighted.max()), f"{prefix}_min": float(weighted.min())}

@@ -53,7 +53,7 @@ def main() -> int:
         out = f(rows, cols - 1)
         am = torch.ones(rows, cols, dtype=torch.uint8, device=dev)
         import ctypes
-        keep, tis, wgt, met, rstat = f(n), f(n), f(n), f(16), f(rows * 20)
+        keep, tis, wgt, met, rstat, parts5 = f(n), f(n), f(n), f(16), f(rows * 20), f(5 * 256)
         c_f = lambda v: ctypes.byref(ctypes.c_float(v))  # noqa: E731
         cases = {  # name: (call, bytes the call reads and writes)
             "ppo_policy_loss": (lambda: lib.skyrl_ppo_policy_loss(p(lp), p(old), p(adv), p(mask), None, n, 0.2, 0.2, 3.0, 0, p(out3),
@@ -67,6 +67,7 @@ def main() -> int:
             "off_policy_correction, all steps": (lambda: lib.skyrl_off_policy_correction(
                 p(old), p(lp), p(mask), rows, cols, 1, 1.5, 1, 0.9, 1.1, c_f(0.5), c_f(3.0), c_f(0.7), c_f(1.5), p(keep), p(tis), p(wgt),
                 p(met), p(rstat), None), 36 * n),
+            "logprob_diff_metrics": (lambda: lib.skyrl_logprob_diff_metrics(p(lp), p(old), p(mask), n, p(out6), p(parts5), None), 12 * n),
             "packed_next_token_labels": (lambda: lib.skyrl_packed_next_token_labels(p(tokens), p(cu), rows, n, p(labels), None), 16 * n),
             "packed_scatter, plain": (lambda: lib.skyrl_packed_scatter_logprobs(p(packed), p(cu), rows, n, None, None, None, None, rows,
                                                                                 cols - 1, p(out), None), 12 * n),

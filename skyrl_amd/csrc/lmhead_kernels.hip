@@ -1548,7 +1548,7 @@ int bwd_entry(const void* hidden, int64_t ld_hidden, const void* weight, int64_t
 
 extern "C" {
 
-int skyrl_lmhead_version(void) { return 18; }
+int skyrl_lmhead_version(void) { return 19; }
 
 const char* skyrl_lmhead_strerror(int status) {
   switch (status) {

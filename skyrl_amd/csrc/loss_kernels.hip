@@ -183,13 +183,107 @@ __global__ __launch_bounds__(1024) void policy_loss_kernel(const float* __restri
 constexpr int kMaxLossSlices = SKYRL_POLICY_LOSS_PARTIALS;
 constexpr int64_t kLossSliceTokens = 8192;  // at least this many tokens per workgroup
 
+// One wave: lane l adds the partial sums of slices l, l + 64, ..., then the lanes meet in a fixed tree -- the same order on
+// every run, and no chain of dependent loads through one thread.
 __global__ __launch_bounds__(64) void policy_loss_finish_kernel(const float* __restrict__ partials, int slices,
                                                                 float* __restrict__ out) {
-  if (threadIdx.x < 3) {
-    float v = 0.f;
-    for (int b = 0; b < slices; ++b) v += partials[threadIdx.x * kMaxLossSlices + b];
-    out[threadIdx.x] = v;
+  float v[3] = {0.f, 0.f, 0.f};
+  for (int b = threadIdx.x; b < slices; b += 64)
+#pragma unroll
+    for (int k = 0; k < 3; ++k) v[k] += partials[k * kMaxLossSlices + b];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1)
+#pragma unroll
+    for (int k = 0; k < 3; ++k) v[k] += __shfl_xor(v[k], off, 64);
+  if (threadIdx.x == 0) out[0] = v[0], out[1] = v[1], out[2] = v[2];
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// Statistics of |logprobs - rollout_logprobs| over the loss tokens of a micro-batch (workers/worker_utils.py:34-58):
+//     mean = sum |d| m / max(sum m, 1),  sq_mean = sum d^2 m / max(sum m, 1),  max / min of |d| m      (m = 1 without a mask:
+//     plain means).  Workgroup b sweeps tokens [b * slice, (b + 1) * slice) and writes its five partial results to
+// part[k * kMaxLossSlices + b]; logprob_diff_finish_kernel merges them in a fixed order.  Maximum and minimum hand a NaN on,
+// as Tensor.max() does.
+// ------------------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float max_nan(float a, float b) { return (a > b || a != a) ? a : b; }
+__device__ __forceinline__ float min_nan(float a, float b) { return (a < b || a != a) ? a : b; }
+
+__global__ __launch_bounds__(1024) void logprob_diff_kernel(const float* __restrict__ lp, const float* __restrict__ rollout,
+                                                            const float* __restrict__ mask, int64_t n, int64_t slice,
+                                                            float* __restrict__ part) {
+  __shared__ float red[5][16];
+  float s_abs = 0.f, s_sq = 0.f, s_m = 0.f, mx = -INFINITY, mn = INFINITY;
+  const int64_t t0 = (int64_t)blockIdx.x * slice, t1 = t0 + slice < n ? t0 + slice : n;
+  auto token = [&](float a, float b, float m) {
+    const float d = fabsf(a - b);
+    const float dm = mask ? d * m : d;
+    s_abs += dm;
+    s_sq += mask ? d * d * m : d * d;
+    s_m += m;
+    mx = max_nan(dm, mx), mn = min_nan(dm, mn);
+  };
+  // 16-byte loads where the slice allows them (slices start at multiples of four tokens when vec is set)
+  const bool vec = (slice & 3) == 0 && (((uintptr_t)lp | (uintptr_t)rollout | (uintptr_t)mask) & 15) == 0;
+  int64_t t = t0;
+  if (vec) {
+    const int64_t quads = (t1 - t0) >> 2;
+    const float4* __restrict__ lp4 = (const float4*)(lp + t0);
+    const float4* __restrict__ ro4 = (const float4*)(rollout + t0);
+    const float4* __restrict__ m4 = mask ? (const float4*)(mask + t0) : nullptr;
+    // four pieces per array in flight per thread: a slice of 16384 tokens is one batch of loads for the 1024 threads
+    for (int64_t i0 = threadIdx.x; i0 < quads; i0 += 4 * (int64_t)blockDim.x) {
+      float4 a[4], b[4], m[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t i = i0 + u * (int64_t)blockDim.x;
+        if (i < quads) {
+          a[u] = lp4[i], b[u] = ro4[i];
+          m[u] = m4 ? m4[i] : make_float4(1.f, 1.f, 1.f, 1.f);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (i0 + u * (int64_t)blockDim.x < quads)
+          token(a[u].x, b[u].x, m[u].x), token(a[u].y, b[u].y, m[u].y), token(a[u].z, b[u].z, m[u].z), token(a[u].w, b[u].w, m[u].w);
+    }
+    t = t0 + (quads << 2);
   }
+  for (t += threadIdx.x; t < t1; t += blockDim.x) token(lp[t], rollout[t], mask ? mask[t] : 1.f);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    s_abs += __shfl_xor(s_abs, off, 64);
+    s_sq += __shfl_xor(s_sq, off, 64);
+    s_m += __shfl_xor(s_m, off, 64);
+    mx = max_nan(__shfl_xor(mx, off, 64), mx);
+    mn = min_nan(__shfl_xor(mn, off, 64), mn);
+  }
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (lane == 0) red[0][wave] = s_abs, red[1][wave] = s_sq, red[2][wave] = s_m, red[3][wave] = mx, red[4][wave] = mn;
+  __syncthreads();
+  if (threadIdx.x < 5) {
+    const int k = threadIdx.x;
+    float v = red[k][0];
+    for (int w = 1; w < 16; ++w) v = k < 3 ? v + red[k][w] : (k == 3 ? max_nan(red[k][w], v) : min_nan(red[k][w], v));
+    part[k * kMaxLossSlices + blockIdx.x] = v;
+  }
+}
+
+__global__ __launch_bounds__(64) void logprob_diff_finish_kernel(const float* __restrict__ part, int slices,
+                                                                 float* __restrict__ out4) {
+  double s_abs = 0.0, s_sq = 0.0, s_m = 0.0;
+  float mx = -INFINITY, mn = INFINITY;
+  for (int b = threadIdx.x; b < slices; b += 64) {  // lane l: slices l, l + 64, ...; then a fixed tree over the lanes
+    s_abs += part[b], s_sq += part[kMaxLossSlices + b], s_m += part[2 * kMaxLossSlices + b];
+    mx = max_nan(part[3 * kMaxLossSlices + b], mx), mn = min_nan(part[4 * kMaxLossSlices + b], mn);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    s_abs += __shfl_xor(s_abs, off, 64), s_sq += __shfl_xor(s_sq, off, 64), s_m += __shfl_xor(s_m, off, 64);
+    mx = max_nan(__shfl_xor(mx, off, 64), mx), mn = min_nan(__shfl_xor(mn, off, 64), mn);
+  }
+  if (threadIdx.x != 0) return;
+  const double den = s_m > 1.0 ? s_m : 1.0;
+  out4[0] = (float)(s_abs / den), out4[1] = (float)(s_sq / den), out4[2] = mx, out4[3] = mn;
 }
 
 constexpr int kRowThreads = 1024;  // one workgroup per row of [B, S]: rows are few and long
@@ -677,6 +771,20 @@ int skyrl_off_policy_correction(const float* old_log_probs, const float* rollout
   hipLaunchKernelGGL(off_policy_finish_kernel, dim3(1), dim3(64), 0, s, a);
   e = hipGetLastError();
   return e == hipSuccess ? SKYRL_LMHEAD_OK : (int)e;
+}
+
+int skyrl_logprob_diff_metrics(const float* logprobs, const float* rollout_logprobs, const float* loss_mask, int64_t n, float* out4,
+                               float* partials, void* stream) {
+  if (!logprobs || !rollout_logprobs || !out4 || !partials) return SKYRL_LMHEAD_ERR_NULL;
+  if (n < 1) return SKYRL_LMHEAD_ERR_SHAPE;
+  int64_t slices = (n + kLossSliceTokens - 1) / kLossSliceTokens;
+  if (slices > kMaxLossSlices) slices = kMaxLossSlices;
+  const int64_t slice = (n + slices - 1) / slices;
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(logprob_diff_kernel, dim3((unsigned)slices), dim3(1024), 0, s, logprobs, rollout_logprobs, loss_mask, n, slice,
+                     partials);
+  hipLaunchKernelGGL(logprob_diff_finish_kernel, dim3(1), dim3(64), 0, s, partials, (int)slices, out4);
+  return (int)hipGetLastError();
 }
 
 }  // extern "C"

@@ -25,7 +25,7 @@ def _read(path):
 def _declared_functions(*headers):
     text = "".join(_read(h) for h in (headers or (HEADER, BENCH_HEADER)))
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(skyrl_(?:lmhead|ppo|packed|approx|masked|actor|softce|logits|off)_\w+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(skyrl_(?:lmhead|ppo|packed|approx|masked|actor|softce|logits|off|logprob)_\w+)\s*\(", text)))
 
 
 def test_library_exports_every_declared_symbol():

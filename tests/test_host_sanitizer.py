@@ -67,6 +67,8 @@ DRIVER = textwrap.dedent("""
     assert lib.skyrl_actor_loss(p, p, p, None, None, None, None, 1 << 40, 1 << 40, 0, 0.2, 0.2, 3.0, 3, 1.0, 1.0, 0.0, 0.0, p, p,
                                 None, None, None) < 0
     assert lib.skyrl_approx_kl(p, p, None, 1 << 40, 4, 3, None, p, p, 0, None, None) < 0
+    for n, out, part in ((0, p, p), (-1, p, p), (16, None, p), (16, p, None)):
+        assert lib.skyrl_logprob_diff_metrics(p, p, None, n, out, part, None) < 0
     assert lib.skyrl_masked_mean(p, None, 1 << 40, 4, p, None, None) < 0
     assert lib.skyrl_actor_loss(p, p, p, None, None, None, p, 1 << 30, 1 << 40, 0, 0.2, 0.2, 3.0, 3, 1.0, 1.0, 0.0, 0.0, p, p,
                                 None, p, None) < 0

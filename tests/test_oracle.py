@@ -1195,3 +1195,26 @@ def test_off_policy_correction_by_hand():
     assert torch.allclose(got, loss * _t([[1, 1.5, .5, 1.5], [1, 1.5, 1, 1], [.25, 1, 1.5, 1]])) and "token_mask_ratio" in m
     assert torch.equal(got_mask, _t([[1, 1, 1, 0], [0, 0, 0, 0], [0, 0, 1, 1]]))
     assert O.apply_off_policy_correction(loss, old, None, mask, _opc_cfg(tis_ratio_type="token")) == (loss, mask, {})
+
+
+def test_minibatch_rollout_logprob_diff_metrics_by_hand():
+    """workers/worker_utils.py:34-58 on six tokens whose differences are 0.5, -1, 2, 0, -0.25, 4."""
+    lp = _t([[-1.0, -2.0, -0.5], [-3.0, -1.25, -0.5]])
+    rollout = _t([[-1.5, -1.0, -2.5], [-3.0, -1.0, -4.5]])
+    assert O.minibatch_rollout_logprob_diff_metrics(lp, None, None) == {}
+    pre = "minibatch_rollout_logprobs_abs_diff"
+    m = O.minibatch_rollout_logprob_diff_metrics(lp, rollout, None)
+    assert sorted(m) == [f"{pre}_max", f"{pre}_mean", f"{pre}_min", f"{pre}_sq_mean"]
+    assert m[f"{pre}_mean"] == pytest.approx(7.75 / 6) and m[f"{pre}_sq_mean"] == pytest.approx((0.25 + 1 + 4 + 0 + 0.0625 + 16) / 6)
+    assert m[f"{pre}_max"] == 4.0 and m[f"{pre}_min"] == 0.0
+    mask = _t([[1, 1, 0], [0, 1, 0]])                              # the tokens with 0.5, 1 and 0.25
+    m = O.minibatch_rollout_logprob_diff_metrics(lp, rollout, mask)
+    assert m[f"{pre}_mean"] == pytest.approx(1.75 / 3) and m[f"{pre}_sq_mean"] == pytest.approx(1.3125 / 3)
+    assert m[f"{pre}_max"] == 1.0 and m[f"{pre}_min"] == 0.0       # masked tokens count as 0 in the extremes
+    half = _t([[0.5, 1, 0], [0, 0, 2]])                           # weights: 0.5 * 0.5, 1 * 1, 2 * 4 over a weight sum of 3.5
+    m = O.minibatch_rollout_logprob_diff_metrics(lp, rollout, half)
+    assert m[f"{pre}_mean"] == pytest.approx(9.25 / 3.5) and m[f"{pre}_sq_mean"] == pytest.approx((0.125 + 1 + 32) / 3.5)
+    assert m[f"{pre}_max"] == 8.0
+    none = torch.zeros(2, 3, dtype=torch.float64)                  # nothing counts: the denominators are clamped at 1
+    m = O.minibatch_rollout_logprob_diff_metrics(lp, rollout, none)
+    assert (m[f"{pre}_mean"], m[f"{pre}_sq_mean"], m[f"{pre}_max"], m[f"{pre}_min"]) == (0.0, 0.0, 0.0, 0.0)
