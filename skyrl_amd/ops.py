@@ -1,7 +1,7 @@
-"""torch.library custom ops over the C ABI: ``skyrl_amd::lmhead_fwd`` and ``skyrl_amd::lmhead_bwd``.
+"""torch.library custom ops over the C ABI for the fused LM head: ``skyrl_amd::lmhead_fwd`` and the ``skyrl_amd::lmhead_bwd*``
+family (fp32 / bf16 weight gradient, hidden gradient alone, all tokens or the tokens with an upstream gradient only).
 
-These are the only two places Python touches the HIP kernels.  Tensors stay torch-owned; the ops pass raw device
-pointers, sizes and the current HIP stream through ctypes.  Scratch is a torch ``uint8`` tensor sized by the library's
+Tensors stay torch-owned; the ops pass raw device pointers, sizes and the current HIP stream through ctypes.  Scratch is a torch ``uint8`` tensor sized by the library's
 own ``*_workspace_bytes`` query, so ``torch.cuda.max_memory_allocated`` sees every byte the path uses.
 
 Shapes: hidden ``[T, H]`` bf16 (row stride a multiple of 8), weight ``[V, H]`` bf16, labels ``[T]`` int64 (a value
