@@ -62,6 +62,10 @@ What pins each function (all in ``tests/test_oracle.py``; none of them re-types 
     written down by hand, and the order of the steps (a row removed as an outlier no longer counts in the token-mask and
     TIS statistics and has sequence ratio 1; the sequence mask sees the tokens the token mask left).
   * log-probability drift statistics: a six-token case worked out by hand, with a mask, with fractional weights and without.
+  * the reference's own unit-test vectors for the off-policy correction, the policy losses and the approximate KL
+    (tests/train/algorithms/test_off_policy_correction.py, tests/train/algorithms/test_losses.py,
+    tests/backends/skyrl_train/utils/test_ppo_utils.py:38-98), transcribed into tests/golden/reference_unit_test_cases.json and run
+    by tests/test_reference_unit_cases.py in fp32 and fp64 at the reference's tolerances.
 No function is left "parity unpinned".
 """
 

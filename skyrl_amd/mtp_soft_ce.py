@@ -11,7 +11,10 @@ chunking with recomputation (:162-197).  Here the loss and its gradient come str
   mtp/adapter.py:51-56);
 * ``draft_soft_ce_from_hidden(...)`` -> the masked-mean scalar, ``draft_soft_ce``'s contract with hidden states in place of
   logits and ``mtp_layer_number`` in place of a pre-rolled teacher;
-* ``shift_mask_for_mtp`` (:37-79) -- the mask roll the caller applies, same signature and results.
+* ``shift_mask_for_mtp`` (:37-79) -- the mask roll the caller applies, same signature and results;
+* ``unpadded_vocab_shard_width`` (:79-95) -- how many rows of a vocabulary shard are real when Megatron padded the vocabulary;
+  where the reference slices both logits tensors to that width (megatron_model_wrapper.py:738-748), the caller here passes
+  ``weight[:width]``.
 
 * ``topk_logits_from_hidden``, ``soft_ce_topk_from_hidden``, ``draft_soft_ce_topk_from_hidden`` -- the top-k variant
   (``draft_soft_ce_topk`` / ``_VocabParallelTopkSoftCE``, :243-341): the teacher's k largest logits per token straight from
@@ -31,7 +34,7 @@ from .ops import _require_device
 
 __all__ = ["soft_ce_from_hidden", "draft_soft_ce_from_hidden", "shift_mask_for_mtp", "softce_fwd", "softce_bwd",
            "topk_logits_from_hidden", "soft_ce_topk_from_hidden", "draft_soft_ce_topk_from_hidden", "topk_logits",
-           "softce_topk_fwd", "softce_topk_bwd"]
+           "softce_topk_fwd", "softce_topk_bwd", "unpadded_vocab_shard_width"]
 
 
 def _check(student: torch.Tensor, teacher: torch.Tensor, weight: torch.Tensor, seq_len: int) -> Tuple[int, int, int]:
@@ -361,3 +364,15 @@ def shift_mask_for_mtp(mask: torch.Tensor, mtp_layer_number: int = 0, cu_seqlens
     ok = target < end
     rolled = torch.where(ok, mask[:, target.clamp(max=S - 1)], torch.zeros((), dtype=mask.dtype, device=mask.device))
     return mask * rolled
+
+
+def unpadded_vocab_shard_width(true_vocab_size: Optional[int], vocab_shard_width: int, tp_rank: int) -> int:
+    """Rows of rank ``tp_rank``'s vocabulary shard that belong to the true vocabulary (reference
+    ``unpadded_vocab_shard_width``, soft_ce.py:79-95): the shard starts at ``tp_rank * vocab_shard_width`` and the padding sits
+    at the end of the padded vocabulary, so the count is what is left of the true vocabulary from that start, between 0 and
+    the shard's width; the whole width when the true size is unknown.  Padded rows are never trained and must not enter the
+    teacher distribution: pass ``weight[:width]`` to the draft-loss functions of this module."""
+    if true_vocab_size is None:
+        return vocab_shard_width
+    remaining = true_vocab_size - tp_rank * vocab_shard_width
+    return min(vocab_shard_width, remaining) if remaining > 0 else 0
