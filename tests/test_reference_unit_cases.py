@@ -365,3 +365,91 @@ def test_hip_draft_losses_reject_an_attached_teacher(cuda_device):
         with pytest.raises(AssertionError, match="must be detached"):
             call(teacher)
         assert bool(torch.isfinite(call(teacher.detach())))
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# the FSDP wrapper's forward tail on the reference's own padded layouts (tests/backends/skyrl_train/gpu/gpu_ci/
+# test_model_wrapper.py:24-33, 200-245): padding on both sides, the last action slot a padding token
+# ----------------------------------------------------------------------------------------------------------------------
+WRAPPER_V, WRAPPER_EOS, WRAPPER_PAD = 1000, 999, 0
+WRAPPER_LAYOUTS = {
+    "one_row": ([[WRAPPER_PAD] * 3 + [10, 14, 200, 3, 40, WRAPPER_EOS] + [WRAPPER_PAD]], [[0] * 3 + [1] * 6 + [0]]),
+    "two_rows": ([[WRAPPER_PAD] * 3 + [10, 14, 200, 3, 40, WRAPPER_EOS] + [WRAPPER_PAD],
+                  [WRAPPER_PAD, 12, 13, 220, 998, 3, 40, WRAPPER_EOS] + [WRAPPER_PAD] * 2], [[0] * 3 + [1] * 6 + [0], [0] + [1] * 7 + [0] * 2]),
+}
+
+
+def _marker_logits(next_tokens, V):
+    """Logits whose log-probability of ``next_tokens[p]`` at position ``p`` is a known function of that token: zeros except a
+    peak ``a = token / 200`` at the token's own column, so log p = a - ln(V - 1 + e^a)."""
+    z = torch.zeros(len(next_tokens), V, dtype=torch.float64)
+    for p, tok in enumerate(next_tokens):
+        z[p, tok] = tok / 200.0
+    return z
+
+
+def _marker_value(tok, V):
+    a = tok / 200.0
+    return a - math.log(V - 1 + math.exp(a))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("layout", list(WRAPPER_LAYOUTS))
+@pytest.mark.parametrize("from_hidden", [False, True])
+def test_hip_wrapper_tail_on_the_reference_layouts(layout, from_hidden, cuda_device):
+    """The reference mocks the per-position log-probability as "the next token's id" and expects the wrapper to hand back the
+    action tokens themselves, with and without sample packing (test_model_wrapper.py:36-103).  Without mocking: logits built
+    so that the log-probability of the next token is a known function of its id; the wrapper must return that function of the
+    last ``num_actions`` tokens.  The last action slot is the padding token behind EOS: without packing its label is that
+    padding token, with packing the roll wraps to the first real token of the stream -- as in the reference.  Then
+    test_actor_entropy_consistency_sample_packing (:200-245): entropy with and without packing agrees on the real tokens."""
+    from skyrl_amd.model_wrapper import action_log_probs_from_hidden, action_log_probs_from_logits
+    ids, am = (torch.tensor(v) for v in WRAPPER_LAYOUTS[layout])
+    B, S = ids.shape
+    A, V = 4, WRAPPER_V
+    nnz = am.flatten().nonzero().flatten()
+    dev = cuda_device
+    results = {}
+    for packed in (False, True):
+        stream = ids.reshape(-1)[nnz][None] if packed else ids
+        rolled = torch.roll(stream, -1, dims=1)
+        logits = torch.stack([_marker_logits(r.tolist(), V) for r in rolled])              # [rows, positions, V]
+        if from_hidden:   # an identity-like head: hidden = logits padded to H = 1024 columns, weight = the matching unit rows
+            H = 1024
+            hidden = torch.zeros(*logits.shape[:2], H, dtype=torch.float64)
+            hidden[..., :V] = logits
+            weight = torch.zeros(V, H, dtype=torch.float64)
+            weight[torch.arange(V), torch.arange(V)] = 1.0
+            alp, out = action_log_probs_from_hidden(hidden.bfloat16().to(dev), weight.bfloat16().to(dev), ids.to(dev), A, am.to(dev), 1.0,
+                                                    return_output=True, compute_entropy=True, entropy_requires_grad=False,
+                                                    nnz_indices=nnz.to(dev) if packed else None)
+            tol = 2e-2                                                                     # the peaks a = token / 200 rounded to bf16
+        else:
+            alp, out = action_log_probs_from_logits(logits.float().to(dev), ids.to(dev), A, am.to(dev), 1.0, return_output=True,
+                                                    compute_entropy=True, entropy_requires_grad=False,
+                                                    nnz_indices=nnz.to(dev) if packed else None)
+            tol = 1e-5
+        assert alp.shape == (B, A)
+        for b in range(B):
+            for j in range(A):
+                pos = S - A - 1 + j                                                        # the position that scores action j
+                if packed and not bool(am[b, pos]):
+                    want = 0.0                                                             # padding put back as zeros
+                elif packed:
+                    k = int((nnz == b * S + pos).nonzero())                               # its place in the packed stream
+                    want = _marker_value(int(rolled[0, k]), V)
+                else:
+                    want = _marker_value(int(ids[b, pos + 1]), V)
+                assert alp[b, j].item() == pytest.approx(want, abs=tol), (packed, b, j)
+        results[packed] = out["entropy"].float().cpu()
+        # cross-check with the oracle's statement of the tail on the same logits
+        want_alp, want_ent = O.hf_wrapper_tail(logits, ids, A, am.double(), 1.0, nnz_indices=nnz if packed else None)
+        assert (alp.cpu().double() - want_alp).abs().max().item() <= tol
+        assert (results[packed].double() - want_ent).abs().max().item() <= (5e-2 if from_hidden else 1e-5)
+    # wherever both runs scored the same next token -- every real token but the last of each row -- the entropies agree;
+    # padding positions are zero in both
+    real = am.bool()
+    same_label = real & torch.roll(am, -1, dims=1).bool()
+    same_label[:, -1] = False
+    assert torch.allclose(results[False][same_label], results[True][same_label], atol=5e-2 if from_hidden else 1e-5)
+    assert bool((results[True][~real] == 0).all()) and bool((results[False][~real] == 0).all())
