@@ -190,9 +190,13 @@ def topk_logits(hidden: torch.Tensor, weight: torch.Tensor, k: int, rcp_temperat
     T, H, V = _check(hidden, hidden, weight, 1)
     dev = _require_device(hidden, weight)
     lib = _lib.load()
+    if not 1 <= int(k) <= min(V, 1024):
+        raise ValueError(f"bad k {k}: must be between 1 and min(V, 1024) = {min(V, 1024)}")
+    if T == 0:  # an empty batch: nothing to launch
+        return torch.empty((0, k), dtype=torch.float32, device=dev), torch.empty((0, k), dtype=torch.int32, device=dev)
     ws_bytes = int(lib.skyrl_lmhead_topk_workspace_bytes(T, H, V, int(k)))
     if ws_bytes == 0:
-        raise ValueError(f"bad k {k}: must be between 1 and min(V, 1024) = {min(V, 1024)}")
+        raise ValueError(f"no top-k workspace for T={T}, H={H}, V={V}, k={k}: an extent is out of range")
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     values = torch.empty((T, k), dtype=torch.float32, device=dev)
     columns = torch.empty((T, k), dtype=torch.int32, device=dev)

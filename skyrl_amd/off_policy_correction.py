@@ -108,7 +108,10 @@ def _run(old_log_probs, rollout_logprobs, loss_mask, cfg, sync_metrics: bool):
     tok_low, tok_high = _get(cfg, "token_mask_is_threshold_low"), _get(cfg, "token_mask_is_threshold_high")
     shape = old_log_probs.shape
     cols = shape[-1] if old_log_probs.dim() else 1
-    flat = lambda t: None if t is None else t.detach().reshape(-1, cols).to(torch.float32).contiguous()  # noqa: E731
+    rows = 1
+    for extent in shape[:-1]:
+        rows *= int(extent)
+    flat = lambda t: None if t is None else t.detach().reshape(rows, cols).to(torch.float32).contiguous()  # noqa: E731
     keep, tis, weight, m = off_policy_correction_terms(
         flat(old_log_probs), flat(rollout_logprobs), flat(loss_mask), _TIS[tis_type], float(tis_cap), _SEQ[seq_metric],
         float(seq_low), float(seq_high), out_low, out_high, tok_low if tok_high is not None else None,

@@ -441,8 +441,6 @@ def _(log_probs, log_probs_base, loss_mask, estimator, grad_mode):
 def _kl_operands(log_probs, log_probs_base, loss_mask, kl_estimator_type):
     if kl_estimator_type not in KL_ESTIMATORS:
         raise ValueError(f"Invalid KL estimator type: {kl_estimator_type}")
-    if log_probs.numel() == 0:
-        raise ValueError("log_probs is empty")
     rows, cols = _rows_cols(log_probs)
     lp = log_probs.detach().to(torch.float32).contiguous().reshape(rows, cols)
     base = _same_f32("log_probs_base", log_probs_base, log_probs).reshape(rows, cols)
@@ -477,6 +475,10 @@ def compute_approx_kl(
     """Per-token KL estimate, same contract as the reference's ``compute_approx_kl`` (ppo_utils.py:88-126): estimators
     ``k1``, ``abs``, ``k2``, ``k3``; masked positions are exactly 0.  fp32 result of the shape of ``log_probs``;
     differentiable with respect to ``log_probs`` (the base policy's log-probabilities are treated as constants)."""
+    if kl_estimator_type not in KL_ESTIMATORS:
+        raise ValueError(f"Invalid KL estimator type: {kl_estimator_type}")
+    if log_probs.numel() == 0:  # nothing to launch: the empty estimate, attached to log_probs as any other
+        return (log_probs - log_probs_base.detach()).to(torch.float32)
     return _ApproxKL.apply(log_probs, log_probs_base, loss_mask, kl_estimator_type, 1)
 
 
@@ -488,6 +490,9 @@ def approx_kl_loss(
 ) -> torch.Tensor:
     """``masked_mean(compute_approx_kl(...), loss_mask, dim=-1).mean()`` -- the KL loss term of the trainer
     (workers/worker.py:1071-1077) -- from one kernel, with its gradient with respect to ``log_probs``."""
+    if log_probs.numel() == 0:  # nothing to launch: the reference's expression on the empty estimate (no rows: NaN; no columns: 0)
+        kld = compute_approx_kl(log_probs, log_probs_base, loss_mask, kl_estimator_type)
+        return masked_mean(kld, loss_mask, dim=-1).mean()
     return _ApproxKL.apply(log_probs, log_probs_base, loss_mask, kl_estimator_type, 2)
 
 
@@ -532,8 +537,14 @@ def masked_mean(tensor: torch.Tensor, mask: Optional[torch.Tensor], dim: Optiona
     """``(tensor * mask).sum(dim) / mask.sum(dim).clamp(min=1)``; ``mask=None``: the plain mean (reference ``masked_mean``,
     torch_utils.py:180-184).  ``dim`` is ``None`` (everything) or the last dimension; fp32 result; differentiable with respect
     to ``tensor``."""
-    if tensor.numel() == 0:
-        raise ValueError("masked_mean of an empty tensor")
+    if tensor.numel() == 0:  # nothing to launch: the reference's expression itself, which is shape arithmetic on an empty tensor
+        t = tensor.to(torch.float32)
+        if mask is None:
+            return t.mean() if dim is None else t.mean(dim=dim)
+        m = mask.to(torch.float32)
+        if dim is None:
+            return (t * m).sum() / m.sum().clamp(min=1.0)
+        return (t * m).sum(dim=dim) / m.sum(dim=dim).clamp(min=1.0)
     if dim is None:
         return _MaskedMean.apply(tensor, mask, 1, tensor.numel(), ())
     if dim not in (-1, tensor.dim() - 1):
@@ -640,6 +651,9 @@ def actor_loss(
     and ``clip_ratio`` (``importance_ratio`` for the importance-sampling loss).
     """
     name = getattr(config, "policy_loss_type", "regular")
+    if log_probs.numel() == 0:
+        raise ValueError(f"actor_loss needs at least one token, got log_probs of shape {tuple(log_probs.shape)}: the mean over "
+                         "the rows of an empty micro-batch is undefined (the reference's KL and entropy terms are NaN there)")
     loss_type, a, b, c, behaviour = _type_parameters(config, name, rollout_logprobs, old_log_probs)
     extra: Dict[str, Any] = {}
     if name not in ("cross_entropy", "importance_sampling"):   # the two losses the reference never corrects (:1056-1142)
