@@ -13,6 +13,7 @@ linear layer):
 Every forward is one HIP kernel that reads the logits once (the reference makes several passes and, in
 ``DistributedLogprob``, keeps an fp32 softmax of the whole tensor for the backward); the backward recomputes the softmax from the
 logits and the saved ``[T]`` row statistics in one read + write pass, over the logits themselves when ``inplace_backward`` says so.
+A sliced view such as ``logits[:, :-1]`` is walked where it lies (one launch per batch entry), not copied.
 """
 
 from __future__ import annotations
@@ -51,6 +52,34 @@ def _rows(logits: torch.Tensor) -> Tuple[int, int, int]:
     return T, V, ld
 
 
+def _pieces(logits: torch.Tensor) -> Tuple[int, int, list]:
+    """``(T, V, pieces)`` of a ``[T, V]`` matrix or a ``[B, S, V]`` tensor: the runs of equally pitched rows the kernels walk,
+    each ``(2-D view, index of its first row)``.  A 3-D tensor whose batch stride is ``S`` row pitches is one run; a view such
+    as ``logits[:, :-1]`` (rows equally pitched inside a batch entry only) is one run per batch entry -- walked where it
+    lies, never copied."""
+    if logits.dim() == 2:
+        T, V, _ = _rows(logits)
+        return T, V, [(logits, 0)]
+    if logits.dim() != 3:
+        raise ValueError(f"expected logits [T, V] or [B, S, V], got {tuple(logits.shape)}")
+    B, S, V = (int(x) for x in logits.shape)
+    if B * S == 0:
+        return 0, V, []
+    flat = None
+    if B == 1:
+        flat = logits[0]
+    elif S == 1:
+        flat = logits[:, 0]
+    elif logits.stride(0) == S * logits.stride(1):
+        flat = logits.as_strided((B * S, V), (logits.stride(1), logits.stride(2)), logits.storage_offset())
+    if flat is not None:
+        _rows(flat)
+        return B * S, V, [(flat, 0)]
+    for b in range(B):
+        _rows(logits[b])
+    return B * S, V, [(logits[b], b * S) for b in range(B)]
+
+
 def _check_rows(name: str, t: Optional[torch.Tensor], T: int, dtype: torch.dtype) -> None:
     if t is not None and (t.dtype != dtype or t.shape != (T,) or not t.is_contiguous()):
         raise ValueError(f"{name} must be a contiguous {dtype} tensor of shape [{T}], got {t.dtype} {tuple(t.shape)}")
@@ -61,7 +90,7 @@ def logits_fwd(logits: torch.Tensor, labels: Optional[torch.Tensor], rcp_tempera
                ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """``(logprobs, entropy, row_lse, row_pz)``, fp32 ``[T]``, of ``logits [T, V] * rcp_temperature``.  Without ``labels`` the
     log-probabilities are zero; without ``want_entropy`` entropy and ``row_pz`` are zero (and cost nothing)."""
-    T, V, ld = _rows(logits)
+    T, V, pieces = _pieces(logits)
     dev = _require_device(logits, labels)
     _check_rows("labels", labels, T, torch.int64)
     f32 = dict(dtype=torch.float32, device=dev)
@@ -69,24 +98,38 @@ def logits_fwd(logits: torch.Tensor, labels: Optional[torch.Tensor], rcp_tempera
     ent, pz = (torch.empty(T, **f32), torch.empty(T, **f32)) if want_entropy else (torch.zeros(T, **f32), torch.zeros(T, **f32))
     if T == 0:
         return lp, ent, lse, pz
+    lib = _lib.load()
     with torch.cuda.device(dev):
-        st = _lib.load().skyrl_logits_fwd(logits.data_ptr(), _DTYPES[logits.dtype], ld, None if labels is None else labels.data_ptr(),
-                                          T, V, float(rcp_temperature), None if labels is None else lp.data_ptr(),
-                                          ent.data_ptr() if want_entropy else None, lse.data_ptr(),
-                                          pz.data_ptr() if want_entropy else None, torch.cuda.current_stream(dev).cuda_stream)
-    _lib.check(st, "skyrl_logits_fwd")
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        for view, r0 in pieces:
+            rows, _, ld = _rows(view)
+            st = lib.skyrl_logits_fwd(view.data_ptr(), _DTYPES[logits.dtype], ld, None if labels is None else labels.data_ptr() + 8 * r0,
+                                      rows, V, float(rcp_temperature), None if labels is None else lp.data_ptr() + 4 * r0,
+                                      ent.data_ptr() + 4 * r0 if want_entropy else None, lse.data_ptr() + 4 * r0,
+                                      pz.data_ptr() + 4 * r0 if want_entropy else None, stream)
+            _lib.check(st, "skyrl_logits_fwd")
     return lp, ent, lse, pz
 
 
 @logits_fwd.register_fake
 def _(logits, labels, rcp_temperature, want_entropy):
-    T = logits.shape[0]
+    T = logits.numel() // max(1, logits.shape[-1])
     return tuple(logits.new_empty(T, dtype=torch.float32) for _ in range(4))
 
 
+def _row_run(pieces: list, r0: int, n: int) -> torch.Tensor:
+    """Rows ``r0 .. r0 + n - 1`` of a tensor given by its pieces, as a 2-D view (the run lies inside one piece)."""
+    for view, first in pieces:
+        if first <= r0 and r0 + n <= first + view.shape[0]:
+            return view[r0 - first:r0 - first + n]
+    raise ValueError("the gradient's layout does not line up with the logits'")
+
+
 def _bwd_into(out: torch.Tensor, logits, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature) -> None:
-    T, V, ld = _rows(logits)
-    _, _, ldd = _rows(out)
+    T, V, pieces = _pieces(logits)
+    To, Vo, out_pieces = _pieces(out)
+    if (To, Vo) != (T, V):
+        raise ValueError(f"the gradient has shape {tuple(out.shape)}, the logits {tuple(logits.shape)}")
     dev = _require_device(logits, labels, row_lse, row_pz, dlogprobs, dentropy, out)
     _check_rows("labels", labels, T, torch.int64)
     for name, t in (("row_lse", row_lse), ("row_pz", row_pz), ("dlogprobs", dlogprobs), ("dentropy", dentropy)):
@@ -95,26 +138,33 @@ def _bwd_into(out: torch.Tensor, logits, labels, row_lse, row_pz, dlogprobs, den
         raise ValueError("the backward needs an upstream gradient: dlogprobs, dentropy or both")
     if T == 0:
         return
-    ptr = lambda t: None if t is None else t.data_ptr()  # noqa: E731
+    runs = pieces if len(pieces) >= len(out_pieces) else out_pieces        # the finer of the two partitions
+    ptr = lambda t, r0, size: None if t is None else t.data_ptr() + size * r0  # noqa: E731
+    lib = _lib.load()
     with torch.cuda.device(dev):
-        st = _lib.load().skyrl_logits_bwd(logits.data_ptr(), _DTYPES[logits.dtype], ld, ptr(labels), row_lse.data_ptr(), ptr(row_pz),
-                                          ptr(dlogprobs), ptr(dentropy), T, V, float(rcp_temperature), out.data_ptr(), ldd,
-                                          torch.cuda.current_stream(dev).cuda_stream)
-    _lib.check(st, "skyrl_logits_bwd")
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        for run, r0 in runs:
+            n = int(run.shape[0])
+            src, dst = _row_run(pieces, r0, n), _row_run(out_pieces, r0, n)
+            _, _, ld = _rows(src)
+            _, _, ldd = _rows(dst)
+            st = lib.skyrl_logits_bwd(src.data_ptr(), _DTYPES[logits.dtype], ld, ptr(labels, r0, 8), ptr(row_lse, r0, 4), ptr(row_pz, r0, 4),
+                                      ptr(dlogprobs, r0, 4), ptr(dentropy, r0, 4), n, V, float(rcp_temperature), dst.data_ptr(), ldd, stream)
+            _lib.check(st, "skyrl_logits_bwd")
 
 
 @torch.library.custom_op("skyrl_amd::logits_bwd", mutates_args=())
 def logits_bwd(logits: torch.Tensor, labels: Optional[torch.Tensor], row_lse: torch.Tensor, row_pz: Optional[torch.Tensor],
                dlogprobs: Optional[torch.Tensor], dentropy: Optional[torch.Tensor], rcp_temperature: float) -> torch.Tensor:
     """d loss / d logits, a new ``[T, V]`` tensor in the logits' dtype."""
-    out = torch.empty((logits.shape[0], logits.shape[1]), dtype=logits.dtype, device=logits.device)
+    out = torch.empty(logits.shape, dtype=logits.dtype, device=logits.device)
     _bwd_into(out, logits, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature)
     return out
 
 
 @logits_bwd.register_fake
 def _(logits, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature):
-    return logits.new_empty((logits.shape[0], logits.shape[1]))
+    return logits.new_empty(logits.shape)
 
 
 @torch.library.custom_op("skyrl_amd::logits_bwd_", mutates_args=("logits",))
@@ -153,11 +203,16 @@ class _FromLogits(torch.autograd.Function):
 
 
 def _flat(logits: torch.Tensor) -> torch.Tensor:
-    """``[..., V]`` as a 2-D matrix without a copy where the layout allows it."""
+    """``[..., V]`` in a form the kernels walk without a copy where the layout allows it: a 2-D matrix, or the ``[B, S, V]``
+    tensor itself when its rows are equally pitched inside every batch entry (a slice such as ``logits[:, :-1]`` stays where
+    it is; the kernels then run once per batch entry)."""
     V = logits.shape[-1]
+    if logits.dtype not in _DTYPES:
+        logits = logits.to(torch.float32)
+    if logits.dim() == 3 and logits.shape[0] > 1 and logits.shape[1] > 1 and (logits.stride(2) == 1 or V == 1) \
+            and logits.stride(1) >= V and logits.stride(0) != logits.shape[1] * logits.stride(1) and logits.stride(0) > 0:
+        return logits          # reshape would copy: the rows of a batch entry are equally pitched, the entries are not adjacent
     flat = logits.reshape(-1, V)
-    if flat.dtype not in _DTYPES:
-        flat = flat.to(torch.float32)
     if flat.stride(1) != 1 and V > 1:
         flat = flat.contiguous()
     return flat

@@ -503,3 +503,51 @@ def test_fsdp_forward_tail_from_logits(cuda_device, packed, compute_entropy, ent
     tol = 1e-4 if dtype == torch.float32 else 2.0 ** -6        # bf16: the entropy reaches the loss rounded to bf16
     assert ((grads[0].cpu().double() - x.grad).abs() / scale)[live].max() <= tol
     assert float(grads[0].cpu()[~live].abs().max() if bool((~live).any()) else 0.0) == 0.0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("view", ["drop_last", "drop_first", "narrow_vocab", "both"])
+def test_sliced_logits_are_walked_where_they_lie(view, dtype, cuda_device):
+    """``logits[:, :-1]`` and its relatives (what a caller that shifts the logits instead of the labels passes): rows equally
+    pitched inside a batch entry, the entries not adjacent.  No copy is made -- the kernels run once per batch entry -- so the
+    results equal those of a contiguous copy bit for bit, and with ``inplace_backward`` the gradient lands in the caller's own
+    storage, the rows outside the view untouched."""
+    from skyrl_amd import torch_utils as TU
+    gen = torch.Generator(device=cuda_device).manual_seed(5)
+    B, S, V = 3, 9, 1000
+    base = (torch.randn(B, S, V, device=cuda_device, generator=gen) * 2).to(dtype)
+    cut = {"drop_last": (slice(None), slice(0, S - 1), slice(None)), "drop_first": (slice(None), slice(1, S), slice(None)),
+           "narrow_vocab": (slice(None), slice(None), slice(0, V - 8)), "both": (slice(None), slice(1, S - 1), slice(8, V))}[view]
+    sub = base[cut]
+    assert not sub.is_contiguous()
+    b, s, v = sub.shape
+    labels = torch.randint(0, v, (b, s), device=cuda_device, generator=gen)
+    g = torch.randn(b, s, device=cuda_device, generator=gen)
+    q = torch.randn(b, s, device=cuda_device, generator=gen) * 0.1
+    # reference run on a contiguous copy
+    copy = sub.clone().requires_grad_(True)
+    lp0, ent0 = TU.logprobs_and_entropy_from_logits(copy, labels, temperature=0.7)
+    ((lp0 * g).sum() + (ent0 * q).sum()).backward()
+    # the view itself, out of place
+    leaf = base.clone().requires_grad_(True)
+    lp1, ent1 = TU.logprobs_and_entropy_from_logits(leaf[cut], labels, temperature=0.7)
+    ((lp1 * g).sum() + (ent1 * q).sum()).backward()
+    assert torch.equal(lp1, lp0) and torch.equal(ent1, ent0)
+    assert torch.equal(leaf.grad[cut], copy.grad)
+    outside = torch.ones_like(base, dtype=torch.bool)
+    outside[cut] = False
+    assert bool((leaf.grad[outside] == 0).all())
+    # in place: the gradient is written over the view's rows of a non-leaf tensor, the rest of its storage keeps the logits
+    leaf2 = base.clone().requires_grad_(True)
+    mid = leaf2 * 1.0
+    before = mid.detach().clone()
+    lp2 = TU.logprobs_from_logits(mid[cut], labels, inplace_backward=True)
+    (lp2 * g).sum().backward()
+    plain = base.clone().requires_grad_(True)
+    (TU.logprobs_from_logits(plain[cut].clone(), labels, inplace_backward=False) * g).sum().backward()
+    assert torch.equal(leaf2.grad, plain.grad)
+    assert torch.equal(mid.detach()[cut], plain.grad[cut]) and torch.equal(mid.detach()[outside], before[outside])
+    # the other wrappers take the same views
+    assert torch.equal(TU.chunked_entropy_from_logits(sub), TU.chunked_entropy_from_logits(sub.clone()))
+    assert torch.equal(TU.logprobs_from_logits_v2(sub, labels), TU.logprobs_from_logits_v2(sub.clone(), labels))
+    assert torch.equal(TU.DistributedLogprob.apply(sub, labels, 0, v, None, True), TU.DistributedLogprob.apply(sub.clone(), labels, 0, v, None, True))
