@@ -52,7 +52,7 @@ int skyrl_lmhead_version(void);
 /* Human-readable text for a status code returned by this library (never NULL). */
 const char* skyrl_lmhead_strerror(int status);
 
-/* Scratch needed by skyrl_lmhead_fwd: per-vocab-tile (max, sum-exp, sum z*exp) partials of one token block,
+/* Scratch needed by skyrl_lmhead_fwd: per-vocab-tile (max, sum-exp, sum (z-max)*exp) partials of one token block,
  * 24 * min(T, 32768) * ceil(V/256) bytes (tokens rounded up to a multiple of 64) plus alignment slack.  The forward walks the
  * tokens in blocks of 32768 and merges a block's partials before the next block overwrites them, so the scratch does not
  * grow with T beyond one block (results are bit-identical to an unblocked run: block boundaries are tile boundaries).

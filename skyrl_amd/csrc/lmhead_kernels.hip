@@ -2,7 +2,7 @@
 //
 // Forward  (2*T*V*H flop):
 //   lmhead_fwd_tiles   one 256(vocab) x 256(token) logits tile per workgroup: bf16 MFMA GEMM, then in registers
-//                      scale by 1/temperature, per-token max / sum-exp / sum z*exp over the tile's vocab rows;
+//                      scale by 1/temperature, per-token max / sum-exp / sum (z-max)*exp over the tile's vocab rows;
 //                      writes one (max, sum, pz) partial per token per 128-row half tile, in blocks of 64 tokens.  Logits
 //                      never leave VGPRs.
 //   lmhead_fwd_merge   per block of 64 tokens: merges the partials (online log-sum-exp), gathers the label logit with an
@@ -66,7 +66,7 @@ __host__ __device__ inline size_t part_elems(size_t nparts, int64_t T) {
 // ------------------------------------------------------------------------------------------------------------
 // Forward tile kernel.  M axis = vocab (A = weight), N axis = tokens (B = hidden).
 // Online softmax statistics follow efficient_entropy_kernel_general_mainloop
-// (fused_linear_logprob_triton.py:296-385): scale, running max, sum exp, sum z*exp; vocab rows past V take no part.
+// (fused_linear_logprob_triton.py:296-385): scale, running max, sum exp, sum z*exp (kept relative to the maximum here); vocab rows past V take no part.
 // The label-logit gather of that kernel (:364-385) is done in lmhead_fwd_merge instead.
 // ------------------------------------------------------------------------------------------------------------
 // PAIRED (the soft cross-entropy, below): token blocks j >= TN / 2 hold teacher rows, and their third statistic weighs the
@@ -76,7 +76,10 @@ __device__ __forceinline__ void fwd_tile_stats(const acc_t& acc, int j, int vbas
                                                float& s_out, float& e_out) {
   const int jy = (PAIRED && j >= TN / 2) ? j - TN / 2 : j;  // j is a constant of the caller's unrolled loop
   // Two read-only passes over the accumulators (they live in AGPRs; writing scaled values back would cost a move each
-  // way).  scale2 > 0, so the maximum commutes with the scaling, and sum z*p = scale2 * sum x*p.
+  // way).  scale2 > 0, so the maximum commutes with the scaling.  The third statistic of an ordinary row is taken relative
+  // to the tile's maximum, sum (z - m) e^(z - m): the exponent is at hand, and the entropy ln s - e / s then comes out of two
+  // small numbers when the row is nearly deterministic, where lse - sum p z would cancel two large ones.  (The paired
+  // statistic of the soft cross-entropy stays sum z_student e^(z_teacher - m): it is an expectation of another row's logit.)
   float mx = -INFINITY;
 #pragma unroll
   for (int i = 0; i < TM; ++i)
@@ -97,19 +100,20 @@ __device__ __forceinline__ void fwd_tile_stats(const acc_t& acc, int j, int vbas
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const float x = acc[i][j][r];
-      float p = __builtin_amdgcn_exp2f(fmaf(x, scale2, -m2));
+      const float t2 = fmaf(x, scale2, -m2);
+      float p = __builtin_amdgcn_exp2f(t2);
       if (MASKED) {
         const int v = vbase + i * MT + kq * 4 + r;
         if (v >= V) p = 0.f;
       }
       s += p;
-      if (ENTROPY) e = fmaf(PAIRED ? acc[i][jy][r] : x, p, e);
+      if (ENTROPY) e = fmaf(PAIRED ? acc[i][jy][r] : t2, p, e);
     }
   s = col_sum(s);
   if (ENTROPY) e = col_sum(e);
   m_out = m2 * kLn2;
   s_out = s;
-  e_out = e * scale2 * kLn2;
+  e_out = PAIRED ? e * scale2 * kLn2 : e * kLn2;
 }
 
 template <bool ENTROPY, bool PAIRED>
@@ -174,6 +178,25 @@ constexpr int kMergeThreads = 1024;
 constexpr int kMergeWaves = kMergeThreads / 64;
 constexpr int kDotLanes = kMergeThreads / kMergeTokens;  // lanes per token in the label-logit phase
 
+// Two partial triples (maximum, sum e^(z - max), third statistic) of one token become one.  RELATIVE: the third statistic
+// is sum (z - max) e^(z - max) and moves with the maximum, e' = c (e + (max - max') s); otherwise it is sum y e^(z - max) of
+// some y that does not depend on the maximum and only scales.
+template <bool RELATIVE>
+__device__ __forceinline__ void merge_partial(float& M, float& S, float& E, float m, float s, float e) {
+  if (!(m > -INFINITY)) return;  // a part without a single vocabulary row
+  if (!(M > -INFINITY)) {
+    M = m, S = s, E = e;
+    return;
+  }
+  const float Mn = fmaxf(M, m);
+  const float da = M - Mn, db = m - Mn;
+  const float ca = expf(da), cb = expf(db);
+  E = RELATIVE ? ca * fmaf(da, S, E) + cb * fmaf(db, s, e) : E * ca + e * cb;
+  S = S * ca + s * cb;
+  M = Mn;
+}
+
+template <bool RELATIVE>
 __global__ __launch_bounds__(kMergeThreads) void lmhead_fwd_merge(const float* __restrict__ part_max,
                                                                   const float* __restrict__ part_sum,
                                                                   const float* __restrict__ part_pz, int nparts, int T,
@@ -204,15 +227,7 @@ __global__ __launch_bounds__(kMergeThreads) void lmhead_fwd_merge(const float* _
           ev[u] = part_pz ? part_pz[idx] : 0.f;
         }
 #pragma unroll
-        for (int u = 0; u < kBatch; ++u) {
-          if (m[u] > -INFINITY) {
-            const float Mn = fmaxf(M, m[u]);
-            const float ca = expf(M - Mn), cb = expf(m[u] - Mn);
-            S = S * ca + sv[u] * cb;
-            E = E * ca + ev[u] * cb;
-            M = Mn;
-          }
-        }
+        for (int u = 0; u < kBatch; ++u) merge_partial<RELATIVE>(M, S, E, m[u], sv[u], ev[u]);
       }
     }
     sm_m[wave][lane] = M;
@@ -220,19 +235,13 @@ __global__ __launch_bounds__(kMergeThreads) void lmhead_fwd_merge(const float* _
     sm_e[wave][lane] = E;
     __syncthreads();
     if (wave == 0) {
-      float Mg = -INFINITY;
-      for (int g = 0; g < kMergeWaves; ++g) Mg = fmaxf(Mg, sm_m[g][lane]);
-      float Sg = 0.f, Eg = 0.f;
-      for (int g = 0; g < kMergeWaves; ++g) {
-        const float m = sm_m[g][lane];
-        if (m > -INFINITY) {
-          const float c = expf(m - Mg);
-          Sg += sm_s[g][lane] * c;
-          Eg += sm_e[g][lane] * c;
-        }
-      }
-      sm_lse[lane] = Mg + logf(Sg);
-      sm_pz[lane] = Eg / Sg;
+      float Mg = -INFINITY, Sg = 0.f, Eg = 0.f;
+      for (int g = 0; g < kMergeWaves; ++g) merge_partial<RELATIVE>(Mg, Sg, Eg, sm_m[g][lane], sm_s[g][lane], sm_e[g][lane]);
+      const float log_s = logf(Sg);
+      sm_lse[lane] = Mg + log_s;
+      // RELATIVE: sm_pz holds the entropy itself, ln s - e / s, and sum p z is recovered as lse - entropy (exactly what the
+      // absolute form would have subtracted the other way round).
+      sm_pz[lane] = RELATIVE ? log_s - Eg / Sg : Eg / Sg;
     }
     __syncthreads();
   }
@@ -263,9 +272,11 @@ __global__ __launch_bounds__(kMergeThreads) void lmhead_fwd_merge(const float* _
 #pragma unroll
   for (int o = 1; o < kDotLanes; o <<= 1) dot += __shfl_xor(dot, o, 64);
   if (sub == 0 && t < T) {
-    const float lse = sm_lse[tl], pz = sm_pz[tl];
+    const float lse = sm_lse[tl];
+    const float ent = RELATIVE ? sm_pz[tl] : lse - sm_pz[tl];
+    const float pz = RELATIVE ? lse - sm_pz[tl] : sm_pz[tl];
     if (logprobs) logprobs[t] = has_label ? dot * rcp_temp - lse : 0.f;
-    if (entropy) entropy[t] = lse - pz;
+    if (entropy) entropy[t] = ent;
     if (row_lse) row_lse[t] = lse;
     if (row_pz) row_pz[t] = pz;
   }
@@ -1173,7 +1184,7 @@ int fwd_token_blocks(const void* hidden, int64_t ld_hidden, const void* weight, 
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
     Timed timed(kFwdMerge, s);
-    hipLaunchKernelGGL(lmhead_fwd_merge, dim3((unsigned)((Tb + kMergeTokens - 1) / kMergeTokens)), dim3(kMergeThreads), 0, s, pmax,
+    hipLaunchKernelGGL(lmhead_fwd_merge<true>, dim3((unsigned)((Tb + kMergeTokens - 1) / kMergeTokens)), dim3(kMergeThreads), 0, s, pmax,
                        psum, want_pz ? ppz : (float*)nullptr, (int)nparts, (int)Tb, Hp, (int)ld_hidden, Wp, (int)ld_weight,
                        labels + t0, (int)H, (int)V, rcp_temperature, logprobs + t0, entropy ? entropy + t0 : (float*)nullptr,
                        row_lse ? row_lse + t0 : (float*)nullptr, row_pz ? row_pz + t0 : (float*)nullptr);
@@ -1712,7 +1723,7 @@ int skyrl_softce_fwd(const void* student_hidden, int64_t ld_student, const void*
   if ((e = hipGetLastError()) != hipSuccess) return (int)e;
   {
     Timed timed(kFwdMerge, s);
-    hipLaunchKernelGGL(lmhead_fwd_merge, dim3((unsigned)((rows + kMergeTokens - 1) / kMergeTokens)), dim3(kMergeThreads), 0, s, w.pmax,
+    hipLaunchKernelGGL(lmhead_fwd_merge<false>, dim3((unsigned)((rows + kMergeTokens - 1) / kMergeTokens)), dim3(kMergeThreads), 0, s, w.pmax,
                        w.psum, w.ppz, (int)w.nparts, (int)rows, w.S, (int)H, Wp, (int)ld_weight, (const int64_t*)nullptr, (int)H,
                        (int)V, rcp_temperature, (float*)nullptr, (float*)nullptr, w.row_lse, w.row_pz);
   }

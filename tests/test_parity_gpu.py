@@ -1599,7 +1599,9 @@ def test_vocab_shards_reproduce_the_full_vocabulary(cuda_device):
     dh_sum = torch.zeros(T, H, dtype=torch.float32, device=dev)
     for (lo, hi), yl in zip(zip(bounds[:-1], bounds[1:]), local_labels):
         dh, dw = ops.lmhead_bwd(h, w[lo:hi].contiguous(), yl, lse, pz, gd, qd, 1.0 / t, 0)
-        torch.testing.assert_close(dw, full_dw[lo:hi], atol=2e-4, rtol=2e-3)   # same dz values up to the merged lse's rounding
+        # same dz values up to the rounding of the merged lse and sum p z: now and then one bf16 dz value lands on the other
+        # side of a rounding boundary (2^-8 of one term of the sum)
+        torch.testing.assert_close(dw, full_dw[lo:hi], atol=1e-3, rtol=5e-3)
         dh_sum += dh.float()
     assert cos(dh_sum, full_dh) >= 0.9999 and rel_l2(dh_sum, full_dh.float()) < 1e-2   # three bf16 roundings instead of one
 
@@ -2241,3 +2243,25 @@ def test_weight_gradient_in_bf16_equals_the_rounded_fp32_one(cuda_device):
     ws = torch.empty(lib.skyrl_lmhead_bwd_workspace_bytes(T, H, V, 0), dtype=torch.uint8, device=cuda_device)
     assert lib.skyrl_lmhead_bwd(p, H, w.data_ptr(), H, y.data_ptr(), lse.data_ptr(), None, gd.data_ptr(), None, T, H, V, 1.0,
                                 dh32.data_ptr(), dw32.data_ptr(), 3, 0, ws.data_ptr(), ws.numel(), None) == -5
+
+
+@pytest.mark.parametrize("temperature", [0.25, 0.1])
+def test_entropy_of_nearly_deterministic_rows(temperature, cuda_device):
+    """Low temperatures make most rows nearly deterministic: entropies of 1e-6 .. 1e-2 nats next to log-sum-exps of 50 and more.
+    lse - sum p z would lose them to cancellation in fp32 (an absolute error of 1e-5); the statistic kept relative to the
+    maximum does not: every entropy above 1e-5 nats is right to 1e-2 relative (the stated tolerance), smaller ones to 1e-7
+    absolute; the log-probabilities and both gradients are unaffected."""
+    T, H, V = 600, 256, 3000
+    hidden, weight, labels, g, q = _rand(T, H, V, seed=77)
+    out = run_hip(cuda_device, hidden, weight, labels, temperature, g, q, True, 1024)
+    ex = O.exact_fwd_bwd(hidden, weight, labels, temperature, g, q)
+    ref_ent = ex["entropy"].double()
+    assert float((ref_ent < 1e-2).float().mean()) > 0.05 and float(ref_ent.min()) < 1e-3     # the case is what it says
+    err = (out["entropy"].double() - ref_ent).abs()
+    assert float((err / ref_ent.clamp_min(1e-5)).max()) <= 1e-2, float((err / ref_ent.clamp_min(1e-5)).max())
+    assert float(err[ref_ent < 1e-5].max() if bool((ref_ent < 1e-5).any()) else 0.0) <= 1e-7
+    assert bool((out["entropy"] >= -1e-7).all())
+    # sum p z, which the backward takes back, is still lse - entropy
+    assert torch.allclose(out["pz"].double(), (ex["logprobs"].double() * 0 + out["lse"].double() - out["entropy"].double()), atol=1e-5)
+    assert (out["logprobs"].double() - ex["logprobs"].double()).abs().max().item() <= 1e-3
+    check_grads(out["d_hidden"], out["d_weight"], ex, f"t={temperature}")
