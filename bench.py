@@ -9,14 +9,20 @@ log-probabilities and the entropy).  The step goes through the C ABI (``skyrl_lm
 as the torch custom ops call it.  One JSON line is printed:
 
   value / unit   tokens per second of forward + backward (whole job; one GPU)
-  roofline       the dominant kernel (``lmhead_bwd_chunk``: logits recompute + dHidden + dWeight, 6*T*V*H of the 8*T*V*H flop)
-                 against the dense bf16 MFMA peak of 2.5 PFLOP/s; its time is measured live with HIP events on the launch stream
+  roofline       the dominant kernel (``lmhead_bwd_gemm``: the dHidden and dWeight products of every vocab chunk, 4*T*V*H of
+                 the 8*T*V*H flop and half of the step) against the dense bf16 MFMA peak of 2.5 PFLOP/s; its time is measured
+                 live with HIP events on the launch stream
   step_roofline  the whole step (8*T*V*H algorithmic flop / step time) against the same peak
   kernels        live HIP-event time per kernel and step
   cpu_baseline   the CPU restatement of the reference's torch implementation, timed on this host on a bounded sample
   mfma_probe     what the matrix pipe of this GPU sustains with the mainloop's MFMA sequence alone (operands in registers, no
                  memory access), on N(0,1) operands and on zeros: with random operands the chip is power-limited well below
                  the published peak, which bounds every bf16 kernel on this benchmark's data
+  vendor_gemm    one ``torch.matmul`` (hipBLASLt) of the same [T,H] x [V,H]^T bf16 product on the same data, HIP-event timed
+  power          board power from the driver's hwmon file while the same steps run again, next to the board's power cap
+  autograd       the same step through ``linear_cross_entropy(...)`` and ``loss.backward()`` on fresh tensors, wall-clock
+                 and peak allocated bytes (the protocol of the reference's own harness)
+The last three legs run after the timed region.
 """
 
 from __future__ import annotations
@@ -72,10 +78,21 @@ def cpu_baseline(cfg, sample_tokens: int):
     O.reference_faithful_fwd_bwd(d["hidden"], d["weight"], d["labels"], cfg.temperature, g, chunk_size=chunk,
                                  want_entropy=cfg.entropy)
     dt = time.perf_counter() - t0
+    cpu_model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    cpu_model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
     return {
         "value": sample_tokens / dt,
         "unit": "tokens/s",
         "cores": torch.get_num_threads(),
+        "cpu_model": cpu_model,
+        "torch_version": torch.__version__,
         "kind": "port",
         "sample": f"{sample_tokens} of {cfg.T} tokens at full H={cfg.H}, V={cfg.V}: logprob forward + entropy metric"
                   f"{' + backward' if cfg.backward else ''} in chunks of {chunk}, bf16 torch.matmul on CPU, {dt:.1f} s; the algorithm is a"
@@ -109,6 +126,113 @@ def mfma_probe(lib, dev):
     return out
 
 
+def vendor_gemm(hidden, weight):
+    """TFLOP/s of the vendor library on the forward's product, same operands: ``hidden @ weight.T`` in bf16 (one [T, V] bf16
+    result, allocated once and freed before returning)."""
+    import torch
+
+    T, H = hidden.shape
+    V = weight.shape[0]
+    out = torch.empty(T, V, dtype=torch.bfloat16, device=hidden.device)
+    wt = weight.t()
+    ms = []
+    for _ in range(4):  # the first call picks the algorithm
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        torch.matmul(hidden, wt, out=out)
+        e1.record()
+        torch.cuda.synchronize()
+        ms.append(e0.elapsed_time(e1))
+    del out
+    best = min(ms[1:])
+    return {"op": f"torch.matmul bf16 [{T},{H}] x [{V},{H}]^T -> bf16 [{T},{V}]", "ms": best,
+            "tflops": 2.0 * T * V * H / (best * 1e-3) / 1e12, "frac_of_peak": 2.0 * T * V * H / (best * 1e-3) / PEAK_BF16_DENSE_FLOPS}
+
+
+def _hwmon(name: str):
+    import glob
+
+    found = sorted(glob.glob(f"/sys/class/drm/card*/device/hwmon/hwmon*/{name}"))
+    return found[0] if found else None
+
+
+def power_while(step, steps: int):
+    """Average board power (W) over ``steps`` more steps, read from the amdgpu hwmon file every few milliseconds by a second
+    thread, and the board's power cap.  None when the files are not readable."""
+    import threading
+
+    import torch
+
+    path = _hwmon("power1_input") or _hwmon("power1_average")
+    cap = _hwmon("power1_cap")
+    if not path:
+        return None
+    samples, stop = [], threading.Event()
+
+    def sample():
+        while not stop.is_set():
+            try:
+                with open(path) as f:
+                    samples.append(int(f.read()) / 1e6)
+            except (OSError, ValueError):
+                pass
+            time.sleep(0.003)
+
+    for _ in range(3):  # reach the steady thermal / power state first
+        step()
+    torch.cuda.synchronize()
+    th = threading.Thread(target=sample, daemon=True)
+    th.start()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    stop.set()
+    th.join()
+    if not samples:
+        return None
+    out = {"avg_watts": sum(samples) / len(samples), "max_watts": max(samples), "samples": len(samples), "source": path}
+    if cap:
+        try:
+            with open(cap) as f:
+                out["cap_watts"] = int(f.read()) / 1e6
+        except (OSError, ValueError):
+            pass
+    return out
+
+
+def autograd_leg(cfg, hidden, weight, labels, g, q, reps: int = 3):
+    """The step as the trainer calls it, timed as skyrl/benchmarks/bench_fused_linear_logprob.py:83-108 times the reference:
+    fresh leaf tensors, ``linear_cross_entropy`` -> a scalar loss -> ``backward()``, synchronize, wall clock; median of ``reps``
+    after one warm-up, and the peak of ``torch.cuda.max_memory_allocated`` above what was allocated before the call."""
+    import torch
+
+    from skyrl_amd.fused_linear_logprob_hip import linear_cross_entropy
+
+    times, peak = [], 0
+    for it in range(reps + 1):
+        h = hidden.detach().clone().requires_grad_(True)
+        w = weight.detach().clone().requires_grad_(True)
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        base = torch.cuda.memory_allocated()
+        t0 = time.perf_counter()
+        logprobs, entropy = linear_cross_entropy(h, w, labels, float(cfg.temperature), "none", None)
+        loss = (logprobs * g).sum()
+        if q is not None:
+            loss = loss + (entropy * q).sum()
+        loss.backward()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        if it > 0:
+            times.append(dt * 1e3)
+            peak = max(peak, torch.cuda.max_memory_allocated() - base)
+        del h, w, logprobs, entropy, loss
+    times.sort()
+    return {"call": "linear_cross_entropy(hidden, weight, labels, temperature, 'none', None); (logprobs*g + entropy*q).sum().backward()",
+            "ms_per_step": times[len(times) // 2], "ms_all": times, "peak_bytes_above_inputs": int(peak),
+            "grad_weight_dtype": "bf16 (the weight's dtype, as the reference returns it)"}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -119,6 +243,8 @@ def main() -> int:
     ap.add_argument("--cpu-sample-tokens", type=int, default=6144)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-mfma-probe", action="store_true")
+    ap.add_argument("--no-extra-legs", action="store_true",
+                    help="skip the legs that run after the timed region: vendor GEMM, board power, the autograd call")
     ap.add_argument("--skip-masked-rows", action="store_true",
                     help="run the backward pass through skyrl_lmhead_bwd_active_rows, which drops the tokens whose upstream "
                          "gradients are zero on the device (the configurations with a response mask); value stays tokens/s "
@@ -224,13 +350,12 @@ def main() -> int:
                      "unit": "TFLOP/s"}
     step_roofline["frac"] = step_roofline["achieved"] / step_roofline["peak"]
 
-    # Dominant kernel: lmhead_bwd_chunk with a backward pass; forward-only workloads are all lmhead_fwd_tiles.
+    # Dominant kernel: lmhead_bwd_gemm with a backward pass (one launch per vocab chunk carries the chunk's dHidden and dWeight
+    # products: over a step 4*T*V*H flop, 2*T*V*H for a frozen LM head); forward-only workloads are all lmhead_fwd_tiles.
     if cfg.backward:
-        # lmhead_bwd_chunk: every backward launch (per vocab chunk one with the dz tiles, one with the gradient GEMM tiles);
-        # over a step the launches add up to the logits recompute, dHidden and dWeight = 6*T*V*H flop.
-        ks = [kernels[n] for n in ("lmhead_bwd_chunk[dz]", "lmhead_bwd_chunk[gemm]")]  # the same kernel, two kinds of launch
-        dom_name, dom_flop = "lmhead_bwd_chunk", 2.0 * bwd_gemms * t_active * V * H
-        dom_ms, dom_launches = sum(k["ms_per_step"] for k in ks), sum(k["launches_per_step"] for k in ks)
+        k = kernels["lmhead_bwd_gemm"]
+        dom_name, dom_flop = "lmhead_bwd_gemm", 2.0 * (bwd_gemms - 1.0) * t_active * V * H
+        dom_ms, dom_launches = k["ms_per_step"], k["launches_per_step"]
     else:
         k = kernels["lmhead_fwd_tiles"]
         dom_name, dom_ms, dom_launches, dom_flop = "lmhead_fwd_tiles", k["ms_per_step"], k["launches_per_step"], 2.0 * T * V * H
@@ -295,8 +420,8 @@ def main() -> int:
     # with nothing else in the loop (the power-limited ceiling of any bf16 kernel on this data).
     kind_flop = {"lmhead_fwd_tiles": 2.0 * T * V * H}
     if cfg.backward:
-        kind_flop["lmhead_bwd_chunk[dz]"] = 2.0 * t_active * V * H
-        kind_flop["lmhead_bwd_chunk[gemm]"] = 2.0 * (bwd_gemms - 1.0) * t_active * V * H
+        kind_flop["lmhead_bwd_dz"] = 2.0 * t_active * V * H
+        kind_flop["lmhead_bwd_gemm"] = 2.0 * (bwd_gemms - 1.0) * t_active * V * H
     probe = None if args.no_mfma_probe else mfma_probe(lib, dev)
     per_kernel = {}
     for name, fl in kind_flop.items():
@@ -308,6 +433,15 @@ def main() -> int:
     if probe:
         out["mfma_probe"] = probe
         out["step_frac_of_mfma_probe_random"] = step_roofline["achieved"] / probe["random_operands_tflops"]
+    if not args.no_extra_legs:
+        power = power_while(step, max(5, args.steps))
+        if power:
+            out["power"] = power
+        if cfg.backward and not skip and not args.frozen_lm_head:
+            del d_weight, ws_b  # the autograd call allocates its own
+            out["autograd"] = autograd_leg(cfg, hidden, weight, labels, g, q)
+            out["autograd"]["vs_c_abi_step"] = out["autograd"]["ms_per_step"] / ms_per_step
+        out["vendor_gemm"] = vendor_gemm(hidden, weight)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_sample_tokens)
     print(json.dumps(out))

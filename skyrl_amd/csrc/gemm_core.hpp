@@ -248,7 +248,7 @@ __device__ __forceinline__ void prefetch_first_tiles(const Operand& a, const Ope
 // MFMA order inside a step: mfma_row() / mfma_col() above (every fragment of the step is in registers before the step
 // starts, so the order is free to serve the power budget).
 template <bool BKM = false>
-__device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int k_begin, int nk, char* lds, acc_t& acc) {
+__device__ __forceinline__ void mainloop_ksteps(const Operand& a, const Operand& b, int k_begin, int nk, char* lds, acc_t& acc) {
   CopyPlan p;
   make_plan<BKM>(p, a, b, k_begin);
   const uint32_t b_stride = b_tile_stride<BKM>(b);
@@ -416,6 +416,204 @@ __device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j) asm volatile("" : "+a"(acc[i][j]));
+}
+
+// ---- accumulator-stationary pairs -------------------------------------------------------------------------------------
+// The same contraction with the MFMAs of a k-tile reordered so that the two k-steps of an accumulator are issued back to
+// back.  With random operands the matrix pipe is power-limited, and an MFMA that accumulates into the register the previous
+// one wrote costs less than one that switches accumulators: a loop of nothing but MFMAs runs 4 % faster in this order, the
+// kernels 2-2.5 %.  Every accumulator still receives its products in the same order (k-tile by k-tile, k-step 0 then 1), so
+// results are bit-identical to mainloop_ksteps().
+//
+// Both k-steps of an accumulator's operands must then be in registers at once.  With the same 128 fragment registers this
+// works quadrant by quadrant: the wave's 8 x 8 accumulators are four 4 x 4 quadrants; a quadrant needs one "half-set" of A
+// (4 row blocks x 2 k-steps = 8 fragments) and one of B.  There are two A slots and two B slots of 8 fragments each.  A
+// k-tile walks its quadrants in a U -- (A0,B0) (A0,B1) (A1,B1) (A1,B0) -- changing one operand per step, and each quadrant
+// loads the one half-set the next step needs into the slot that just died: 8 fragment reads per 32 MFMAs, 32 per k-tile, as
+// before.  The last quadrant of a tile still holds one A and one B slot, so the next tile starts from the other two and
+// walks the U backwards -- (A1,B0) (A1,B1) (A0,B1) (A0,B0) -- after which the first pattern fits again: tiles alternate
+// between two schedules ("even" / "odd"), fixed at compile time in kQuadPlan.  The ring of LDS slots, the copies (one
+// behind every eighth MFMA) and the single barrier per k-tile (now between the second and third quadrant: the first half of
+// a tile reads the rest of its own LDS slots, the second half the first half-sets of the next tile's) are those of
+// mainloop_ksteps().
+//
+// nk must be even and >= 2: with one fixed sequence of tile bodies (steady-state pair, then even, then odd) the
+// accumulators pass through no join of different bodies; any remainder handling by branches made the register allocator
+// move accumulators between AGPRs and VGPRs right behind the MFMAs that wrote them.  Callers pick mainloop_ksteps() for an
+// odd number of k-tiles.
+// Order of the 16 accumulators of a 4 x 4 quadrant: a zigzag inside strips of two rows.
+__host__ __device__ constexpr int quad_row(int p) { return (p / 8) * 2 + ((p % 8 + 1) / 2) % 2; }
+__host__ __device__ constexpr int quad_col(int p) { return (p / 8) % 2 ? 3 - (p % 8) / 2 : (p % 8) / 2; }
+
+// One quadrant of a k-tile: which halves of the wave's A rows / B columns it multiplies, the fragment slots that hold them,
+// and the half-set it loads meanwhile (operand, half, of this k-tile or the next, destination slot).
+struct QuadPlan {
+  int a_half, b_half, a_slot, b_slot;
+  int ld_is_b, ld_half, ld_next, ld_slot;
+};
+constexpr QuadPlan kQuadPlan[2][4] = {
+    {{0, 0, 0, 0, 1, 1, 0, 1}, {0, 1, 0, 1, 0, 1, 0, 1}, {1, 1, 1, 1, 0, 1, 1, 0}, {1, 0, 1, 0, 1, 0, 1, 1}},
+    {{1, 0, 0, 1, 1, 1, 0, 0}, {1, 1, 0, 0, 0, 0, 0, 1}, {0, 1, 1, 0, 0, 0, 1, 0}, {0, 0, 1, 1, 1, 0, 1, 0}}};
+
+template <bool BKM = false>
+__device__ __forceinline__ void mainloop_pairs(const Operand& a, const Operand& b, int k_begin, int nk, char* lds, acc_t& acc) {
+  CopyPlan p;
+  make_plan<BKM>(p, a, b, k_begin);
+  const uint32_t b_stride = b_tile_stride<BKM>(b);
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int lrow = lane & 15;
+  const int xsw = ((lane >> 4) ^ swz(lrow)) << 4;
+  const uint32_t w0 = wave_copy_base(lds);
+  const int rel = -(wave * 1024);
+  typedef const __attribute__((address_space(3))) bf16x8* frag_ptr;
+  typedef __attribute__((address_space(3))) i16x4* half_ptr;
+  constexpr int NB = BKM ? 4 : 2;  // B address registers per k-tile
+  // Lane offsets inside a slot: A (and K-contiguous B) per k-step; K-major B per column of a half (see mainloop_ksteps).
+  int a_off[2], b_off[NB];
+  a_off[0] = (wm * WM + lrow) * ROW_BYTES + xsw + rel;
+  a_off[1] = (wm * WM + lrow) * ROW_BYTES + (xsw ^ 64) + rel;
+  if constexpr (BKM) {
+    const int kq = lane >> 4, s = lane & 15, r = s >> 2;
+    const int sigma = ((r >> 1) & 1) + 2 * (kq & 1);
+    const int base = (kq * 4 + (r >> 1)) * 1024 + wn * (WN / 16) * 64 + (r & 1) * 32 + (s & 3) * 8 + rel;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) b_off[e] = base + ((e ^ sigma) * 64);
+  } else {
+    b_off[0] = (wn * WN + lrow) * ROW_BYTES + xsw + rel;
+    b_off[1] = (wn * WN + lrow) * ROW_BYTES + (xsw ^ 64) + rel;
+  }
+  constexpr int kKStepBytes = 16 * 1024;
+  constexpr int kHalfBytes = 2 * 1024;
+
+  // Fragment slots: two for A half-sets, two for B half-sets; a half-set is 4 row blocks x 2 k-steps, index r * 2 + ks.
+  bf16x8 sa[2][8], sb[2][BKM ? 1 : 8];
+  i16x4 sbh[2][BKM ? 8 : 1][2];
+  auto b_frag = [&](int slot, int f) -> bf16x8 {
+    if constexpr (BKM) {
+      typedef __attribute__((ext_vector_type(8))) short i16x8;
+      const i16x8 v = __builtin_shufflevector(sbh[slot][f][0], sbh[slot][f][1], 0, 1, 2, 3, 4, 5, 6, 7);
+      return __builtin_bit_cast(bf16x8, v);
+    } else {
+      return sb[slot][f];
+    }
+  };
+  struct Addr {
+    uint32_t a[2], b[NB];
+  };
+  constexpr int A_READS = 8, B_READS = BKM ? 16 : 8;
+  // Read instruction y of a half-set load.
+  auto read_a = [&](const Addr& ad, int half, int slot, int y) {
+    const int r = y / 2, ks = y % 2;
+    sa[slot][y] = *(frag_ptr)(uintptr_t)(ad.a[ks] + (half * 4 + r) * MT * ROW_BYTES);
+  };
+  auto read_b = [&](const Addr& ad, int half, int slot, int y) {
+    if constexpr (BKM) {
+      const int c = y / 4, ks = (y / 2) % 2, hf = y % 2;
+      const uint32_t addr = ad.b[c] + half * 256 + hf * kHalfBytes + ks * kKStepBytes;
+      sbh[slot][c * 2 + ks][hf] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((half_ptr)(uintptr_t)addr);
+    } else {
+      const int r = y / 2, ks = y % 2;
+      sb[slot][y] = *(frag_ptr)(uintptr_t)(ad.b[ks] + (half * 4 + r) * MT * ROW_BYTES);
+    }
+  };
+
+  if (nk > 1) wait_copies_and_barrier<2 * COPIES_PER_OPERAND>(); else wait_copies_and_barrier<0>();  // tile 0 has landed
+  uint32_t o0 = w0, o1 = w0 + OPERAND_BYTES, o2 = w0 + 2 * OPERAND_BYTES, o3 = w0 + 3 * OPERAND_BYTES, o4 = w0 + 4 * OPERAND_BYTES;
+  Addr X, Y;
+#pragma unroll
+  for (int e = 0; e < 2; ++e) X.a[e] = Y.a[e] = o0 + a_off[e];
+#pragma unroll
+  for (int e = 0; e < NB; ++e) X.b[e] = Y.b[e] = o1 + b_off[e];
+#pragma unroll
+  for (int y = 0; y < A_READS; ++y) read_a(X, 0, 0, y);
+#pragma unroll
+  for (int y = 0; y < B_READS; ++y) read_b(X, 0, 0, y);
+
+  auto pinned_add = [](uint32_t slot_off, int lane_off) {
+    uint32_t r;
+    asm volatile("v_add_u32_e32 %0, %1, %2" : "=v"(r) : "s"(slot_off), "v"(lane_off));
+    return r;
+  };
+  const char* ga = p.a_bytes + 2 * (BK * 2);
+  const char* gb = p.b_bytes + 2 * (size_t)b_stride;
+
+  // One k-tile = four quadrants of 32 MFMAs.  cur: fragment addresses of this k-tile's slots, nxt: of the next k-tile's
+  // (formed here, in MFMA shadows of the first half; they are this tile's second-half addresses and the next tile's cur).
+  auto tile_step = [&](auto par, auto has_next, auto load2, Addr& cur, Addr& nxt) {
+    constexpr int PAR = decltype(par)::value;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      constexpr QuadPlan const* plans = kQuadPlan[PAR];
+      const QuadPlan pl = plans[q];
+      if (q == 2 && has_next) {
+        if (load2) wait_copies_and_barrier<COPIES_PER_OPERAND>();  // A(kt+2) may still be in flight
+        else wait_copies_and_barrier<0>();
+      }
+      const bool do_load = q < 2 || has_next;
+      const int nreads = pl.ld_is_b ? B_READS : A_READS;
+#pragma unroll
+      for (int pos = 0; pos < 32; ++pos) {
+        const int pr = pos / 2, ks = pos % 2;
+        const int r = quad_row(pr), c = quad_col(pr);
+        mfma_16x16x32(acc[pl.a_half * 4 + r][pl.b_half * 4 + c], sa[pl.a_slot][r * 2 + ks], b_frag(pl.b_slot, c * 2 + ks));
+        __builtin_amdgcn_sched_barrier(0);
+        if (do_load && pos % 2 == 0 && pos / 2 < nreads) {
+          if (pl.ld_is_b) read_b(pl.ld_next ? nxt : cur, pl.ld_half, pl.ld_slot, pos / 2);
+          else read_a(pl.ld_next ? nxt : cur, pl.ld_half, pl.ld_slot, pos / 2);
+        }
+        if (load2 && pos % 8 == 5) {
+          if (q < 2) copy_part(ga, p.a_src, o4, q * 4 + pos / 8, 1);
+          else copy_part(gb, p.b_src, o0, (q - 2) * 4 + pos / 8, 1);
+        }
+        if (load2 && pos == 31 && q == 1) {
+          ga += BK * 2;
+          asm volatile("" : "+s"(ga));
+        }
+        if (load2 && pos == 31 && q == 3) {
+          gb += b_stride;
+          asm volatile("" : "+s"(gb));
+        }
+        if (has_next && q == 0) {  // next k-tile's fragment addresses, one add per MFMA shadow, in gaps without a read or a copy
+          if (pos == 1) nxt.a[0] = pinned_add(o2, a_off[0]);
+          if (pos == 3) nxt.a[1] = pinned_add(o2, a_off[1]);
+          if (pos == 7) nxt.b[0] = pinned_add(o3, b_off[0]);
+          if (pos == 9) nxt.b[1] = pinned_add(o3, b_off[1]);
+          if (NB == 4 && pos == 11) nxt.b[NB - 2] = pinned_add(o3, b_off[NB - 2]);
+          if (NB == 4 && pos == 15) nxt.b[NB - 1] = pinned_add(o3, b_off[NB - 1]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    const uint32_t t0 = o0, t1 = o1;
+    o0 = o2, o1 = o3, o2 = o4, o3 = t0, o4 = t1;
+  };
+  std::integral_constant<int, 0> even;
+  std::integral_constant<int, 1> odd;
+  std::true_type yes;
+  std::false_type no;
+  // nk is even: tiles alternate even, odd and the sequence is a straight line.
+  for (int kt = 0; kt + 3 < nk; kt += 2) {
+    tile_step(even, yes, yes, X, Y);
+    tile_step(odd, yes, yes, Y, X);
+  }
+  tile_step(even, yes, no, X, Y);
+  tile_step(odd, no, no, Y, X);
+  wait_copies_and_barrier<0>();
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) asm volatile("" : "+a"(acc[i][j]));
+}
+
+// The mainloop of a tile: EVEN_NK (the caller guarantees an even number of k-tiles, at least two) takes the
+// accumulator-stationary order, anything else the k-step order.  Both leave identical accumulators.
+template <bool BKM = false, bool EVEN_NK = false>
+__device__ __forceinline__ void mainloop(const Operand& a, const Operand& b, int k_begin, int nk, char* lds, acc_t& acc) {
+  if constexpr (EVEN_NK) mainloop_pairs<BKM>(a, b, k_begin, nk, lds, acc);
+  else mainloop_ksteps<BKM>(a, b, k_begin, nk, lds, acc);
 }
 
 // Work item id -> tile coordinates.

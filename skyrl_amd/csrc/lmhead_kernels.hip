@@ -9,10 +9,11 @@
 //                      fp32 dot product hidden[t] . weight[label], writes logprob / entropy / lse / pz.
 // Backward (6*T*V*H flop), looped over vocab chunks of `vocab_chunk` columns:
 //   transpose_bf16     hidden^T once per call (and weight^T only when V is not a multiple of 64).
-//   lmhead_bwd_chunk   dz tiles: recompute a logits tile, form dz in registers and write it (bf16) into one token-major
-//                      panel of the chunk.  GEMM tiles: dHidden (+)= dz . weight and dW[chunk] = dz^T . hidden with fp32
-//                      accumulation, both from that panel -- dW reads it K-major, dHidden reads the weight K-major in
-//                      place -- through the transposing LDS read (gemm_core.hpp).
+//   lmhead_bwd_dz      recompute a logits tile, form dz in registers and write it (bf16) into one token-major panel of
+//                      the chunk.
+//   lmhead_bwd_gemm    dHidden (+)= dz . weight and dW[chunk] = dz^T . hidden with fp32 accumulation, both from that
+//                      panel -- dW reads it K-major, dHidden reads the weight K-major in place -- through the transposing
+//                      LDS read (gemm_core.hpp).
 // Soft cross-entropy of a draft head against the policy (10*T*V*H flop): softce_pack_rows stacks the two hidden rows of every
 //   token, softce_fwd_tiles is the forward tile with a paired third statistic, softce_dz_tiles the matching dz producer; merge
 //   and dHidden GEMM are the kernels above.
@@ -40,11 +41,16 @@ constexpr float kLn2 = 0.6931471805599453f;
 #define LMHEAD_GROUP_M 4  // measured best of 2, 4, 6, 8, 16, 32 on both passes
 #endif
 constexpr int kGroupM = LMHEAD_GROUP_M;
+#ifndef LMHEAD_DZ_FLUSH_LOG2
+#define LMHEAD_DZ_FLUSH_LOG2 0
+#endif
 // Scratch matrices get 64 extra elements (128 B) per row: with a power-of-two row pitch (T' = 16384 -> 32 KiB) the 256 rows of
 // an operand tile would all start in the same L2 channel and set.
 constexpr int kLdPad = 64;
 
 __host__ __device__ inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+// An even number of k-tiles selects the accumulator-stationary mainloop (the EVEN instantiation of a tile kernel).
+inline bool even_ktiles(int64_t contraction) { return (contraction / BK) % 2 == 0; }
 
 // Scratch of skyrl_lmhead_fwd_static_scratch, the entry point for callers that cannot allocate: one fixed array in every
 // device's memory, held until the process ends.  In host code this name is only a handle for hipGetSymbolAddress (see
@@ -116,7 +122,8 @@ __device__ __forceinline__ void fwd_tile_stats(const acc_t& acc, int j, int vbas
   e_out = PAIRED ? e * scale2 * kLn2 : e * kLn2;
 }
 
-template <bool ENTROPY, bool PAIRED>
+// EVEN: H / 64 is even, which selects the accumulator-stationary mainloop (gemm_core.hpp).
+template <bool ENTROPY, bool PAIRED, bool EVEN>
 __device__ __forceinline__ void fwd_tile(const uint16_t* __restrict__ W, int ldw, const uint16_t* __restrict__ Hd, int ldh, int T,
                                          int H, int V, float rcp_temp, float* __restrict__ part_max,
                                          float* __restrict__ part_sum, float* __restrict__ part_pz, char* lds) {
@@ -130,7 +137,7 @@ __device__ __forceinline__ void fwd_tile(const uint16_t* __restrict__ W, int ldw
   acc_t acc;
   zero_acc(acc);
   prefetch_first_tiles(a, b, 0, H / BK, lds);
-  mainloop(a, b, 0, H / BK, lds, acc);
+  mainloop<false, EVEN>(a, b, 0, H / BK, lds, acc);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
@@ -156,13 +163,13 @@ __device__ __forceinline__ void fwd_tile(const uint16_t* __restrict__ W, int ldw
   }
 }
 
-template <bool ENTROPY>
+template <bool ENTROPY, bool EVEN>
 __global__ __launch_bounds__(NTHREADS) void lmhead_fwd_tiles(const uint16_t* __restrict__ W, int ldw,
                                                              const uint16_t* __restrict__ Hd, int ldh, int T, int H, int V,
                                                              float rcp_temp, float* __restrict__ part_max,
                                                              float* __restrict__ part_sum, float* __restrict__ part_pz) {
   __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
-  fwd_tile<ENTROPY, false>(W, ldw, Hd, ldh, T, H, V, rcp_temp, part_max, part_sum, part_pz, lds);
+  fwd_tile<ENTROPY, false, EVEN>(W, ldw, Hd, ldh, T, H, V, rcp_temp, part_max, part_sum, part_pz, lds);
 }
 
 // ------------------------------------------------------------------------------------------------------------
@@ -315,7 +322,7 @@ struct DzArgs {
   float* label_resid;
 };
 
-template <bool ENTGRAD>
+template <bool ENTGRAD, bool EVEN>
 __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
   const uint16_t* __restrict__ W = z.W;
   const uint16_t* __restrict__ Hd = z.Hd;
@@ -361,6 +368,17 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
     gs_[j] = g * rcp_temp;
     c0_[j] = -(g - q * pz) * rcp_temp;
     c1_[j] = -q * rcp_temp * rcp_temp;
+#if LMHEAD_DZ_FLUSH_LOG2
+    // Probabilities below 2^-LMHEAD_DZ_FLUSH_LOG2 count as zero: the exponent is moved down so that v_exp_f32 -- which
+    // returns 0 where the result would be a denormal, below 2^-126 -- does the flush, and the two coefficients carry
+    // the power of two back (exact).  Not for coefficients so large that the scaled ones could overflow.
+    if (fabsf(c0_[j]) < 0x1p30f && fabsf(c1_[j]) < 0x1p20f) {
+      constexpr float kShift = 126.f - LMHEAD_DZ_FLUSH_LOG2;
+      lse2_[j] += kShift;
+      c0_[j] *= __builtin_exp2f(kShift);
+      c1_[j] *= __builtin_exp2f(kShift);
+    }
+#endif
   }
 
   Operand a{W, ldw, vc0 + tm * BM, V};
@@ -368,7 +386,7 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
   acc_t acc;
   zero_acc(acc);
   prefetch_first_tiles(a, b, 0, H / BK, lds);
-  mainloop(a, b, 0, H / BK, lds, acc);
+  mainloop<false, EVEN>(a, b, 0, H / BK, lds, acc);
 
   // The wave's 128 x 128 dz block leaves through LDS so that the panel is written with 16-byte stores: a lane holds four
   // consecutive vocab rows of one token, an 8-byte piece of a D row.  mainloop() left LDS free and every wave uses a
@@ -475,13 +493,13 @@ __global__ __launch_bounds__(256) void softce_pack_rows(const uint16_t* __restri
     *(uint4*)(dst + c) = src ? *(const uint4*)(src + c) : make_uint4(0, 0, 0, 0);
 }
 
-template <bool ENTROPY>
+template <bool ENTROPY, bool EVEN>
 __global__ __launch_bounds__(NTHREADS) void softce_fwd_tiles(const uint16_t* __restrict__ W, int ldw,
                                                              const uint16_t* __restrict__ Hd, int ldh, int T, int H, int V,
                                                              float rcp_temp, float* __restrict__ part_max,
                                                              float* __restrict__ part_sum, float* __restrict__ part_pz) {
   __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
-  fwd_tile<ENTROPY, true>(W, ldw, Hd, ldh, T, H, V, rcp_temp, part_max, part_sum, part_pz, lds);
+  fwd_tile<ENTROPY, true, EVEN>(W, ldw, Hd, ldh, T, H, V, rcp_temp, part_max, part_sum, part_pz, lds);
 }
 
 // Per token: the merged statistics of its two stacked rows -> loss and the two log-sum-exps the backward needs.
@@ -511,6 +529,7 @@ struct SoftCeDzArgs {
   int ldd;
 };
 
+template <bool EVEN>
 __global__ __launch_bounds__(NTHREADS) void softce_dz_tiles(const SoftCeDzArgs z) {
   __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
   const uint16_t* __restrict__ W = z.W;
@@ -544,7 +563,7 @@ __global__ __launch_bounds__(NTHREADS) void softce_dz_tiles(const SoftCeDzArgs z
   acc_t acc;
   zero_acc(acc);
   prefetch_first_tiles(a, b, 0, H / BK, lds);
-  mainloop(a, b, 0, H / BK, lds, acc);
+  mainloop<false, EVEN>(a, b, 0, H / BK, lds, acc);
 
   // Staging as in dz_tile: a private region per wave, 64 token rows of 128 vocab columns, then 16-byte non-temporal stores.
   constexpr int kTokRow = WM * 2 + 16;
@@ -631,7 +650,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, int bid, char* lds)
     const int count = __builtin_amdgcn_readfirstlane(*p.T_dev);
     if (p.t_role == kTokensOnM) M = count;
     else if (p.t_role == kTokensOnN) N = count;
-    else nk = (count + BK - 1) / BK;
+    else nk = (count + 2 * BK - 1) / (2 * BK) * 2;  // whole pairs of k-tiles: the rows up to the next multiple of 256 are zeros
     // Nothing to contract: C += 0 needs no work; a C that is overwritten or converted still goes through the epilogue.
     if (nk == 0 && !p.Cb && p.Cin == p.Cf) return;
   }
@@ -649,7 +668,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, int bid, char* lds)
   zero_acc(acc);
   if (nk > 0) {
     prefetch_first_tiles<BKM>(a, b, 0, nk, lds);
-    mainloop<BKM>(a, b, 0, nk, lds, acc);
+    mainloop<BKM, true>(a, b, 0, nk, lds, acc);  // nk is even for every gradient GEMM (make_gemm checks)
   }
 
   const float* __restrict__ Cin = p.Cin;
@@ -722,22 +741,22 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, int bid, char* lds)
   }
 }
 
-// One kernel for both kinds of backward tile: workgroups [0, gemm_tiles) run gradient GEMM tiles, the rest dz tiles.
-// The host launches it twice per vocab chunk: dz tiles only (gemm_tiles == 0), then the two GEMMs (grid == gemm_tiles).
-template <bool ENTGRAD>
-__global__ __launch_bounds__(NTHREADS) void lmhead_bwd_chunk(const DzArgs z, const GemmArgs p0, const GemmArgs p1, int tiles0,
-                                                             int gemm_tiles) {
+// The two kinds of backward launch per vocab chunk, as kernels of their own so that a kernel trace tells them apart:
+// the dz tiles of the chunk, then its two gradient GEMMs in one launch (workgroups [0, tiles0) work on p0, the rest on p1).
+template <bool ENTGRAD, bool EVEN>
+__global__ __launch_bounds__(NTHREADS) void lmhead_bwd_dz(const DzArgs z) {
+  __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
+  dz_tile<ENTGRAD, EVEN>(z, blockIdx.x, lds);
+}
+
+__global__ __launch_bounds__(NTHREADS) void lmhead_bwd_gemm(const GemmArgs p0, const GemmArgs p1, int tiles0) {
   __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
   const int id = blockIdx.x;
   // dW always reads the dz panel K-major (K = tokens); dHidden either reads the weight itself K-major (K = vocab) or,
-  // when the vocabulary is not a multiple of the k-tile, a transposed, zero-padded copy of it with K contiguous.
+  // when the vocabulary is not a multiple of two k-tiles, a transposed, zero-padded copy of it with K contiguous.
   const bool second = id >= tiles0;
-  if (id < gemm_tiles) {
-    if (second || p0.b_kmajor) gemm_tile<true>(second ? p1 : p0, second ? id - tiles0 : id, lds);
-    else gemm_tile<false>(p0, id, lds);
-  } else {
-    dz_tile<ENTGRAD>(z, id - gemm_tiles, lds);
-  }
+  if (second || p0.b_kmajor) gemm_tile<true>(second ? p1 : p0, second ? id - tiles0 : id, lds);
+  else gemm_tile<false>(p0, id, lds);
 }
 
 // Measurement aid: the mainloop's MFMA sequence (two 32-k steps of 64 MFMAs, same order, accumulators in AGPRs) with
@@ -990,7 +1009,7 @@ enum KernelKind {
   kNumKernelKinds
 };
 const char* const kKernelNames[kNumKernelKinds] = {"lmhead_fwd_tiles", "lmhead_fwd_merge", "transpose_bf16",
-                                                   "lmhead_bwd_chunk[dz]", "lmhead_bwd_chunk[gemm]", "softce_pack_rows",
+                                                   "lmhead_bwd_dz", "lmhead_bwd_gemm", "softce_pack_rows",
                                                    "softce_fwd_tiles", "softce_finish", "softce_dz_tiles",
                                                    "active_rows[compact+gather+scatter]", "split_operand_rows",
                                                    "topk_filter_tiles", "topk_select", "topk_softce_rows",
@@ -1174,12 +1193,10 @@ int fwd_token_blocks(const void* hidden, int64_t ld_hidden, const void* weight, 
     const dim3 grid((unsigned)(tiles_m * tiles_n)), block(NTHREADS);
     {
       Timed timed(kFwdTiles, s);
-      if (want_pz)
-        hipLaunchKernelGGL(lmhead_fwd_tiles<true>, grid, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)Tb, (int)H,
-                           (int)V, rcp_temperature, pmax, psum, ppz);
-      else
-        hipLaunchKernelGGL(lmhead_fwd_tiles<false>, grid, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)Tb, (int)H,
-                           (int)V, rcp_temperature, pmax, psum, ppz);
+      auto kernel = want_pz ? (even_ktiles(H) ? lmhead_fwd_tiles<true, true> : lmhead_fwd_tiles<true, false>)
+                            : (even_ktiles(H) ? lmhead_fwd_tiles<false, true> : lmhead_fwd_tiles<false, false>);
+      hipLaunchKernelGGL(kernel, grid, block, 0, s, Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)Tb, (int)H, (int)V,
+                         rcp_temperature, pmax, psum, ppz);
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
@@ -1232,10 +1249,10 @@ struct BwdWorkspace {
   size_t bytes;
 };
 
-// The dHidden GEMM contracts over the vocabulary.  When V is a multiple of the k-tile it reads the weight rows where they
-// are (K-major B operand); otherwise the last k-tile would reach past the weight's last row, and a transposed copy,
-// zero-padded to whole tiles, is made in the workspace instead.
-inline bool reads_weight_in_place(int64_t V) { return V % BK == 0; }
+// The dHidden GEMM contracts over the vocabulary.  When V is a multiple of two k-tiles (the gradient GEMMs run whole pairs
+// of k-tiles) it reads the weight rows where they are (K-major B operand); otherwise the last pair would reach past the
+// weight's last row, and a transposed copy, zero-padded to whole tiles, is made in the workspace instead.
+inline bool reads_weight_in_place(int64_t V) { return V % (2 * BK) == 0; }
 
 inline int64_t bwd_block_tokens(int64_t T) { return T < kBwdTokenBlock ? T : kBwdTokenBlock; }
 inline int64_t bwd_num_blocks(int64_t T) { return (T + kBwdTokenBlock - 1) / kBwdTokenBlock; }
@@ -1277,17 +1294,27 @@ GemmArgs make_gemm(const uint16_t* A, int64_t lda, int64_t a_rows, const uint16_
 
 unsigned gemm_tiles(const GemmArgs& g) { return (unsigned)(((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN)); }
 
-// gemm == false: dz tiles only; dz_tiles == 0: GEMM tiles only.
-hipError_t launch_bwd_chunk(hipStream_t s, bool entgrad, const DzArgs& z, unsigned dz_tiles, bool gemm, const GemmArgs& p0,
-                            const GemmArgs& p1) {
-  const unsigned t0 = gemm ? gemm_tiles(p0) : 0, t1 = gemm ? gemm_tiles(p1) : 0;
-  Timed timed(gemm ? kBwdChunkGemm : kBwdChunkDz, s);
-  if (entgrad)
-    hipLaunchKernelGGL(lmhead_bwd_chunk<true>, dim3(t0 + t1 + dz_tiles), dim3(NTHREADS), 0, s, z, p0, p1, (int)t0,
-                       (int)(t0 + t1));
-  else
-    hipLaunchKernelGGL(lmhead_bwd_chunk<false>, dim3(t0 + t1 + dz_tiles), dim3(NTHREADS), 0, s, z, p0, p1, (int)t0,
-                       (int)(t0 + t1));
+hipError_t launch_bwd_dz(hipStream_t s, bool entgrad, const DzArgs& z, unsigned dz_tiles) {
+  Timed timed(kBwdChunkDz, s);
+  const bool even = even_ktiles(z.H);
+  const dim3 grid(dz_tiles), block(NTHREADS);
+  if (entgrad) {
+    if (even) hipLaunchKernelGGL((lmhead_bwd_dz<true, true>), grid, block, 0, s, z);
+    else hipLaunchKernelGGL((lmhead_bwd_dz<true, false>), grid, block, 0, s, z);
+  } else {
+    if (even) hipLaunchKernelGGL((lmhead_bwd_dz<false, true>), grid, block, 0, s, z);
+    else hipLaunchKernelGGL((lmhead_bwd_dz<false, false>), grid, block, 0, s, z);
+  }
+  return hipGetLastError();
+}
+
+// Both problems (p1 may be empty) must have an even number of k-tiles: every caller contracts over padded extents that
+// are multiples of 256, or over vocabulary rows that reads_weight_in_place() admits.
+hipError_t launch_bwd_gemm(hipStream_t s, const GemmArgs& p0, const GemmArgs& p1) {
+  if ((p0.nk & 1) || (p1.nk & 1)) return hipErrorInvalidValue;
+  const unsigned t0 = gemm_tiles(p0), t1 = gemm_tiles(p1);
+  Timed timed(kBwdChunkGemm, s);
+  hipLaunchKernelGGL(lmhead_bwd_gemm, dim3(t0 + t1), dim3(NTHREADS), 0, s, p0, p1, (int)t0);
   return hipGetLastError();
 }
 
@@ -1427,7 +1454,7 @@ int bwd_token_block(const uint16_t* Hp, int64_t ld_hidden, const uint16_t* Wp, i
     const int64_t vc0 = ci * vc, vcw = chunk_width(ci);
     const DzArgs z{Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)Tb, (int)Hk, (int)V, rcp_temperature, labels, row_lse, row_pz,
                    dlogprobs, dentropy, (int)vc0, (int)(vcw / 256), tiles_t, w.D, (int)(vcw + kLdPad), T_dev, resid};
-    e = launch_bwd_chunk(s, dentropy != nullptr, z, (unsigned)(vcw / 256 * tiles_t), false, none, none);
+    e = launch_bwd_dz(s, dentropy != nullptr, z, (unsigned)(vcw / 256 * tiles_t));
     if (e != hipSuccess) return (int)e;
     // dHidden[t, h] (+)= sum_v D[t, v] . weight^T[h, vc0 + v]        (A = weight^T rows at k offset vc0, B = D rows)
     // dW[vc0 + v, h]  (+)= sum_t D[t, v] . hidden^T[h, t]             (A = hidden^T rows, B = D read K-major)
@@ -1453,7 +1480,7 @@ int bwd_token_block(const uint16_t* Hp, int64_t ld_hidden, const uint16_t* Wp, i
                                             dw_bf16 ? dw_bf16 + dw_off : (uint16_t*)nullptr, H, nullptr, nullptr, T_dev,
                                             kTokensOnK)
                                 : none;
-    e = launch_bwd_chunk(s, dentropy != nullptr, DzArgs{}, 0, true, gh, gw);
+    e = launch_bwd_gemm(s, gh, gw);
     if (e != hipSuccess) return (int)e;
   }
   if (resid) {
@@ -1717,8 +1744,9 @@ int skyrl_softce_fwd(const void* student_hidden, int64_t ld_student, const void*
   const int tiles_m = (int)((V + BM - 1) / BM), tiles_n = (int)(rows / BN);
   {
     Timed timed(kSoftCeFwdTiles, s);
-    hipLaunchKernelGGL(softce_fwd_tiles<true>, dim3((unsigned)(tiles_m * tiles_n)), dim3(NTHREADS), 0, s, Wp, (int)ld_weight, w.S,
-                       (int)H, (int)rows, (int)H, (int)V, rcp_temperature, w.pmax, w.psum, w.ppz);
+    auto kernel = even_ktiles(H) ? softce_fwd_tiles<true, true> : softce_fwd_tiles<true, false>;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(tiles_m * tiles_n)), dim3(NTHREADS), 0, s, Wp, (int)ld_weight, w.S, (int)H,
+                       (int)rows, (int)H, (int)V, rcp_temperature, w.pmax, w.psum, w.ppz);
   }
   if ((e = hipGetLastError()) != hipSuccess) return (int)e;
   {
@@ -1773,7 +1801,8 @@ int skyrl_softce_bwd(const void* student_hidden, int64_t ld_student, const void*
                          dloss, (int)vc0, (int)(vcw / 256), (int)(2 * Tp / BN), w.D, (int)(vcw + kLdPad)};
     {
       Timed timed(kSoftCeDz, s);
-      hipLaunchKernelGGL(softce_dz_tiles, dim3((unsigned)(z.tiles_m * z.tiles_n)), dim3(NTHREADS), 0, s, z);
+      auto kernel = even_ktiles(H) ? softce_dz_tiles<true> : softce_dz_tiles<false>;
+      hipLaunchKernelGGL(kernel, dim3((unsigned)(z.tiles_m * z.tiles_n)), dim3(NTHREADS), 0, s, z);
     }
     if ((e = hipGetLastError()) != hipSuccess) return (int)e;
     // d student hidden [t, h] (+)= sum_v D[t, v] . weight[vc0 + v, h]: the dHidden GEMM of the log-probability backward,
@@ -1788,7 +1817,7 @@ int skyrl_softce_bwd(const void* student_hidden, int64_t ld_student, const void*
                                H, nullptr, nullptr, dh_out, H, dh_in, dh_keep)
                    : make_gemm(w.Wt + vc0, Vpad + kLdPad, H, w.D, vcw + kLdPad, Tp, false, false, vcw / BK, H, T, nullptr,
                                nullptr, dh_out, H, dh_in, dh_keep);
-    e = launch_bwd_chunk(s, false, DzArgs{}, 0, true, gh, none);
+    e = launch_bwd_gemm(s, gh, none);
     if (e != hipSuccess) return (int)e;
   }
   return SKYRL_LMHEAD_OK;
@@ -1833,7 +1862,8 @@ int skyrl_lmhead_topk_logits(const void* hidden, int64_t ld_hidden, const void* 
                          (int)w.cap};
       {
         Timed timed(kTopkFilter, s);
-        hipLaunchKernelGGL(topk::topk_filter_tiles, dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(NTHREADS), 0, s, a);
+        auto kernel = even_ktiles(H) ? topk::topk_filter_tiles<true> : topk::topk_filter_tiles<false>;
+        hipLaunchKernelGGL(kernel, dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(NTHREADS), 0, s, a);
       }
       if ((e = hipGetLastError()) != hipSuccess) return (int)e;
       {

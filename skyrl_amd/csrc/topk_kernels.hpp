@@ -56,6 +56,7 @@ struct FilterArgs {
   int cap;             // >= columns of a chunk, so that a list cannot overflow
 };
 
+template <bool EVEN>
 __global__ __launch_bounds__(NTHREADS) void topk_filter_tiles(const FilterArgs a) {
   __shared__ __attribute__((aligned(1024))) char lds[LDS_BYTES];
   int tm, tn;
@@ -66,7 +67,7 @@ __global__ __launch_bounds__(NTHREADS) void topk_filter_tiles(const FilterArgs a
   acc_t acc;
   zero_acc(acc);
   prefetch_first_tiles(oa, ob, 0, a.H / BK, lds);
-  mainloop(oa, ob, 0, a.H / BK, lds, acc);
+  mainloop<false, EVEN>(oa, ob, 0, a.H / BK, lds, acc);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;

@@ -51,7 +51,7 @@ def kernels(tmp_path_factory):
 
 def test_mfma_kernels_found(kernels):
     names = " ".join(kernels)
-    for expect in ("lmhead_fwd_tiles", "lmhead_bwd_chunk", "mfma_probe"):
+    for expect in ("lmhead_fwd_tiles", "lmhead_bwd_dz", "lmhead_bwd_gemm", "mfma_probe"):
         assert expect in names, f"no MFMA kernel named *{expect}* in the assembly: {list(kernels)}"
 
 
