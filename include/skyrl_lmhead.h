@@ -40,7 +40,7 @@ extern "C" {
 
 #define SKYRL_LMHEAD_OK 0
 #define SKYRL_LMHEAD_ERR_NULL (-1)      /* a required pointer is NULL, or only some of seg_row / seg_col / seg_len are given */
-#define SKYRL_LMHEAD_ERR_SHAPE (-2)     /* T, V < 1, H not a positive multiple of 64, a leading dimension < H, a weight (or a 32768-token block of hidden rows) of 4 GiB or more, a negative count */
+#define SKYRL_LMHEAD_ERR_SHAPE (-2)     /* T, V < 1, H not a positive multiple of 64, a leading dimension < H or > 4194304 elements, a negative count */
 #define SKYRL_LMHEAD_ERR_ALIGN (-3)     /* a pointer is not 16-byte aligned or a leading dimension is not a multiple of 8 */
 #define SKYRL_LMHEAD_ERR_WORKSPACE (-4) /* workspace is NULL or smaller than the matching *_workspace_bytes() */
 #define SKYRL_LMHEAD_ERR_TOO_LARGE (-6) /* skyrl_lmhead_fwd_static_scratch only: V beyond SKYRL_LMHEAD_STATIC_SCRATCH_MAX_V */

@@ -96,7 +96,7 @@ struct Operand {
   const uint16_t* ptr;  // bf16 bits, row-major, K contiguous
   int ld;               // elements between rows (multiple of 8)
   int row0;             // first row of this tile
-  int rows;             // total valid rows; rows past the end are clamped (their results are masked later)
+  int rows;             // total valid rows (> row0); rows past the end are clamped (their results are masked later)
 };
 // A B operand may instead be "K-major": the same matrix stored transposed, ptr[k * ld + n], so that a 16-byte chunk
 // holds eight consecutive n of one k (what a producer writes when n is its contiguous axis).  Then row0 is the first
@@ -124,8 +124,9 @@ __device__ __forceinline__ void wait_copies_and_barrier() {
 // One MFMA, accumulating in place in AGPRs.  Written as inline assembly because the register allocator, given 64
 // separate four-register accumulators through the builtin, rotates them through the loop (MFMA destination != source)
 // and repairs the permutation with hundreds of v_accvgpr moves per iteration.  The compiler does not know this is an
-// MFMA, so the two hazards it would otherwise pad are handled by construction: an accumulator is reused only after
-// 63 other MFMAs, and mainloop() ends with explicit wait states before anything reads the accumulators.
+// MFMA, so the hazards it would otherwise pad are handled by construction: an MFMA that reads as its C operand exactly the
+// registers the previous MFMA wrote is interlocked by the hardware (that is what mainloop_pairs() issues back to back), and
+// every mainloop ends with explicit wait states before anything else reads the accumulators.
 __device__ __forceinline__ void mfma_16x16x32(f32x4& c, const bf16x8& a, const bf16x8& b) {
   asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
@@ -149,8 +150,11 @@ __device__ __forceinline__ void zero_acc(acc_t& acc) {
 
 // Per-lane plan of the global->LDS copies of one output tile: which global 16-byte chunk lands in which LDS chunk.
 // One copy instruction of one wave fills 64 consecutive 16-byte chunks of a slot (8 rows); the lane picks the global
-// chunk whose swizzled home is its LDS chunk.  Offsets are 32-bit byte offsets from the operand base (operands are
-// smaller than 4 GiB, checked on the host); the k offset is added to the uniform base pointer.
+// chunk whose swizzled home is its LDS chunk.  Offsets are 32-bit byte offsets from the tile's first row (K-contiguous
+// operand) or first column (K-major operand), which the 64-bit uniform base pointer carries together with the k offset:
+// an operand may be of any size as long as 256 of its rows (64 for a K-major one) span less than 4 GiB, i.e. its row
+// pitch stays below kMaxRowPitch elements (checked on the host).
+constexpr int64_t kMaxRowPitch = (int64_t)1 << 22;  // elements: 256 rows of 8 MiB are 2 GiB of 32-bit offsets
 struct CopyPlan {
   const char* a_bytes;
   const char* b_bytes;
@@ -166,24 +170,26 @@ __device__ __forceinline__ void make_plan(CopyPlan& p, const Operand& a, const O
     const int c = (j * NWAVES + wave) * 64 + lane;  // chunk index inside the slot
     const int row = c >> 3;
     const int kc = (c & 7) ^ swz(row);
-    int ga = a.row0 + row;
-    ga = ga < a.rows ? ga : a.rows - 1;
-    p.a_src[j] = (uint32_t)ga * (uint32_t)a.ld * 2u + (uint32_t)(kc * 16);
+    int ra = a.row0 + row < a.rows ? row : a.rows - 1 - a.row0;  // row inside the tile; rows past the end re-read the last one
+    p.a_src[j] = (uint32_t)ra * (uint32_t)a.ld * 2u + (uint32_t)(kc * 16);
     if (BKM) {
       const int block = j * NWAVES + wave;             // rows 2 * block, 2 * block + 1 of the k-tile
       const int q = (lane >> 2) ^ kmajor_sigma(block);  // the pair whose home is this lane's window
       const int krow = 2 * block + ((lane >> 1) & 1);
-      int n = b.row0 + q * 16 + (lane & 1) * 8;
-      n = n < b.rows - 8 ? n : b.rows - 8;
+      int n = q * 16 + (lane & 1) * 8;  // column inside the tile
+      n = b.row0 + n < b.rows - 8 ? n : b.rows - 8 - b.row0;
       p.b_src[j] = (uint32_t)krow * (uint32_t)b.ld * 2u + (uint32_t)(n * 2);
     } else {
-      int gb = b.row0 + row;
-      gb = gb < b.rows ? gb : b.rows - 1;
-      p.b_src[j] = (uint32_t)gb * (uint32_t)b.ld * 2u + (uint32_t)(kc * 16);
+      int rb = b.row0 + row < b.rows ? row : b.rows - 1 - b.row0;
+      p.b_src[j] = (uint32_t)rb * (uint32_t)b.ld * 2u + (uint32_t)(kc * 16);
     }
   }
-  p.a_bytes = (const char*)a.ptr + (size_t)k_begin * 2;
-  p.b_bytes = (const char*)b.ptr + (BKM ? (size_t)k_begin * (size_t)b.ld * 2 : (size_t)k_begin * 2);
+  // The tile origins are wave-uniform, but they come out of integer divisions that the compiler runs on the vector unit:
+  // readfirstlane puts them (and with them the two base pointers) back into scalar registers.
+  const size_t a_row0 = (size_t)__builtin_amdgcn_readfirstlane(a.row0), b_row0 = (size_t)__builtin_amdgcn_readfirstlane(b.row0);
+  p.a_bytes = (const char*)a.ptr + (a_row0 * (size_t)a.ld + (size_t)k_begin) * 2;
+  p.b_bytes = (const char*)b.ptr +
+              (BKM ? ((size_t)k_begin * (size_t)b.ld + b_row0) * 2 : (b_row0 * (size_t)b.ld + (size_t)k_begin) * 2);
 }
 
 // Bytes between consecutive k-tiles of the B operand.

@@ -1053,21 +1053,20 @@ struct Carver {
 
 inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
-// Largest T, H, V or leading dimension any entry point accepts (the 4 GiB limit per matrix is far tighter in practice);
-// the workspace queries answer 0 beyond it instead of computing with sizes that no call would accept.
+// Largest T, H or V any entry point accepts (row pitches are limited to kMaxRowPitch, far below it); the workspace queries
+// answer 0 beyond it instead of computing with sizes that no call would accept.
 constexpr int64_t kMaxExtent = (int64_t)1 << 30;
 
 // The two bf16 operands of every entry point: hidden rows [T, H] and weight rows [V, H].
-// hidden_in_blocks: the entry point walks the hidden rows in token blocks (each below 4 GiB), so only a block counts.
+// Matrices may be of any size: the copy plan addresses a tile with 32-bit offsets from the tile's own first row, so only
+// the row pitch is limited (256 rows must span less than 4 GiB: kMaxRowPitch elements).
 int check_operands(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, int64_t T, int64_t H, int64_t V,
                    float rcp_temperature, bool hidden_in_blocks = false) {
   if (!hidden || !weight) return SKYRL_LMHEAD_ERR_NULL;
   if (T < 1 || V < 1 || H < BK || H % BK != 0 || ldh < H || ldw < H) return SKYRL_LMHEAD_ERR_SHAPE;
-  if (T > kMaxExtent || V > kMaxExtent || ldh > kMaxExtent || ldw > kMaxExtent) return SKYRL_LMHEAD_ERR_SHAPE;
-  // The copy plan addresses an operand with 32-bit byte offsets: each operand (and each backward scratch matrix, which is
-  // never larger than these two transposed) must stay below 4 GiB.
-  const int64_t kMaxBytes = (int64_t)1 << 32;
-  if ((hidden_in_blocks ? BN : T) * ldh * 2 >= kMaxBytes || V * ldw * 2 >= kMaxBytes) return SKYRL_LMHEAD_ERR_SHAPE;
+  if (T > kMaxExtent || V > kMaxExtent) return SKYRL_LMHEAD_ERR_SHAPE;
+  (void)hidden_in_blocks;
+  if (ldh > kMaxRowPitch || ldw > kMaxRowPitch) return SKYRL_LMHEAD_ERR_SHAPE;
   if (!aligned16(hidden) || !aligned16(weight) || ldh % 8 != 0 || ldw % 8 != 0) return SKYRL_LMHEAD_ERR_ALIGN;
   if (!(rcp_temperature > 0.f) || !isfinite(rcp_temperature)) return SKYRL_LMHEAD_ERR_ARG;
   return SKYRL_LMHEAD_OK;
@@ -1168,11 +1167,10 @@ size_t fwd_partials_bytes(int64_t tokens, int64_t V) {
 // for any block size.
 constexpr int64_t kFwdTokenBlock = 32768;
 
-// Tokens per block such that a block of hidden rows stays below the 4 GiB the copy plan can address.
+// Tokens per block: what the caller's scratch allows, at least one 256-token tile.
 int64_t fwd_block_tokens(int64_t wanted, int64_t ld_hidden) {
-  const int64_t by_bytes = (((int64_t)1 << 32) - 1) / (ld_hidden * 2) / BN * BN;
-  int64_t b = wanted < by_bytes ? wanted : by_bytes;
-  return b < BN ? BN : b;
+  (void)ld_hidden;
+  return wanted < BN ? BN : wanted;
 }
 
 int fwd_token_blocks(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight, const int64_t* labels,
@@ -1365,9 +1363,8 @@ int check_softce(const void* student, int64_t lds_, const void* teacher, int64_t
   if (!teacher) return SKYRL_LMHEAD_ERR_NULL;
   int st = check_operands(student, lds_, weight, ldw, T, H, V, rcp_temperature);
   if (st) return st;
-  if (ldt < H || ldt > (int64_t)1 << 30 || T * ldt * 2 >= ((int64_t)1 << 32)) return SKYRL_LMHEAD_ERR_SHAPE;
+  if (ldt < H || ldt > kMaxRowPitch) return SKYRL_LMHEAD_ERR_SHAPE;
   if (seq_len < 1 || T % seq_len != 0 || shift < 0) return SKYRL_LMHEAD_ERR_SHAPE;
-  if (2 * round_up(T, kPairTile) * H * 2 >= ((int64_t)1 << 32)) return SKYRL_LMHEAD_ERR_SHAPE;  // the stacked rows
   if (!aligned16(teacher) || ldt % 8 != 0) return SKYRL_LMHEAD_ERR_ALIGN;
   return SKYRL_LMHEAD_OK;
 }
@@ -1509,9 +1506,8 @@ int bwd_entry(const void* hidden, int64_t ld_hidden, const void* weight, int64_t
   const int64_t Tb = bwd_block_tokens(T), Tbpad = round_up(Tb, 256), Vpad = round_up(V, 256);
   int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(Tb, H, V);
   if (vc > Vpad) vc = Vpad;
-  // 32-bit byte offsets inside a block of hidden rows and inside the scratch matrices (weight^T, hidden^T, the dz panel)
-  if (Tb * ld_hidden * 2 >= ((int64_t)1 << 32) || Tb * Hk * 2 >= ((int64_t)1 << 32) || H * (Vpad + kLdPad) * 2 >= ((int64_t)1 << 32) ||
-      H * (Tbpad + kLdPad) * 2 >= ((int64_t)1 << 32) || Tbpad * (vc + kLdPad) * 2 >= ((int64_t)1 << 32))
+  // Row pitches of the scratch matrices (weight^T, hidden^T, the dz panel) under the copy plan's limit; Hk <= ld_hidden is.
+  if ((!reads_weight_in_place(V) && Vpad + kLdPad > kMaxRowPitch) || Tbpad + kLdPad > kMaxRowPitch || vc + kLdPad > kMaxRowPitch)
     return SKYRL_LMHEAD_ERR_SHAPE;
   if (!workspace || workspace_bytes < bwd_workspace_bytes(T, H, V, vc, compact, terms)) return SKYRL_LMHEAD_ERR_WORKSPACE;
   if ((uintptr_t)workspace & 255u) return SKYRL_LMHEAD_ERR_ALIGN;
@@ -1593,7 +1589,7 @@ const char* skyrl_lmhead_strerror(int status) {
     case SKYRL_LMHEAD_OK: return "ok";
     case SKYRL_LMHEAD_ERR_NULL: return "a required pointer is NULL (or only some of seg_row, seg_col, seg_len are given)";
     case SKYRL_LMHEAD_ERR_SHAPE:
-      return "bad shape: need T >= 1, V >= 1, H a positive multiple of 64, leading dimensions >= H, every matrix under 4 GiB; "
+      return "bad shape: need T >= 1, V >= 1, H a positive multiple of 64, leading dimensions >= H and at most 4194304 elements; "
              "packed-sequence calls: counts >= 0, rows == num_seqs with an attention mask";
     case SKYRL_LMHEAD_ERR_ALIGN: return "bad alignment: pointers must be 16-byte aligned, leading dimensions multiples of 8";
     case SKYRL_LMHEAD_ERR_WORKSPACE: return "workspace is NULL or too small";
@@ -1776,8 +1772,7 @@ int skyrl_softce_bwd(const void* student_hidden, int64_t ld_student, const void*
   const int64_t Tp = round_up(T, kPairTile), Vpad = round_up(V, 256);
   int64_t vc = vocab_chunk ? vocab_chunk : default_vocab_chunk(T, H, V);
   if (vc > Vpad) vc = Vpad;
-  if (H * (Vpad + kLdPad) * 2 >= ((int64_t)1 << 32) || Tp * (vc + kLdPad) * 2 >= ((int64_t)1 << 32))
-    return SKYRL_LMHEAD_ERR_SHAPE;
+  if ((!reads_weight_in_place(V) && Vpad + kLdPad > kMaxRowPitch) || vc + kLdPad > kMaxRowPitch) return SKYRL_LMHEAD_ERR_SHAPE;
   if (!workspace || workspace_bytes < skyrl_softce_bwd_workspace_bytes(T, H, V, vc)) return SKYRL_LMHEAD_ERR_WORKSPACE;
   if ((uintptr_t)workspace & 255u) return SKYRL_LMHEAD_ERR_ALIGN;
 

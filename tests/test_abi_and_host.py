@@ -92,7 +92,8 @@ def test_forward_argument_errors_are_reported_before_any_launch():
     assert _call_fwd(lib, H=100, ldh=104, ldw=104) == -2  # H not a multiple of 64
     assert _call_fwd(lib, T=0) == -2
     assert _call_fwd(lib, ldh=64) == -2  # leading dimension < H
-    assert _call_fwd(lib, V=300000, H=8192, ldh=8192, ldw=8192, wsb=1 << 40) == -2  # weight of 4 GiB or more
+    # matrices of any size are accepted (a tile is addressed from its own first row); only the row pitch is limited
+    assert _call_fwd(lib, ldw=(1 << 22) + 8) == -2 and _call_fwd(lib, ldh=(1 << 22) + 8) == -2
     assert _call_fwd(lib, hidden=0x1008) == -3
     assert _call_fwd(lib, ldw=132) == -3
     assert _call_fwd(lib, ws=None) == -4
@@ -116,7 +117,7 @@ def test_static_scratch_forward_argument_errors():
     assert call(hidden=0x1008) == -3
     assert call(rt=0.0) == -5
     assert call(V=1398017, H=64) == -6  # a 256-token tile of partials no longer fits the 32 MiB array
-    assert call(V=300000, H=8192) == -2  # the weight limit is reported first
+    assert call(V=1398017, H=64, ldw=(1 << 22) + 8) == -2  # the row-pitch limit is reported first
 
 
 def test_split_operand_argument_errors():

@@ -341,6 +341,41 @@ def test_fp32_weight_matches_the_fp32_product(hidden_dtype, with_oov_targets, cu
     assert rel_l2(compact[1], dense[1]) < 1e-5
 
 
+@pytest.mark.parametrize("weight_dtype,V,H", [(torch.float32, 152064, 8192), (torch.bfloat16, 139264, 16384)])
+def test_operands_beyond_four_gib(weight_dtype, V, H, cuda_device):
+    """A weight whose bf16 form exceeds 4 GiB -- the fp32 output layer of a 70B-class model as stacked bf16 terms
+    ([152064, 2 * 8192], 4.98 GB), and a plain bf16 [139264, 16384] (4.56 GB): the copy plan addresses every tile from its own
+    first row, so rows beyond the 4 GiB mark are read and written like any other.  Half of the labels lie beyond it.  Checked
+    on the GPU against the library's fp32 product, log-softmax and autograd (test_fused_linear_logprob.py:71-95)."""
+    dev = cuda_device
+    T = 192
+    gen = torch.Generator(device=dev).manual_seed(11)
+    hidden = torch.randn(T, H, generator=gen, device=dev).to(torch.bfloat16)
+    weight = (torch.randn(V, H, generator=gen, device=dev) * (2.0 / H ** 0.5)).to(weight_dtype)
+    first_high = (1 << 32) // (2 * (2 * H if weight_dtype == torch.float32 else H)) + 1   # first row wholly beyond 4 GiB
+    assert first_high < V - 1000
+    labels = torch.cat([torch.randint(0, V, (T // 2,), generator=gen, device=dev),
+                        torch.randint(first_high, V, (T - T // 2,), generator=gen, device=dev)])
+    g = torch.randn(T, generator=gen, device=dev)
+    h = hidden.clone().requires_grad_(True)
+    w = weight.clone().requires_grad_(True)
+    out = FusedLinearLogprobHip.apply(h.view(1, T, H), w, labels.view(1, T), 0, V, 1024, None, False).view(T)
+    out.backward(g)
+    hr = hidden.float().requires_grad_(True)
+    wr = weight.float().requires_grad_(True)
+    ref = torch.log_softmax(hr @ wr.t(), -1).gather(-1, labels[:, None])[:, 0]
+    (ref * g).sum().backward()
+    assert float((out.detach() - ref.detach()).abs().max()) <= (1e-4 if weight_dtype == torch.float32 else 2e-3)
+    assert w.grad.dtype == weight_dtype and h.grad.dtype == torch.bfloat16
+    for got, want, what in ((h.grad.float(), hr.grad, "grad_hidden"), (w.grad.float(), wr.grad, "grad_weight"),
+                            (w.grad[first_high:].float(), wr.grad[first_high:], "grad_weight beyond 4 GiB")):
+        c = float(torch.nn.functional.cosine_similarity(got.flatten().double(), want.flatten().double(), dim=0))
+        r = float((got.double() - want.double()).norm() / want.double().norm())
+        assert c >= 0.9999 and r < GRAD_REL_L2, (what, c, r)   # dz and grad_hidden are rounded to bf16 once each
+    hot = labels[T // 2:]                                  # label rows beyond the mark carry the one-hot term
+    assert float((w.grad[hot].float() - wr.grad[hot]).abs().max()) <= 2e-2 * float(wr.grad[hot].abs().max())
+
+
 def test_extreme_logits(cuda_device):
     # one dominant logit -> logprob, entropy -> 0; all logits very negative -> the split merge must not underflow
     T, H, V = 40, 64, 700
@@ -1643,6 +1678,7 @@ def _full_size_check(cfg, dev, n_rows=24, n_vocab=12):
     assert (lp <= 0).all() and torch.isfinite(lp).all()
     want_lse = torch.logsumexp(z, -1)
     assert (lse.cpu()[rows].double() - want_lse).abs().max() <= 1e-3
+    _check_every_token_against_the_library(cfg, h, w, y, lp, ent if (cfg.entropy or cfg.entropy_grad) else None, lse)
     if not cfg.backward:
         return
 
@@ -1695,6 +1731,86 @@ def _full_size_check(cfg, dev, n_rows=24, n_vocab=12):
     scale = dw.abs().sum(0).max().item()
     assert col < 2e-3 * scale
     assert torch.isfinite(dh).all() and torch.isfinite(dw).all()
+
+
+def _check_every_token_against_the_library(cfg, h, w, y, lp, ent, lse, slab=512):
+    """Log-sum-exp, log-probability and entropy of ALL tokens against an independent computation on the GPU with library
+    routines only: fp32 ``torch.matmul`` of 512-token slabs with the weight (a [512, V] fp32 slab, never T x V), then
+    ``torch.logsumexp`` / ``gather`` / ``softmax``.  The sampled fp64 rows above pin the library's result; this pins every
+    row of the kernel's -- the expected dW rows below are built from the kernel's own lse of all tokens."""
+    T, V = cfg.T, cfg.V
+    w32 = w.float()
+    rt = 1.0 / cfg.temperature
+    worst_lse = worst_lp = worst_ent = 0.0
+    for t0 in range(0, T, slab):
+        t1 = min(T, t0 + slab)
+        z = torch.matmul(h[t0:t1].float(), w32.t()) * rt
+        ref_lse = torch.logsumexp(z, -1)
+        worst_lse = max(worst_lse, float((lse[t0:t1] - ref_lse).abs().max()))
+        ref_lp = z.gather(-1, y[t0:t1, None])[:, 0] - ref_lse
+        worst_lp = max(worst_lp, float((lp[t0:t1] - ref_lp).abs().max()))
+        if ent is not None:
+            ref_ent = ref_lse - (torch.softmax(z, -1) * z).sum(-1)
+            worst_ent = max(worst_ent, float(((ent[t0:t1] - ref_ent).abs() / ref_ent.abs().clamp(min=1e-3)).max()))
+        del z
+    assert worst_lse <= 1e-3 and worst_lp <= 1e-3 and worst_ent <= 2e-3, (worst_lse, worst_lp, worst_ent)
+
+
+def test_full_size_packed_wrapper_qwen7b(cuda_device):
+    """The 7B configuration as the Megatron worker feeds it: one packed stream of 16384 tokens with the configuration's own
+    ``cu_seqlens`` through ``from_parallel_hidden_to_logprobs_packed_sequences`` and autograd (model_utils.py:773-883).
+    Checked: every landed log-probability against the flat op on the rolled labels (bit-exact: same kernels), padding exactly
+    zero, sampled rows against fp64, and the gradients against the flat backward on the scattered-back upstream gradient."""
+    from skyrl_amd.model_utils import from_parallel_hidden_to_logprobs_packed_sequences
+
+    dev = cuda_device
+    cfg = CONFIGS["qwen2.5-7b-fwdbwd"]
+    d = make_inputs(cfg)
+    T, H, V = cfg.T, cfg.H, cfg.V
+    cu = d["cu_seqlens"]
+    lens = (cu[1:] - cu[:-1]).tolist()
+    n, L = len(lens), max(lens)
+    hidden = d["hidden"].to(dev).requires_grad_(True)
+    weight = d["weight"].to(dev).requires_grad_(True)
+    tokens = d["labels"].to(dev)                     # the packed input ids; the wrapper rolls them per sequence
+    out = from_parallel_hidden_to_logprobs_packed_sequences(hidden.unsqueeze(0), weight, tokens.unsqueeze(0), cu.to(dev), L, 0, V,
+                                                            None, temperature=cfg.temperature, fused_backend="hip")
+    assert out.shape == (n, L - 1) and out.dtype == torch.float32
+    gen = torch.Generator().manual_seed(5)
+    up = torch.randn(n, L - 1, generator=gen)
+    out.backward(up.to(dev))
+
+    # expectation by a per-sequence loop on the host: successor labels, landing positions, upstream gradient per token
+    rolled = torch.empty(T, dtype=torch.int64)
+    g_tok = torch.zeros(T)
+    landed = torch.zeros(n, L - 1, dtype=torch.bool)
+    for i, ln in enumerate(lens):
+        a = int(cu[i])
+        rolled[a:a + ln] = torch.roll(d["labels"][a:a + ln], -1)
+        g_tok[a:a + ln - 1] = up[i, :ln - 1]
+        landed[i, :ln - 1] = True
+    lp_flat, _, lse, _ = ops.lmhead_fwd(hidden.detach(), weight.detach(), rolled.to(dev), 1.0 / cfg.temperature, False)
+    got = out.detach().cpu()
+    assert float(got[~landed].abs().max()) == 0.0
+    for i, ln in enumerate(lens):
+        a = int(cu[i])
+        assert torch.equal(got[i, :ln - 1], lp_flat[a:a + ln - 1].cpu())
+    rows = torch.randperm(T, generator=gen)[:16]
+    z = (d["hidden"][rows].double() @ d["weight"].double().t()) / cfg.temperature
+    want = torch.log_softmax(z, -1).gather(-1, rolled[rows][:, None])[:, 0]
+    assert float((lp_flat.cpu()[rows].double() - want).abs().max()) <= 1e-3
+    dh, dw = ops.lmhead_bwd(hidden.detach(), weight.detach(), rolled.to(dev), lse, None, g_tok.to(dev), None, 1.0 / cfg.temperature, 0)
+    assert hidden.grad.dtype == torch.bfloat16 and weight.grad.dtype == torch.bfloat16
+    last = torch.tensor([int(cu[i + 1]) - 1 for i in range(n)])
+    assert float(hidden.grad[last.to(dev)].abs().max()) == 0.0          # the last token of a sequence predicts nothing
+    assert torch.equal(hidden.grad, dh)                                    # rows dropped or not, same products
+    assert rel_l2(weight.grad.float(), dw) < 5e-3                          # bf16 rounding of the fp32 sums
+    p = torch.softmax(z, -1)
+    gg = g_tok[rows].double()
+    dz = -p * gg[:, None]
+    dz[torch.arange(len(rows)), rolled[rows]] += gg
+    want_dh = (dz / cfg.temperature) @ d["weight"].double()
+    assert cos(hidden.grad.cpu()[rows].double(), want_dh) >= GRAD_COS
 
 
 def test_full_size_forward_qwen05b(cuda_device):
