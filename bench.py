@@ -302,7 +302,7 @@ def main() -> int:
     skip = bool(args.skip_masked_rows and cfg.backward)
     t_active = int(((g != 0) | ((q != 0) if q is not None else False)).sum().item()) if skip else T
 
-    def step():
+    def step(bwd_options: int = 0):
         st = lib.skyrl_lmhead_fwd(hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), labels.data_ptr(),
                                   T, H, V, rcp_t, logprobs.data_ptr(), ptr(entropy), row_lse.data_ptr(), ptr(row_pz),
                                   ws_f.data_ptr(), ws_f.numel(), stream)
@@ -311,7 +311,7 @@ def main() -> int:
             st = bwd_entry(hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0),
                                       labels.data_ptr(), row_lse.data_ptr(), ptr(row_pz) if q is not None else None,
                                       g.data_ptr(), ptr(q), T, H, V, rcp_t, d_hidden.data_ptr(),
-                                      None if args.frozen_lm_head else d_weight.data_ptr(), 0,
+                                      None if args.frozen_lm_head else d_weight.data_ptr(), bwd_options,
                                       args.vocab_chunk, ws_b.data_ptr(), ws_b.numel(), stream)
             _lib.check(st, "skyrl_lmhead_bwd")
 
@@ -437,6 +437,24 @@ def main() -> int:
         power = power_while(step, max(5, args.steps))
         if power:
             out["power"] = power
+        if cfg.backward:
+            # The same K steps with the backward's optional flush of softmax probabilities below 2^-24 (SKYRL_BWD_FLUSH_TINY_DZ,
+            # off in `value`): same products, a dz panel that is mostly zeros, and with it a higher clock under the power limit.
+            for _ in range(2):
+                step(ops.FLUSH_TINY_DZ_BIT)
+            torch.cuda.synchronize()
+            with _lib.KernelProfile() as prof_f:
+                t0 = time.perf_counter()
+                for _ in range(args.steps):
+                    step(ops.FLUSH_TINY_DZ_BIT)
+                torch.cuda.synchronize()
+                ms_f = (time.perf_counter() - t0) * 1e3 / args.steps
+            out["with_tiny_dz_flushed"] = {
+                "option": "SKYRL_BWD_FLUSH_TINY_DZ: p < 2^-24 taken as 0 when dz is formed; not part of `value`",
+                "ms_per_step": ms_f, "tokens_per_s": T * 1e3 / ms_f,
+                "pct_of_bf16_mfma_peak": 100.0 * step_flop / (ms_f * 1e-3) / PEAK_BF16_DENSE_FLOPS,
+                "kernels_ms_per_step": {k: ms / args.steps for k, (ms, n) in prof_f.results.items() if n},
+            }
         if cfg.backward and not skip and not args.frozen_lm_head:
             del d_weight, ws_b  # the autograd call allocates its own
             out["autograd"] = autograd_leg(cfg, hidden, weight, labels, g, q)

@@ -119,6 +119,15 @@ size_t skyrl_lmhead_static_scratch_bytes(void);
 #define SKYRL_DW_FP32 0
 #define SKYRL_DW_FP32_ACCUMULATE 1
 #define SKYRL_DW_BF16 2
+/*
+ * Option bit, OR-ed into dw_mode of any backward entry point (no counterpart in the reference; off unless asked for):
+ * softmax probabilities below 2^-24 -- the unit round-off of the fp32 in which p is formed; 1 - p rounds to 1 for them --
+ * are taken as exactly zero when dz is formed.  Every product of the two gradient GEMMs is still computed; what changes is
+ * the data: on peaked distributions most of the dz panel becomes zeros, and on an MI355X, whose matrix pipe is power-limited
+ * on random operands, the gradient GEMMs then run at a higher clock.  The gradients differ from the exact ones by at most
+ * the flushed probability mass of a row (below V * 2^-24, in practice far less) times |g| / temperature per dz row.
+ */
+#define SKYRL_BWD_FLUSH_TINY_DZ 0x100
 int skyrl_lmhead_bwd(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight,
                      const int64_t* labels, const float* row_lse, const float* row_pz,
                      const float* dlogprobs, const float* dentropy,

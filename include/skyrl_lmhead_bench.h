@@ -25,6 +25,15 @@ extern "C" {
  */
 int skyrl_lmhead_mfma_probe(const void* operands, int workgroups, int iters, float* sink, void* stream);
 
+/*
+ * Measurement aid (no counterpart in the reference): the fp32 atomic adds that a fully fused backward -- the variant
+ * efficient_entropy_backward_kernel_general_mainloop_MN of fused_linear_logprob_triton.py:807-996, which this library does
+ * not build -- would have to issue, and nothing else: one workgroup per 256 x 256 (vocab, token) tile adds 1.0 to its
+ * [256, H] slice of d_weight (fp32 [V, H]) and of d_hidden (fp32 [T, H]); T and V multiples of 256.  Its duration is a lower
+ * bound of that variant's, to set against the split backward's.  Both buffers are overwritten with counts.
+ */
+int skyrl_lmhead_atomic_floor_probe(float* d_weight, float* d_hidden, int64_t T, int64_t H, int64_t V, void* stream);
+
 /* Measurement aid (no counterpart in the reference): compute units and maximum shader clock (kHz) of the current device, the
  * two figures the published matrix peak is made of (compute units x 4096 bf16 flop per clock x clock). */
 int skyrl_lmhead_device_info(int* compute_units, int* max_clock_khz);

@@ -11,7 +11,7 @@ import os
 import threading
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libskyrl_lmhead.so")
-ABI_VERSION = 19
+ABI_VERSION = 20
 
 _c_i64 = ctypes.c_int64
 _c_p = ctypes.c_void_p
@@ -104,6 +104,7 @@ SIGNATURES = {
         [_c_p, ctypes.c_int, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_p, _c_i64, _c_i64, ctypes.c_float, _c_p, _c_i64, _c_p]),
     "skyrl_logprob_diff_metrics": (ctypes.c_int, [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_p]),
     "skyrl_lmhead_mfma_probe": (ctypes.c_int, [_c_p, ctypes.c_int, ctypes.c_int, _c_p, _c_p]),
+    "skyrl_lmhead_atomic_floor_probe": (ctypes.c_int, [_c_p, _c_p, _c_i64, _c_i64, _c_i64, _c_p]),
     "skyrl_lmhead_device_info": (ctypes.c_int, [ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]),
     "skyrl_lmhead_num_kernel_kinds": (ctypes.c_int, []),
     "skyrl_lmhead_kernel_name": (ctypes.c_char_p, [ctypes.c_int]),

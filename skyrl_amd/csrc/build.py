@@ -35,15 +35,17 @@ def lib_path() -> str:
     return os.path.join(HERE, LIB_NAME)
 
 
-def build(verbose: bool = False) -> str:
+def build(verbose: bool = False, extra_flags=(), out: str | None = None) -> str:
+    """Compile the library.  ``extra_flags`` / ``out``: a variant build (the timing-only ablations of
+    ``skyrl_amd/bench_ablations.py``) written somewhere else than the product library."""
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(hipcc):
         raise RuntimeError("hipcc not found: the fused LM-head library can only be built with the ROCm toolchain")
-    out = lib_path()
+    out = out or lib_path()
     # Compile into a temporary name and rename, so a failed build never leaves a half-written library behind.
-    fd, tmp = tempfile.mkstemp(suffix=".so", dir=HERE)
+    fd, tmp = tempfile.mkstemp(suffix=".so", dir=os.path.dirname(out) or ".")
     os.close(fd)
-    cmd = [hipcc, *HIPCC_FLAGS, "-o", tmp, *[os.path.join(HERE, s) for s in SOURCES]]
+    cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, "-o", tmp, *[os.path.join(HERE, s) for s in SOURCES]]
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)

@@ -41,8 +41,12 @@ constexpr float kLn2 = 0.6931471805599453f;
 #define LMHEAD_GROUP_M 4  // measured best of 2, 4, 6, 8, 16, 32 on both passes
 #endif
 constexpr int kGroupM = LMHEAD_GROUP_M;
-#ifndef LMHEAD_DZ_FLUSH_LOG2
-#define LMHEAD_DZ_FLUSH_LOG2 0
+// Timing-only ablations for skyrl_amd/bench_ablations.py (results are wrong with any of them; 0 in the product build):
+//   1  forward tiles skip their statistics epilogue        2  dz tiles skip their epilogue (arithmetic, staging, stores)
+//   4  dz tiles do everything but the global stores        8  forward and dz tiles read the operand panels of one 4 x 8 patch
+//  16  the same for the gradient-GEMM tiles                   of tiles, so that every operand read hits the XCD's L2
+#ifndef LMHEAD_ABLATE
+#define LMHEAD_ABLATE 0
 #endif
 // Scratch matrices get 64 extra elements (128 B) per row: with a power-of-two row pitch (T' = 16384 -> 32 KiB) the 256 rows of
 // an operand tile would all start in the same L2 channel and set.
@@ -132,12 +136,20 @@ __device__ __forceinline__ void fwd_tile(const uint16_t* __restrict__ W, int ldw
   int tm, tn;
   tile_coords(blockIdx.x, tiles_m, tiles_n, kGroupM, tm, tn);
 
+#if LMHEAD_ABLATE & 8
+  Operand a{W, ldw, (tm % 4) * BM, V};
+  Operand b{Hd, ldh, (tn % 8) * BN, T};
+#else
   Operand a{W, ldw, tm * BM, V};
   Operand b{Hd, ldh, tn * BN, T};
+#endif
   acc_t acc;
+  prefetch_first_tiles(a, b, 0, H / BK, lds);  // the first copies travel while the accumulators are cleared
   zero_acc(acc);
-  prefetch_first_tiles(a, b, 0, H / BK, lds);
   mainloop<false, EVEN>(a, b, 0, H / BK, lds, acc);
+#if LMHEAD_ABLATE & 1
+  return;
+#endif
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
@@ -320,6 +332,8 @@ struct DzArgs {
   // of the row is of order p; the caller adds what the bf16 product dropped of it (label_residual_update) so that the label
   // rows of dW keep fp32 accuracy.
   float* label_resid;
+  // 0, or 126 - n: softmax probabilities below 2^-n are treated as zero (SKYRL_BWD_FLUSH_TINY_DZ).
+  float p_shift;
 };
 
 template <bool ENTGRAD, bool EVEN>
@@ -368,25 +382,32 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
     gs_[j] = g * rcp_temp;
     c0_[j] = -(g - q * pz) * rcp_temp;
     c1_[j] = -q * rcp_temp * rcp_temp;
-#if LMHEAD_DZ_FLUSH_LOG2
-    // Probabilities below 2^-LMHEAD_DZ_FLUSH_LOG2 count as zero: the exponent is moved down so that v_exp_f32 -- which
-    // returns 0 where the result would be a denormal, below 2^-126 -- does the flush, and the two coefficients carry
-    // the power of two back (exact).  Not for coefficients so large that the scaled ones could overflow.
-    if (fabsf(c0_[j]) < 0x1p30f && fabsf(c1_[j]) < 0x1p20f) {
-      constexpr float kShift = 126.f - LMHEAD_DZ_FLUSH_LOG2;
-      lse2_[j] += kShift;
-      c0_[j] *= __builtin_exp2f(kShift);
-      c1_[j] *= __builtin_exp2f(kShift);
+    // Optional (DzArgs::p_shift > 0): probabilities below 2^(p_shift - 126) count as zero.  The exponent is moved down by
+    // p_shift so that v_exp_f32 -- which returns 0 where the result would be a denormal, below 2^-126 -- does the flush,
+    // and the two coefficients carry the power of two back (exact).  Not for coefficients so large that the scaled ones
+    // could overflow.
+    if (z.p_shift > 0.f && fabsf(c0_[j]) < 0x1p30f && fabsf(c1_[j]) < 0x1p20f) {
+      const float up = __builtin_amdgcn_exp2f(z.p_shift);
+      lse2_[j] += z.p_shift;
+      c0_[j] *= up;
+      c1_[j] *= up;
     }
-#endif
   }
 
+#if LMHEAD_ABLATE & 8
+  Operand a{W, ldw, vc0 + (tm % 4) * BM, V};
+  Operand b{Hd, ldh, (tn % 8) * BN, T};
+#else
   Operand a{W, ldw, vc0 + tm * BM, V};
   Operand b{Hd, ldh, tn * BN, T};
+#endif
   acc_t acc;
+  prefetch_first_tiles(a, b, 0, H / BK, lds);  // the first copies travel while the accumulators are cleared
   zero_acc(acc);
-  prefetch_first_tiles(a, b, 0, H / BK, lds);
   mainloop<false, EVEN>(a, b, 0, H / BK, lds, acc);
+#if LMHEAD_ABLATE & 2
+  return;
+#endif
 
   // The wave's 128 x 128 dz block leaves through LDS so that the panel is written with 16-byte stores: a lane holds four
   // consecutive vocab rows of one token, an 8-byte piece of a D row.  mainloop() left LDS free and every wave uses a
@@ -408,7 +429,11 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
       const int idx = it * 64 + lane;
       const int n = j * MT + (idx >> 4), c = idx & 15;  // token row, 8-vocab piece
       const u32x4 v = *(const u32x4*)(stage + n * kTokRow + c * 16);
+#if LMHEAD_ABLATE & 4
+      asm volatile("" ::"v"(v));  // staged and read back, not stored
+#else
       __builtin_nontemporal_store(v, (u32x4*)(D + (size_t)(tbase + n) * (size_t)ldd + vloc_base + c * 8));
+#endif
     }
   };
 #pragma unroll
@@ -561,8 +586,8 @@ __global__ __launch_bounds__(NTHREADS) void softce_dz_tiles(const SoftCeDzArgs z
   Operand a{W, z.ldw, vc0 + tm * BM, V};
   Operand b{S, H, tn * BN, 2 * z.Tp};
   acc_t acc;
+  prefetch_first_tiles(a, b, 0, H / BK, lds);  // the first copies travel while the accumulators are cleared
   zero_acc(acc);
-  prefetch_first_tiles(a, b, 0, H / BK, lds);
   mainloop<false, EVEN>(a, b, 0, H / BK, lds, acc);
 
   // Staging as in dz_tile: a private region per wave, 64 token rows of 128 vocab columns, then 16-byte non-temporal stores.
@@ -662,12 +687,17 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, int bid, char* lds)
   if (bid >= tiles_m * tiles_n) return;
   int tm, tn;
   tile_coords(bid, tiles_m, tiles_n, kGroupM, tm, tn);
+#if LMHEAD_ABLATE & 16
+  Operand a{p.A, p.lda, (tm % 4) * BM, p.a_rows};
+  Operand b{p.B, p.ldb, (tn % 8) * BN, p.b_rows};
+#else
   Operand a{p.A, p.lda, tm * BM, p.a_rows};
   Operand b{p.B, p.ldb, tn * BN, p.b_rows};
+#endif
   acc_t acc;
+  if (nk > 0) prefetch_first_tiles<BKM>(a, b, 0, nk, lds);
   zero_acc(acc);
   if (nk > 0) {
-    prefetch_first_tiles<BKM>(a, b, 0, nk, lds);
     mainloop<BKM, true>(a, b, 0, nk, lds, acc);  // nk is even for every gradient GEMM (make_gemm checks)
   }
 
@@ -791,6 +821,32 @@ __global__ __launch_bounds__(NTHREADS) void mfma_probe(const bf16x8* __restrict_
       sum += acc[i][j][0] + acc[i][j][1] + acc[i][j][2] + acc[i][j][3];
     }
   sink[blockIdx.x * NTHREADS + threadIdx.x] = sum;
+}
+
+// Measurement aid: the fp32 atomic traffic of a fully fused backward (efficient_entropy_backward_kernel_general_mainloop_MN,
+// fused_linear_logprob_triton.py:807-996) and nothing else.  Such a kernel forms the dz tile of 256 vocab rows x 256 tokens and
+// has to add its contribution to dW[256, H] and to dHidden[256, H] in memory, because no workgroup can hold a [256, H]
+// accumulator.  One workgroup per (vocab tile, token tile) issues exactly those adds -- in the accumulator layout, a lane's
+// four values contiguous -- with no logits recompute and no MFMA: a lower bound of what the fused variant costs.
+__global__ __launch_bounds__(NTHREADS) void atomic_floor_probe(float* __restrict__ dW, float* __restrict__ dH, int tiles_v, int H) {
+  const int tv = blockIdx.x % tiles_v, tt = blockIdx.x / tiles_v;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N, lrow = lane & 15, kq = lane >> 4;
+  for (int c0 = 0; c0 < H; c0 += BN) {
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      float* dst = half ? dH + (size_t)tt * BM * (size_t)H : dW + (size_t)tv * BM * (size_t)H;
+#pragma unroll 4
+      for (int x = 0; x < TM * TN; ++x) {
+        const int i = x / TN, j = x % TN;
+        const int n = c0 + wn * WN + j * MT + lrow;          // column of the [256, H] slice
+        if (n >= H) continue;
+        const int m = wm * WM + i * MT + kq * 4;             // this lane adds rows m .. m+3
+#pragma unroll
+        for (int r = 0; r < 4; ++r) atomicAdd(dst + (size_t)(m + r) * (size_t)H + n, 1.0f);
+      }
+    }
+  }
 }
 
 // dst[c, r] = src[r, c] for r < R, c < C;  dst[c, r] = 0 for R <= r < Rpad.  bf16 bits, 64 x 64 tiles.
@@ -1424,7 +1480,8 @@ size_t bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t vocab_chunk,
 int bwd_token_block(const uint16_t* Hp, int64_t ld_hidden, const uint16_t* Wp, int64_t ld_weight, const int64_t* labels,
                     const float* row_lse, const float* row_pz, const float* dlogprobs, const float* dentropy, int64_t Tb,
                     const int* T_dev, int64_t H, int64_t Hk, int64_t V, float rcp_temperature, uint16_t* d_hidden, bool want_dw,
-                    const float* dw_in, float* dw_f32, uint16_t* dw_bf16, int64_t vc, const BwdWorkspace& w, hipStream_t s) {
+                    const float* dw_in, float* dw_f32, uint16_t* dw_bf16, int64_t vc, const BwdWorkspace& w, float p_shift,
+                    hipStream_t s) {
   const int64_t Tpad = round_up(Tb, 256), Vpad = round_up(V, 256);
   const bool w_in_place = reads_weight_in_place(V);
   hipError_t e;
@@ -1450,7 +1507,7 @@ int bwd_token_block(const uint16_t* Hp, int64_t ld_hidden, const uint16_t* Wp, i
     // width, and it needs a second panel.
     const int64_t vc0 = ci * vc, vcw = chunk_width(ci);
     const DzArgs z{Wp, (int)ld_weight, Hp, (int)ld_hidden, (int)Tb, (int)Hk, (int)V, rcp_temperature, labels, row_lse, row_pz,
-                   dlogprobs, dentropy, (int)vc0, (int)(vcw / 256), tiles_t, w.D, (int)(vcw + kLdPad), T_dev, resid};
+                   dlogprobs, dentropy, (int)vc0, (int)(vcw / 256), tiles_t, w.D, (int)(vcw + kLdPad), T_dev, resid, p_shift};
     e = launch_bwd_dz(s, dentropy != nullptr, z, (unsigned)(vcw / 256 * tiles_t));
     if (e != hipSuccess) return (int)e;
     // dHidden[t, h] (+)= sum_v D[t, v] . weight^T[h, vc0 + v]        (A = weight^T rows at k offset vc0, B = D rows)
@@ -1493,6 +1550,9 @@ int bwd_entry(const void* hidden, int64_t ld_hidden, const void* weight, int64_t
               int64_t V, float rcp_temperature, void* d_hidden, void* d_weight, int dw_mode, int64_t vocab_chunk,
               void* workspace, size_t workspace_bytes, hipStream_t s, bool compact, int64_t terms = 1) {
   if (terms < 1 || terms > 3 || H < 1 || H > kMaxExtent / 4) return SKYRL_LMHEAD_ERR_ARG;
+  // dw_mode carries one option bit next to the mode: softmax probabilities below 2^-24 count as zero in dz.
+  const float p_shift = (dw_mode & SKYRL_BWD_FLUSH_TINY_DZ) ? 126.f - 24.f : 0.f;
+  if (dw_mode >= 0) dw_mode &= ~SKYRL_BWD_FLUSH_TINY_DZ;
   const int64_t Hk = terms * H;
   int st = check_common(hidden, ld_hidden, weight, ld_weight, labels, T, Hk, V, rcp_temperature, true);
   if (st) return st;
@@ -1560,12 +1620,12 @@ int bwd_entry(const void* hidden, int64_t ld_hidden, const void* weight, int64_t
       st = bwd_token_block(w.hidden_c + (size_t)t0 * (size_t)Hk, Hk, Wp, ld_weight, w.labels_c + t0, w.lse_c + t0,
                            dentropy ? w.pz_c + t0 : nullptr, w.g_c + t0, dentropy ? w.q_c + t0 : nullptr, Tcur,
                            w.counts + 1 + b, H, Hk, V, rcp_temperature, w.d_hidden_c + (size_t)t0 * (size_t)H, d_weight != nullptr,
-                           dw_in, dw_f32, dw_bf16, vc, w, s);
+                           dw_in, dw_f32, dw_bf16, vc, w, p_shift, s);
     } else {
       st = bwd_token_block(Hp + (size_t)t0 * (size_t)ld_hidden, ld_hidden, Wp, ld_weight, labels + t0, row_lse + t0,
                            row_pz ? row_pz + t0 : nullptr, dlogprobs + t0, dentropy ? dentropy + t0 : nullptr, Tcur, nullptr, H,
                            Hk, V, rcp_temperature, (uint16_t*)d_hidden + (size_t)t0 * (size_t)H, d_weight != nullptr, dw_in, dw_f32,
-                           dw_bf16, vc, w, s);
+                           dw_bf16, vc, w, p_shift, s);
     }
     if (st) return st;
   }
@@ -1582,7 +1642,7 @@ int bwd_entry(const void* hidden, int64_t ld_hidden, const void* weight, int64_t
 
 extern "C" {
 
-int skyrl_lmhead_version(void) { return 19; }
+int skyrl_lmhead_version(void) { return 20; }
 
 const char* skyrl_lmhead_strerror(int status) {
   switch (status) {
@@ -1929,6 +1989,16 @@ int skyrl_lmhead_mfma_probe(const void* operands, int workgroups, int iters, flo
   if (!aligned16(operands)) return SKYRL_LMHEAD_ERR_ALIGN;
   hipLaunchKernelGGL(mfma_probe, dim3((unsigned)workgroups), dim3(NTHREADS), 0, (hipStream_t)stream, (const bf16x8*)operands, iters,
                      sink);
+  return (int)hipGetLastError();
+}
+
+int skyrl_lmhead_atomic_floor_probe(float* d_weight, float* d_hidden, int64_t T, int64_t H, int64_t V, void* stream) {
+  if (!d_weight || !d_hidden) return SKYRL_LMHEAD_ERR_NULL;
+  if (T < BN || V < BM || T % BN != 0 || V % BM != 0 || H < 1 || T > kMaxExtent || V > kMaxExtent) return SKYRL_LMHEAD_ERR_SHAPE;
+  const int64_t tiles = (T / BN) * (V / BM);
+  if (tiles > ((int64_t)1 << 30)) return SKYRL_LMHEAD_ERR_SHAPE;
+  hipLaunchKernelGGL(atomic_floor_probe, dim3((unsigned)tiles), dim3(NTHREADS), 0, (hipStream_t)stream, d_weight, d_hidden,
+                     (int)(V / BM), (int)H);
   return (int)hipGetLastError();
 }
 

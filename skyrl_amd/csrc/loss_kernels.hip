@@ -543,6 +543,12 @@ __device__ __forceinline__ float block_max(float v, float* red) {
   return s;
 }
 
+// exp of a log-ratio clamped to +-20 (utils/off_policy_correction_utils.py: _safe_exp_delta).  fmaxf / fminf drop a NaN;
+// torch.clamp passes it on, and so does this: a NaN log-probability must show in the weights, the metrics and the loss.
+__device__ __forceinline__ float safe_exp_delta(float delta) {
+  return delta != delta ? delta : expf(fminf(fmaxf(delta, -20.f), 20.f));
+}
+
 __global__ __launch_bounds__(kRowThreads) void off_policy_rows_kernel(const OffPolicyArgs a) {
   __shared__ float red[kRowThreads / 64];
   const int64_t row0 = (int64_t)blockIdx.x * a.cols;
@@ -551,10 +557,12 @@ __global__ __launch_bounds__(kRowThreads) void off_policy_rows_kernel(const OffP
   float over = 0.f, under = 0.f, pos = 0.f, oob = 0.f, dm2 = 0.f, m2s = 0.f, pos2 = 0.f, capped = 0.f;
   for (int64_t c = threadIdx.x; c < a.cols; c += kRowThreads) {
     const float delta = a.old[row0 + c] - a.rollout[row0 + c];
-    const float r = expf(fminf(fmaxf(delta, -20.f), 20.f));
+    const float r = safe_exp_delta(delta);
     const float m = a.mask ? a.mask[row0 + c] : 1.f;
     const float x = r * m;
-    s_rm += x, s_m += m, s_x += x, s_xx += x * x;
+    // the two sums behind the standard deviation are taken of x - 1 (the variance does not move with the shift): ratios sit
+    // near 1, and sums of x and x^2 themselves would cancel to nothing when the spread is far below the mean
+    s_rm += x, s_m += m, s_x += x - 1.f, s_xx += (x - 1.f) * (x - 1.f);
     mx = fmaxf(mx, x), mn = fminf(mn, x);
     const bool live = m > 0.f;
     if (a.use_outlier_high && live && r > a.outlier_high) over = 1.f;
@@ -570,31 +578,32 @@ __global__ __launch_bounds__(kRowThreads) void off_policy_rows_kernel(const OffP
   }
   s_rm = block_sum(s_rm, red), s_m = block_sum(s_m, red), s_x = block_sum(s_x, red), s_xx = block_sum(s_xx, red);
   mx = block_max(mx, red), mn = -block_max(-mn, red);
+  if (s_x != s_x) mx = mn = s_x;  // a NaN ratio in the row: the extremes are NaN as well (fmaxf had dropped it)
   over = block_max(over, red), under = block_max(under, red);
   pos = block_sum(pos, red), oob = block_sum(oob, red), dm2 = block_sum(dm2, red), m2s = block_sum(m2s, red);
   pos2 = block_sum(pos2, red), capped = block_sum(capped, red);
   const bool valid = !(outlier && (over > 0.f || under > 0.f));
   if (!valid) pos = 0.f, oob = 0.f, dm2 = 0.f, m2s = 0.f, pos2 = 0.f, capped = 0.f;  // the row's mask is gone from step 1 on
-  const float seq_ratio = expf(fminf(fmaxf(dm2, -20.f), 20.f));
+  const float seq_ratio = safe_exp_delta(dm2);
   float tis_row = 1.f, seq_capped = 0.f;
   if (a.tis_type == 2) {
     seq_capped = seq_ratio > a.tis_cap ? 1.f : 0.f;
-    tis_row = fminf(seq_ratio, a.tis_cap);
+    tis_row = seq_ratio != seq_ratio ? seq_ratio : fminf(seq_ratio, a.tis_cap);
   }
   float seq_over = 0.f, seq_under = 0.f;
   if (a.seq_metric) {
-    const float v = a.seq_metric == 1 ? expf(fminf(fmaxf(dm2 / fmaxf(m2s, 1.f), -20.f), 20.f)) : seq_ratio;
+    const float v = a.seq_metric == 1 ? safe_exp_delta(dm2 / fmaxf(m2s, 1.f)) : seq_ratio;
     seq_over = v > a.seq_high ? 1.f : 0.f;
     seq_under = v < a.seq_low ? 1.f : 0.f;
   }
   const bool keep_row = valid && seq_over == 0.f && seq_under == 0.f;
   for (int64_t c = threadIdx.x; c < a.cols; c += kRowThreads) {
     const float delta = a.old[row0 + c] - a.rollout[row0 + c];
-    const float r = expf(fminf(fmaxf(delta, -20.f), 20.f));
+    const float r = safe_exp_delta(delta);
     const float m = a.mask ? a.mask[row0 + c] : 1.f;
     const bool in_bounds = !a.use_token_mask || (r >= a.token_low && r <= a.token_high);
     const float keep = (keep_row && (in_bounds || m == 0.f)) ? 1.f : 0.f;
-    const float tis = a.tis_type == 1 ? fminf(r, a.tis_cap) : tis_row;
+    const float tis = a.tis_type == 1 ? (r != r ? r : fminf(r, a.tis_cap)) : tis_row;  // torch.clamp keeps a NaN
     if (a.keep_out) a.keep_out[row0 + c] = keep;
     if (a.tis_out) a.tis_out[row0 + c] = tis;
     if (a.weight_out) a.weight_out[row0 + c] = tis * keep;
@@ -623,7 +632,8 @@ __global__ __launch_bounds__(64) void off_policy_finish_kernel(const OffPolicyAr
     for (int64_t r = threadIdx.x; r < a.rows; r += 64) {
       const float* st = a.row_stats + r * kOpRowStats;
       for (int k = 0; k < kOpRowStats; ++k) s[k] += (double)st[k];
-      mx = fmax(mx, (double)st[kOpMaxX]), mn = fmin(mn, (double)st[kOpMinX]);
+      const double rx = (double)st[kOpMaxX], rn = (double)st[kOpMinX];
+      mx = (rx != rx || mx != mx) ? NAN : fmax(mx, rx), mn = (rn != rn || mn != mn) ? NAN : fmin(mn, rn);
     }
     for (int k = 0; k < kOpRowStats; ++k) part[threadIdx.x][k] = s[k];
     part_max[threadIdx.x] = mx, part_min[threadIdx.x] = mn;
@@ -635,13 +645,15 @@ __global__ __launch_bounds__(64) void off_policy_finish_kernel(const OffPolicyAr
   double mx = -INFINITY, mn = INFINITY;
   for (int l = 0; l < 64; ++l) {
     for (int k = 0; k < kOpRowStats; ++k) s[k] += part[l][k];
-    mx = fmax(mx, part_max[l]), mn = fmin(mn, part_min[l]);
+    mx = (part_max[l] != part_max[l] || mx != mx) ? NAN : fmax(mx, part_max[l]);
+    mn = (part_min[l] != part_min[l] || mn != mn) ? NAN : fmin(mn, part_min[l]);
   }
   const double n = (double)a.rows * (double)a.cols, rows = (double)a.rows;
   float* o = a.metrics;
   o[0] = (float)(s[kOpSumRatioMask] / fmax(s[kOpSumMask], 1.0));
-  // unbiased, as Tensor.std(): NaN for a single element
-  o[1] = n > 1.0 ? (float)sqrt(fmax((s[kOpSumXX] - s[kOpSumX] * s[kOpSumX] / n) / (n - 1.0), 0.0)) : NAN;
+  // unbiased, as Tensor.std(): NaN for a single element (the two sums are of x - 1, see the row kernel)
+  const double var = (s[kOpSumXX] - s[kOpSumX] * s[kOpSumX] / n) / (n - 1.0);
+  o[1] = (n > 1.0 && var == var) ? (float)sqrt(fmax(var, 0.0)) : NAN;  // fmax would turn a NaN variance into 0
   o[2] = (float)mx, o[3] = (float)mn;
   o[4] = (float)(s[kOpRowInvalid] / rows), o[5] = (float)(s[kOpRowOver] / rows), o[6] = (float)(s[kOpRowUnder] / rows);
   o[7] = (float)(s[kOpMaskedTokens] / fmax(s[kOpValidTokens], 1.0));

@@ -65,8 +65,8 @@ __global__ __launch_bounds__(NTHREADS) void topk_filter_tiles(const FilterArgs a
   Operand oa{a.W, a.ldw, tm * BM, a.vrows};
   Operand ob{a.Hd, a.ldh, tn * BN, a.T};
   acc_t acc;
-  zero_acc(acc);
   prefetch_first_tiles(oa, ob, 0, a.H / BK, lds);
+  zero_acc(acc);
   mainloop<false, EVEN>(oa, ob, 0, a.H / BK, lds, acc);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -268,6 +268,11 @@ __global__ __launch_bounds__(64 * kSelectWaves) void topk_select(int T, int k, k
       for (int o = 0; o < n_have; ++o) rank += list[o] > mine ? 1 : 0;
       final_vals[(size_t)t * (size_t)k + rank] = key_value(mine);
       final_idx[(size_t)t * (size_t)k + rank] = key_column(mine);
+    } else {
+      // Fewer than k comparable logits: the row holds NaNs (a NaN never passes the filter's comparison).  torch.topk ranks
+      // NaN first and the loss built on it is NaN (mtp/soft_ce.py:258-305); the ranks nobody filled say the same.
+      final_vals[(size_t)t * (size_t)k + e] = NAN;
+      final_idx[(size_t)t * (size_t)k + e] = 0;
     }
   }
   if (lane == 0) cnt[t] = 0u;

@@ -28,6 +28,32 @@ _OOV_LABEL_SENTINEL = torch.iinfo(torch.int64).max
 _REDUCTIONS = ("none", "sum", "mean")
 
 
+class EntropyReductionEnum:
+    """Reduction of the log-probability output, as numbers (``fused_linear_logprob_triton.py:146-152``)."""
+
+    _None = 0
+    _Sum = 1
+    _Mean = 2
+
+
+_REDUCTION_NUMBER = {"none": EntropyReductionEnum._None, "sum": EntropyReductionEnum._Sum, "mean": EntropyReductionEnum._Mean}
+
+
+def get_entropy_reduction_enum_number(reduction: str) -> int:
+    """``"none" | "sum" | "mean"`` -> 0 | 1 | 2; anything else is a ``ValueError`` (``fused_linear_logprob_triton.py:155-166``)."""
+    try:
+        return _REDUCTION_NUMBER[reduction]
+    except KeyError:
+        raise ValueError(f"Invalid reduction: {reduction}") from None
+
+
+def get_entropy_reduction_enum(ce_reduction: int) -> int:
+    """The inverse check: 0, 1 or 2 is returned as it is, anything else is a ``ValueError`` (``...triton.py:169-180``)."""
+    if ce_reduction not in _REDUCTION_NUMBER.values():
+        raise ValueError(f"Invalid ce_reduction: {ce_reduction}")
+    return int(ce_reduction)
+
+
 class BackwardEnum:
     """The backward methods verl's kernels offer (``fused_linear_logprob_triton.py:185-195``).  One of them is built here:
     ``_Split_Dlogits_N`` -- d_logits formed one vocabulary chunk at a time and fed to two GEMMs -- which is also the

@@ -265,6 +265,21 @@ def lmhead_bwd_active_rows(
     return lmhead_bwd_hidden(*args), None
 
 
+# SKYRL_BWD_FLUSH_TINY_DZ of include/skyrl_lmhead.h: an option of every backward call made through this module, off by default.
+FLUSH_TINY_DZ_BIT = 0x100
+_flush_tiny_dz = False
+
+
+def set_flush_tiny_dz(enabled: bool) -> bool:
+    """Switch on / off the backward option that takes softmax probabilities below 2^-24 as exactly zero when dz is formed
+    (``SKYRL_BWD_FLUSH_TINY_DZ``; no counterpart in the reference).  Returns the previous setting.  Results stay inside the
+    path's tolerances (the flushed mass of a row is below V * 2^-24); the gradient GEMMs run faster on a power-limited GPU
+    because most of the dz panel becomes zeros.  A process-wide setting: set it once, before training starts."""
+    global _flush_tiny_dz
+    previous, _flush_tiny_dz = _flush_tiny_dz, bool(enabled)
+    return previous
+
+
 def _bwd_into(lib, hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy, rcp_temperature, vocab_chunk, d_hidden,
               d_weight, accumulate_dw: bool, active_rows: bool = False) -> None:
     T, H = hidden.shape
@@ -293,7 +308,8 @@ def _bwd_into(lib, hidden, weight, labels, row_lse, row_pz, dlogprobs, dentropy,
             hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), labels.data_ptr(),
             row_lse.data_ptr(), _ptr(row_pz if dentropy is not None else None), dlogprobs.data_ptr(), _ptr(dentropy),
             T, H, terms, V, float(rcp_temperature), d_hidden.data_ptr(), _ptr(d_weight),
-            2 if (d_weight is not None and d_weight.dtype == torch.bfloat16) else int(bool(accumulate_dw)),
+            (2 if (d_weight is not None and d_weight.dtype == torch.bfloat16) else int(bool(accumulate_dw)))
+            | (FLUSH_TINY_DZ_BIT if _flush_tiny_dz else 0),
             int(vocab_chunk), int(bool(active_rows)), ws.data_ptr(), ws_bytes, stream,
         )
     _lib.check(st, "skyrl_lmhead_bwd_split")

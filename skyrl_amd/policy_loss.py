@@ -254,21 +254,24 @@ _POLICY_LOSS_NAMES = ("regular", "dual_clip", "cross_entropy", "importance_sampl
 
 
 def _elementwise_loss(name: str, log_probs, old_log_probs, advantages, config, loss_mask, rollout_logprobs, loss_weight,
-                      sync_metrics: bool):
+                      sync_metrics: bool, read_clip_ratio: bool = True):
     loss_type, a, b, c, behaviour = _type_parameters(config, name, rollout_logprobs, old_log_probs)
     loss_weight, extra = _with_off_policy_correction(config, old_log_probs, rollout_logprobs, loss_mask, loss_weight, sync_metrics)
     loss, sums = _PolicyLoss.apply(log_probs, behaviour, advantages, loss_mask, loss_weight, a, b, c, loss_type)
+    if not read_clip_ratio:  # a loss whose clip statistic is a constant: no device value, no read-back
+        return loss, dict(extra)
     clip_ratio = sums[1] / sums[2].clamp(min=1.0)
     return loss, {"clip_ratio": clip_ratio.item() if sync_metrics else clip_ratio, **extra}
 
 
 def sapo_policy_loss(log_probs, old_log_probs, advantages, config, loss_mask=None, rollout_logprobs=None, *,
-                     loss_weight=None) -> Tuple[torch.Tensor, Dict[str, Any]]:
+                     loss_weight=None, sync_metrics: bool = True) -> Tuple[torch.Tensor, Dict[str, Any]]:
     """Soft adaptive policy optimisation (reference ``sapo_policy_loss``, ppo_utils.py:590-660): the gate
     ``sigmoid(tau (r - 1)) 4 / tau`` replaces the clipped ratio, ``tau = config.sapo.tau_pos`` where the advantage is
-    positive, ``tau_neg`` elsewhere.  ``clip_ratio`` is 0.0 as in the reference."""
+    positive, ``tau_neg`` elsewhere.  ``clip_ratio`` is 0.0 as in the reference (a constant: nothing is read back for it);
+    ``sync_metrics=False`` leaves the off-policy-correction metrics as 0-dim tensors, so that nothing waits for the device."""
     loss, metrics = _elementwise_loss("sapo", log_probs, old_log_probs, advantages, config, loss_mask, rollout_logprobs, loss_weight,
-                                      True)
+                                      sync_metrics, read_clip_ratio=False)
     metrics["clip_ratio"] = 0.0
     return loss, metrics
 

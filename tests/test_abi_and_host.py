@@ -460,3 +460,17 @@ def test_product_never_touches_the_oracle_or_the_working_folder():
             assert not uses or fn.name == allowed, f"{script}:{fn.name} imports the oracle"
         top_level = [n for n in tree.body if isinstance(n, (ast.Import, ast.ImportFrom))]
         assert not any(isinstance(n, ast.ImportFrom) and n.module == "oracle" for n in top_level)
+
+
+def test_reduction_enum_of_the_verl_interface():
+    """EntropyReductionEnum and its two helpers (fused_linear_logprob_triton.py:146-180): same numbers, same errors."""
+    from skyrl_amd import fused_linear_logprob_hip as F
+
+    assert (F.EntropyReductionEnum._None, F.EntropyReductionEnum._Sum, F.EntropyReductionEnum._Mean) == (0, 1, 2)
+    assert [F.get_entropy_reduction_enum_number(r) for r in ("none", "sum", "mean")] == [0, 1, 2]
+    assert [F.get_entropy_reduction_enum(n) for n in (0, 1, 2)] == [0, 1, 2]
+    for bad in ("NONE", "max", ""):
+        with pytest.raises(ValueError, match="Invalid reduction"):
+            F.get_entropy_reduction_enum_number(bad)
+    with pytest.raises(ValueError, match="Invalid ce_reduction"):
+        F.get_entropy_reduction_enum(3)

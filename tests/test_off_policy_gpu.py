@@ -358,3 +358,38 @@ def test_off_policy_correction_replays_from_a_hip_graph(cuda_device):
         eager = OPC.off_policy_correction_terms(o, r, k, *args)
         torch.cuda.synchronize()
         assert all(torch.equal(a, b) for a, b in zip(captured, eager)), seed
+
+
+def test_nan_log_probabilities_reach_weights_and_metrics(cuda_device):
+    """torch.clamp passes a NaN on, so the reference's ratio of a NaN log-probability is NaN and shows in the importance
+    weight of its token, in the ratio statistics and in the sequence-level decisions of its row
+    (utils/off_policy_correction_utils.py: _safe_exp_delta and its callers).  The kernel's clamp must not swallow it."""
+    cfg = _cfg(tis_ratio_type="token", token_tis_ratio_clip_high=1.5)
+    old, rollout, mask = _batch()
+    old[6, 10] = float("nan")
+    mask[6, 10] = 1.0
+    want_tis, want_metrics, _ = O.off_policy_correction(old.double(), rollout.double(), mask.double(), cfg)
+    tis, metrics, _ = OPC.compute_off_policy_correction(old.to(cuda_device), rollout.to(cuda_device), mask.to(cuda_device), cfg)
+    assert bool(torch.isnan(want_tis[6, 10])) and bool(torch.isnan(tis[6, 10]))
+    clean = torch.ones_like(mask, dtype=torch.bool)
+    clean[6, 10] = False
+    assert torch.allclose(tis.cpu().double()[clean], want_tis[clean], rtol=2e-5)
+    for key in ("is_ratio_mean", "is_ratio_std", "is_ratio_max", "is_ratio_min"):
+        assert want_metrics[key] != want_metrics[key] and metrics[key] != metrics[key], key   # NaN on both sides
+
+
+def test_ratio_spread_far_below_its_mean(cuda_device):
+    """Ratios within 1e-4 of 1: the standard deviation of the ratios is four orders of magnitude below their mean, where sums of x
+    and x^2 in fp32 would cancel to nothing (the kernel sums x - 1 instead)."""
+    cfg = _cfg(tis_ratio_type="token", token_tis_ratio_clip_high=2.0)
+    gen = torch.Generator().manual_seed(9)
+    B, S = 64, 2048
+    rollout = torch.randn(B, S, generator=gen) * 0.7 - 1.5
+    old = rollout + torch.randn(B, S, generator=gen) * 1e-4
+    mask = torch.ones(B, S)
+    _, want, _ = O.off_policy_correction(old.double(), rollout.double(), mask.double(), cfg)
+    _, got, _ = OPC.compute_off_policy_correction(old.to(cuda_device), rollout.to(cuda_device), mask.to(cuda_device), cfg)
+    assert 5e-5 < want["is_ratio_std"] < 2e-4
+    # the inputs are fp32: the log-ratios themselves carry 2e-7 of rounding, 2e-3 of this spread
+    assert got["is_ratio_std"] == pytest.approx(want["is_ratio_std"], rel=1e-2)
+    assert got["is_ratio_mean"] == pytest.approx(want["is_ratio_mean"], rel=1e-6)

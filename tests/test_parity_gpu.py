@@ -376,6 +376,53 @@ def test_operands_beyond_four_gib(weight_dtype, V, H, cuda_device):
     assert float((w.grad[hot].float() - wr.grad[hot]).abs().max()) <= 2e-2 * float(wr.grad[hot].abs().max())
 
 
+@pytest.mark.parametrize("entgrad", [False, True])
+def test_tiny_dz_flush_option(entgrad, cuda_device):
+    """SKYRL_BWD_FLUSH_TINY_DZ (off by default; no counterpart in the reference): softmax probabilities below 2^-24 are taken
+    as zero when dz is formed.  The gradients stay inside the path's tolerances against the fp64 statement and close to the
+    exact path's; a vocabulary row that no token gives a probability of 2^-24 gets an exactly zero weight gradient, and one
+    that some token does keeps that token's term; switched off again, the backward is bit-identical to before."""
+    dev = cuda_device
+    T, H, V, temperature = 300, 128, 5000, 0.5
+    hidden, weight, labels, g, q = _rand(T, H, V, seed=31)
+    if not entgrad:
+        q = None
+    # 200 vocabulary rows that every token finds hopeless: a feature all tokens share, against a large negative weight
+    low = torch.arange(100, 300)
+    hidden[:, 0] = 4.0
+    weight[:, 0] = 0.0
+    weight[low, 0] = -8.0
+    labels[(labels >= 100) & (labels < 300)] = 7
+    ex = O.exact_fwd_bwd(hidden, weight, labels, temperature, g, q)
+    h, w, y = hidden.to(dev), weight.to(dev), labels.to(dev)
+    _, _, lse, pz = ops.lmhead_fwd(h, w, y, 1.0 / temperature, True)
+    args = (h, w, y, lse, pz if entgrad else None, g.to(dev), None if q is None else q.to(dev), 1.0 / temperature, 1024)
+    exact = ops.lmhead_bwd(*args)
+    assert ops.set_flush_tiny_dz(True) is False
+    try:
+        flushed = ops.lmhead_bwd(*args)
+    finally:
+        assert ops.set_flush_tiny_dz(False) is True
+    again = ops.lmhead_bwd(*args)
+    assert torch.equal(again[0], exact[0]) and torch.equal(again[1], exact[1])
+    check_grads(flushed[0].cpu(), flushed[1].cpu(), ex, "tiny dz flushed")
+    assert rel_l2(flushed[0].float(), exact[0].float()) < 1e-3 and rel_l2(flushed[1], exact[1]) < 1e-3
+    # probabilities in fp64: which vocabulary rows are below / above the threshold for every / some token
+    z = (hidden.double() @ weight.double().t()) / temperature
+    p = torch.softmax(z, -1)
+    is_label = torch.zeros(V, dtype=torch.bool)
+    is_label[labels] = True
+    never = (p.max(0).values < 2.0 ** -25) & ~is_label
+    some = (p.max(0).values > 2.0 ** -20) & ~is_label
+    assert int(never.sum()) > 50 and int(some.sum()) > 50, (int(never.sum()), int(some.sum()))
+    assert float(flushed[1][never.to(dev)].abs().max()) == 0.0
+    assert float(exact[1][never.to(dev)].abs().max()) > 0.0
+    kept = flushed[1][some.to(dev)].cpu().double()
+    assert rel_l2(kept, ex["d_weight"][some]) < GRAD_REL_L2
+    share = float((p < 2.0 ** -24).double().mean())
+    assert share > 0.5                                       # most of the panel is zeros on a peaked distribution
+
+
 def test_extreme_logits(cuda_device):
     # one dominant logit -> logprob, entropy -> 0; all logits very negative -> the split merge must not underflow
     T, H, V = 40, 64, 700

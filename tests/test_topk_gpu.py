@@ -347,3 +347,18 @@ def test_topk_draft_loss_replays_from_a_hip_graph(cuda_device):
         torch.cuda.synchronize()
         for a, b in zip(got, want):
             assert torch.equal(a, b)
+
+
+def test_topk_of_a_nan_row_is_nan(cuda_device):
+    """A token whose hidden row holds a NaN has NaN logits everywhere: torch.topk ranks NaN first, and the reference's draft loss
+    on it is NaN (mtp/soft_ce.py:258-305).  No logit of such a row passes the kernel's comparisons; the ranks it cannot fill
+    come back as NaN with column 0, never as uninitialised memory, and the rows around it are untouched."""
+    T, H, V, k = 130, 64, 3000, 16
+    hidden, weight = _operands(T, H, V, seed=3)
+    clean_vals, clean_idx = M.topk_logits_from_hidden(hidden.to(cuda_device), weight.to(cuda_device), k)
+    hidden[77, 5] = float("nan")
+    vals, idx = M.topk_logits_from_hidden(hidden.to(cuda_device), weight.to(cuda_device), k)
+    assert bool(torch.isnan(vals[77]).all()) and bool((idx[77] == 0).all())
+    others = torch.arange(T) != 77
+    assert torch.equal(vals[others.to(cuda_device)], clean_vals[others.to(cuda_device)])
+    assert torch.equal(idx[others.to(cuda_device)], clean_idx[others.to(cuda_device)])
