@@ -157,22 +157,27 @@ __device__ __forceinline__ void fwd_tile(const uint16_t* __restrict__ W, int ldw
   const int vbase = tm * BM + wm * WM;
   const int part = tm * WAVES_M + wm, nparts = tiles_m * WAVES_M;
   const float scale2 = rcp_temp * kLog2e;
+  // Whether the wave's 128 vocab rows all exist (0), partly (1: the last vocab tile) or not at all (2) is the same for the
+  // whole wave: decided once, outside the unrolled loop over the token blocks.
+  const int rows_kind = __builtin_amdgcn_readfirstlane(vbase + WM <= V ? 0 : (vbase < V ? 1 : 2));
+  auto token_blocks = [&](auto kind) {
+    constexpr int KIND = decltype(kind)::value;
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int t = tn * BN + wn * WN + j * MT + lrow;
-    float m = -INFINITY, s = 0.f, e = 0.f;
-    if (vbase + WM <= V) {
-      fwd_tile_stats<ENTROPY, false, PAIRED>(acc, j, vbase, V, scale2, kq, m, s, e);
-    } else if (vbase < V) {
-      fwd_tile_stats<ENTROPY, true, PAIRED>(acc, j, vbase, V, scale2, kq, m, s, e);
+    for (int j = 0; j < TN; ++j) {
+      const int t = tn * BN + wn * WN + j * MT + lrow;
+      float m = -INFINITY, s = 0.f, e = 0.f;
+      if (KIND < 2) fwd_tile_stats<ENTROPY, KIND == 1, PAIRED>(acc, j, vbase, V, scale2, kq, m, s, e);
+      if (kq == 0 && t < T) {
+        const size_t idx = part_index(part, t, nparts);
+        part_max[idx] = m;
+        part_sum[idx] = s;
+        if (ENTROPY) part_pz[idx] = e;
+      }
     }
-    if (kq == 0 && t < T) {
-      const size_t idx = part_index(part, t, nparts);
-      part_max[idx] = m;
-      part_sum[idx] = s;
-      if (ENTROPY) part_pz[idx] = e;
-    }
-  }
+  };
+  if (rows_kind == 0) token_blocks(std::integral_constant<int, 0>{});
+  else if (rows_kind == 1) token_blocks(std::integral_constant<int, 1>{});
+  else token_blocks(std::integral_constant<int, 2>{});
 }
 
 template <bool ENTROPY, bool EVEN>
@@ -436,11 +441,14 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
 #endif
     }
   };
-#pragma unroll
-  for (int j = 0; j < TN; ++j) {
+  // One token block: eight i-steps of four values per lane.  What is the same for the whole wave -- rows past the
+  // vocabulary's end (RAGGED: only the last vocab tile), a label of some token inside the wave's rows (LABEL, decided per
+  // token block by a ballot), the fp32 residual of the label's value (fp32 operands only) -- is decided once outside the
+  // unrolled loops: as tests inside them they cost three branches per i-step, a third of the epilogue's time.
+  auto token_block = [&](int j, auto ragged, auto label) {
+    constexpr bool RAGGED = decltype(ragged)::value, LABEL = decltype(label)::value;
     const float gs = gs_[j], c0 = c0_[j], c1 = c1_[j], lse2 = lse2_[j];
     const int yrel = yrel_[j];
-    const bool any_label = __any(yrel >= 0);  // some token of this column tile has its label inside the wave's rows
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       float d[4];
@@ -451,12 +459,12 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
         d[r] = ENTGRAD ? p * fmaf(c1, x, c0) : p * c0;
       }
       const int vl = i * MT + kq * 4;  // vocab row inside the wave block; this lane holds vl .. vl+3
-      if (any_label) {
+      if (LABEL) {
 #pragma unroll
         for (int r = 0; r < 4; ++r)
           if (yrel == vl + r) d[r] += gs;
       }
-      if (!full) {
+      if (RAGGED) {
 #pragma unroll
         for (int r = 0; r < 4; ++r)
           if (vbase + vl + r >= V) d[r] = 0.f;
@@ -464,13 +472,25 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
       f32x4 v4 = {d[0], d[1], d[2], d[3]};
       const bf16x4 b4 = __builtin_convertvector(v4, bf16x4);
       *(uint2*)(stage + (j * MT + lrow) * kTokRow + vl * 2) = *(const uint2*)&b4;
-      if (any_label && z.label_resid) {
+      if (LABEL && z.label_resid) {
 #pragma unroll
         for (int r = 0; r < 4; ++r)
           if (yrel == vl + r) z.label_resid[tbase + j * MT + lrow] = d[r];
       }
       if (i == TM / 2 - 1 && j > 0) flush_block(j - 1);
     }
+  };
+  std::true_type yes;
+  std::false_type no;
+  if (__builtin_amdgcn_readfirstlane((int)full)) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      if (__any(yrel_[j] >= 0)) token_block(j, no, yes);  // some token of this block has its label inside the wave's rows
+      else token_block(j, no, no);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) token_block(j, yes, yes);
   }
   flush_block(TN - 1);
 }
