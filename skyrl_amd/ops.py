@@ -256,6 +256,12 @@ def lmhead_bwd_active_rows(
     (``skyrl_lmhead_bwd_active_rows``): the host never reads the count, nothing synchronises, shapes are static, and the
     call can sit inside a captured HIP graph.  With ``want_dweight=False`` (the weight takes no gradient) the dW product is
     skipped and ``None`` is returned in its place; ``dweight_dtype`` is fp32 or bf16 (rounded in the GEMM epilogue).
+
+    With every token active the compaction is pure overhead: one scan, one copy of the hidden rows, one scatter of d_hidden.
+    Measured through ``linear_cross_entropy(...).backward()`` at T=16384, H=3584, V=152064 with all tokens active: 48.45 ms
+    against 48.09 ms for the dense C-ABI step (``bench.py``, ``autograd``), custom-op dispatch and the bf16 dW included.
+    ``d_hidden`` is bf16 also for an fp32 ``hidden`` (the adapters cast it back): one rounding of 2^-9 relative, inside the
+    reference's 2e-3 tolerance for grad_hidden, where the reference returns an fp32-accurate tensor.
     """
     if dweight_dtype not in (torch.float32, torch.bfloat16):
         raise TypeError(f"d_weight is fp32 or bf16, not {dweight_dtype}")

@@ -123,3 +123,32 @@ def test_steady_state_loop_is_clean(kernels):
                 assert not bad, f"{name}: steady-state loop has spill / accumulator traffic: {bad[:4]}"
         if any(ln.startswith("global_load_lds") for ln in lines):
             assert matched >= 1, f"{name}: no steady-state loop block recognised"
+
+
+def test_even_kernels_issue_both_k_steps_of_an_accumulator_back_to_back(kernels):
+    """The accumulator-stationary mainloop (gemm_core.hpp: mainloop_pairs) is what the EVEN instantiations and the gradient
+    GEMMs run: in their steady-state loop every MFMA shares its accumulator with the MFMA before or after it.  The k-step
+    mainloop of the other instantiations never repeats an accumulator within a step."""
+    acc = re.compile(r"v_mfma_f32_16x16x32_bf16 (a\[\d+:\d+\])")
+    seen_pairs = seen_ksteps = 0
+    for name, lines in kernels.items():
+        blocks, cur = [], []
+        for ln in lines:
+            if re.match(r"^\.LBB\w+:", ln):
+                blocks.append(cur)
+                cur = []
+            cur.append(ln)
+        blocks.append(cur)
+        for b in blocks:
+            regs = [acc.match(ln).group(1) for ln in b if ln.startswith("v_mfma")]
+            n_copy = sum(ln.startswith("global_load_lds") for ln in b)
+            if not regs or len(regs) % 128 or n_copy * 8 != len(regs):
+                continue  # not a steady-state loop body
+            paired = sum(1 for k in range(0, len(regs) - 1, 2) if regs[k] == regs[k + 1])
+            if len(regs) == 256:      # two k-tiles per body: the pairs loop
+                assert paired == 128, f"{name}: {paired} of 128 accumulator pairs in the steady-state loop"
+                seen_pairs += 1
+            else:                     # one k-tile per body: the k-step loop
+                assert paired == 0, f"{name}: the k-step loop repeats an accumulator"
+                seen_ksteps += 1
+    assert seen_pairs >= 3 and seen_ksteps >= 2, (seen_pairs, seen_ksteps)

@@ -423,6 +423,26 @@ def test_tiny_dz_flush_option(entgrad, cuda_device):
     assert share > 0.5                                       # most of the panel is zeros on a peaked distribution
 
 
+def test_fp32_weight_gradient_spread_run_to_run(cuda_device):
+    """The one place with atomics: on the fp32-weight path the label term of dW is added with fp32 atomic adds (tokens may
+    share a label), so the last bits of those rows depend on the order of the adds.  Many tokens on few labels, several runs:
+    d_hidden is bit-identical, d_weight rows without a label are bit-identical, label rows agree to fp32 rounding."""
+    dev = cuda_device
+    T, H, V = 2048, 128, 1024
+    gen = torch.Generator().manual_seed(3)
+    hidden = torch.randn(T, H, generator=gen).to(torch.bfloat16).to(dev)
+    weight = (torch.randn(V, H, generator=gen) * 3 / H ** 0.5).to(dev)          # fp32
+    labels = torch.randint(0, 16, (T,), generator=gen).to(dev)                   # 128 tokens per label
+    g = torch.randn(T, generator=gen).to(dev)
+    _, _, lse, _ = ops.lmhead_fwd(hidden, weight, labels, 1.0, False)
+    runs = [ops.lmhead_bwd(hidden, weight, labels, lse, None, g, None, 1.0, 0) for _ in range(4)]
+    for dh, dw in runs[1:]:
+        assert torch.equal(dh, runs[0][0])
+        assert torch.equal(dw[16:], runs[0][1][16:])
+        spread = float((dw[:16] - runs[0][1][:16]).abs().max())
+        assert spread <= 1e-5 * float(runs[0][1][:16].abs().max()), spread
+
+
 def test_extreme_logits(cuda_device):
     # one dominant logit -> logprob, entropy -> 0; all logits very negative -> the split merge must not underflow
     T, H, V = 40, 64, 700
