@@ -215,8 +215,10 @@ __device__ __forceinline__ void merge_partial(float& M, float& S, float& E, floa
   const float Mn = fmaxf(M, m);
   const float da = M - Mn, db = m - Mn;
   const float ca = expf(da), cb = expf(db);
-  E = RELATIVE ? ca * fmaf(da, S, E) + cb * fmaf(db, s, e) : E * ca + e * cb;
-  S = S * ca + s * cb;
+  // Explicit fused multiply-adds: which of the two products of a * b + c * d the compiler would contract is its choice, and it
+  // need not make the same one in every build.
+  E = RELATIVE ? fmaf(ca, fmaf(da, S, E), cb * fmaf(db, s, e)) : fmaf(E, ca, e * cb);
+  S = fmaf(S, ca, s * cb);
   M = Mn;
 }
 
