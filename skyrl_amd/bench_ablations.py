@@ -9,8 +9,9 @@ without the piece.  The forward and the dz launches of a variant are always fed 
 so that the data every other kernel sees stay what they are in the product.  Variants alternate inside every round (same
 box, same thermal state).  Around the table the script also prints what else is needed to judge it: the board power while
 the product steps run against the board's cap, the matrix pipe's own rate on random and on zero operands, the vendor
-library's GEMM on the same operands, the product step with the backward's tiny-probability flush, and the duration of the
-fp32 atomic adds alone that a fully fused backward would issue.
+library's GEMM on the same operands, the product step with the backward's tiny-probability flush, the board power by kind of
+work (idle, matrix pipe alone, HBM copy alone, forward launches, backward launches), and the duration of the fp32 atomic adds
+alone that a fully fused backward would issue.
 """
 
 from __future__ import annotations
@@ -173,6 +174,27 @@ def main() -> int:
     extra["power_product_steps"] = bench_py.power_while(product_step, 10)
     extra["power_flushed_steps"] = bench_py.power_while(lambda: (fwd(base, (lp, ent, lse, pz)), bwd(base, ops.FLUSH_TINY_DZ_BIT)), 10)
     extra["mfma_probe"] = bench_py.mfma_probe(base, dev)
+
+    # Board power by kind of work: which launches sit at the board's cap, and what the matrix pipe alone, HBM alone draw.
+    def watts(fn, n):
+        p = bench_py.power_while(fn, n)
+        return None if p is None else round(p["avg_watts"], 1)
+
+    by_work = {"idle": watts(lambda: time.sleep(0.05), 10)}
+    sink = torch.empty(256 * 256, **f32)
+    for name, operands in (("mfma_only_zero_operands", torch.zeros(65536)), ("mfma_only_random_operands", torch.randn(65536))):
+        o = operands.to(torch.bfloat16).to(dev)
+        by_work[name] = watts(lambda: _lib.check(base.skyrl_lmhead_mfma_probe(o.data_ptr(), 256, 20000, sink.data_ptr(), stream), "probe"), 12)
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    by_work["hbm_copy"] = watts(lambda: dst.copy_(src), 400)
+    del src, dst
+    by_work["forward_launches"] = watts(lambda: fwd(base, (lp, ent, lse, pz)), 30)
+    by_work["backward_launches"] = watts(lambda: bwd(base), 10)
+    by_work["backward_launches_l2_only_gemm"] = watts(lambda: bwd(libs["l2_only_gemm"]), 10)
+    fwd(base, (lp, ent, lse, pz))
+    bwd(base)
+    extra["avg_watts_by_kind_of_work"] = by_work
     extra["vendor_gemm"] = bench_py.vendor_gemm(h, w)
     # the atomic traffic of a fully fused backward, alone
     dh32 = torch.zeros(T, H, **f32)
