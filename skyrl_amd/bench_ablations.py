@@ -27,6 +27,7 @@ from . import _lib
 from .csrc import build as B
 
 VARIANT_DIR = os.path.join(B.HERE, "ablations")
+_ALL = ("lmhead_fwd_tiles", "lmhead_bwd_dz", "lmhead_bwd_gemm")
 VARIANTS = [
     # name, LMHEAD_ABLATE, the kernels whose time the variant changes, what is left out
     ("product", 0, (), "nothing"),
@@ -35,6 +36,11 @@ VARIANTS = [
     ("dz_no_stores", 4, ("lmhead_bwd_dz",), "the global stores of the dz panel (arithmetic and staging stay)"),
     ("l2_only_fwd_dz", 8, ("lmhead_fwd_tiles", "lmhead_bwd_dz"), "operand traffic beyond L2: every tile reads one 4 x 8 patch of tiles"),
     ("l2_only_gemm", 16, ("lmhead_bwd_gemm",), "the same for the gradient-GEMM tiles"),
+    # what the mainloop's energy goes into (the launches are power-limited: time is energy)
+    ("no_epilogues", 1 | 2, ("lmhead_fwd_tiles", "lmhead_bwd_dz"), "both epilogues: the three mainloops alone"),
+    ("mainloops_no_lds_reads", 1 | 2 | 32, _ALL, "epilogues, and every fragment read from LDS inside the k loop"),
+    ("mainloops_no_copies", 1 | 2 | 64, _ALL, "epilogues, and every global -> LDS copy behind the first two k-tiles"),
+    ("mainloops_mfma_only", 1 | 2 | 32 | 64, _ALL, "epilogues, fragment reads and copies: the MFMAs of the k loop alone"),
 ]
 
 

@@ -41,6 +41,13 @@
 
 #include <type_traits>
 
+// Timing-only ablations (skyrl_amd/bench_ablations.py): 32 = mainloop_pairs() without its fragment reads from LDS (the MFMAs
+// run on the fragments read before the loop), 64 = without its global -> LDS copies behind the first two k-tiles.  Results
+// are wrong with either; 0 in the product.
+#ifndef LMHEAD_ABLATE
+#define LMHEAD_ABLATE 0
+#endif
+
 namespace lmhead {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -565,11 +572,11 @@ __device__ __forceinline__ void mainloop_pairs(const Operand& a, const Operand& 
         const int r = quad_row(pr), c = quad_col(pr);
         mfma_16x16x32(acc[pl.a_half * 4 + r][pl.b_half * 4 + c], sa[pl.a_slot][r * 2 + ks], b_frag(pl.b_slot, c * 2 + ks));
         __builtin_amdgcn_sched_barrier(0);
-        if (do_load && pos % 2 == 0 && pos / 2 < nreads) {
+        if (!(LMHEAD_ABLATE & 32) && do_load && pos % 2 == 0 && pos / 2 < nreads) {
           if (pl.ld_is_b) read_b(pl.ld_next ? nxt : cur, pl.ld_half, pl.ld_slot, pos / 2);
           else read_a(pl.ld_next ? nxt : cur, pl.ld_half, pl.ld_slot, pos / 2);
         }
-        if (load2 && pos % 8 == 5) {
+        if (!(LMHEAD_ABLATE & 64) && load2 && pos % 8 == 5) {
           if (q < 2) copy_part(ga, p.a_src, o4, q * 4 + pos / 8, 1);
           else copy_part(gb, p.b_src, o0, (q - 2) * 4 + pos / 8, 1);
         }

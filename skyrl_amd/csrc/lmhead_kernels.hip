@@ -45,6 +45,7 @@ constexpr int kGroupM = LMHEAD_GROUP_M;
 //   1  forward tiles skip their statistics epilogue        2  dz tiles skip their epilogue (arithmetic, staging, stores)
 //   4  dz tiles do everything but the global stores        8  forward and dz tiles read the operand panels of one 4 x 8 patch
 //  16  the same for the gradient-GEMM tiles                   of tiles, so that every operand read hits the XCD's L2
+//  32, 64  in gemm_core.hpp: the mainloop without its LDS fragment reads / without its global -> LDS copies
 #ifndef LMHEAD_ABLATE
 #define LMHEAD_ABLATE 0
 #endif
