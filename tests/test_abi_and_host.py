@@ -474,3 +474,34 @@ def test_reduction_enum_of_the_verl_interface():
             F.get_entropy_reduction_enum_number(bad)
     with pytest.raises(ValueError, match="Invalid ce_reduction"):
         F.get_entropy_reduction_enum(3)
+
+
+def test_ablation_variants_name_bits_the_kernel_sources_test_for():
+    """The timing-only variants of skyrl_amd/bench_ablations.py: unique names, the product first and unmodified, every bit a
+    variant sets is tested for by the kernel sources, and the sources default to no ablation."""
+    import re
+
+    from skyrl_amd import bench_ablations as A
+
+    names = [v[0] for v in A.VARIANTS]
+    assert len(set(names)) == len(names) and A.VARIANTS[0][:2] == ("product", 0)
+    csrc = os.path.join(ROOT, "skyrl_amd", "csrc")
+    sources = _read(os.path.join(csrc, "lmhead_kernels.hip")) + _read(os.path.join(csrc, "gemm_core.hpp"))
+    known = {int(b) for b in re.findall(r"LMHEAD_ABLATE & (\d+)", sources)}
+    assert known == {1, 2, 4, 8, 16, 32, 64}
+    for name, bits, touched, what in A.VARIANTS:
+        assert all(bits & b == 0 or b in known for b in (1 << i for i in range(16))), name
+        assert bits < 2 * max(known) and what
+        assert set(touched) <= {"lmhead_fwd_tiles", "lmhead_bwd_dz", "lmhead_bwd_gemm"}
+        assert A.variant_path(name).startswith(os.path.join(csrc, "ablations"))
+    assert sources.count("#define LMHEAD_ABLATE 0") == 2  # each file's default, under #ifndef
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py --gpus N with N > 1 exits with a message instead of measuring anything."""
+    import subprocess
+    import sys
+
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=300)
+    assert proc.returncode != 0
+    assert "ONE GPU" in (proc.stdout + proc.stderr)
