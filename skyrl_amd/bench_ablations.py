@@ -200,7 +200,7 @@ def main() -> int:
     by_work["backward_launches_l2_only_gemm"] = watts(lambda: bwd(libs["l2_only_gemm"]), 10)
     fwd(base, (lp, ent, lse, pz))
     bwd(base)
-    extra["avg_watts_by_kind_of_work"] = by_work
+    extra["avg_watts_by_workload_kind"] = by_work
     extra["vendor_gemm"] = bench_py.vendor_gemm(h, w)
     # the atomic traffic of a fully fused backward, alone
     dh32 = torch.zeros(T, H, **f32)
