@@ -186,21 +186,21 @@ def main() -> int:
         p = bench_py.power_while(fn, n)
         return None if p is None else round(p["avg_watts"], 1)
 
-    by_work = {"idle": watts(lambda: time.sleep(0.05), 10)}
+    watts_by = {"idle": watts(lambda: time.sleep(0.05), 10)}
     sink = torch.empty(256 * 256, **f32)
     for name, operands in (("mfma_only_zero_operands", torch.zeros(65536)), ("mfma_only_random_operands", torch.randn(65536))):
         o = operands.to(torch.bfloat16).to(dev)
-        by_work[name] = watts(lambda: _lib.check(base.skyrl_lmhead_mfma_probe(o.data_ptr(), 256, 20000, sink.data_ptr(), stream), "probe"), 12)
+        watts_by[name] = watts(lambda: _lib.check(base.skyrl_lmhead_mfma_probe(o.data_ptr(), 256, 20000, sink.data_ptr(), stream), "probe"), 12)
     src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
     dst = torch.empty_like(src)
-    by_work["hbm_copy"] = watts(lambda: dst.copy_(src), 400)
+    watts_by["hbm_copy"] = watts(lambda: dst.copy_(src), 400)
     del src, dst
-    by_work["forward_launches"] = watts(lambda: fwd(base, (lp, ent, lse, pz)), 30)
-    by_work["backward_launches"] = watts(lambda: bwd(base), 10)
-    by_work["backward_launches_l2_only_gemm"] = watts(lambda: bwd(libs["l2_only_gemm"]), 10)
+    watts_by["forward_launches"] = watts(lambda: fwd(base, (lp, ent, lse, pz)), 30)
+    watts_by["backward_launches"] = watts(lambda: bwd(base), 10)
+    watts_by["backward_launches_l2_only_gemm"] = watts(lambda: bwd(libs["l2_only_gemm"]), 10)
     fwd(base, (lp, ent, lse, pz))
     bwd(base)
-    extra["avg_watts_by_workload_kind"] = by_work
+    extra["avg_watts_by_workload_kind"] = watts_by
     extra["vendor_gemm"] = bench_py.vendor_gemm(h, w)
     # the atomic traffic of a fully fused backward, alone
     dh32 = torch.zeros(T, H, **f32)
