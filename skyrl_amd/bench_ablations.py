@@ -200,7 +200,7 @@ def main() -> int:
     watts_by["backward_launches_l2_only_gemm"] = watts(lambda: bwd(libs["l2_only_gemm"]), 10)
     fwd(base, (lp, ent, lse, pz))
     bwd(base)
-    extra["avg_watts_by_workload_kind"] = watts_by
+    extra["avg_watts_by_kind"] = watts_by
     extra["vendor_gemm"] = bench_py.vendor_gemm(h, w)
     # the atomic traffic of a fully fused backward, alone
     dh32 = torch.zeros(T, H, **f32)
