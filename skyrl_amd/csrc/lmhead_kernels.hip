@@ -373,33 +373,22 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
   const bool full = vbase + WM <= V;
   const float scale2 = rcp_temp * kLog2e;
 
-  // Per-token inputs of the epilogue, loaded before the mainloop so that their latency is not paid after it.
-  float gs_[TN], c0_[TN], c1_[TN], lse2_[TN];
-  int yrel_[TN];
+  // Per-token inputs of the epilogue.  The loads are issued here, before the mainloop, and their values are first touched
+  // behind it, so the mainloop hides their latency; they are unconditional loads from a clamped token index (a load under
+  // `t < T` becomes a branch with its own wait: one memory round trip per token block before the first copy is issued).  Lane
+  // l loads tokens l and 64 + l of the wave's 128 -- twelve registers to carry through the mainloop -- and the values reach
+  // the lanes that need them (token j * 16 + lrow for every token block j) through LDS afterwards.
+  float g_[2], q_[2], lse_[2], pz_[2];
+  int64_t y_[2];
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int t = tbase + j * MT + lrow;
-    const bool valid = t < T;
-    const float g = valid ? dlogprobs[t] : 0.f;
-    const float q = (ENTGRAD && valid) ? dentropy[t] : 0.f;
-    lse2_[j] = valid ? row_lse[t] * kLog2e : INFINITY;
-    const float pz = (ENTGRAD && valid) ? row_pz[t] : 0.f;
-    const int64_t y = valid ? labels[t] : (int64_t)-1;
-    const int64_t yrel64 = y - (int64_t)vbase;
-    yrel_[j] = (y >= 0 && y < (int64_t)V && yrel64 >= 0 && yrel64 < WM) ? (int)yrel64 : -1;
-    gs_[j] = g * rcp_temp;
-    c0_[j] = -(g - q * pz) * rcp_temp;
-    c1_[j] = -q * rcp_temp * rcp_temp;
-    // Optional (DzArgs::p_shift > 0): probabilities below 2^(p_shift - 126) count as zero.  The exponent is moved down by
-    // p_shift so that v_exp_f32 -- which returns 0 where the result would be a denormal, below 2^-126 -- does the flush,
-    // and the two coefficients carry the power of two back (exact).  Not for coefficients so large that the scaled ones
-    // could overflow.
-    if (z.p_shift > 0.f && fabsf(c0_[j]) < 0x1p30f && fabsf(c1_[j]) < 0x1p20f) {
-      const float up = __builtin_amdgcn_exp2f(z.p_shift);
-      lse2_[j] += z.p_shift;
-      c0_[j] *= up;
-      c1_[j] *= up;
-    }
+  for (int u = 0; u < 2; ++u) {
+    const int t = tbase + u * 64 + lane;
+    const int tc = t < T ? t : T - 1;  // T >= 1 here: a tile without a token has returned above
+    g_[u] = dlogprobs[tc];
+    q_[u] = ENTGRAD ? dentropy[tc] : 0.f;
+    lse_[u] = row_lse[tc];
+    pz_[u] = ENTGRAD ? row_pz[tc] : 0.f;
+    y_[u] = labels[tc];
   }
 
 #if LMHEAD_ABLATE & 8
@@ -417,14 +406,52 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
   return;
 #endif
 
+  constexpr int kTokRow = WM * 2 + 16;  // dz staging (below): 128 token rows x (128 vocab x 2 B + pad) per wave
+  constexpr int kStage = WN * kTokRow;
+  // The wave's per-token values, through a private 3 KiB of LDS behind the four staging regions (LDS operations of one wave
+  // execute in order, so no barrier).
+  constexpr int kTokBytes = WN * 24;
+  static_assert(NWAVES * (kStage + kTokBytes) <= LDS_BYTES, "dz staging and per-token values do not fit LDS");
+  char* tokv = lds + NWAVES * kStage + wave * kTokBytes;  // float4 {g, q, lse, pz} [128], then int64 label [128]
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const f32x4 v = {g_[u], q_[u], lse_[u], pz_[u]};
+    *(f32x4*)(tokv + (u * 64 + lane) * 16) = v;
+    *(int64_t*)(tokv + WN * 16 + (u * 64 + lane) * 8) = y_[u];
+  }
+  float gs_[TN], c0_[TN], c1_[TN], lse2_[TN];
+  int yrel_[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const bool valid = tbase + j * MT + lrow < T;
+    const f32x4 v = *(const f32x4*)(tokv + (j * MT + lrow) * 16);
+    const float g = valid ? v[0] : 0.f;
+    const float q = (ENTGRAD && valid) ? v[1] : 0.f;
+    lse2_[j] = valid ? v[2] * kLog2e : INFINITY;
+    const float pz = (ENTGRAD && valid) ? v[3] : 0.f;
+    const int64_t y = valid ? *(const int64_t*)(tokv + WN * 16 + (j * MT + lrow) * 8) : (int64_t)-1;
+    const int64_t yrel64 = y - (int64_t)vbase;
+    yrel_[j] = (y >= 0 && y < (int64_t)V && yrel64 >= 0 && yrel64 < WM) ? (int)yrel64 : -1;
+    gs_[j] = g * rcp_temp;
+    c0_[j] = -(g - q * pz) * rcp_temp;
+    c1_[j] = -q * rcp_temp * rcp_temp;
+    // Optional (DzArgs::p_shift > 0): probabilities below 2^(p_shift - 126) count as zero.  The exponent is moved down by
+    // p_shift so that v_exp_f32 -- which returns 0 where the result would be a denormal, below 2^-126 -- does the flush,
+    // and the two coefficients carry the power of two back (exact).  Not for coefficients so large that the scaled ones
+    // could overflow.
+    if (z.p_shift > 0.f && fabsf(c0_[j]) < 0x1p30f && fabsf(c1_[j]) < 0x1p20f) {
+      const float up = __builtin_amdgcn_exp2f(z.p_shift);
+      lse2_[j] += z.p_shift;
+      c0_[j] *= up;
+      c1_[j] *= up;
+    }
+  }
+
   // The wave's 128 x 128 dz block leaves through LDS so that the panel is written with 16-byte stores: a lane holds four
   // consecutive vocab rows of one token, an 8-byte piece of a D row.  mainloop() left LDS free and every wave uses a
   // private region, so no barrier is needed (LDS operations of one wave execute in order).  The stores are marked
   // non-temporal: the panel is a gigabyte that is read back only by the next launch, and letting it displace the operand
   // panels from L2 costs the mainloops of the neighbouring tiles more than the stores themselves.
-  constexpr int kTokRow = WM * 2 + 16;  // staging: 128 token rows x (128 vocab x 2 B + pad)
-  constexpr int kStage = WN * kTokRow;
-  static_assert(NWAVES * kStage <= LDS_BYTES, "dz staging does not fit LDS");
   char* stage = lds + wave * kStage;
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
