@@ -623,14 +623,16 @@ __global__ __launch_bounds__(NTHREADS) void softce_dz_tiles(const SoftCeDzArgs z
   const bool full = vbase + WM <= V;
   const float scale2 = z.rcp_temp * kLog2e;
 
+  // Per-token inputs: unconditional loads from a clamped index, issued before the mainloop and first touched behind it (as
+  // in dz_tile: a load under `t < T` is a branch with its own wait in front of the first copy).
   float gs_[TN / 2], ls2_[TN / 2], lt2_[TN / 2];
 #pragma unroll
   for (int j = 0; j < TN / 2; ++j) {
     const int t = tokbase + j * MT + lrow;
-    const bool valid = t < T;
-    gs_[j] = valid ? z.dloss[t] * z.rcp_temp : 0.f;
-    ls2_[j] = valid ? z.lse_student[t] * kLog2e : INFINITY;
-    lt2_[j] = valid ? z.lse_teacher[t] * kLog2e : INFINITY;
+    const int tc = t < T ? t : T - 1;  // T >= 1: the host launches nothing for an empty batch
+    gs_[j] = z.dloss[tc];
+    ls2_[j] = z.lse_student[tc];
+    lt2_[j] = z.lse_teacher[tc];
   }
 
   Operand a{W, z.ldw, vc0 + tm * BM, V};
@@ -639,6 +641,13 @@ __global__ __launch_bounds__(NTHREADS) void softce_dz_tiles(const SoftCeDzArgs z
   prefetch_first_tiles(a, b, 0, H / BK, lds);  // the first copies travel while the accumulators are cleared
   zero_acc(acc);
   mainloop<false, EVEN>(a, b, 0, H / BK, lds, acc);
+#pragma unroll
+  for (int j = 0; j < TN / 2; ++j) {
+    const bool valid = tokbase + j * MT + lrow < T;
+    gs_[j] = valid ? gs_[j] * z.rcp_temp : 0.f;
+    ls2_[j] = valid ? ls2_[j] * kLog2e : INFINITY;
+    lt2_[j] = valid ? lt2_[j] * kLog2e : INFINITY;
+  }
 
   // Staging as in dz_tile: a private region per wave, 64 token rows of 128 vocab columns, then 16-byte non-temporal stores.
   constexpr int kTokRow = WM * 2 + 16;

@@ -62,6 +62,18 @@ __global__ __launch_bounds__(NTHREADS) void topk_filter_tiles(const FilterArgs a
   int tm, tn;
   tile_coords(blockIdx.x, a.tiles_m, a.tiles_n, a.group_m, tm, tn);
 
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int lrow = lane & 15, kq = lane >> 4;
+  // The tokens' thresholds (fixed for the launch): unconditional loads from a clamped index, issued before the mainloop and
+  // first touched behind it -- a load under `t < T` is a branch with its own wait, eight memory round trips in a row.
+  float th[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int t = tn * BN + wn * WN + j * MT + lrow;
+    th[j] = a.thr[t < a.T ? t : a.T - 1];
+  }
+
   Operand oa{a.W, a.ldw, tm * BM, a.vrows};
   Operand ob{a.Hd, a.ldh, tn * BN, a.T};
   acc_t acc;
@@ -69,17 +81,13 @@ __global__ __launch_bounds__(NTHREADS) void topk_filter_tiles(const FilterArgs a
   zero_acc(acc);
   mainloop<false, EVEN>(oa, ob, 0, a.H / BK, lds, acc);
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-  const int lrow = lane & 15, kq = lane >> 4;
   const int vbase = tm * BM + wm * WM;  // first row of this wave inside the chunk
   if (vbase >= a.vrows) return;
   const float s = a.rcp_temp;
-  float th[TN];
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int t = tn * BN + wn * WN + j * MT + lrow;
-    th[j] = t < a.T ? a.thr[t] : NAN;  // rows past the last token never pass: every comparison with NaN is false
+    if (t >= a.T) th[j] = NAN;  // rows past the last token never pass: every comparison with NaN is false
   }
   // A lane holds 32 logits of each of its eight tokens.  First sweep: how many of them pass (a wave-wide vote on the largest
   // of four skips the blocks in which nothing does -- nearly all of them once a threshold exists; rounding is monotone and

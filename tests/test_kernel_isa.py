@@ -152,3 +152,21 @@ def test_even_kernels_issue_both_k_steps_of_an_accumulator_back_to_back(kernels)
                 assert paired == 0, f"{name}: the k-step loop repeats an accumulator"
                 seen_ksteps += 1
     assert seen_pairs >= 3 and seen_ksteps >= 2, (seen_pairs, seen_ksteps)
+
+
+def test_nothing_waits_on_memory_before_the_first_copy(kernels):
+    """A tile's first global -> LDS copies must leave before anything waits for a vector-memory load: per-token inputs of
+    the epilogues are issued in front of them as unconditional loads and first used behind the mainloop.  (Loaded under a
+    `t < T` condition they become branches with a wait each -- several memory round trips at the head of every tile.)"""
+    checked = 0
+    for name, lines in kernels.items():
+        if not any(k in name for k in ("fwd_tiles", "bwd_dz", "bwd_gemm", "dz_tiles", "filter_tiles")):
+            continue
+        first = next(i for i, ln in enumerate(lines) if ln.startswith("global_load_lds_dwordx4"))
+        head = lines[:first]
+        waits = [ln for ln in head if ln.startswith("s_waitcnt") and "vmcnt" in ln]
+        assert not waits, f"{name}: {waits[:3]} before the first copy"
+        if "bwd_dz" in name or "dz_tiles" in name or "filter_tiles" in name:
+            assert any(ln.startswith("global_load_dword") for ln in head), f"{name}: per-token loads not in front of the copies"
+        checked += 1
+    assert checked >= 8
