@@ -454,21 +454,28 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
   // panels from L2 costs the mainloops of the neighbouring tiles more than the stores themselves.
   char* stage = lds + wave * kStage;
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  // Every staging address is one per-lane base plus a compile-time constant (an immediate of the LDS instruction), and the
+  // panel rows are walked with one running pointer: written as (j * 16 + row) * pitch the compiler keeps eight row indices
+  // alive across the whole epilogue and spills them, and a spill reload waits for vmcnt(0) -- i.e. for every panel store in flight.
+  char* const st_w = stage + lrow * kTokRow + kq * 8;                      // + (j * MT) * kTokRow + i * MT * 2
+  const char* const st_r = stage + (lane >> 4) * kTokRow + (lane & 15) * 16;  // + (j * MT + it * 4) * kTokRow
+  uint16_t* d_row = D + (size_t)(tbase + (lane >> 4)) * (size_t)ldd + vloc_base + (lane & 15) * 8;  // four rows further per store
+  const size_t d_step = (size_t)4 * (size_t)ldd;
 
   // A token block j (16 token rows x 128 vocab, 4 KiB of the staging region) is complete after its eight i-steps; its 256
   // 16-byte pieces (4 per lane; 16 lanes cover one token row of 256 bytes) go out in the middle of block j + 1, so that the
-  // read-back and the store issue hide behind that block's arithmetic instead of forming a tail of their own.
+  // read-back and the store issue hide behind that block's arithmetic instead of forming a tail of their own.  Blocks are
+  // flushed in order, j = 0 .. TN - 1.
   auto flush_block = [&](int j) {
 #pragma unroll
     for (int it = 0; it < 4; ++it) {
-      const int idx = it * 64 + lane;
-      const int n = j * MT + (idx >> 4), c = idx & 15;  // token row, 8-vocab piece
-      const u32x4 v = *(const u32x4*)(stage + n * kTokRow + c * 16);
+      const u32x4 v = *(const u32x4*)(st_r + (j * MT + it * 4) * kTokRow);
 #if LMHEAD_ABLATE & 4
       asm volatile("" ::"v"(v));  // staged and read back, not stored
 #else
-      __builtin_nontemporal_store(v, (u32x4*)(D + (size_t)(tbase + n) * (size_t)ldd + vloc_base + c * 8));
+      __builtin_nontemporal_store(v, (u32x4*)d_row);
 #endif
+      d_row += d_step;
     }
   };
   // One token block: eight i-steps of four values per lane.  What is the same for the whole wave -- rows past the
@@ -501,7 +508,7 @@ __device__ __forceinline__ void dz_tile(const DzArgs& z, int id, char* lds) {
       }
       f32x4 v4 = {d[0], d[1], d[2], d[3]};
       const bf16x4 b4 = __builtin_convertvector(v4, bf16x4);
-      *(uint2*)(stage + (j * MT + lrow) * kTokRow + vl * 2) = *(const uint2*)&b4;
+      *(uint2*)(st_w + (j * MT) * kTokRow + i * (MT * 2)) = *(const uint2*)&b4;
       if (LABEL && z.label_resid) {
 #pragma unroll
         for (int r = 0; r < 4; ++r)
